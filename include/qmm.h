@@ -1,0 +1,128 @@
+/*
+ * qmm.h -- C ABI of libqmm.so: quantized-weight matmul for AMD MI355X (gfx950).
+ *
+ * This is the boundary a host runtime binds to replace MAX's
+ * `max.graph.ops.qmatmul(encoding, config, lhs, *rhs)` and the
+ * `QuantizationEncoding` block parameters.  MAX itself is not part of the
+ * reference snapshot (it is the binary dependency pinned at
+ * magic.lock:135-137), so each entry point cites the in-tree interface whose
+ * conventions it follows:
+ *   - plain C symbols resolved with dlopen/dlsym, POD arguments only
+ *     (stdlib/src/sys/ffi.mojo:118-367, external_call at :471-502,
+ *     C scalar aliases at :29-60);
+ *   - the callee borrows every buffer and never frees or reallocates one
+ *     (stdlib/src/python/_bindings.mojo:222-243,252-260);
+ *   - errors come back as a status plus a message, never as an abort
+ *     (stdlib/src/python/_bindings.mojo:285-291).
+ *
+ * All pointers are device pointers on the current HIP device unless a
+ * parameter is documented as host memory.  Kernels are enqueued on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream) and the calls
+ * return without synchronising.  The library allocates no device memory:
+ * scratch space is passed in as `workspace`.
+ *
+ * Every function returns QMM_OK (0) or a negative qmm_status;
+ * qmm_last_error() then holds a thread-local description.
+ */
+#ifndef QMM_H
+#define QMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* QuantizationEncoding values (GGUF block encodings + GPTQ). */
+enum qmm_encoding {
+    QMM_Q4_0 = 0, /* 32 weights / 18 bytes : f16 d, 16 B nibbles            */
+    QMM_Q4_K = 1, /* 256 weights / 144 bytes: f16 d, dmin, 12 B 6-bit, 128 B */
+    QMM_Q6_K = 2, /* 256 weights / 210 bytes: ql[128] qh[64] i8 sc[16] f16 d */
+    QMM_GPTQ = 3, /* AutoGPTQ v1 tensors: qweight, scales, qzeros[, g_idx]   */
+    QMM_Q8_0 = 8  /* 32 values / 34 bytes  : f16 d, 32 x i8 (activations)    */
+};
+
+enum qmm_dtype { QMM_F32 = 0, QMM_BF16 = 1, QMM_F16 = 2 };
+
+enum qmm_status {
+    QMM_OK = 0,
+    QMM_ERR_INVALID = -1,     /* bad argument: shape, alignment, null, enum */
+    QMM_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for */
+    QMM_ERR_HIP = -3,         /* HIP runtime error at launch                */
+    QMM_ERR_WORKSPACE = -4    /* workspace missing or too small             */
+};
+
+/* QuantizationConfig of the reference API (GPTQ only). */
+typedef struct qmm_gptq_config {
+    int32_t bits;       /* 4                                      */
+    int32_t group_size; /* 128 (any multiple of 32 dividing K)    */
+    int32_t desc_act;   /* 0: g_idx[k] = k / group_size           */
+    int32_t sym;        /* 1: stored zero-point 7 (true zero 8)   */
+} qmm_gptq_config;
+
+int qmm_version(void);
+const char* qmm_last_error(void);
+
+/* QuantizationEncoding.block_parameters: elements and bytes per block. */
+int qmm_block_params(int encoding, int64_t* elements_per_block, int64_t* bytes_per_block);
+
+/* Number of compute units and peak engine clock (kHz) of the current device,
+ * for roofline reports (the role of the reference's
+ * stdlib/src/sys/info.mojo:789-818 core-count queries). */
+int qmm_device_info(int32_t* compute_units, int32_t* clock_khz);
+
+/*
+ * Block unpack / dequantise: rhs uint8[n, k/epb*bpb] -> out[n, k] in
+ * out_dtype (QMM_F32 or QMM_BF16, bf16 by round-to-nearest-even as
+ * stdlib/src/builtin/simd.mojo:3279-3300).  Q4_0, Q4_K, Q6_K.
+ */
+int qmm_dequantize(int encoding, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
+                   void* stream);
+
+/* GPTQ tensors -> out[n, k] (the transposed, GGUF-like orientation). */
+int qmm_dequantize_gptq(const qmm_gptq_config* cfg, const void* qweight, const void* scales,
+                        const void* qzeros, const void* g_idx, int64_t n, int64_t k, void* out,
+                        int out_dtype, void* stream);
+
+/*
+ * Quantisers.  x fp32[rows, k] -> packed blocks uint8[rows, k/epb*bpb].
+ * QMM_Q4_0 and QMM_Q8_0 follow the GGUF reference quantisers; QMM_Q4_K and
+ * QMM_Q6_K use a direct (non-iterative) min/max fit.
+ */
+int qmm_quantize(int encoding, const float* x, int64_t rows, int64_t k, void* out, void* stream);
+
+/* w fp32[n, k] -> AutoGPTQ tensors (symmetric 4-bit, desc_act = 0). */
+int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int64_t k,
+                      void* qweight, void* scales, void* qzeros, void* g_idx, void* stream);
+
+/* Bytes of device scratch qmm_matmul needs for this problem (may be 0). */
+int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
+
+/*
+ * ops.qmatmul: out fp32[m, n] = lhs[m, k] . dequant(rhs)^T.
+ *   encoding Q4_0/Q4_K/Q6_K: n_rhs = 1, rhs[0] = uint8[n, k/epb*bpb];
+ *   encoding GPTQ: cfg required, n_rhs = 3 or 4,
+ *     rhs = {qweight i32[k/8, n], scales f16[k/g, n], qzeros i32[k/g, n/8], g_idx i32[k]}.
+ *   lhs_dtype QMM_F32 or QMM_BF16.  Q4_0 quantises lhs rows to Q8_0 and takes
+ *   integer block dots (the reference CPU path); the others keep lhs as given.
+ *   flags: bit 0 (QMM_FLAG_W_BF16) rounds dequantised weights to bf16 before
+ *   the product in the M > 16 kernels.
+ * rhs is a host array of device pointers.
+ */
+#define QMM_FLAG_W_BF16 1
+int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m,
+               int64_t k, const void* const* rhs, int n_rhs, int64_t n, float* out,
+               void* workspace, int64_t workspace_bytes, int flags, void* stream);
+
+/*
+ * Test hook for the bit-exact integer check: raw int32 block sums
+ * out[m, n, k/32] = sum_32 (q4 - 8) * q8 of Q8_0 lhs blocks (uint8[m, k/32*34])
+ * against Q4_0 rhs blocks.
+ */
+int qmm_block_dots_q4_0(const void* lhs_q8_0, const void* rhs_q4_0, int64_t m, int64_t n,
+                        int64_t k, int32_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QMM_H */

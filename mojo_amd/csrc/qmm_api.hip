@@ -1,0 +1,232 @@
+// C ABI of libqmm.so: argument validation and dispatch by encoding and shape.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "qmm_internal.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_status(hipError_t e, const char* what) {
+    if (e == hipSuccess) return QMM_OK;
+    return fail(QMM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+bool block_params(int enc, int64_t& epb, int64_t& bpb) {
+    switch (enc) {
+        case QMM_Q4_0: epb = 32; bpb = 18; return true;
+        case QMM_Q8_0: epb = 32; bpb = 34; return true;
+        case QMM_Q4_K: epb = 256; bpb = 144; return true;
+        case QMM_Q6_K: epb = 256; bpb = 210; return true;
+        default: return false;
+    }
+}
+
+int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+int check_gptq(const qmm_gptq_config* cfg, int64_t n, int64_t k) {
+    if (!cfg) return fail(QMM_ERR_INVALID, "GPTQ requires a config");
+    if (cfg->bits != 4) return fail(QMM_ERR_UNSUPPORTED, "GPTQ bits=%d: only 4-bit is supported", cfg->bits);
+    if (cfg->desc_act) return fail(QMM_ERR_UNSUPPORTED, "GPTQ desc_act=True is not supported");
+    if (!cfg->sym) return fail(QMM_ERR_UNSUPPORTED, "GPTQ sym=False is not supported");
+    if (cfg->group_size <= 0 || cfg->group_size % 32 || k % cfg->group_size)
+        return fail(QMM_ERR_INVALID, "GPTQ group_size=%d must be a multiple of 32 dividing K=%lld", cfg->group_size,
+                    (long long)k);
+    if (n % 8) return fail(QMM_ERR_INVALID, "GPTQ needs N %% 8 == 0 (N=%lld)", (long long)n);
+    return QMM_OK;
+}
+
+// Workspace layout of the Q4_0 path: int8 codes [m,k], fp32 scales [m,k/32], int32 sums [m,k/32].
+struct Q8Planes {
+    int8_t* codes;
+    float* scale;
+    int32_t* sum;
+    int64_t bytes;
+};
+Q8Planes q8_planes(void* ws, int64_t m, int64_t k) {
+    Q8Planes p;
+    int64_t codes = align_up(m * k, 256), sc = align_up(m * (k / 32) * 4, 256);
+    p.codes = (int8_t*)ws;
+    p.scale = (float*)((char*)ws + codes);
+    p.sum = (int32_t*)((char*)ws + codes + sc);
+    p.bytes = codes + 2 * sc;
+    return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+int qmm_version(void) { return 100; }
+
+const char* qmm_last_error(void) { return g_err; }
+
+int qmm_block_params(int encoding, int64_t* elements_per_block, int64_t* bytes_per_block) {
+    int64_t e, b;
+    if (!elements_per_block || !bytes_per_block) return fail(QMM_ERR_INVALID, "null output pointer");
+    if (!block_params(encoding, e, b)) return fail(QMM_ERR_INVALID, "encoding %d has no block layout", encoding);
+    *elements_per_block = e;
+    *bytes_per_block = b;
+    return QMM_OK;
+}
+
+int qmm_device_info(int32_t* compute_units, int32_t* clock_khz) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e, "hipGetDevice");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return hip_status(e, "hipGetDeviceProperties");
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    return QMM_OK;
+}
+
+int qmm_dequantize(int encoding, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype, void* stream) {
+    int64_t epb, bpb;
+    if (encoding == QMM_Q8_0 || !block_params(encoding, epb, bpb))
+        return fail(QMM_ERR_INVALID, "qmm_dequantize: encoding %d is not a GGUF weight encoding", encoding);
+    if (!rhs || !out) return fail(QMM_ERR_INVALID, "qmm_dequantize: null pointer");
+    if (n <= 0 || k <= 0 || k % epb)
+        return fail(QMM_ERR_INVALID, "qmm_dequantize: N=%lld, K=%lld; K must be a positive multiple of %lld",
+                    (long long)n, (long long)k, (long long)epb);
+    if (out_dtype != QMM_F32 && out_dtype != QMM_BF16)
+        return fail(QMM_ERR_INVALID, "qmm_dequantize: out_dtype must be f32 or bf16");
+    if (encoding == QMM_Q4_K && !aligned(rhs, 16))
+        return fail(QMM_ERR_INVALID, "qmm_dequantize: Q4_K rhs must be 16-byte aligned");
+    return hip_status(qmm::launch_dequant(encoding, rhs, n, k, out, out_dtype, (hipStream_t)stream),
+                      "qmm_dequantize");
+}
+
+int qmm_dequantize_gptq(const qmm_gptq_config* cfg, const void* qweight, const void* scales, const void* qzeros,
+                        const void* g_idx, int64_t n, int64_t k, void* out, int out_dtype, void* stream) {
+    if (!qweight || !scales || !qzeros || !out) return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: null pointer");
+    if (n <= 0 || k <= 0) return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: empty shape");
+    if (int rc = check_gptq(cfg, n, k)) return rc;
+    if (out_dtype != QMM_F32 && out_dtype != QMM_BF16)
+        return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: out_dtype must be f32 or bf16");
+    return hip_status(qmm::launch_dequant_gptq(qweight, scales, qzeros, g_idx, n, k, cfg->group_size, out, out_dtype,
+                                               (hipStream_t)stream),
+                      "qmm_dequantize_gptq");
+}
+
+int qmm_quantize(int encoding, const float* x, int64_t rows, int64_t k, void* out, void* stream) {
+    int64_t epb, bpb;
+    if (!block_params(encoding, epb, bpb)) return fail(QMM_ERR_INVALID, "qmm_quantize: unknown encoding %d", encoding);
+    if (!x || !out) return fail(QMM_ERR_INVALID, "qmm_quantize: null pointer");
+    if (rows <= 0 || k <= 0 || k % epb)
+        return fail(QMM_ERR_INVALID, "qmm_quantize: rows=%lld, K=%lld; K must be a positive multiple of %lld",
+                    (long long)rows, (long long)k, (long long)epb);
+    return hip_status(qmm::launch_quantize(encoding, x, rows, k, out, (hipStream_t)stream), "qmm_quantize");
+}
+
+int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int64_t k, void* qweight, void* scales,
+                      void* qzeros, void* g_idx, void* stream) {
+    if (!w || !qweight || !scales || !qzeros || !g_idx) return fail(QMM_ERR_INVALID, "qmm_quantize_gptq: null pointer");
+    if (n <= 0 || k <= 0) return fail(QMM_ERR_INVALID, "qmm_quantize_gptq: empty shape");
+    if (int rc = check_gptq(cfg, n, k)) return rc;
+    return hip_status(
+        qmm::launch_quantize_gptq(w, n, k, cfg->group_size, qweight, scales, qzeros, g_idx, (hipStream_t)stream),
+        "qmm_quantize_gptq");
+}
+
+int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    (void)lhs_dtype;
+    (void)n;
+    if (m <= 0 || k <= 0) return 0;
+    if (encoding == QMM_Q4_0) return q8_planes(nullptr, m, k).bytes;
+    return 0;
+}
+
+int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
+               const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
+               int flags, void* stream) {
+    (void)flags;
+    hipStream_t s = (hipStream_t)stream;
+    if (!lhs || !rhs || !out) return fail(QMM_ERR_INVALID, "qmm_matmul: null pointer");
+    if (m <= 0 || n <= 0 || k <= 0)
+        return fail(QMM_ERR_INVALID, "qmm_matmul: M=%lld N=%lld K=%lld must all be positive", (long long)m,
+                    (long long)n, (long long)k);
+    if (m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return fail(QMM_ERR_INVALID, "qmm_matmul: dimension too large");
+    if (lhs_dtype != QMM_F32 && lhs_dtype != QMM_BF16)
+        return fail(QMM_ERR_INVALID, "qmm_matmul: lhs dtype must be f32 or bf16");
+    if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul: lhs must be 16-byte aligned");
+    int64_t esz = lhs_dtype == QMM_F32 ? 4 : 2;
+    int64_t need = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(QMM_ERR_WORKSPACE, "qmm_matmul: workspace of %lld bytes required, %lld given", (long long)need,
+                    (long long)workspace_bytes);
+    if (need > 0 && !aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul: workspace must be 256-byte aligned");
+
+    if (encoding == QMM_GPTQ) {
+        if (n_rhs != 3 && n_rhs != 4)
+            return fail(QMM_ERR_INVALID, "qmm_matmul: GPTQ takes rhs = (qweight, scales, qzeros[, g_idx]), got %d", n_rhs);
+        if (int rc = check_gptq(cfg, n, k)) return rc;
+        for (int i = 0; i < 3; i++)
+            if (!rhs[i] || !aligned(rhs[i], 4)) return fail(QMM_ERR_INVALID, "qmm_matmul: GPTQ rhs[%d] null or misaligned", i);
+        for (int64_t m0 = 0; m0 < m; m0 += 16) {
+            int mt = (int)(m - m0 < 16 ? m - m0 : 16);
+            hipError_t e = qmm::launch_gemv_gptq((const char*)lhs + m0 * k * esz, lhs_dtype, (const uint32_t*)rhs[0],
+                                                 (const uint16_t*)rhs[1], (const uint32_t*)rhs[2], mt, n, k,
+                                                 cfg->group_size, out + m0 * n, n, s);
+            if (e != hipSuccess) return hip_status(e, "qmm_matmul(GPTQ)");
+        }
+        return QMM_OK;
+    }
+
+    int64_t epb, bpb;
+    if (encoding == QMM_Q8_0 || !block_params(encoding, epb, bpb))
+        return fail(QMM_ERR_INVALID, "qmm_matmul: unknown encoding %d", encoding);
+    if (n_rhs != 1 || !rhs[0]) return fail(QMM_ERR_INVALID, "qmm_matmul: GGUF encodings take exactly one rhs tensor");
+    if (k % epb)
+        return fail(QMM_ERR_INVALID, "qmm_matmul: K=%lld is not a multiple of the block size %lld", (long long)k,
+                    (long long)epb);
+    const uint8_t* w = (const uint8_t*)rhs[0];
+    if (encoding == QMM_Q4_K && !aligned(w, 16)) return fail(QMM_ERR_INVALID, "qmm_matmul: Q4_K rhs must be 16-byte aligned");
+    if (!aligned(w, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: rhs must be 2-byte aligned");
+
+    if (encoding == QMM_Q4_0) {
+        Q8Planes p = q8_planes(workspace, m, k);
+        hipError_t e = qmm::launch_quantize_q8_0(lhs, lhs_dtype, m, k, nullptr, p.codes, p.scale, p.sum, s);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q8_0 quantise)");
+        for (int64_t m0 = 0; m0 < m; m0 += 16) {
+            int mt = (int)(m - m0 < 16 ? m - m0 : 16);
+            e = qmm::launch_gemv_q4_0(p.codes + m0 * k, p.scale + m0 * (k / 32), p.sum + m0 * (k / 32), w, mt, n, k,
+                                      out + m0 * n, n, s);
+            if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_0)");
+        }
+        return QMM_OK;
+    }
+
+    for (int64_t m0 = 0; m0 < m; m0 += 16) {
+        int mt = (int)(m - m0 < 16 ? m - m0 : 16);
+        const void* a = (const char*)lhs + m0 * k * esz;
+        hipError_t e = encoding == QMM_Q4_K ? qmm::launch_gemv_q4_k(a, lhs_dtype, w, mt, n, k, out + m0 * n, n, s)
+                                            : qmm::launch_gemv_q6_k(a, lhs_dtype, w, mt, n, k, out + m0 * n, n, s);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul");
+    }
+    return QMM_OK;
+}
+
+int qmm_block_dots_q4_0(const void* lhs_q8_0, const void* rhs_q4_0, int64_t m, int64_t n, int64_t k, int32_t* out,
+                        void* stream) {
+    if (!lhs_q8_0 || !rhs_q4_0 || !out) return fail(QMM_ERR_INVALID, "qmm_block_dots_q4_0: null pointer");
+    if (m <= 0 || n <= 0 || k <= 0 || k % 32) return fail(QMM_ERR_INVALID, "qmm_block_dots_q4_0: bad shape");
+    return hip_status(qmm::launch_block_dots_q4_0((const uint8_t*)lhs_q8_0, (const uint8_t*)rhs_q4_0, m, n, k, out,
+                                                  (hipStream_t)stream),
+                      "qmm_block_dots_q4_0");
+}
+
+}  // extern "C"

@@ -1,0 +1,58 @@
+// Device-side helpers shared by every kernel: half conversions, block layouts
+// of the GGUF encodings, nibble / 6-bit field decoding, wave reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qmm {
+
+constexpr int kWave = 64;
+
+constexpr int Q4_0_EPB = 32, Q4_0_BPB = 18;
+constexpr int Q8_0_EPB = 32, Q8_0_BPB = 34;
+constexpr int Q4_K_EPB = 256, Q4_K_BPB = 144;
+constexpr int Q6_K_EPB = 256, Q6_K_BPB = 210;
+
+__device__ __forceinline__ float h2f(uint16_t h) {
+    union { uint16_t u; _Float16 f; } v;
+    v.u = h;
+    return (float)v.f;
+}
+__device__ __forceinline__ uint16_t f2h(float f) {
+    union { uint16_t u; _Float16 h; } v;
+    v.h = (_Float16)f;  // v_cvt_f16_f32: round-to-nearest-even
+    return v.u;
+}
+__device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+// Round-to-nearest-even with canonical NaN, the rule of the reference's
+// software bf16 narrowing (stdlib/src/builtin/simd.mojo:3279-3300).
+__device__ __forceinline__ uint16_t f2bf(float f) {
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)(((x >> 16) & 0x8000u) | 0x7fc0u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return (uint16_t)(x >> 16);
+}
+
+__device__ __forceinline__ uint32_t byte_of(uint32_t w, int i) { return (w >> (8 * i)) & 0xffu; }
+
+// Q4_K: 6-bit scale and min of sub-block j (0..7) from the 12 packed bytes,
+// given as three little-endian dwords s[0..2].
+__device__ __forceinline__ void q4k_scale_min(int j, const uint32_t s[3], uint32_t& sc, uint32_t& mn) {
+    if (j < 4) {
+        sc = byte_of(s[0], j) & 63u;
+        mn = byte_of(s[1], j) & 63u;
+    } else {
+        uint32_t hi = byte_of(s[2], j - 4);
+        sc = (hi & 0xFu) | ((byte_of(s[0], j - 4) >> 6) << 4);
+        mn = (hi >> 4) | ((byte_of(s[1], j - 4) >> 6) << 4);
+    }
+}
+
+// Sum over the 64 lanes of a wavefront; every lane gets the total.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+}  // namespace qmm

@@ -1,0 +1,37 @@
+// Host-side launch functions shared between the kernel translation units and
+// the C ABI in qmm_api.hip.  Each returns the hipError_t of its launch.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qmm.h"
+#include "qmm_device.h"
+
+namespace qmm {
+
+hipError_t launch_dequant(int enc, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
+                          hipStream_t s);
+hipError_t launch_dequant_gptq(const void* qweight, const void* scales, const void* qzeros,
+                               const void* g_idx, int64_t n, int64_t k, int group, void* out,
+                               int out_dtype, hipStream_t s);
+hipError_t launch_quantize(int enc, const float* x, int64_t rows, int64_t k, void* out, hipStream_t s);
+hipError_t launch_quantize_q8_0(const void* x, int x_dtype, int64_t rows, int64_t k, void* blocks,
+                                void* codes, void* dscale, void* csum, hipStream_t s);
+hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group, void* qweight,
+                                void* scales, void* qzeros, void* g_idx, hipStream_t s);
+
+// Decode-shape kernels (m <= 16 rows of lhs per launch).
+hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const int32_t* a_sum,
+                            const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
+                            hipStream_t s);
+hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
+                            float* out, int64_t ldo, hipStream_t s);
+hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
+                            float* out, int64_t ldo, hipStream_t s);
+hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
+                            const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
+                            int64_t ldo, hipStream_t s);
+hipError_t launch_block_dots_q4_0(const uint8_t* a_q8, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                                  int32_t* out, hipStream_t s);
+
+}  // namespace qmm

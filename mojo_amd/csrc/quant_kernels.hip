@@ -1,0 +1,395 @@
+// Block unpack / dequantise kernels and the quantisers (fp32 -> packed blocks).
+//
+// Layouts are the on-disk GGUF ones (ggml-common.h) and AutoGPTQ v1 tensors.
+// The quantisers are written as separate IEEE multiplies, adds and divides
+// (this file is compiled with -ffp-contract=off) so that their packed output is
+// bit-identical to a scalar CPU evaluation of the same formulas.
+#include "qmm_internal.h"
+
+namespace qmm {
+
+// ---------------------------------------------------------------------------
+// dequantise: one thread per output element, coalesced stores
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ float dequant_q4_0_elem(const uint8_t* b, int pos) {
+    float d = h2f((uint16_t)(b[0] | (b[1] << 8)));
+    uint32_t byte = b[2 + (pos & 15)];
+    int q = (pos < 16) ? (int)(byte & 15u) : (int)(byte >> 4);
+    return (float)(q - 8) * d;
+}
+
+__device__ __forceinline__ float dequant_q4_k_elem(const uint8_t* b, int pos) {
+    const uint32_t* w = (const uint32_t*)b;  // blocks are 16-byte aligned
+    uint32_t hdr = w[0];
+    float d = h2f((uint16_t)(hdr & 0xffffu)), dmin = h2f((uint16_t)(hdr >> 16));
+    uint32_t s[3] = {w[1], w[2], w[3]};
+    int j = pos >> 5, c = pos >> 6, l = pos & 31;
+    uint32_t sc, mn;
+    q4k_scale_min(j, s, sc, mn);
+    uint32_t byte = b[16 + 32 * c + l];
+    uint32_t q = (j & 1) ? (byte >> 4) : (byte & 15u);
+    return (d * (float)sc) * (float)q - (dmin * (float)mn);
+}
+
+__device__ __forceinline__ float dequant_q6_k_elem(const uint8_t* b, int pos) {
+    int h = pos >> 7, r = pos & 127, quarter = r >> 5, l = r & 31;
+    const uint8_t* ql = b + 64 * h;
+    const uint8_t* qh = b + 128 + 32 * h;
+    const int8_t* sc = (const int8_t*)(b + 192 + 8 * h);
+    float d = h2f((uint16_t)(b[208] | (b[209] << 8)));
+    uint32_t lb = ql[l + 32 * (quarter & 1)];
+    uint32_t lo = (quarter & 2) ? (lb >> 4) : (lb & 15u);
+    uint32_t hi = ((uint32_t)qh[l] >> (2 * quarter)) & 3u;
+    int q = (int)(lo | (hi << 4)) - 32;
+    return d * (float)sc[(l >> 4) + 2 * quarter] * (float)q;
+}
+
+template <int ENC, typename OutT>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, int64_t total,
+                                                      OutT* __restrict__ out) {
+    constexpr int EPB = ENC == QMM_Q4_0 ? Q4_0_EPB : 256;
+    constexpr int BPB = ENC == QMM_Q4_0 ? Q4_0_BPB : (ENC == QMM_Q4_K ? Q4_K_BPB : Q6_K_BPB);
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
+        int64_t blk = e / EPB;
+        int pos = (int)(e % EPB);
+        const uint8_t* b = w + blk * BPB;
+        float v;
+        if (ENC == QMM_Q4_0) v = dequant_q4_0_elem(b, pos);
+        else if (ENC == QMM_Q4_K) v = dequant_q4_k_elem(b, pos);
+        else v = dequant_q6_k_elem(b, pos);
+        if constexpr (sizeof(OutT) == 4) out[e] = v;
+        else out[e] = f2bf(v);
+    }
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void dequant_gptq_kernel(const uint32_t* __restrict__ qweight,
+                                                           const uint16_t* __restrict__ scales,
+                                                           const uint32_t* __restrict__ qzeros,
+                                                           const int32_t* __restrict__ g_idx, int64_t n,
+                                                           int64_t k, int group, OutT* __restrict__ out) {
+    int64_t total = n * k;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
+        int64_t col = e / k, kk = e % k;
+        int64_t g = g_idx ? g_idx[kk] : kk / group;
+        int q = (int)((qweight[(kk >> 3) * n + col] >> (4 * (kk & 7))) & 0xFu);
+        int z = (int)((qzeros[g * (n >> 3) + (col >> 3)] >> (4 * (col & 7))) & 0xFu) + 1;
+        float v = h2f(scales[g * n + col]) * (float)(q - z);
+        if constexpr (sizeof(OutT) == 4) out[e] = v;
+        else out[e] = f2bf(v);
+    }
+}
+
+static int grid_for(int64_t total, int threads) {
+    int64_t g = (total + threads - 1) / threads;
+    const int64_t cap = 256 * 64;
+    return (int)(g < cap ? (g > 0 ? g : 1) : cap);
+}
+
+hipError_t launch_dequant(int enc, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
+                          hipStream_t s) {
+    int64_t total = n * k;
+    dim3 grid(grid_for(total, 256)), block(256);
+    const uint8_t* w = (const uint8_t*)rhs;
+#define QMM_DQ(E)                                                                              \
+    if (out_dtype == QMM_F32) dequant_kernel<E, float><<<grid, block, 0, s>>>(w, total, (float*)out); \
+    else dequant_kernel<E, uint16_t><<<grid, block, 0, s>>>(w, total, (uint16_t*)out)
+    if (enc == QMM_Q4_0) { QMM_DQ(QMM_Q4_0); }
+    else if (enc == QMM_Q4_K) { QMM_DQ(QMM_Q4_K); }
+    else { QMM_DQ(QMM_Q6_K); }
+#undef QMM_DQ
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant_gptq(const void* qweight, const void* scales, const void* qzeros,
+                               const void* g_idx, int64_t n, int64_t k, int group, void* out,
+                               int out_dtype, hipStream_t s) {
+    dim3 grid(grid_for(n * k, 256)), block(256);
+    if (out_dtype == QMM_F32)
+        dequant_gptq_kernel<float><<<grid, block, 0, s>>>((const uint32_t*)qweight, (const uint16_t*)scales,
+                                                          (const uint32_t*)qzeros, (const int32_t*)g_idx, n, k,
+                                                          group, (float*)out);
+    else
+        dequant_gptq_kernel<uint16_t><<<grid, block, 0, s>>>((const uint32_t*)qweight, (const uint16_t*)scales,
+                                                             (const uint32_t*)qzeros, (const int32_t*)g_idx, n, k,
+                                                             group, (uint16_t*)out);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Q8_0 / Q4_0 quantisers: 32 lanes per block, two blocks per wavefront
+// ---------------------------------------------------------------------------
+
+template <typename InT>
+__device__ __forceinline__ float load_f32(const InT* p, int64_t i) {
+    if constexpr (sizeof(InT) == 4) return p[i];
+    else return bf2f(p[i]);
+}
+
+// Writes GGUF Q8_0 blocks (blocks != null) and/or the planar form the Q4_0
+// matmul kernels read: codes int8[rows, k], scales fp32[rows, k/32] (the fp16
+// block scale widened) and code sums int32[rows, k/32].
+template <typename InT>
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const InT* __restrict__ x, int64_t nblocks,
+                                                            uint8_t* __restrict__ blocks,
+                                                            int8_t* __restrict__ codes,
+                                                            float* __restrict__ dscale,
+                                                            int32_t* __restrict__ csum) {
+    int64_t blk = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    int l = threadIdx.x & 31;
+    if (blk >= nblocks) return;
+    float v = load_f32(x, blk * 32 + l);
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
+    float d = amax / 127.0f;
+    float id = d != 0.0f ? 1.0f / d : 0.0f;
+    int q = (int)roundf(v * id);
+    uint16_t dh = f2h(d);
+    int sum = q;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 32);
+    if (blocks) {
+        uint8_t* ob = blocks + blk * Q8_0_BPB;
+        if (l == 0) {
+            ob[0] = (uint8_t)(dh & 0xff);
+            ob[1] = (uint8_t)(dh >> 8);
+        }
+        ob[2 + l] = (uint8_t)(int8_t)q;
+    }
+    if (codes) {
+        codes[blk * 32 + l] = (int8_t)q;
+        if (l == 0) {
+            dscale[blk] = h2f(dh);
+            csum[blk] = sum;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void quantize_q4_0_kernel(const float* __restrict__ x, int64_t nblocks,
+                                                            uint8_t* __restrict__ out) {
+    int64_t blk = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    int l = threadIdx.x & 31;
+    if (blk >= nblocks) return;
+    float v = x[blk * 32 + l];
+    // signed value of the first element with the largest magnitude
+    float amax = fabsf(v);
+    int idx = l;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+        float oa = __shfl_xor(amax, off, 32);
+        int oi = __shfl_xor(idx, off, 32);
+        if (oa > amax || (oa == amax && oi < idx)) {
+            amax = oa;
+            idx = oi;
+        }
+    }
+    float mx = __shfl(v, idx, 32);
+    if (amax == 0.0f) mx = 0.0f;  // all-zero block keeps max = +0
+    float d = mx / -8.0f;
+    float id = d != 0.0f ? 1.0f / d : 0.0f;
+    float t = v * id;
+    t = t + 8.5f;
+    int q = (int)t;
+    if (q > 15) q = 15;
+    int qhi = __shfl_down(q, 16, 32);
+    uint8_t* ob = out + blk * Q4_0_BPB;
+    if (l == 0) {
+        uint16_t dh = f2h(d);
+        ob[0] = (uint8_t)(dh & 0xff);
+        ob[1] = (uint8_t)(dh >> 8);
+    }
+    if (l < 16) ob[2 + l] = (uint8_t)(q | (qhi << 4));
+}
+
+// ---------------------------------------------------------------------------
+// K-quant packers: direct min/max fit, one thread per 256-weight super-block
+// ---------------------------------------------------------------------------
+
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+__global__ __launch_bounds__(64) void quantize_q4_k_kernel(const float* __restrict__ x, int64_t nblocks,
+                                                           uint8_t* __restrict__ out) {
+    int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (blk >= nblocks) return;
+    const float* xb = x + blk * 256;
+    uint8_t* ob = out + blk * Q4_K_BPB;
+    float scale[8], minv[8];
+    float max_scale = 0.0f, max_min = 0.0f;
+    for (int j = 0; j < 8; j++) {
+        float lo = 0.0f, hi = 0.0f;
+        for (int l = 0; l < 32; l++) {
+            float v = xb[j * 32 + l];
+            if (v < lo) lo = v;
+            if (v > hi) hi = v;
+        }
+        scale[j] = (hi - lo) / 15.0f;
+        minv[j] = -lo;
+        if (scale[j] > max_scale) max_scale = scale[j];
+        if (minv[j] > max_min) max_min = minv[j];
+    }
+    float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    uint32_t sc[8], mn[8];
+    for (int j = 0; j < 8; j++) {
+        sc[j] = (uint32_t)clampi((int)rintf(inv_scale * scale[j]), 0, 63);
+        mn[j] = (uint32_t)clampi((int)rintf(inv_min * minv[j]), 0, 63);
+    }
+    uint16_t dh = f2h(max_scale / 63.0f), mh = f2h(max_min / 63.0f);
+    uint8_t s[12];
+    for (int j = 0; j < 12; j++) s[j] = 0;
+    for (int j = 0; j < 8; j++) {
+        if (j < 4) {
+            s[j] |= (uint8_t)sc[j];
+            s[j + 4] |= (uint8_t)mn[j];
+        } else {
+            s[j + 4] = (uint8_t)((sc[j] & 0xFu) | ((mn[j] & 0xFu) << 4));
+            s[j - 4] |= (uint8_t)((sc[j] >> 4) << 6);
+            s[j] |= (uint8_t)((mn[j] >> 4) << 6);
+        }
+    }
+    ob[0] = (uint8_t)(dh & 0xff);
+    ob[1] = (uint8_t)(dh >> 8);
+    ob[2] = (uint8_t)(mh & 0xff);
+    ob[3] = (uint8_t)(mh >> 8);
+    for (int j = 0; j < 12; j++) ob[4 + j] = s[j];
+    float d = h2f(dh), dmin = h2f(mh);
+    for (int c = 0; c < 4; c++) {
+        float d1 = d * (float)sc[2 * c], m1 = dmin * (float)mn[2 * c];
+        float d2 = d * (float)sc[2 * c + 1], m2 = dmin * (float)mn[2 * c + 1];
+        for (int l = 0; l < 32; l++) {
+            int q1 = 0, q2 = 0;
+            if (d1 != 0.0f) q1 = clampi((int)rintf((xb[64 * c + l] + m1) / d1), 0, 15);
+            if (d2 != 0.0f) q2 = clampi((int)rintf((xb[64 * c + 32 + l] + m2) / d2), 0, 15);
+            ob[16 + 32 * c + l] = (uint8_t)(q1 | (q2 << 4));
+        }
+    }
+}
+
+__global__ __launch_bounds__(64) void quantize_q6_k_kernel(const float* __restrict__ x, int64_t nblocks,
+                                                           uint8_t* __restrict__ out) {
+    int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (blk >= nblocks) return;
+    const float* xb = x + blk * 256;
+    uint8_t* ob = out + blk * Q6_K_BPB;
+    float scale[16];
+    float amax_scale = 0.0f, max_scale = 0.0f;
+    for (int j = 0; j < 16; j++) {
+        float amax = 0.0f, mx = 0.0f;
+        for (int l = 0; l < 16; l++) {
+            float v = xb[j * 16 + l];
+            if (amax < fabsf(v)) {
+                amax = fabsf(v);
+                mx = v;
+            }
+        }
+        scale[j] = mx / -32.0f;
+        if (amax_scale < fabsf(scale[j])) {
+            amax_scale = fabsf(scale[j]);
+            max_scale = scale[j];
+        }
+    }
+    if (amax_scale == 0.0f) {
+        for (int i = 0; i < 128; i++) ob[i] = 0;
+        for (int i = 0; i < 64; i++) ob[128 + i] = 0xAA;
+        for (int i = 192; i < 210; i++) ob[i] = 0;
+        return;
+    }
+    float iscale = -128.0f / max_scale;
+    uint16_t dh = f2h(1.0f / iscale);
+    float d = h2f(dh);
+    ob[208] = (uint8_t)(dh & 0xff);
+    ob[209] = (uint8_t)(dh >> 8);
+    float dl[16];
+    for (int j = 0; j < 16; j++) {
+        int s = clampi((int)rintf(iscale * scale[j]), -128, 127);
+        ob[192 + j] = (uint8_t)(int8_t)s;
+        dl[j] = d * (float)s;
+    }
+    for (int h = 0; h < 2; h++) {
+        const float* xx = xb + 128 * h;
+        for (int l = 0; l < 32; l++) {
+            int q[4];
+            for (int t = 0; t < 4; t++) {
+                float dd = dl[8 * h + (l >> 4) + 2 * t];
+                int v = 0;
+                if (dd != 0.0f) v = clampi((int)rintf(xx[l + 32 * t] / dd), -32, 31);
+                q[t] = v + 32;
+            }
+            ob[64 * h + l] = (uint8_t)((q[0] & 0xF) | ((q[2] & 0xF) << 4));
+            ob[64 * h + l + 32] = (uint8_t)((q[1] & 0xF) | ((q[3] & 0xF) << 4));
+            ob[128 + 32 * h + l] = (uint8_t)((q[0] >> 4) | ((q[1] >> 4) << 2) | ((q[2] >> 4) << 4) | ((q[3] >> 4) << 6));
+        }
+    }
+}
+
+// GPTQ symmetric 4-bit: one thread per (group, output column).
+__global__ __launch_bounds__(256) void quantize_gptq_kernel(const float* __restrict__ w, int64_t n, int64_t k,
+                                                            int group, uint32_t* __restrict__ qweight,
+                                                            uint16_t* __restrict__ scales,
+                                                            uint32_t* __restrict__ qzeros,
+                                                            int32_t* __restrict__ g_idx) {
+    int64_t ng = k / group;
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < k) g_idx[t] = (int32_t)(t / group);
+    if (t < ng * (n >> 3)) qzeros[t] = 0x77777777u;
+    if (t >= ng * n) return;
+    int64_t g = t / n, col = t % n;
+    const float* wc = w + col * k + g * group;
+    float amax = 0.0f;
+    for (int i = 0; i < group; i++) amax = fmaxf(amax, fabsf(wc[i]));
+    float scale = 2.0f * amax / 15.0f;
+    scales[g * n + col] = f2h(scale);
+    for (int i8 = 0; i8 < group / 8; i8++) {
+        uint32_t word = 0;
+        for (int i = 0; i < 8; i++) {
+            int q = 8;
+            if (scale != 0.0f) q = clampi((int)rintf(wc[i8 * 8 + i] / scale) + 8, 0, 15);
+            word |= (uint32_t)q << (4 * i);
+        }
+        qweight[(g * (group / 8) + i8) * n + col] = word;
+    }
+}
+
+hipError_t launch_quantize_q8_0(const void* x, int x_dtype, int64_t rows, int64_t k, void* blocks, void* codes,
+                                void* dscale, void* csum, hipStream_t s) {
+    int64_t nblocks = rows * (k / 32);
+    dim3 block(256), grid((unsigned)((nblocks * 32 + 255) / 256));
+    if (x_dtype == QMM_F32)
+        quantize_q8_0_kernel<float><<<grid, block, 0, s>>>((const float*)x, nblocks, (uint8_t*)blocks,
+                                                           (int8_t*)codes, (float*)dscale, (int32_t*)csum);
+    else
+        quantize_q8_0_kernel<uint16_t><<<grid, block, 0, s>>>((const uint16_t*)x, nblocks, (uint8_t*)blocks,
+                                                              (int8_t*)codes, (float*)dscale, (int32_t*)csum);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize(int enc, const float* x, int64_t rows, int64_t k, void* out, hipStream_t s) {
+    if (enc == QMM_Q8_0) return launch_quantize_q8_0(x, QMM_F32, rows, k, out, nullptr, nullptr, nullptr, s);
+    if (enc == QMM_Q4_0) {
+        int64_t nblocks = rows * (k / 32);
+        quantize_q4_0_kernel<<<dim3((unsigned)((nblocks * 32 + 255) / 256)), dim3(256), 0, s>>>(x, nblocks,
+                                                                                                  (uint8_t*)out);
+    } else {
+        int64_t nblocks = rows * (k / 256);
+        dim3 grid((unsigned)((nblocks + 63) / 64)), block(64);
+        if (enc == QMM_Q4_K) quantize_q4_k_kernel<<<grid, block, 0, s>>>(x, nblocks, (uint8_t*)out);
+        else quantize_q6_k_kernel<<<grid, block, 0, s>>>(x, nblocks, (uint8_t*)out);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group, void* qweight, void* scales,
+                                void* qzeros, void* g_idx, hipStream_t s) {
+    int64_t ng = k / group;
+    int64_t threads = ng * n;
+    if (threads < k) threads = k;
+    quantize_gptq_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s>>>(
+        w, n, k, group, (uint32_t*)qweight, (uint16_t*)scales, (uint32_t*)qzeros, (int32_t*)g_idx);
+    return hipGetLastError();
+}
+
+}  // namespace qmm

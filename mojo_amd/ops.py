@@ -1,0 +1,204 @@
+"""Host side of ``qmatmul``: shape/dtype checks, tensor allocation, C-ABI calls.
+
+PyTorch is used only to allocate device memory and to name the stream; every
+number is produced by the HIP kernels in ``libqmm.so``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from .quantization import QuantizationConfig, QuantizationEncoding
+
+_DTYPES = {torch.float32: _lib.QMM_F32, torch.bfloat16: _lib.QMM_BF16}
+
+
+def _stream(t: torch.Tensor) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {t.device}); there is no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _gptq_cfg(config: Optional[QuantizationConfig]) -> _lib.GptqConfig:
+    if config is None:
+        raise ValueError("GPTQ needs a QuantizationConfig")
+    if config.quant_method != "gptq":
+        raise ValueError(f"unsupported quant_method {config.quant_method!r}")
+    return _lib.GptqConfig(int(config.bits), int(config.group_size), int(bool(config.desc_act)), int(bool(config.sym)))
+
+
+def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], lhs: torch.Tensor,
+            *rhs: torch.Tensor, w_bf16: bool = False) -> torch.Tensor:
+    """``out[..., N] = lhs[..., K] @ dequantize(rhs)^T`` in fp32.
+
+    GGUF encodings take one ``uint8[N, K/epb*bpb]`` tensor of packed blocks (the
+    transposed, quantised weight).  GPTQ takes the AutoGPTQ tensors
+    ``(qweight int32[K/8, N], scales float16[K/g, N], qzeros int32[K/g, N/8][, g_idx int32[K]])``.
+    ``lhs`` is float32 or bfloat16.  Q4_0 quantises ``lhs`` to Q8_0 blocks and
+    takes integer block dots; the other encodings use ``lhs`` as given.
+    """
+    if not isinstance(encoding, QuantizationEncoding):
+        raise TypeError("encoding must be a QuantizationEncoding")
+    _require_gpu(lhs, "lhs")
+    if lhs.dtype not in _DTYPES:
+        raise TypeError(f"lhs must be float32 or bfloat16, got {lhs.dtype}")
+    if lhs.dim() < 1:
+        raise ValueError("lhs must have at least one dimension")
+    k = lhs.shape[-1]
+    lead = lhs.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    lib = _lib.load()
+    if encoding == QuantizationEncoding.GPTQ:
+        if len(rhs) not in (3, 4):
+            raise TypeError(f"GPTQ qmatmul takes (qweight, scales, qzeros[, g_idx]); got {len(rhs)} rhs tensors")
+        qweight, scales, qzeros = rhs[:3]
+        for t, name, dt in ((qweight, "qweight", torch.int32), (scales, "scales", torch.float16),
+                            (qzeros, "qzeros", torch.int32)):
+            _require_gpu(t, name)
+            if t.dtype != dt or t.dim() != 2:
+                raise TypeError(f"{name} must be a rank-2 {dt} tensor")
+        n = qweight.shape[1]
+        cfg = _gptq_cfg(config)
+        g = cfg.group_size
+        if qweight.shape[0] * 8 != k:
+            raise ValueError(f"qweight has K={qweight.shape[0] * 8}, lhs has K={k}")
+        if g <= 0 or k % g or tuple(scales.shape) != (k // g, n) or tuple(qzeros.shape) != (k // g, n // 8):
+            raise ValueError("scales/qzeros shapes do not match (K/group, N) and (K/group, N/8)")
+        if len(rhs) == 4:
+            _require_gpu(rhs[3], "g_idx")
+            if rhs[3].dtype != torch.int32 or tuple(rhs[3].shape) != (k,):
+                raise TypeError("g_idx must be int32[K]")
+        cfg_p = C.byref(cfg)
+    elif encoding.is_gguf:
+        if len(rhs) != 1:
+            raise TypeError(f"{encoding.name} qmatmul takes exactly one rhs tensor; got {len(rhs)}")
+        (w,) = rhs
+        _require_gpu(w, "rhs")
+        if w.dtype != torch.uint8 or w.dim() != 2:
+            raise TypeError("rhs must be a rank-2 uint8 tensor of packed blocks")
+        n = w.shape[0]
+        if w.shape[1] != encoding.packed_row_bytes(k):
+            raise ValueError(
+                f"rhs rows hold {w.shape[1]} bytes; K={k} in {encoding.name} needs {encoding.packed_row_bytes(k)}")
+        cfg_p = None
+    else:
+        raise ValueError(f"{encoding.name} is not a weight encoding of qmatmul")
+    if m == 0 or n == 0:
+        raise ValueError("qmatmul of an empty tensor")
+    out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+    lhs_dt = _DTYPES[lhs.dtype]
+    need = lib.qmm_matmul_workspace_bytes(encoding.code, lhs_dt, m, n, k)
+    ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
+    ptrs = (C.c_void_p * len(rhs))(*[t.data_ptr() for t in rhs])
+    rc = lib.qmm_matmul(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), _ptr(ws),
+                        need, _lib.QMM_FLAG_W_BF16 if w_bf16 else 0, _stream(lhs))
+    _lib.check(rc, "qmatmul")
+    return out.reshape(*lead, n)
+
+
+def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Optional[int] = None,
+               config: Optional[QuantizationConfig] = None, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Unpack ``uint8[N, K/epb*bpb]`` blocks (or GPTQ tensors) to ``dtype[N, K]``."""
+    if dtype not in _DTYPES:
+        raise TypeError("dtype must be float32 or bfloat16")
+    lib = _lib.load()
+    if encoding == QuantizationEncoding.GPTQ:
+        if len(quantized) not in (3, 4):
+            raise TypeError("GPTQ dequantize takes (qweight, scales, qzeros[, g_idx])")
+        for t in quantized:
+            _require_gpu(t, "GPTQ tensor")
+        qweight, scales, qzeros = quantized[:3]
+        g_idx = quantized[3] if len(quantized) == 4 else None
+        cfg = _gptq_cfg(config)
+        kk, n = qweight.shape[0] * 8, qweight.shape[1]
+        out = torch.empty((n, kk), dtype=dtype, device=qweight.device)
+        rc = lib.qmm_dequantize_gptq(C.byref(cfg), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(g_idx), n, kk,
+                                     _ptr(out), _DTYPES[dtype], _stream(qweight))
+        _lib.check(rc, "dequantize")
+        return out
+    if not encoding.is_gguf:
+        raise ValueError(f"{encoding.name} cannot be dequantized here")
+    (w,) = quantized
+    _require_gpu(w, "quantized")
+    if w.dtype != torch.uint8 or w.dim() != 2:
+        raise TypeError("quantized must be a rank-2 uint8 tensor")
+    bp = encoding.block_parameters
+    if w.shape[1] % bp.block_size:
+        raise ValueError(f"row length {w.shape[1]} is not a multiple of the {encoding.name} block size {bp.block_size}")
+    kk = w.shape[1] // bp.block_size * bp.elements_per_block
+    if k is not None and k != kk:
+        raise ValueError(f"K={k} does not match the packed row length (K={kk})")
+    n = w.shape[0]
+    if n == 0 or kk == 0:
+        raise ValueError("dequantize of an empty tensor")
+    out = torch.empty((n, kk), dtype=dtype, device=w.device)
+    rc = lib.qmm_dequantize(encoding.code, _ptr(w), n, kk, _ptr(out), _DTYPES[dtype], _stream(w))
+    _lib.check(rc, "dequantize")
+    return out
+
+
+def quantize(encoding: QuantizationEncoding, x: torch.Tensor) -> torch.Tensor:
+    """fp32 ``[rows, K]`` -> packed ``uint8[rows, K/epb*bpb]`` (Q4_0, Q8_0, Q4_K, Q6_K)."""
+    _require_gpu(x, "x")
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise TypeError("x must be a rank-2 float32 tensor")
+    rows, k = x.shape
+    out = torch.empty((rows, encoding.packed_row_bytes(k)), dtype=torch.uint8, device=x.device)
+    if rows == 0 or k == 0:
+        raise ValueError("quantize of an empty tensor")
+    rc = _lib.load().qmm_quantize(encoding.code, _ptr(x), rows, k, _ptr(out), _stream(x))
+    _lib.check(rc, "quantize")
+    return out
+
+
+def quantize_gptq(w: torch.Tensor, config: QuantizationConfig = QuantizationConfig()) -> Sequence[torch.Tensor]:
+    """fp32 ``[N, K]`` -> ``(qweight, scales, qzeros, g_idx)`` in the AutoGPTQ v1 layout."""
+    _require_gpu(w, "w")
+    if w.dtype != torch.float32 or w.dim() != 2:
+        raise TypeError("w must be a rank-2 float32 tensor")
+    n, k = w.shape
+    cfg = _gptq_cfg(config)
+    g = cfg.group_size
+    if g <= 0 or k % g or k % 8 or n % 8:
+        raise ValueError("GPTQ needs K % group_size == 0 and N % 8 == 0")
+    dev = w.device
+    qweight = torch.empty((k // 8, n), dtype=torch.int32, device=dev)
+    scales = torch.empty((k // g, n), dtype=torch.float16, device=dev)
+    qzeros = torch.empty((k // g, n // 8), dtype=torch.int32, device=dev)
+    g_idx = torch.empty((k,), dtype=torch.int32, device=dev)
+    rc = _lib.load().qmm_quantize_gptq(C.byref(cfg), _ptr(w), n, k, _ptr(qweight), _ptr(scales), _ptr(qzeros),
+                                       _ptr(g_idx), _stream(w))
+    _lib.check(rc, "quantize_gptq")
+    return qweight, scales, qzeros, g_idx
+
+
+def block_dots_q4_0(lhs_q8_0: torch.Tensor, rhs_q4_0: torch.Tensor) -> torch.Tensor:
+    """Raw int32 block sums ``[M, N, K/32]`` of Q8_0 lhs blocks against Q4_0 rhs blocks."""
+    _require_gpu(lhs_q8_0, "lhs_q8_0")
+    _require_gpu(rhs_q4_0, "rhs_q4_0")
+    if lhs_q8_0.dtype != torch.uint8 or rhs_q4_0.dtype != torch.uint8:
+        raise TypeError("both operands must be uint8 block tensors")
+    m, n = lhs_q8_0.shape[0], rhs_q4_0.shape[0]
+    if lhs_q8_0.shape[1] % 34 or rhs_q4_0.shape[1] % 18 or lhs_q8_0.shape[1] // 34 != rhs_q4_0.shape[1] // 18:
+        raise ValueError("operands disagree on K")
+    nb = rhs_q4_0.shape[1] // 18
+    out = torch.empty((m, n, nb), dtype=torch.int32, device=rhs_q4_0.device)
+    rc = _lib.load().qmm_block_dots_q4_0(_ptr(lhs_q8_0), _ptr(rhs_q4_0), m, n, nb * 32, _ptr(out), _stream(rhs_q4_0))
+    _lib.check(rc, "block_dots_q4_0")
+    return out

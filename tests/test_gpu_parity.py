@@ -1,0 +1,172 @@
+"""GPU parity: every kernel behind the C ABI against the CPU oracle on the same seeded inputs.
+
+Bars: packed bytes, dequantised weights and int8 block dots bit-exact; fp32
+matmul outputs within rtol 1e-3 / atol 1e-4 under the reference's symmetric
+isclose (stdlib/src/math/math.mojo:1023-1030).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from conftest import synth
+from mojo_amd import QuantizationConfig, QuantizationEncoding as QE
+from mojo_amd import block_dots_q4_0, dequantize, qmatmul, quantize, quantize_gptq
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-3, 1e-4
+ENC = {QE.Q4_0: O.Q4_0, QE.Q4_K: O.Q4_K, QE.Q6_K: O.Q6_K}
+DEV = "cuda:0"
+
+
+def gpu(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(DEV)
+
+
+def assert_close(got, want, what):
+    got = got.detach().cpu().numpy() if isinstance(got, torch.Tensor) else got
+    ok = O.isclose(got, want, RTOL, ATOL)
+    if not ok.all():
+        bad = np.argwhere(~ok)
+        i = tuple(bad[0])
+        raise AssertionError(
+            f"{what}: {len(bad)}/{ok.size} outside rtol={RTOL} atol={ATOL}; first {i}: got {got[i]} want {want[i]}; "
+            f"max abs err {np.abs(got - want).max()}")
+
+
+def bits(x):
+    return x.detach().cpu().contiguous().view(torch.uint8).numpy()
+
+
+# ------------------------------------------------------------------ quantisers
+@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q6_K])
+def test_quantize_bytes_match_oracle(enc):
+    w, _ = synth(3, 96, 1024, 1)
+    w[5, 256:512] = 0.0  # an all-zero super-block
+    w[7, :32] = 0.0
+    w[9, 0:32] = -w[9, 0:32].max()  # ties in the max search
+    got = quantize(enc, gpu(w)).cpu().numpy()
+    want = O.quantize(ENC[enc], w)
+    assert np.array_equal(got, want)
+
+
+def test_quantize_q8_0_bytes_match_oracle():
+    _, a = synth(4, 8, 2048, 16)
+    a[3, 64:96] = 0.0
+    a[2, 0:8] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.0]  # x/d lands on .5 ties when amax = 127
+    got = quantize(QE.Q8_0, gpu(a)).cpu().numpy()
+    assert np.array_equal(got, O.quantize_q8_0(a))
+
+
+def test_quantize_gptq_matches_oracle():
+    w, _ = synth(5, 64, 512, 1)
+    qw, sc, qz, gi = [t.cpu().numpy() for t in quantize_gptq(gpu(w))]
+    oqw, osc, oqz, ogi = O.quantize_gptq(w)
+    assert np.array_equal(qw, oqw) and np.array_equal(sc.view(np.uint16), osc)
+    assert np.array_equal(qz, oqz) and np.array_equal(gi, ogi)
+
+
+# ------------------------------------------------------------------ dequantisers (bit-exact)
+@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q6_K])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_dequantize_bit_exact(enc, dtype):
+    w, _ = synth(6, 128, 2048, 1)
+    packed = O.quantize(ENC[enc], w)
+    # random bytes in the code/scale fields exercise every bit pattern, fp16 fields stay finite
+    rng = np.random.default_rng(1)
+    noisy = packed.copy()
+    epb, bpb = O.BLOCK[ENC[enc]]
+    blocks = noisy.reshape(-1, bpb)
+    keep = {O.Q4_0: slice(0, 2), O.Q4_K: slice(0, 4), O.Q6_K: slice(208, 210)}[ENC[enc]]
+    rnd = rng.integers(0, 256, blocks.shape, dtype=np.uint8)
+    rnd[:, keep] = blocks[:, keep]
+    blocks[64:] = rnd[64:]
+    want = O.dequantize(ENC[enc], noisy, 2048)
+    got = dequantize(enc, gpu(noisy), dtype=dtype)
+    if dtype == torch.float32:
+        assert np.array_equal(bits(got), want.view(np.uint8).reshape(128, -1))
+    else:
+        assert np.array_equal(bits(got).view(np.uint16), O.f32_to_bf16(want))
+
+
+def test_dequantize_gptq_bit_exact():
+    w, _ = synth(7, 128, 1024, 1)
+    qw, sc, qz, gi = O.quantize_gptq(w)
+    want = O.dequantize_gptq(qw, sc, qz)
+    cfg = QuantizationConfig()
+    got = dequantize(QE.GPTQ, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi), config=cfg)
+    assert np.array_equal(bits(got), want.view(np.uint8).reshape(128, -1))
+    got = dequantize(QE.GPTQ, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), config=cfg)
+    assert np.array_equal(bits(got), want.view(np.uint8).reshape(128, -1))
+
+
+# ------------------------------------------------------------------ Q4_0: integer dots and matmul
+def test_block_dots_bit_exact():
+    w, a = synth(0, 256, 1024, 4)
+    wq, aq = O.quantize(O.Q4_0, w), O.quantize_q8_0(a)
+    got = block_dots_q4_0(gpu(aq), gpu(wq)).cpu().numpy()
+    assert np.array_equal(got, O.block_dots_q4_0_q8_0(aq, wq, 1024))
+
+
+def test_block_dots_extremes():
+    # all codes 0 (-8) against all -127 / +127, and all codes 15 (+7)
+    wq = np.zeros((2, 18), np.uint8)
+    wq[:, :2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    wq[1, 2:] = 0xFF
+    aq = np.zeros((2, 34), np.uint8)
+    aq[0, 2:] = np.int8(-127).view(np.uint8)
+    aq[1, 2:] = 127
+    got = block_dots_q4_0(gpu(aq), gpu(wq)).cpu().numpy()[:, :, 0]
+    assert got.tolist() == [[32 * 8 * 127, -32 * 7 * 127], [-32 * 8 * 127, 32 * 7 * 127]]
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (16, 1024, 4096), (5, 130, 64), (3, 7, 32), (33, 64, 256)])
+def test_q4_0_matmul(m, n, k):
+    w, a = synth(0, n, k, m)
+    wq = O.quantize(O.Q4_0, w)
+    want = O.matmul_q4_0(a, wq)
+    got = qmatmul(QE.Q4_0, None, gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_0 {m}x{n}x{k}")
+
+
+# ------------------------------------------------------------------ Q4_K / Q6_K with fp32 activations
+@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K])
+@pytest.mark.parametrize("m,n,k", [(1, 1024, 4096), (4, 512, 4096), (16, 256, 2048), (3, 5, 256), (2, 66, 14336),
+                                   (20, 64, 512)])
+def test_kquant_matmul_f32(enc, m, n, k):
+    w, a = synth(3, n, k, m)
+    wq = O.quantize(ENC[enc], w)
+    want = O.matmul_f32(ENC[enc], a, wq)
+    truth = O.matmul_f64(ENC[enc], a, wq)
+    got = qmatmul(enc, None, gpu(a), gpu(wq))
+    assert_close(got, want, f"{enc.name} {m}x{n}x{k} vs fp32 oracle")
+    assert_close(got, truth, f"{enc.name} {m}x{n}x{k} vs fp64 truth")
+
+
+@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K])
+def test_kquant_matmul_bf16_lhs(enc):
+    w, a = synth(5, 256, 1024, 4)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(ENC[enc], w)
+    want = O.matmul_f32(ENC[enc], a, wq)
+    got = qmatmul(enc, None, gpu(a).to(torch.bfloat16), gpu(wq))
+    assert_close(got, want, f"{enc.name} bf16 lhs")
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256)])
+def test_gptq_matmul(m, n, k):
+    w, a = synth(5, n, k, m)
+    qw, sc, qz, gi = O.quantize_gptq(w)
+    want = O.matmul_gptq(a, qw, sc, qz)
+    got = qmatmul(QE.GPTQ, QuantizationConfig(), gpu(a), gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, want, f"GPTQ {m}x{n}x{k}")
+
+
+def test_leading_dims_broadcast():
+    w, a = synth(8, 64, 512, 6)
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq).reshape(2, 3, 64)
+    got = qmatmul(QE.Q4_K, None, gpu(a).reshape(2, 3, 512), gpu(wq))
+    assert got.shape == (2, 3, 64)
+    assert_close(got, want, "leading dims")
