@@ -1,0 +1,264 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Q4_K decode GEMV over the Llama-3-8B projection set on one MI355X.
+
+A step is one pass of the seven projections of one transformer layer
+(q, k, v, o, gate, up, down) at M=1 with fp32 activations through ``qmm_matmul``.
+Steps rotate over several distinct layers' weights so that no step finds its
+weights in the 256 MB Infinity Cache.  The value is algorithmic bytes per step
+(packed weight bytes + fp32 activations + fp32 outputs) over wall time, in GB/s.
+
+Prints ONE JSON line.  ``roofline`` covers the dominant kernel (the Q4_K GEMV),
+timed with HIP events on the launch stream; ``cpu_baseline`` is the CPU oracle
+(a port of the reference CPU path, not the MAX binary) on a bounded sample of the
+same workload; ``extra`` carries per-shape and secondary-config rates.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from mojo_amd import QuantizationConfig, QuantizationEncoding as QE  # noqa: E402
+from mojo_amd import _lib, qmatmul, quantize, quantize_gptq  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+BF16_PEAK_TFLOPS = 2500.0
+
+# (name, N, K) of the Llama-3-8B projections
+PROJ = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+        ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
+
+
+def alg_bytes(enc: QE, m: int, n: int, k: int) -> int:
+    return n * enc.packed_row_bytes(k) + 4 * m * k + 4 * m * n
+
+
+class Gemv:
+    """One preallocated qmm_matmul call (no Python-side allocation when launched)."""
+
+    def __init__(self, enc: QE, w: torch.Tensor, a: torch.Tensor):
+        self.lib = _lib.load()
+        self.enc, self.w, self.a = enc, w, a
+        self.m, self.k = a.shape
+        self.n = w.shape[0]
+        self.out = torch.empty((self.m, self.n), dtype=torch.float32, device=a.device)
+        dt = _lib.QMM_F32 if a.dtype == torch.float32 else _lib.QMM_BF16
+        need = self.lib.qmm_matmul_workspace_bytes(enc.code, dt, self.m, self.n, self.k)
+        self.ws = torch.empty((max(need, 1),), dtype=torch.uint8, device=a.device)
+        self.need = need
+        self.dt = dt
+        self.ptrs = (C.c_void_p * 1)(w.data_ptr())
+
+    def launch(self, stream_ptr: int) -> None:
+        rc = self.lib.qmm_matmul(self.enc.code, None, C.c_void_p(self.a.data_ptr()), self.dt, self.m, self.k,
+                                 self.ptrs, 1, self.n, C.c_void_p(self.out.data_ptr()),
+                                 C.c_void_p(self.ws.data_ptr()), self.need, 0, C.c_void_p(stream_ptr))
+        _lib.check(rc, "qmm_matmul")
+
+
+def make_weight(enc: QE, n: int, k: int, gen: torch.Generator) -> torch.Tensor:
+    w = torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02
+    return quantize(enc, w)
+
+
+def capture(calls) -> torch.cuda.CUDAGraph:
+    """Record a list of Gemv launches into one HIP graph on a side stream."""
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for c in calls:  # warm the kernels outside capture
+            c.launch(s.cuda_stream)
+        s.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            sp = torch.cuda.current_stream().cuda_stream
+            for c in calls:
+                c.launch(sp)
+    torch.cuda.current_stream().wait_stream(s)
+    return g
+
+
+def time_graphs(graphs, steps: int, warmup: int) -> float:
+    """Seconds for exactly `steps` replays (graph i % len), HIP events on the launch stream."""
+    for i in range(warmup):
+        graphs[i % len(graphs)].replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        graphs[i % len(graphs)].replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return e0.elapsed_time(e1) * 1e-3, wall
+
+
+def cpu_baseline(layer_w, m: int, budget_s: float = 12.0):
+    """Oracle (port of the reference CPU path) on one layer's seven projections, OpenMP over N."""
+    import numpy as np
+
+    import oracle as O
+
+    threads = min(O.num_threads(), 16)
+    O.set_num_threads(threads)
+    rng = np.random.Generator(np.random.PCG64(3))
+    host = [(w.cpu().numpy(), n, k) for (w, (_, n, k)) in zip(layer_w, PROJ)]
+    acts = {k: rng.standard_normal((m, k), dtype=np.float32) for k in (4096, 14336)}
+    nbytes = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
+    for w, n, k in host:  # warm-up pass
+        O.matmul_f32(O.Q4_K, acts[k], w)
+    passes, t0 = 0, O.now()
+    while True:
+        for w, n, k in host:
+            O.matmul_f32(O.Q4_K, acts[k], w)
+        passes += 1
+        el = O.now() - t0
+        if el > budget_s or passes >= 5000:
+            break
+    return {"value": round(nbytes * passes / el / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{passes} passes of one layer's 7 Q4_K projections at M={m} ({nbytes} B each), "
+                      f"{el:.1f} s, OpenMP over N, host has {os.cpu_count()} logical cpus"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
+    ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip per-shape and secondary-config timings")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this path runs on a single MI355X and --gpus {args.gpus} is not "
+              "supported (sharding by N is described in DESIGN.md).", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(3)
+    m = args.m
+    acts = {k: torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}
+    layers = []
+    for _ in range(args.layers):
+        layers.append([make_weight(QE.Q4_K, n, k, gen) for _, n, k in PROJ])
+    calls = [[Gemv(QE.Q4_K, w, acts[k]) for w, (_, n, k) in zip(lw, PROJ)] for lw in layers]
+    graphs = [capture(c) for c in calls]
+    step_bytes = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
+
+    dev_s, wall_s = time_graphs(graphs, args.steps, args.warmup)
+    ms_per_step = dev_s * 1e3 / args.steps
+    value = step_bytes * args.steps / dev_s / 1e9
+    launches = args.steps * len(PROJ)
+    avg_launch_us = dev_s * 1e6 / launches
+    avg_launch_bytes = step_bytes / len(PROJ)
+    achieved = avg_launch_bytes / (avg_launch_us * 1e-6) / 1e9
+
+    cu, khz = C.c_int32(0), C.c_int32(0)
+    _lib.load().qmm_device_info(C.byref(cu), C.byref(khz))
+
+    extra = {"wall_ms_per_step": round(wall_s * 1e3 / args.steps, 5), "avg_launch_us": round(avg_launch_us, 3),
+             "compute_units": cu.value, "clock_mhz": khz.value / 1000.0}
+    if not args.no_extra:
+        extra.update(extra_timings(layers, acts, gen))
+
+    result = {
+        "metric": "Q4_K decode GEMV HBM GB/s",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"Q4_K decode GEMV, Llama-3-8B projection set (q,k,v,o,gate,up,down), M={m}, fp32 "
+                        f"activations, fp32 out; weights 0.02*N(0,1) quantised to Q4_K on the GPU, activations "
+                        f"N(0,1); {args.layers} distinct layers rotated (cold cache); one step = one layer "
+                        f"= 7 launches, {step_bytes} algorithmic bytes",
+            "m": m, "layers": args.layers, "bytes_per_step": step_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "gemv_q4_k_kernel",
+            "bytes_per_launch": avg_launch_bytes,
+            "launch_us": round(avg_launch_us, 3),
+        },
+        "extra": extra,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(layers[0], m)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+    return 0
+
+
+def extra_timings(layers, acts, gen):
+    """Per-shape cold-cache rates for the headline set, M=4, and the other configs."""
+    out = {}
+    m = acts[4096].shape[0]
+    # per projection shape, rotating over the layers' copies of that shape
+    per_shape = {}
+    for idx, (name, n, k) in enumerate(PROJ):
+        if name in ("v", "up"):
+            continue
+        cs = [Gemv(QE.Q4_K, lw[idx], acts[k]) for lw in layers]
+        if name in ("q", "k"):  # small matrices: add the same-shape sibling so the rotation exceeds the cache
+            cs += [Gemv(QE.Q4_K, lw[idx + (3 if name == "q" else 1)], acts[k]) for lw in layers]
+        g = capture(cs)
+        dev_s, _ = time_graphs([g], 50, 5)
+        us = dev_s * 1e6 / (50 * len(cs))
+        b = alg_bytes(QE.Q4_K, m, n, k)
+        per_shape[f"{name}_{n}x{k}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1)}
+    out["q4_k_per_shape"] = per_shape
+    # M=4 over the same set
+    if m == 1:
+        acts4 = {k: torch.randn((4, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}
+        graphs = [capture([Gemv(QE.Q4_K, w, acts4[k]) for w, (_, n, k) in zip(lw, PROJ)]) for lw in layers]
+        dev_s, _ = time_graphs(graphs, 100, 10)
+        b = sum(alg_bytes(QE.Q4_K, 4, n, k) for _, n, k in PROJ)
+        out["q4_k_m4_GB/s"] = round(b * 100 / dev_s / 1e9, 1)
+    # cfg4: Q6_K lm_head, M=1 (431 MB: larger than the cache by itself)
+    w6 = make_weight(QE.Q6_K, 128256, 4096, gen)
+    a1 = torch.randn((1, 4096), dtype=torch.float32, device="cuda:0", generator=gen)
+    g = capture([Gemv(QE.Q6_K, w6, a1)])
+    dev_s, _ = time_graphs([g], 20, 3)
+    b = alg_bytes(QE.Q6_K, 1, 128256, 4096)
+    out["q6_k_lm_head"] = {"us": round(dev_s * 1e6 / 20, 2), "GB/s": round(b * 20 / dev_s / 1e9, 1)}
+    del w6
+    # cfg1 / cfg2: Q4_0 with Q8_0 activations
+    for tag, mm, n, k, copies in (("q4_0_m1_4096x4096", 1, 4096, 4096, 32), ("q4_0_m16_14336x4096", 16, 14336, 4096, 10)):
+        am = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen)
+        cs = [Gemv(QE.Q4_0, make_weight(QE.Q4_0, n, k, gen), am) for _ in range(copies)]
+        g = capture(cs)
+        dev_s, _ = time_graphs([g], 20, 3)
+        us = dev_s * 1e6 / (20 * copies)
+        out[tag] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q4_0, mm, n, k) / us / 1e3, 1)}
+        del cs
+    return out
+
+
+if __name__ == "__main__":
+    sys.exit(main())
