@@ -3,6 +3,8 @@
 // The packed weights are streamed once; every wavefront owns one weight row,
 // keeps one fp32 accumulator per lhs row and finishes with a cross-lane sum.
 // No matrix-core instructions are used here.
+#include <stdlib.h>
+
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -300,8 +302,21 @@ __global__ __launch_bounds__(256) void gemv_gptq_kernel(const uint32_t* __restri
     else if (m <= 8) { CALL(8); } \
     else { CALL(16); }
 
+// Kernel choice for Q4_K decode shapes.  Measured on MI355X: with one or two lhs rows the
+// vector-ALU kernel below is faster on the Llama-3-8B projection shapes; from three rows on its
+// cost grows with m while the matrix-core kernel's does not.  QMM_Q4K_GEMV=valu|mfma overrides.
+static bool q4k_use_valu(int m) {
+    static const int forced = [] {
+        const char* e = getenv("QMM_Q4K_GEMV");
+        return !e ? 0 : (e[0] == 'v' ? 1 : (e[0] == 'm' ? 2 : 0));
+    }();
+    if (forced) return forced == 1;
+    return m <= 2;
+}
+
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
+    if (!q4k_use_valu(m)) return launch_gemv_q4_k_mfma(a, a_dtype, w, m, n, k, out, ldo, s);
     dim3 grid((unsigned)((n + 3) / 4)), block(256);
 #define CALL(MT)                                                                                          \
     if (a_dtype == QMM_F32)                                                                               \

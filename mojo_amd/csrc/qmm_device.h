@@ -33,6 +33,13 @@ __device__ __forceinline__ uint16_t f2bf(float f) {
     return (uint16_t)(x >> 16);
 }
 
+// lhs element i as fp32; InT is float or a bf16 bit pattern (uint16_t).
+template <typename InT>
+__device__ __forceinline__ float load_f32(const InT* p, int64_t i) {
+    if constexpr (sizeof(InT) == 4) return p[i];
+    else return bf2f(p[i]);
+}
+
 __device__ __forceinline__ uint32_t byte_of(uint32_t w, int i) { return (w >> (8 * i)) & 0xffu; }
 
 // Q4_K: 6-bit scale and min of sub-block j (0..7) from the 12 packed bytes,
@@ -53,6 +60,35 @@ __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
     return v;
+}
+
+// Cross-lane data movement inside the VALU (DPP), no LDS round trip.
+// CTRL: 0xB1 swap lane pairs, 0x4E swap pairs of a quad, 0x141 mirror 8 lanes, 0x140 mirror 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over each aligned group of 8 lanes; every lane of the group gets it.
+__device__ __forceinline__ float sum8(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    return v;
+}
+
+// Largest value of a non-negative float over the 64 lanes, as its bit pattern (wave-uniform).
+__device__ __forceinline__ uint32_t wave_max_nonneg_bits(float v) {
+    v = fmaxf(v, dpp_move<0xB1>(v));
+    v = fmaxf(v, dpp_move<0x4E>(v));
+    v = fmaxf(v, dpp_move<0x141>(v));
+    v = fmaxf(v, dpp_move<0x140>(v));
+    const int b = __float_as_int(v);
+    uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane(b, 0), r1 = (uint32_t)__builtin_amdgcn_readlane(b, 16);
+    uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane(b, 32), r3 = (uint32_t)__builtin_amdgcn_readlane(b, 48);
+    r0 = r0 > r1 ? r0 : r1;
+    r2 = r2 > r3 ? r2 : r3;
+    return r0 > r2 ? r0 : r2;
 }
 
 }  // namespace qmm

@@ -123,12 +123,6 @@ hipError_t launch_dequant_gptq(const void* qweight, const void* scales, const vo
 // Q8_0 / Q4_0 quantisers: 32 lanes per block, two blocks per wavefront
 // ---------------------------------------------------------------------------
 
-template <typename InT>
-__device__ __forceinline__ float load_f32(const InT* p, int64_t i) {
-    if constexpr (sizeof(InT) == 4) return p[i];
-    else return bf2f(p[i]);
-}
-
 // Writes GGUF Q8_0 blocks (blocks != null) and/or the planar form the Q4_0
 // matmul kernels read: codes int8[rows, k], scales fp32[rows, k/32] (the fp16
 // block scale widened) and code sums int32[rows, k/32].
