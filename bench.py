@@ -248,6 +248,15 @@ def extra_timings(layers, acts, gen):
     b = alg_bytes(QE.Q6_K, 1, 128256, 4096)
     out["q6_k_lm_head"] = {"us": round(dev_s * 1e6 / 20, 2), "GB/s": round(b * 20 / dev_s / 1e9, 1)}
     del w6
+    # cfg5: Q4_K prefill, bf16 lhs [2048, 4096] x [14336, 4096]
+    ab = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
+    wp = make_weight(QE.Q4_K, 14336, 4096, gen)
+    g = capture([Gemv(QE.Q4_K, wp, ab)])
+    dev_s, _ = time_graphs([g], 20, 3)
+    us = dev_s * 1e6 / 20
+    tf = 2 * 2048 * 14336 * 4096 / us / 1e6
+    out["q4_k_prefill_m2048"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
+    del wp
     # cfg1 / cfg2: Q4_0 with Q8_0 activations
     for tag, mm, n, k, copies in (("q4_0_m1_4096x4096", 1, 4096, 4096, 32), ("q4_0_m16_14336x4096", 16, 14336, 4096, 10)):
         am = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen)

@@ -1,0 +1,364 @@
+// Q4_K prefill kernel (m > 16 lhs rows): matrix-core GEMM over exact integer codes.
+//
+// Arithmetic.  As in the decode kernel, a masked nibble is the fp16 subnormal
+// q*2^-24 and one packed fp16 multiply folds the 6-bit sub-block scale in
+// (q*sc <= 945, exact).  lhs values are scaled per row by a power of two and
+// narrowed to fp16 (exact for bf16 inputs of ordinary range), so every product
+// inside v_mfma_f32_32x32x16_f16 is exact and the sums are fp32.  Per 256-wide
+// super-block b the matrix cores produce P_b[m][n] = sum_k a[m][k]*(sc*q)[n][k];
+// the fp32 super-block scale is applied in the lanes, acc += d[n,b] * P_b.  The
+// min term  -sum_{b,j} (dmin*mn_j)[n] * (sum_{k in j} a[m][k])  is itself a matrix
+// product over the 8 sub-blocks of a super-block: dmin*mn (17 bits) is split
+// exactly into two fp16 values and the activation sums into hi + lo, and the two
+// extra products per super-block accumulate straight into acc.
+//
+// A workgroup of 8 wavefronts computes a 128 x 256 output tile; wavefront
+// (wm, wn) owns the 64 x 64 sub-tile at (64*wm, 64*wn).  lhs tiles go through
+// LDS (double buffered, one 64-wide chunk per step); the packed weights are
+// loaded by the lanes that use them and unpacked in registers.
+#include <stdlib.h>
+
+#include "qmm_internal.h"
+
+namespace qmm {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BM = 128, BN = 256;   // workgroup tile
+constexpr int A_STRIDE = 72;        // halfs per LDS row of a 64-wide chunk (144 bytes: conflict-free b128 reads)
+constexpr float kTwo24 = 16777216.0f;
+
+union HalfPack {
+    uint32_t u[4];
+    half8 h;
+};
+__device__ __forceinline__ half8 pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    HalfPack p;
+    p.u[0] = a; p.u[1] = b; p.u[2] = c; p.u[3] = d;
+    return p.h;
+}
+__device__ __forceinline__ uint32_t pack_half2(float x, float y) {
+    return (uint32_t)f2h(x) | ((uint32_t)f2h(y) << 16);
+}
+__device__ __forceinline__ uint32_t pk_mul(uint32_t x, uint32_t s) {
+    union { uint32_t u; half2v h; } a, b, r;
+    a.u = x; b.u = s;
+    r.h = a.h * b.h;
+    return r.u;
+}
+// x*s + c on packed fp16 pairs, fused (single rounding)
+__device__ __forceinline__ uint32_t pk_fma(uint32_t x, uint32_t s, uint32_t c) {
+    union { uint32_t u; half2v h; } a, b, d, r;
+    a.u = x; b.u = s; d.u = c;
+    r.h = __builtin_elementwise_fma(a.h, b.h, d.h);
+    return r.u;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// lhs preparation: per-row power-of-two scale, fp16 narrowing in operand order,
+// per-sub-block sums.  One workgroup of 256 threads per lhs row.
+//   a16  [m][k] fp16: inside every 64-wide chunk, position f*16 + g*8 + slot holds
+//        k = 32*(f/2) + 16*g + 8*(f%2) + perm[slot], perm = (0,2,1,3,4,6,5,7)
+//   asum [m][k/256][16] fp16: hi parts of the 8 sub-block sums, then their lo parts
+//   inv  [m] fp32: inverse of the row scale
+// PART = 0 writes the narrowed values, PART = 1 the residual (fp32 lhs only).
+// ---------------------------------------------------------------------------
+template <typename AT>
+__global__ __launch_bounds__(256) void q4k_prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
+                                                           _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum,
+                                                           float* __restrict__ inv) {
+    __shared__ uint32_t wmax[4];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const AT* ar = a + (int64_t)row * k;
+    float mx = 0.0f;
+    for (int i = tid * 4; i < k; i += 1024) {
+        float x0 = load_f32(ar, i), x1 = load_f32(ar, i + 1), x2 = load_f32(ar, i + 2), x3 = load_f32(ar, i + 3);
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3))));
+    }
+    const uint32_t mb = wave_max_nonneg_bits(mx);
+    if (lane == 0) wmax[wave] = mb;
+    __syncthreads();
+    uint32_t mxb = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+    int e = (int)((mxb >> 23) & 0xffu) - 127;
+    if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite row: leave unscaled
+    const float s = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
+    if (tid == 0) inv[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+    for (int i = tid * 4; i < k; i += 1024) {
+        const float x0 = load_f32(ar, i) * s, x1 = load_f32(ar, i + 1) * s, x2 = load_f32(ar, i + 2) * s,
+                    x3 = load_f32(ar, i + 3) * s;
+        const float h0 = h2f(f2h(x0)), h1 = h2f(f2h(x1)), h2 = h2f(f2h(x2)), h3 = h2f(f2h(x3));
+        const int kl = i & 63, hin = kl >> 5, gg = (kl >> 4) & 1, odd = (kl >> 3) & 1;
+        const int pos = (2 * hin + odd) * 16 + gg * 8 + (kl & 4);
+        const int64_t o = (int64_t)row * k + (i & ~63) + pos;
+        *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
+        if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
+        const float sum = sum8((x0 + x1) + (x2 + x3));  // 8 consecutive lanes = one 32-wide sub-block
+        if ((lane & 7) == 0) {
+            const int blk = i >> 8, j = (i >> 5) & 7;
+            const float sh = h2f(f2h(sum));
+            _Float16* as = asum + ((int64_t)row * (k >> 8) + blk) * 16;
+            as[j] = (_Float16)sh;
+            as[8 + j] = (_Float16)(sum - sh);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// main kernel
+// ---------------------------------------------------------------------------
+template <int NPART>
+__global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restrict__ w, const _Float16* __restrict__ a16,
+                                                        const _Float16* __restrict__ a16_lo,
+                                                        const _Float16* __restrict__ asum,
+                                                        const float* __restrict__ inv, float* __restrict__ out, int m,
+                                                        int n, int k, int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][NPART][BM * A_STRIDE];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_s[BM * 16];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 2, wn = wave & 3;
+    const int nl = lane & 31, g = lane >> 5;
+    const int nblk = k >> 8;
+    const int64_t row_bytes = (int64_t)nblk * Q4_K_BPB;
+
+    // Tile order: consecutive workgroup ids land on different XCDs, so give each XCD a
+    // contiguous range of an order that keeps two lhs tile rows fixed while walking N.
+    int tile_m, tile_n;
+    {
+        const int total = tiles_m * tiles_n;
+        const int per_xcd = (total + 7) / 8;
+        const int o = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+        if (o >= total) return;
+        const int gm = 2, span = gm * tiles_n;
+        const int grp = o / span, rem = o - grp * span;
+        const int rows_here = min(gm, tiles_m - grp * gm);
+        tile_n = rem / rows_here;
+        tile_m = grp * gm + rem - tile_n * rows_here;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // lhs chunk loader: 128 rows x 64 halfs = 1024 x 16 bytes; 512 threads x 2
+    const int a_row = tid >> 2, a_seg = tid & 3;  // rows a_row and a_row (+0), two 16-byte segments each
+    auto a_src = [&](const _Float16* base, int chunk, int seg) {
+        int row = m0 + a_row;
+        if (row >= m) row = m - 1;
+        return (const uint4*)(base + (int64_t)row * k + (int64_t)chunk * 64 + seg * 8);
+    };
+    uint4 a_pref[NPART][2];
+    auto a_load = [&](int chunk) {
+        a_pref[0][0] = *a_src(a16, chunk, a_seg);
+        a_pref[0][1] = *a_src(a16, chunk, a_seg + 4);
+        if constexpr (NPART == 2) {
+            a_pref[1][0] = *a_src(a16_lo, chunk, a_seg);
+            a_pref[1][1] = *a_src(a16_lo, chunk, a_seg + 4);
+        }
+    };
+    auto a_store = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < NPART; p++) {
+            *(uint4*)(&lds_a[buf][p][a_row * A_STRIDE + a_seg * 8]) = a_pref[p][0];
+            *(uint4*)(&lds_a[buf][p][a_row * A_STRIDE + (a_seg + 4) * 8]) = a_pref[p][1];
+        }
+    };
+
+    // this lane's two weight columns
+    const uint8_t* wcol[2];
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        int col = n0 + wn * 64 + ni * 32 + nl;
+        if (col >= n) col = n - 1;
+        wcol[ni] = w + (int64_t)col * row_bytes;
+    }
+
+    float16v acc[2][2], P[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mi][ni][r] = 0.0f;
+
+    uint4 q_pref[2];
+    auto q_load = [&](int blk, int c) {
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) q_pref[ni] = *(const uint4*)(wcol[ni] + (int64_t)blk * Q4_K_BPB + 16 + 32 * c + 16 * g);
+    };
+
+    a_load(0);
+    q_load(0, 0);
+    a_store(0);
+    __syncthreads();
+
+    const int nsteps = nblk * 4;
+    float dscale[2] = {0.f, 0.f};
+    uint32_t sp[2][8];
+    for (int blk = 0; blk < nblk; blk++) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) {  // compile-time chunk index: register arrays stay in registers
+        const int step = blk * 4 + c, buf = c & 1;
+        const uint4 qc[2] = {q_pref[0], q_pref[1]};
+        if (step + 1 < nsteps) {
+            a_load(step + 1);
+            q_load((step + 1) >> 2, (step + 1) & 3);
+        }
+        if (c == 0) {
+            // ---- super-block start: sub-block sums to LDS, header decode, min-term products
+            if (tid < 256) {
+                int row = m0 + (tid >> 1);
+                if (row >= m) row = m - 1;
+                *(uint4*)(&lds_s[(tid >> 1) * 16 + (tid & 1) * 8]) =
+                    *(const uint4*)(asum + ((int64_t)row * nblk + blk) * 16 + (tid & 1) * 8);
+            }
+            uint32_t dmn_hi[2][4], dmn_lo[2][4];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++) {
+                const uint4 hdr = *(const uint4*)(wcol[ni] + (int64_t)blk * Q4_K_BPB);
+                dscale[ni] = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo24;
+                const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
+                const uint32_t sc_lo = s0 & 0x3F3F3F3Fu, sc_hi = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
+                const uint32_t mn_lo = s1 & 0x3F3F3F3Fu, mn_hi = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+                const float e0 = (float)(sc_lo & 0xffu), e1 = 0.0625f * (float)((sc_lo >> 8) & 0xffu);
+                const float e2 = (float)((sc_lo >> 16) & 0xffu), e3 = 0.0625f * (float)(sc_lo >> 24);
+                const float e4 = (float)(sc_hi & 0xffu), e5 = 0.0625f * (float)((sc_hi >> 8) & 0xffu);
+                const float e6 = (float)((sc_hi >> 16) & 0xffu), e7 = 0.0625f * (float)(sc_hi >> 24);
+                sp[ni][0] = pack_half2(e0, e0); sp[ni][1] = pack_half2(e1, e1);
+                sp[ni][2] = pack_half2(e2, e2); sp[ni][3] = pack_half2(e3, e3);
+                sp[ni][4] = pack_half2(e4, e4); sp[ni][5] = pack_half2(e5, e5);
+                sp[ni][6] = pack_half2(e6, e6); sp[ni][7] = pack_half2(e7, e7);
+                // -(dmin * mn_j) as exact fp16 hi + lo, sub-blocks (0,1) (2,3) (4,5) (6,7)
+                const uint32_t ndm = ((hdr.x >> 16) ^ 0x8000u) * 0x00010001u;  // (-dmin, -dmin)
+                const uint32_t mp[4] = {
+                    pack_half2((float)(mn_lo & 0xffu), (float)((mn_lo >> 8) & 0xffu)),
+                    pack_half2((float)((mn_lo >> 16) & 0xffu), (float)(mn_lo >> 24)),
+                    pack_half2((float)(mn_hi & 0xffu), (float)((mn_hi >> 8) & 0xffu)),
+                    pack_half2((float)((mn_hi >> 16) & 0xffu), (float)(mn_hi >> 24))};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    dmn_hi[ni][i] = pk_mul(ndm, mp[i]);
+                    dmn_lo[ni][i] = pk_fma(ndm, mp[i], dmn_hi[ni][i] ^ 0x80008000u);
+                }
+            }
+            __syncthreads();  // lds_s visible (also orders this step's lds_a reads after the previous stores)
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+                // A operand: lanes g=0 carry the hi parts of the 8 sub-block sums, g=1 the lo parts
+                const half8 av = *(const half8*)(&lds_s[(wm * 64 + mi * 32 + nl) * 16 + g * 8]);
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        av, pack4(dmn_hi[ni][0], dmn_hi[ni][1], dmn_hi[ni][2], dmn_hi[ni][3]), acc[mi][ni], 0, 0, 0);
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        av, pack4(dmn_lo[ni][0], dmn_lo[ni][1], dmn_lo[ni][2], dmn_lo[ni][3]), acc[mi][ni], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) P[mi][ni][r] = 0.0f;
+        }
+
+        // ---- one 64-wide chunk: four 16-wide operand slices
+        const uint32_t M1 = 0x000F000Fu, M2 = 0x00F000F0u;
+#pragma unroll
+        for (int f = 0; f < 4; f++) {
+            half8 bfrag[2];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++) {
+                const uint32_t x0 = (f & 1) ? qc[ni].z : qc[ni].x, x1 = (f & 1) ? qc[ni].w : qc[ni].y;
+                const uint32_t mask = (f & 2) ? M2 : M1;
+                const uint32_t s = sp[ni][2 * c + (f >> 1)];
+                bfrag[ni] = pack4(pk_mul(x0 & mask, s), pk_mul((x0 >> 8) & mask, s), pk_mul(x1 & mask, s),
+                                  pk_mul((x1 >> 8) & mask, s));
+            }
+#pragma unroll
+            for (int p = 0; p < NPART; p++) {
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++) {
+                    const half8 afrag = *(const half8*)(&lds_a[buf][p][(wm * 64 + mi * 32 + nl) * A_STRIDE + f * 16 + g * 8]);
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++)
+                        P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[ni], P[mi][ni], 0, 0, 0);
+                }
+            }
+        }
+        if (c == 3) {
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[mi][ni][r] = fmaf(dscale[ni], P[mi][ni][r], acc[mi][ni][r]);
+        }
+        if (step + 1 < nsteps) {
+            a_store(buf ^ 1);
+            if (c != 3) __syncthreads();  // a super-block start has its own barrier
+        }
+      }
+    }
+
+    // ---- epilogue: undo the row scale, store
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (row < m) {
+                const float is = inv[row];
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    const int col = n0 + wn * 64 + ni * 32 + nl;
+                    if (col < n) out[(int64_t)row * n + col] = acc[mi][ni][r] * is;
+                }
+            }
+        }
+    }
+}
+
+// Workspace: a16 [m][k] fp16 (+ the residual part for fp32 lhs), asum [m][k/256][16] fp16, inv [m] fp32.
+int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) {
+    const int64_t parts = lhs_dtype == QMM_F32 ? 2 : 1;
+    auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
+    return parts * up(m * k * 2) + up(m * (k / 256) * 32) + up(m * 4);
+}
+
+hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                            float* out, void* workspace, hipStream_t s) {
+    auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
+    char* ws = (char*)workspace;
+    _Float16* a16 = (_Float16*)ws;
+    ws += up(m * k * 2);
+    _Float16* a16_lo = nullptr;
+    if (lhs_dtype == QMM_F32) {
+        a16_lo = (_Float16*)ws;
+        ws += up(m * k * 2);
+    }
+    _Float16* asum = (_Float16*)ws;
+    ws += up(m * (k / 256) * 32);
+    float* inv = (float*)ws;
+    if (lhs_dtype == QMM_F32)
+        q4k_prep_lhs_kernel<float><<<dim3((unsigned)m), dim3(256), 0, s>>>((const float*)lhs, (int)k, a16, a16_lo, asum, inv);
+    else
+        q4k_prep_lhs_kernel<uint16_t><<<dim3((unsigned)m), dim3(256), 0, s>>>((const uint16_t*)lhs, (int)k, a16, nullptr, asum, inv);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int tiles_m = (int)((m + BM - 1) / BM), tiles_n = (int)((n + BN - 1) / BN);
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    dim3 grid((unsigned)(per_xcd * 8)), block(512);
+    if (lhs_dtype == QMM_F32)
+        gemm_q4_k_kernel<2><<<grid, block, 0, s>>>(w, a16, a16_lo, asum, inv, out, (int)m, (int)n, (int)k, tiles_m, tiles_n);
+    else
+        gemm_q4_k_kernel<1><<<grid, block, 0, s>>>(w, a16, nullptr, asum, inv, out, (int)m, (int)n, (int)k, tiles_m, tiles_n);
+    return hipGetLastError();
+}
+
+}  // namespace qmm

@@ -147,6 +147,7 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     (void)n;
     if (m <= 0 || k <= 0) return 0;
     if (encoding == QMM_Q4_0) return q8_planes(nullptr, m, k).bytes;
+    if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, k);
     return 0;
 }
 
@@ -209,6 +210,9 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         }
         return QMM_OK;
     }
+
+    if (encoding == QMM_Q4_K && m > 16)
+        return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");
 
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         int mt = (int)(m - m0 < 16 ? m - m0 : 16);

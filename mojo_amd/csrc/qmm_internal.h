@@ -33,6 +33,11 @@ hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m,
 hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                             const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                             int64_t ldo, hipStream_t s);
+// Prefill-shape kernels (m > 16).
+int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
+hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                            float* out, void* workspace, hipStream_t s);
+
 hipError_t launch_block_dots_q4_0(const uint8_t* a_q8, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                   int32_t* out, hipStream_t s);
 

@@ -170,3 +170,38 @@ def test_leading_dims_broadcast():
     got = qmatmul(QE.Q4_K, None, gpu(a).reshape(2, 3, 512), gpu(wq))
     assert got.shape == (2, 3, 64)
     assert_close(got, want, "leading dims")
+
+
+# ------------------------------------------------------------------ prefill shapes (m > 16)
+@pytest.mark.parametrize("m,n,k", [(128, 256, 256), (17, 40, 512), (200, 300, 1024), (256, 512, 4096), (130, 64, 2048)])
+def test_q4_k_gemm_bf16_lhs(m, n, k):
+    """bf16 lhs (exact in the kernel's fp16 operands): against the fp32-weight oracle and fp64 truth."""
+    w, a = synth(11, n, k, m)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq)
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a).to(torch.bfloat16), gpu(wq))
+    assert_close(got, want, f"Q4_K GEMM {m}x{n}x{k} vs fp32 oracle")
+    assert_close(got, truth, f"Q4_K GEMM {m}x{n}x{k} vs fp64 truth")
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 128, 512), (33, 64, 256)])
+def test_q4_k_gemm_f32_lhs(m, n, k):
+    w, a = synth(12, n, k, m)
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_K GEMM fp32 lhs {m}x{n}x{k}")
+
+
+def test_q4_k_gemm_wide_range_lhs():
+    """Rows of very different magnitude: the per-row power-of-two scaling keeps fp16 operands exact."""
+    w, a = synth(13, 96, 512, 40)
+    a *= np.logspace(-6, 5, 40, dtype=np.float32)[:, None]
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a).to(torch.bfloat16), gpu(wq)).cpu().numpy()
+    scale = np.abs(truth).max(axis=1, keepdims=True)
+    assert np.all(np.abs(got - truth) <= 1e-4 * scale + 1e-3 * np.abs(truth))
