@@ -1,0 +1,118 @@
+"""C-ABI surface and host-side (Python) logic, runnable without a GPU: no kernel is launched."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import mojo_amd
+from mojo_amd import QuantizationConfig, QuantizationEncoding as QE, _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qmm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(_lib.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 11
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in include/qmm.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signatures out of step with the header"
+
+
+def test_block_params_and_errors_from_c():
+    lib = _lib.load()
+    assert lib.qmm_version() >= 100
+    e, b = C.c_int64(), C.c_int64()
+    for code, want in ((0, (32, 18)), (1, (256, 144)), (2, (256, 210)), (8, (32, 34))):
+        assert lib.qmm_block_params(code, C.byref(e), C.byref(b)) == 0
+        assert (e.value, b.value) == want
+    assert lib.qmm_block_params(3, C.byref(e), C.byref(b)) == -1  # GPTQ has no fixed block
+    assert b"no block layout" in lib.qmm_last_error()
+    assert lib.qmm_block_params(0, None, None) == -1
+
+
+def test_argument_validation_happens_before_any_launch():
+    """Every invalid-argument status is produced on the host; pointers here are never dereferenced."""
+    lib = _lib.load()
+    fake = C.c_void_p(0x1000)
+    rhs = (C.c_void_p * 1)(0x2000)
+
+    def matmul(enc, m, k, n, cfg=None, n_rhs=1, lhs=fake, dt=0, ws=None, ws_bytes=0, rhs_arr=rhs):
+        return lib.qmm_matmul(enc, cfg, lhs, dt, m, k, rhs_arr, n_rhs, n, fake, ws, ws_bytes, 0, None)
+
+    assert matmul(1, 1, 4100, 8) == -1 and b"multiple of the block size" in lib.qmm_last_error()
+    assert matmul(1, 0, 4096, 8) == -1 and b"positive" in lib.qmm_last_error()
+    assert matmul(1, 1, 4096, 8, lhs=None) == -1
+    assert matmul(7, 1, 4096, 8) == -1 and b"unknown encoding" in lib.qmm_last_error()
+    assert matmul(1, 1, 4096, 8, dt=2) == -1  # fp16 lhs is not part of the contract
+    assert matmul(1, 1, 4096, 8, n_rhs=2) == -1
+    assert matmul(1, 1, 4096, 8, lhs=C.c_void_p(0x1004)) == -1 and b"aligned" in lib.qmm_last_error()
+    assert matmul(1, 1, 4096, 8, rhs_arr=(C.c_void_p * 1)(0x2008)) == -1  # Q4_K blocks need 16-byte alignment
+    assert matmul(0, 2, 4096, 8) == -4 and b"workspace" in lib.qmm_last_error()  # Q4_0 needs its Q8_0 planes
+    assert matmul(3, 1, 4096, 8) == -1 and b"GPTQ" in lib.qmm_last_error()
+    bad = _lib.GptqConfig(8, 128, 0, 1)
+    rhs3 = (C.c_void_p * 3)(0x2000, 0x3000, 0x4000)
+    assert matmul(3, 1, 4096, 8, cfg=C.byref(bad), n_rhs=3, rhs_arr=rhs3) == -2
+    for cfg in (_lib.GptqConfig(4, 128, 1, 1), _lib.GptqConfig(4, 128, 0, 0)):
+        assert matmul(3, 1, 4096, 8, cfg=C.byref(cfg), n_rhs=3, rhs_arr=rhs3) == -2
+    assert matmul(3, 1, 4096, 8, cfg=C.byref(_lib.GptqConfig(4, 100, 0, 1)), n_rhs=3, rhs_arr=rhs3) == -1
+    assert lib.qmm_dequantize(1, fake, 4, 100, fake, 0, None) == -1
+    assert lib.qmm_dequantize(8, fake, 4, 256, fake, 0, None) == -1
+    assert lib.qmm_quantize(1, fake, 0, 256, fake, None) == -1
+    assert lib.qmm_matmul_workspace_bytes(0, 0, 16, 4096, 4096) == 16 * 4096 + 2 * 16 * 128 * 4
+    assert lib.qmm_matmul_workspace_bytes(1, 0, 4, 4096, 4096) == 0
+    assert lib.qmm_matmul_workspace_bytes(1, 1, 2048, 14336, 4096) >= 2048 * 4096 * 2
+
+
+def test_quantization_encoding_metadata():
+    assert QE.Q4_0.block_parameters == mojo_amd.BlockParameters(32, 18)
+    assert QE.Q4_K.block_parameters.block_size == 144 and QE.Q6_K.block_parameters.block_size == 210
+    assert QE.Q4_K.is_gguf and QE.Q6_K.is_gguf and QE.Q4_0.is_gguf and not QE.GPTQ.is_gguf
+    assert QE.Q4_K.name == "Q4_K" and QE.GPTQ.code == 3
+    assert QE.Q4_K.packed_row_bytes(4096) == 2304 and QE.Q6_K.packed_row_bytes(4096) == 3360
+    with pytest.raises(ValueError):
+        QE.Q4_K.packed_row_bytes(4100)
+    with pytest.raises(ValueError):
+        QE.GPTQ.block_parameters
+    cfg = QuantizationConfig()
+    assert (cfg.quant_method, cfg.bits, cfg.group_size, cfg.desc_act, cfg.sym) == ("gptq", 4, 128, False, True)
+
+
+def test_host_shim_rejects_bad_calls_without_touching_the_gpu():
+    a = torch.zeros(1, 256)
+    w = torch.zeros(4, 144, dtype=torch.uint8)
+    with pytest.raises(ValueError, match="GPU"):
+        mojo_amd.qmatmul(QE.Q4_K, None, a, w)  # no CPU fallback, by design
+    with pytest.raises(TypeError):
+        mojo_amd.qmatmul("Q4_K", None, a, w)
+    with pytest.raises(TypeError):
+        mojo_amd.qmatmul(QE.Q4_K, None, np.zeros((1, 256), np.float32), w)
+    with pytest.raises(ValueError, match="GPU"):
+        mojo_amd.dequantize(QE.Q4_K, w)
+    with pytest.raises(ValueError, match="GPU"):
+        mojo_amd.quantize(QE.Q4_0, a)
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(ROOT, "mojo_amd", "does_not_exist.so"))
+    with pytest.raises(RuntimeError, match="not built"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    """The shipped package and the C sources must not reference the oracle directory."""
+    for base, _, files in os.walk(os.path.join(ROOT, "mojo_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(base, f), errors="ignore").read()
+                assert "import oracle" not in text and "qmm_oracle" not in text and "oracle/" not in text, f
