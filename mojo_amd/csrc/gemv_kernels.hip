@@ -317,6 +317,7 @@ static bool q4k_use_valu(int m) {
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
     if (!q4k_use_valu(m)) return launch_gemv_q4_k_mfma(a, a_dtype, w, m, n, k, out, ldo, s);
+    if (m <= 2 && !getenv("QMM_Q4K_V1")) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
     dim3 grid((unsigned)((n + 3) / 4)), block(256);
 #define CALL(MT)                                                                                          \
     if (a_dtype == QMM_F32)                                                                               \
