@@ -64,6 +64,19 @@ class Gemv:
         _lib.check(rc, "qmm_matmul")
 
 
+class ReadProbe:
+    """qmm_read_probe over an existing tensor: the plain-read yardstick for the same bytes."""
+
+    def __init__(self, t: torch.Tensor):
+        self.lib = _lib.load()
+        self.t = t
+        self.nbytes = t.numel() * t.element_size() // 16 * 16
+
+    def launch(self, stream_ptr: int) -> None:
+        _lib.check(self.lib.qmm_read_probe(C.c_void_p(self.t.data_ptr()), self.nbytes, C.c_void_p(stream_ptr)),
+                   "qmm_read_probe")
+
+
 def make_weight(enc: QE, n: int, k: int, gen: torch.Generator) -> torch.Tensor:
     w = torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02
     return quantize(enc, w)
@@ -233,6 +246,11 @@ def extra_timings(layers, acts, gen):
         b = alg_bytes(QE.Q4_K, m, n, k)
         per_shape[f"{name}_{n}x{k}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1)}
     out["q4_k_per_shape"] = per_shape
+    # the same seven weight tensors per layer, only read (no arithmetic): what the memory system gives
+    graphs = [capture([ReadProbe(w) for w in lw]) for lw in layers]
+    dev_s, _ = time_graphs(graphs, 100, 10)
+    wbytes = sum(n * QE.Q4_K.packed_row_bytes(k) for _, n, k in PROJ)
+    out["plain_read_same_set"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(wbytes * 100 / dev_s / 1e9, 1)}
     # M=4 over the same set
     if m == 1:
         acts4 = {k: torch.randn((4, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}

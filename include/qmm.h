@@ -72,6 +72,15 @@ int qmm_block_params(int encoding, int64_t* elements_per_block, int64_t* bytes_p
 int qmm_device_info(int32_t* compute_units, int32_t* clock_khz);
 
 /*
+ * Roofline calibration: a plain read of `bytes` bytes (16-byte coalesced loads, grid-stride,
+ * nothing written) on `stream`.  Timing it gives the read bandwidth this device sustains at a
+ * given footprint, and profiling it gives the FETCH_SIZE a known number of bytes produces.  The
+ * reference times its kernels with its own benchmark harness (stdlib/docs/bencher/Bench.md);
+ * this is the device-side yardstick for the same purpose.  `buf` must be 16-byte aligned.
+ */
+int qmm_read_probe(const void* buf, int64_t bytes, void* stream);
+
+/*
  * Block unpack / dequantise: rhs uint8[n, k/epb*bpb] -> out[n, k] in
  * out_dtype (QMM_F32 or QMM_BF16, bf16 by round-to-nearest-even as
  * stdlib/src/builtin/simd.mojo:3279-3300).  Q4_0, Q4_K, Q6_K.

@@ -94,6 +94,12 @@ int qmm_device_info(int32_t* compute_units, int32_t* clock_khz) {
     return QMM_OK;
 }
 
+int qmm_read_probe(const void* buf, int64_t bytes, void* stream) {
+    if (!buf || bytes < 16) return fail(QMM_ERR_INVALID, "qmm_read_probe: needs a buffer of at least 16 bytes");
+    if (!aligned(buf, 16)) return fail(QMM_ERR_INVALID, "qmm_read_probe: buffer must be 16-byte aligned");
+    return hip_status(qmm::launch_read_probe(buf, bytes, (hipStream_t)stream), "qmm_read_probe");
+}
+
 int qmm_dequantize(int encoding, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype, void* stream) {
     int64_t epb, bpb;
     if (encoding == QMM_Q8_0 || !block_params(encoding, epb, bpb))

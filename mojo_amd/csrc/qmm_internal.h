@@ -9,6 +9,7 @@
 
 namespace qmm {
 
+hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
 hipError_t launch_dequant(int enc, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
                           hipStream_t s);
 hipError_t launch_dequant_gptq(const void* qweight, const void* scales, const void* qzeros,
