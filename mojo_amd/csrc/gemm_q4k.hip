@@ -18,6 +18,8 @@
 // loaded by the lanes that use them and unpacked in registers.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -144,38 +146,43 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    // lhs chunk loader: 128 rows x 64 halfs = 1024 x 16 bytes; 512 threads x 2
-    const int a_row = tid >> 2, a_seg = tid & 3;  // rows a_row and a_row (+0), two 16-byte segments each
-    auto a_src = [&](const _Float16* base, int chunk, int seg) {
-        int row = m0 + a_row;
-        if (row >= m) row = m - 1;
-        return (const uint4*)(base + (int64_t)row * k + (int64_t)chunk * 64 + seg * 8);
-    };
-    uint4 a_pref[NPART][2];
-    auto a_load = [&](int chunk) {
-        a_pref[0][0] = *a_src(a16, chunk, a_seg);
-        a_pref[0][1] = *a_src(a16, chunk, a_seg + 4);
-        if constexpr (NPART == 2) {
-            a_pref[1][0] = *a_src(a16_lo, chunk, a_seg);
-            a_pref[1][1] = *a_src(a16_lo, chunk, a_seg + 4);
-        }
-    };
-    auto a_store = [&](int buf) {
-#pragma unroll
-        for (int p = 0; p < NPART; p++) {
-            *(uint4*)(&lds_a[buf][p][a_row * A_STRIDE + a_seg * 8]) = a_pref[p][0];
-            *(uint4*)(&lds_a[buf][p][a_row * A_STRIDE + (a_seg + 4) * 8]) = a_pref[p][1];
-        }
-    };
+    // lhs chunk loader: 128 rows x 64 halfs = 1024 x 16 bytes; 512 threads x 2.  Base pointers are
+    // fixed per thread; a step only adds the chunk offset.  Two register sets (parity of the
+    // step) keep two steps of loads in flight.
+    const int nsteps = nblk * 4;
+    const int a_row = tid >> 2, a_seg = tid & 3;
+    const int64_t a_off = (int64_t)min(m0 + a_row, m - 1) * k + a_seg * 8;
+    const uint4* a_base0 = (const uint4*)(a16 + a_off);
+    const uint4* a_base1 = NPART == 2 ? (const uint4*)(a16_lo + a_off) : nullptr;
+    // register sets as plain variables (set, part, segment)
+    uint4 ax0_p0s0, ax0_p0s1, ax0_p1s0, ax0_p1s1, ax1_p0s0, ax1_p0s1, ax1_p1s0, ax1_p1s1;
+    ax0_p1s0 = ax0_p1s1 = ax1_p1s0 = ax1_p1s1 = make_uint4(0, 0, 0, 0);
+    _Float16* a_dst = &lds_a[0][0][a_row * A_STRIDE + a_seg * 8];
+#define QMM_A_LOAD(SET, STEP)                                         \
+    do {                                                              \
+        const int chunk_ = min((STEP), nsteps - 1);                   \
+        SET##_p0s0 = a_base0[chunk_ * 8];                             \
+        SET##_p0s1 = a_base0[chunk_ * 8 + 4];                         \
+        if constexpr (NPART == 2) {                                   \
+            SET##_p1s0 = a_base1[chunk_ * 8];                         \
+            SET##_p1s1 = a_base1[chunk_ * 8 + 4];                     \
+        }                                                             \
+    } while (0)
+#define QMM_A_STORE(SET, BUF)                                                     \
+    do {                                                                          \
+        _Float16* d_ = a_dst + (size_t)(BUF) * NPART * BM * A_STRIDE;             \
+        *(uint4*)d_ = SET##_p0s0;                                                 \
+        *(uint4*)(d_ + 32) = SET##_p0s1;                                          \
+        if constexpr (NPART == 2) {                                               \
+            *(uint4*)(d_ + BM * A_STRIDE) = SET##_p1s0;                           \
+            *(uint4*)(d_ + BM * A_STRIDE + 32) = SET##_p1s1;                      \
+        }                                                                         \
+    } while (0)
 
     // this lane's two weight columns
-    const uint8_t* wcol[2];
-#pragma unroll
-    for (int ni = 0; ni < 2; ni++) {
-        int col = n0 + wn * 64 + ni * 32 + nl;
-        if (col >= n) col = n - 1;
-        wcol[ni] = w + (int64_t)col * row_bytes;
-    }
+    const uint8_t* wcol0 = w + (int64_t)min(n0 + wn * 64 + nl, n - 1) * row_bytes;
+    const uint8_t* wcol1 = w + (int64_t)min(n0 + wn * 64 + 32 + nl, n - 1) * row_bytes;
+    const int q_lane_off = 16 + 16 * g;
 
     float16v acc[2][2], P[2][2];
 #pragma unroll
@@ -183,43 +190,66 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
 #pragma unroll
         for (int ni = 0; ni < 2; ni++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[mi][ni][r] = 0.0f;
+            for (int r = 0; r < 16; r++) {
+                acc[mi][ni][r] = 0.0f;
+                P[mi][ni][r] = 0.0f;
+            }
 
-    uint4 q_pref[2];
-    auto q_load = [&](int blk, int c) {
-#pragma unroll
-        for (int ni = 0; ni < 2; ni++) q_pref[ni] = *(const uint4*)(wcol[ni] + (int64_t)blk * Q4_K_BPB + 16 + 32 * c + 16 * g);
+    uint4 qx0_c0, qx0_c1, qx1_c0, qx1_c1;  // code units of the two columns, two register sets
+#define QMM_Q_LOAD(SET, STEP)                                                              \
+    do {                                                                                   \
+        const int st_ = min((STEP), nsteps - 1);                                           \
+        const int off_ = (st_ >> 2) * Q4_K_BPB + 32 * (st_ & 3) + q_lane_off;              \
+        SET##_c0 = *(const uint4*)(wcol0 + off_);                                          \
+        SET##_c1 = *(const uint4*)(wcol1 + off_);                                          \
+    } while (0)
+
+    // block headers and sub-block sums are fetched one super-block ahead
+    uint4 hdr_n0, hdr_n1, as_n = make_uint4(0, 0, 0, 0);
+    const uint4* as_src = (const uint4*)(asum + (int64_t)min(m0 + (tid >> 1), m - 1) * nblk * 16 + (tid & 1) * 8);
+    auto hdr_prefetch = [&](int blk) {
+        const int bc = min(blk, nblk - 1);
+        hdr_n0 = *(const uint4*)(wcol0 + bc * Q4_K_BPB);
+        hdr_n1 = *(const uint4*)(wcol1 + bc * Q4_K_BPB);
     };
-
-    a_load(0);
-    q_load(0, 0);
-    a_store(0);
+    auto as_prefetch = [&](int blk) {
+        if (tid < 256) as_n = as_src[min(blk, nblk - 1) * 2];
+    };
+    hdr_prefetch(0);
+    as_prefetch(0);
+    QMM_A_LOAD(ax0, 0);
+    QMM_Q_LOAD(qx0, 0);
+    QMM_Q_LOAD(qx1, 1);
+    QMM_A_STORE(ax0, 0);
+    if (tid < 256) *(uint4*)(&lds_s[(tid >> 1) * 16 + (tid & 1) * 8]) = as_n;
+    QMM_A_LOAD(ax1, 1);
+    QMM_A_LOAD(ax0, 2);
+    as_prefetch(1);
     __syncthreads();
 
-    const int nsteps = nblk * 4;
     float dscale[2] = {0.f, 0.f};
     uint32_t sp[2][8];
-    for (int blk = 0; blk < nblk; blk++) {
-#pragma unroll
-      for (int c = 0; c < 4; c++) {  // compile-time chunk index: register arrays stay in registers
+    // One step = one 64-wide chunk c of super-block blk.  The chunk index is a compile-time
+    // constant so that register arrays and the parity-selected prefetch sets stay in registers.
+    auto do_step = [&](int blk, auto CC) {
+        constexpr int c = decltype(CC)::value;
         const int step = blk * 4 + c, buf = c & 1;
-        const uint4 qc[2] = {q_pref[0], q_pref[1]};
-        if (step + 1 < nsteps) {
-            a_load(step + 1);
-            q_load((step + 1) >> 2, (step + 1) & 3);
+        uint4 qc0, qc1;
+        if constexpr (c & 1) {
+            qc0 = qx1_c0; qc1 = qx1_c1;
+            QMM_Q_LOAD(qx1, step + 2);
+        } else {
+            qc0 = qx0_c0; qc1 = qx0_c1;
+            QMM_Q_LOAD(qx0, step + 2);
         }
         if (c == 0) {
-            // ---- super-block start: sub-block sums to LDS, header decode, min-term products
-            if (tid < 256) {
-                int row = m0 + (tid >> 1);
-                if (row >= m) row = m - 1;
-                *(uint4*)(&lds_s[(tid >> 1) * 16 + (tid & 1) * 8]) =
-                    *(const uint4*)(asum + ((int64_t)row * nblk + blk) * 16 + (tid & 1) * 8);
-            }
+            // ---- super-block start: header decode, min-term products (sums already in lds_s)
+            const uint4 hdr_c0 = hdr_n0, hdr_c1 = hdr_n1;
+            hdr_prefetch(blk + 1);
             uint32_t dmn_hi[2][4], dmn_lo[2][4];
 #pragma unroll
             for (int ni = 0; ni < 2; ni++) {
-                const uint4 hdr = *(const uint4*)(wcol[ni] + (int64_t)blk * Q4_K_BPB);
+                const uint4 hdr = ni == 0 ? hdr_c0 : hdr_c1;
                 dscale[ni] = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo24;
                 const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
                 const uint32_t sc_lo = s0 & 0x3F3F3F3Fu, sc_hi = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
@@ -245,7 +275,6 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
                     dmn_lo[ni][i] = pk_fma(ndm, mp[i], dmn_hi[ni][i] ^ 0x80008000u);
                 }
             }
-            __syncthreads();  // lds_s visible (also orders this step's lds_a reads after the previous stores)
 #pragma unroll
             for (int mi = 0; mi < 2; mi++) {
                 // A operand: lanes g=0 carry the hi parts of the 8 sub-block sums, g=1 the lo parts
@@ -273,7 +302,8 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
             half8 bfrag[2];
 #pragma unroll
             for (int ni = 0; ni < 2; ni++) {
-                const uint32_t x0 = (f & 1) ? qc[ni].z : qc[ni].x, x1 = (f & 1) ? qc[ni].w : qc[ni].y;
+                const uint4 qq = ni == 0 ? qc0 : qc1;
+                const uint32_t x0 = (f & 1) ? qq.z : qq.x, x1 = (f & 1) ? qq.w : qq.y;
                 const uint32_t mask = (f & 2) ? M2 : M1;
                 const uint32_t s = sp[ni][2 * c + (f >> 1)];
                 bfrag[ni] = pack4(pk_mul(x0 & mask, s), pk_mul((x0 >> 8) & mask, s), pk_mul(x1 & mask, s),
@@ -290,6 +320,15 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
                 }
             }
         }
+        // Ask the scheduler to interleave the unpack arithmetic with the matrix-core instructions
+        // (one MFMA, then a group of vector ALU ops), so the two pipes run concurrently inside a
+        // wavefront instead of in two phases.
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // 6 VALU
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+        }
         if (c == 3) {
 #pragma unroll
             for (int mi = 0; mi < 2; mi++)
@@ -298,13 +337,30 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
 #pragma unroll
                     for (int r = 0; r < 16; r++) acc[mi][ni][r] = fmaf(dscale[ni], P[mi][ni][r], acc[mi][ni][r]);
         }
-        if (step + 1 < nsteps) {
-            a_store(buf ^ 1);
-            if (c != 3) __syncthreads();  // a super-block start has its own barrier
+        // next step's lhs chunk to the other LDS buffer; its register set then takes the loads of step + 3
+        if constexpr (c & 1) {
+            QMM_A_STORE(ax0, buf ^ 1);
+            QMM_A_LOAD(ax0, step + 3);
+        } else {
+            QMM_A_STORE(ax1, buf ^ 1);
+            QMM_A_LOAD(ax1, step + 3);
         }
-      }
+        if (c == 3) {  // next super-block's sub-block sums
+            if (tid < 256) *(uint4*)(&lds_s[(tid >> 1) * 16 + (tid & 1) * 8]) = as_n;
+            as_prefetch(blk + 2);
+        }
+        __syncthreads();
+    };
+    for (int blk = 0; blk < nblk; blk++) {
+        do_step(blk, std::integral_constant<int, 0>{});
+        do_step(blk, std::integral_constant<int, 1>{});
+        do_step(blk, std::integral_constant<int, 2>{});
+        do_step(blk, std::integral_constant<int, 3>{});
     }
 
+#undef QMM_A_LOAD
+#undef QMM_A_STORE
+#undef QMM_Q_LOAD
     // ---- epilogue: undo the row scale, store
 #pragma unroll
     for (int mi = 0; mi < 2; mi++) {
