@@ -64,6 +64,28 @@ class Gemv:
         _lib.check(rc, "qmm_matmul")
 
 
+class GptqMatmul:
+    """One preallocated GPTQ qmm_matmul call on (qweight, scales, qzeros)."""
+
+    def __init__(self, tensors, a: torch.Tensor, group: int = 128):
+        self.lib = _lib.load()
+        self.t, self.a = tensors, a
+        self.m, self.k = a.shape
+        self.n = tensors[0].shape[1]
+        self.out = torch.empty((self.m, self.n), dtype=torch.float32, device=a.device)
+        self.dt = _lib.QMM_F32 if a.dtype == torch.float32 else _lib.QMM_BF16
+        self.need = self.lib.qmm_matmul_workspace_bytes(QE.GPTQ.code, self.dt, self.m, self.n, self.k)
+        self.ws = torch.empty((max(self.need, 1),), dtype=torch.uint8, device=a.device)
+        self.cfg = _lib.GptqConfig(4, group, 0, 1)
+        self.ptrs = (C.c_void_p * 3)(*[t.data_ptr() for t in tensors[:3]])
+
+    def launch(self, stream_ptr: int) -> None:
+        rc = self.lib.qmm_matmul(QE.GPTQ.code, C.byref(self.cfg), C.c_void_p(self.a.data_ptr()), self.dt, self.m,
+                                 self.k, self.ptrs, 3, self.n, C.c_void_p(self.out.data_ptr()),
+                                 C.c_void_p(self.ws.data_ptr()), self.need, 0, C.c_void_p(stream_ptr))
+        _lib.check(rc, "qmm_matmul")
+
+
 class ReadProbe:
     """qmm_read_probe over an existing tensor: the plain-read yardstick for the same bytes."""
 
@@ -275,6 +297,14 @@ def extra_timings(layers, acts, gen):
     tf = 2 * 2048 * 14336 * 4096 / us / 1e6
     out["q4_k_prefill_m2048"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
     del wp
+    # cfg5, second weight set: GPTQ (group 128) prefill on the same shape
+    wg = quantize_gptq(torch.randn((14336, 4096), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
+    g = capture([GptqMatmul(wg, ab)])
+    dev_s, _ = time_graphs([g], 20, 3)
+    us = dev_s * 1e6 / 20
+    tf = 2 * 2048 * 14336 * 4096 / us / 1e6
+    out["gptq_prefill_m2048"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
+    del wg
     # cfg1 / cfg2: Q4_0 with Q8_0 activations
     for tag, mm, n, k, copies in (("q4_0_m1_4096x4096", 1, 4096, 4096, 32), ("q4_0_m16_14336x4096", 16, 14336, 4096, 10)):
         am = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen)

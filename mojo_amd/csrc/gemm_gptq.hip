@@ -1,0 +1,321 @@
+// GPTQ (4-bit, AutoGPTQ v1 packing) prefill kernel for m > 16 lhs rows: the same
+// matrix-core scheme as the Q4_K prefill kernel, on the [K/8, N] int32 layout.
+//
+// A packed dword holds 8 consecutive k of one output column.  With the lhs stored in
+// the order (0,4,1,5,2,6,3,7) inside each 8-group and its odd columns pre-multiplied
+// by 1/16, the four fp16 pairs  x & 0x000F000F,  x & 0x00F000F0,  (x>>8) & 0x000F000F,
+// (x>>8) & 0x00F000F0  are the matrix-core B operand directly: fp16 subnormals q*2^-24
+// (or 16q*2^-24), no multiply needed because the scale is per group, not per 32.
+// Per group g the matrix cores produce  P[m][n] = sum_k a[m][k]*q[k][n]  exactly (fp32
+// sums), and the lanes apply  acc += scale[g][n] * P.  The zero-point term
+// -scale*zero * sum_k a[m][k]  is a second small matrix product over the 32-wide
+// sub-block sums of a 256-column chunk, with scale*zero split exactly into two fp16
+// values; zero = stored + 1 (AutoGPTQ v1 convention).
+//
+// Tile shape and data movement as in the Q4_K kernel: 128 x 256 outputs per workgroup of
+// 8 wavefronts, lhs chunks through double-buffered LDS, weights loaded by the lanes that
+// use them (a wavefront load covers 32 consecutive columns of two k8 rows: 128-byte runs).
+#include <stdlib.h>
+
+#include <type_traits>
+
+#include "gemm_lhs.h"
+#include "qmm_internal.h"
+
+namespace qmm {
+
+namespace {
+
+constexpr int BM = 128, BN = 256;
+constexpr int A_STRIDE = 72;
+constexpr float kTwo24 = 16777216.0f;
+
+}  // namespace
+
+// GB = groups per 256-column chunk (group size 256 / GB: 256, 128 or 64).
+template <int NPART, int GB>
+__global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restrict__ qweight,
+                                                        const uint16_t* __restrict__ scales,
+                                                        const uint32_t* __restrict__ qzeros,
+                                                        const _Float16* __restrict__ a16,
+                                                        const _Float16* __restrict__ a16_lo,
+                                                        const _Float16* __restrict__ asum, const float* __restrict__ inv,
+                                                        float* __restrict__ out, int m, int n, int k, int tiles_m,
+                                                        int tiles_n) {
+    __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][NPART][BM * A_STRIDE];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_s[BM * 16];
+    constexpr int SPG = 4 / GB;  // 64-wide steps per group
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 2, wn = wave & 3;
+    const int nl = lane & 31, g = lane >> 5;
+    const int nblk = k >> 8;
+
+    int tile_m, tile_n;
+    {
+        const int total = tiles_m * tiles_n;
+        const int per_xcd = (total + 7) / 8;
+        const int o = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+        if (o >= total) return;
+        const int gm = 2, span = gm * tiles_n;
+        const int grp = o / span, rem = o - grp * span;
+        const int rows_here = min(gm, tiles_m - grp * gm);
+        tile_n = rem / rows_here;
+        tile_m = grp * gm + rem - tile_n * rows_here;
+    }
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int nsteps = nblk * 4;
+    const int a_row = tid >> 2, a_seg = tid & 3;
+    const int64_t a_off = (int64_t)min(m0 + a_row, m - 1) * k + a_seg * 8;
+    const uint4* a_base0 = (const uint4*)(a16 + a_off);
+    const uint4* a_base1 = NPART == 2 ? (const uint4*)(a16_lo + a_off) : nullptr;
+    uint4 ax0_p0s0, ax0_p0s1, ax0_p1s0, ax0_p1s1, ax1_p0s0, ax1_p0s1, ax1_p1s0, ax1_p1s1;
+    ax0_p1s0 = ax0_p1s1 = ax1_p1s0 = ax1_p1s1 = make_uint4(0, 0, 0, 0);
+    _Float16* a_dst = &lds_a[0][0][a_row * A_STRIDE + a_seg * 8];
+#define QMM_A_LOAD(SET, STEP)                                         \
+    do {                                                              \
+        const int chunk_ = min((STEP), nsteps - 1);                   \
+        SET##_p0s0 = a_base0[chunk_ * 8];                             \
+        SET##_p0s1 = a_base0[chunk_ * 8 + 4];                         \
+        if constexpr (NPART == 2) {                                   \
+            SET##_p1s0 = a_base1[chunk_ * 8];                         \
+            SET##_p1s1 = a_base1[chunk_ * 8 + 4];                     \
+        }                                                             \
+    } while (0)
+#define QMM_A_STORE(SET, BUF)                                                     \
+    do {                                                                          \
+        _Float16* d_ = a_dst + (size_t)(BUF) * NPART * BM * A_STRIDE;             \
+        *(uint4*)d_ = SET##_p0s0;                                                 \
+        *(uint4*)(d_ + 32) = SET##_p0s1;                                          \
+        if constexpr (NPART == 2) {                                               \
+            *(uint4*)(d_ + BM * A_STRIDE) = SET##_p1s0;                           \
+            *(uint4*)(d_ + BM * A_STRIDE + 32) = SET##_p1s1;                      \
+        }                                                                         \
+    } while (0)
+
+    // this lane's two weight columns; the lane half g takes the odd k8 rows
+    const int col0 = min(n0 + wn * 64 + nl, n - 1), col1 = min(n0 + wn * 64 + 32 + nl, n - 1);
+    // Loads are written as (wave-uniform pointer)[per-lane 32-bit offset] so that the address
+    // arithmetic stays in scalar registers.
+    const int64_t ldq = n;  // dwords per k8 row
+    const int qoff0 = g * n + col0, qoff1 = g * n + col1;
+
+    float16v acc[2][2], P[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[mi][ni][r] = 0.0f;
+                P[mi][ni][r] = 0.0f;
+            }
+
+    // code dwords of the two columns (4 k8 rows each), two register sets
+    uint32_t qx0_a0, qx0_a1, qx0_a2, qx0_a3, qx0_b0, qx0_b1, qx0_b2, qx0_b3;
+    uint32_t qx1_a0, qx1_a1, qx1_a2, qx1_a3, qx1_b0, qx1_b1, qx1_b2, qx1_b3;
+#define QMM_Q_LOAD(SET, STEP)                                                       \
+    do {                                                                            \
+        const uint32_t* r_ = qweight + (int64_t)min((STEP), nsteps - 1) * 8 * ldq;  \
+        SET##_a0 = r_[qoff0];                                                       \
+        SET##_a1 = (r_ + 2 * ldq)[qoff0];                                           \
+        SET##_a2 = (r_ + 4 * ldq)[qoff0];                                           \
+        SET##_a3 = (r_ + 6 * ldq)[qoff0];                                           \
+        SET##_b0 = r_[qoff1];                                                       \
+        SET##_b1 = (r_ + 2 * ldq)[qoff1];                                           \
+        SET##_b2 = (r_ + 4 * ldq)[qoff1];                                           \
+        SET##_b3 = (r_ + 6 * ldq)[qoff1];                                           \
+    } while (0)
+
+    // group scales and zero words of the next 256-column chunk
+    uint32_t sc_n[2][GB], zw_n[2][GB];
+    const int zshift0 = 4 * (col0 & 7), zshift1 = 4 * (col1 & 7);
+    const int ldz = n >> 3, zcol0 = col0 >> 3, zcol1 = col1 >> 3;
+    auto hdr_prefetch = [&](int blk) {
+        const int64_t g0 = (int64_t)min(blk, nblk - 1) * GB;
+#pragma unroll
+        for (int i = 0; i < GB; i++) {
+            const uint16_t* sr = scales + (g0 + i) * n;
+            const uint32_t* zr = qzeros + (g0 + i) * ldz;
+            sc_n[0][i] = sr[col0];
+            sc_n[1][i] = sr[col1];
+            zw_n[0][i] = zr[zcol0];
+            zw_n[1][i] = zr[zcol1];
+        }
+    };
+    uint4 as_n = make_uint4(0, 0, 0, 0);
+    const uint4* as_src = (const uint4*)(asum + (int64_t)min(m0 + (tid >> 1), m - 1) * nblk * 16 + (tid & 1) * 8);
+    auto as_prefetch = [&](int blk) {
+        if (tid < 256) as_n = as_src[min(blk, nblk - 1) * 2];
+    };
+    hdr_prefetch(0);
+    as_prefetch(0);
+    QMM_A_LOAD(ax0, 0);
+    QMM_Q_LOAD(qx0, 0);
+    QMM_Q_LOAD(qx1, 1);
+    QMM_A_STORE(ax0, 0);
+    if (tid < 256) *(uint4*)(&lds_s[(tid >> 1) * 16 + (tid & 1) * 8]) = as_n;
+    QMM_A_LOAD(ax1, 1);
+    QMM_A_LOAD(ax0, 2);
+    as_prefetch(1);
+    __syncthreads();
+
+    float gscale[2][GB];
+    auto do_step = [&](int blk, auto CC) {
+        constexpr int c = decltype(CC)::value;
+        const int step = blk * 4 + c, buf = c & 1;
+        uint32_t qa[4], qb[4];
+        if constexpr (c & 1) {
+            qa[0] = qx1_a0; qa[1] = qx1_a1; qa[2] = qx1_a2; qa[3] = qx1_a3;
+            qb[0] = qx1_b0; qb[1] = qx1_b1; qb[2] = qx1_b2; qb[3] = qx1_b3;
+            QMM_Q_LOAD(qx1, step + 2);
+        } else {
+            qa[0] = qx0_a0; qa[1] = qx0_a1; qa[2] = qx0_a2; qa[3] = qx0_a3;
+            qb[0] = qx0_b0; qb[1] = qx0_b1; qb[2] = qx0_b2; qb[3] = qx0_b3;
+            QMM_Q_LOAD(qx0, step + 2);
+        }
+        if (c == 0) {
+            // ---- chunk start: group scales, zero-point term (sub-block sums already in lds_s)
+            uint32_t sz_hi[2][GB], sz_lo[2][GB];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++) {
+#pragma unroll
+                for (int i = 0; i < GB; i++) {
+                    const uint32_t sb = sc_n[ni][i] & 0xffffu;
+                    gscale[ni][i] = h2f((uint16_t)sb) * kTwo24;
+                    const float z = (float)(((zw_n[ni][i] >> (ni == 0 ? zshift0 : zshift1)) & 0xFu) + 1u);
+                    const uint32_t nsc = (sb ^ 0x8000u) * 0x00010001u;  // (-scale, -scale)
+                    const uint32_t zp = pack_half2(z, z);
+                    sz_hi[ni][i] = pk_mul(nsc, zp);
+                    sz_lo[ni][i] = pk_fma(nsc, zp, sz_hi[ni][i] ^ 0x80008000u);
+                }
+            }
+            hdr_prefetch(blk + 1);
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+                // A operand: lanes g=0 carry the hi parts of the 8 sub-block sums, g=1 the lo parts
+                const half8 av = *(const half8*)(&lds_s[(wm * 64 + mi * 32 + nl) * 16 + g * 8]);
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    // sub-block pair p (columns 64p..64p+63) belongs to group p*GB/4
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        av, pack4(sz_hi[ni][0], sz_hi[ni][GB / 4], sz_hi[ni][GB / 2], sz_hi[ni][3 * GB / 4]),
+                        acc[mi][ni], 0, 0, 0);
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        av, pack4(sz_lo[ni][0], sz_lo[ni][GB / 4], sz_lo[ni][GB / 2], sz_lo[ni][3 * GB / 4]),
+                        acc[mi][ni], 0, 0, 0);
+                }
+            }
+        }
+
+        // ---- one 64-wide chunk: four 16-wide operand slices, one packed dword per column each
+        const uint32_t M1 = 0x000F000Fu, M2 = 0x00F000F0u;
+#pragma unroll
+        for (int f = 0; f < 4; f++) {
+            half8 bfrag[2];
+            bfrag[0] = pack4(qa[f] & M1, qa[f] & M2, (qa[f] >> 8) & M1, (qa[f] >> 8) & M2);
+            bfrag[1] = pack4(qb[f] & M1, qb[f] & M2, (qb[f] >> 8) & M1, (qb[f] >> 8) & M2);
+#pragma unroll
+            for (int p = 0; p < NPART; p++) {
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++) {
+                    const half8 afrag = *(const half8*)(&lds_a[buf][p][(wm * 64 + mi * 32 + nl) * A_STRIDE + f * 16 + g * 8]);
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++)
+                        P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[ni], P[mi][ni], 0, 0, 0);
+                }
+            }
+        }
+        if constexpr ((c + 1) % SPG == 0) {  // group end: apply its scale
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        acc[mi][ni][r] = fmaf(gscale[ni][c / SPG], P[mi][ni][r], acc[mi][ni][r]);
+                        P[mi][ni][r] = 0.0f;
+                    }
+            // Pin the updated accumulators here.  Otherwise the compiler sinks these multiply-adds
+            // to the end of the chunk and keeps every group's P alive until then.
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) asm volatile("" : "+v"(acc[mi][ni]));
+        }
+        if constexpr (c & 1) {
+            QMM_A_STORE(ax0, buf ^ 1);
+            QMM_A_LOAD(ax0, step + 3);
+        } else {
+            QMM_A_STORE(ax1, buf ^ 1);
+            QMM_A_LOAD(ax1, step + 3);
+        }
+        if (c == 3) {  // next chunk's sub-block sums
+            if (tid < 256) *(uint4*)(&lds_s[(tid >> 1) * 16 + (tid & 1) * 8]) = as_n;
+            as_prefetch(blk + 2);
+        }
+        __syncthreads();
+    };
+    for (int blk = 0; blk < nblk; blk++) {
+        do_step(blk, std::integral_constant<int, 0>{});
+        do_step(blk, std::integral_constant<int, 1>{});
+        do_step(blk, std::integral_constant<int, 2>{});
+        do_step(blk, std::integral_constant<int, 3>{});
+    }
+#undef QMM_A_LOAD
+#undef QMM_A_STORE
+#undef QMM_Q_LOAD
+
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+            if (row < m) {
+                const float is = inv[row];
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    const int col = n0 + wn * 64 + ni * 32 + nl;
+                    if (col < n) out[(int64_t)row * n + col] = acc[mi][ni][r] * is;
+                }
+            }
+        }
+    }
+}
+
+bool gemm_gptq_supported(int64_t k, int group) {
+    return k % 256 == 0 && (group == 64 || group == 128 || group == 256);
+}
+
+int64_t gemm_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return lhs_planes(nullptr, lhs_dtype, m, k).bytes; }
+
+hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales,
+                            const uint32_t* qzeros, int64_t m, int64_t n, int64_t k, int group, float* out,
+                            void* workspace, hipStream_t s) {
+    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
+    hipError_t e = launch_prep_lhs<kLhsOrderGPTQ>(lhs, lhs_dtype, m, k, p, s);
+    if (e != hipSuccess) return e;
+    const int tiles_m = (int)((m + BM - 1) / BM), tiles_n = (int)((n + BN - 1) / BN);
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    dim3 grid((unsigned)(per_xcd * 8)), block(512);
+#define QMM_GPTQ_LAUNCH(GB_)                                                                                          \
+    do {                                                                                                              \
+        if (lhs_dtype == QMM_F32)                                                                                     \
+            gemm_gptq_kernel<2, GB_><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.a16_lo, p.asum, p.inv,  \
+                                                            out, (int)m, (int)n, (int)k, tiles_m, tiles_n);          \
+        else                                                                                                          \
+            gemm_gptq_kernel<1, GB_><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, nullptr, p.asum, p.inv,   \
+                                                            out, (int)m, (int)n, (int)k, tiles_m, tiles_n);          \
+    } while (0)
+    if (group == 256) QMM_GPTQ_LAUNCH(1);
+    else if (group == 128) QMM_GPTQ_LAUNCH(2);
+    else if (group == 64) QMM_GPTQ_LAUNCH(4);
+    else return hipErrorInvalidValue;
+#undef QMM_GPTQ_LAUNCH
+    return hipGetLastError();
+}
+
+}  // namespace qmm

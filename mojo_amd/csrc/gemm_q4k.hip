@@ -20,13 +20,10 @@
 
 #include <type_traits>
 
+#include "gemm_lhs.h"
 #include "qmm_internal.h"
 
 namespace qmm {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef float float16v __attribute__((ext_vector_type(16)));
 
 namespace {
 
@@ -34,82 +31,7 @@ constexpr int BM = 128, BN = 256;   // workgroup tile
 constexpr int A_STRIDE = 72;        // halfs per LDS row of a 64-wide chunk (144 bytes: conflict-free b128 reads)
 constexpr float kTwo24 = 16777216.0f;
 
-union HalfPack {
-    uint32_t u[4];
-    half8 h;
-};
-__device__ __forceinline__ half8 pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-    HalfPack p;
-    p.u[0] = a; p.u[1] = b; p.u[2] = c; p.u[3] = d;
-    return p.h;
-}
-__device__ __forceinline__ uint32_t pack_half2(float x, float y) {
-    return (uint32_t)f2h(x) | ((uint32_t)f2h(y) << 16);
-}
-__device__ __forceinline__ uint32_t pk_mul(uint32_t x, uint32_t s) {
-    union { uint32_t u; half2v h; } a, b, r;
-    a.u = x; b.u = s;
-    r.h = a.h * b.h;
-    return r.u;
-}
-// x*s + c on packed fp16 pairs, fused (single rounding)
-__device__ __forceinline__ uint32_t pk_fma(uint32_t x, uint32_t s, uint32_t c) {
-    union { uint32_t u; half2v h; } a, b, d, r;
-    a.u = x; b.u = s; d.u = c;
-    r.h = __builtin_elementwise_fma(a.h, b.h, d.h);
-    return r.u;
-}
-
 }  // namespace
-
-// ---------------------------------------------------------------------------
-// lhs preparation: per-row power-of-two scale, fp16 narrowing in operand order,
-// per-sub-block sums.  One workgroup of 256 threads per lhs row.
-//   a16  [m][k] fp16: inside every 64-wide chunk, position f*16 + g*8 + slot holds
-//        k = 32*(f/2) + 16*g + 8*(f%2) + perm[slot], perm = (0,2,1,3,4,6,5,7)
-//   asum [m][k/256][16] fp16: hi parts of the 8 sub-block sums, then their lo parts
-//   inv  [m] fp32: inverse of the row scale
-// PART = 0 writes the narrowed values, PART = 1 the residual (fp32 lhs only).
-// ---------------------------------------------------------------------------
-template <typename AT>
-__global__ __launch_bounds__(256) void q4k_prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
-                                                           _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum,
-                                                           float* __restrict__ inv) {
-    __shared__ uint32_t wmax[4];
-    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const AT* ar = a + (int64_t)row * k;
-    float mx = 0.0f;
-    for (int i = tid * 4; i < k; i += 1024) {
-        float x0 = load_f32(ar, i), x1 = load_f32(ar, i + 1), x2 = load_f32(ar, i + 2), x3 = load_f32(ar, i + 3);
-        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3))));
-    }
-    const uint32_t mb = wave_max_nonneg_bits(mx);
-    if (lane == 0) wmax[wave] = mb;
-    __syncthreads();
-    uint32_t mxb = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
-    int e = (int)((mxb >> 23) & 0xffu) - 127;
-    if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite row: leave unscaled
-    const float s = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
-    if (tid == 0) inv[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
-    for (int i = tid * 4; i < k; i += 1024) {
-        const float x0 = load_f32(ar, i) * s, x1 = load_f32(ar, i + 1) * s, x2 = load_f32(ar, i + 2) * s,
-                    x3 = load_f32(ar, i + 3) * s;
-        const float h0 = h2f(f2h(x0)), h1 = h2f(f2h(x1)), h2 = h2f(f2h(x2)), h3 = h2f(f2h(x3));
-        const int kl = i & 63, hin = kl >> 5, gg = (kl >> 4) & 1, odd = (kl >> 3) & 1;
-        const int pos = (2 * hin + odd) * 16 + gg * 8 + (kl & 4);
-        const int64_t o = (int64_t)row * k + (i & ~63) + pos;
-        *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
-        if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
-        const float sum = sum8((x0 + x1) + (x2 + x3));  // 8 consecutive lanes = one 32-wide sub-block
-        if ((lane & 7) == 0) {
-            const int blk = i >> 8, j = (i >> 5) & 7;
-            const float sh = h2f(f2h(sum));
-            _Float16* as = asum + ((int64_t)row * (k >> 8) + blk) * 16;
-            as[j] = (_Float16)sh;
-            as[8 + j] = (_Float16)(sum - sh);
-        }
-    }
-}
 
 // ---------------------------------------------------------------------------
 // main kernel
@@ -379,41 +301,21 @@ __global__ __launch_bounds__(512) void gemm_q4_k_kernel(const uint8_t* __restric
     }
 }
 
-// Workspace: a16 [m][k] fp16 (+ the residual part for fp32 lhs), asum [m][k/256][16] fp16, inv [m] fp32.
-int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) {
-    const int64_t parts = lhs_dtype == QMM_F32 ? 2 : 1;
-    auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
-    return parts * up(m * k * 2) + up(m * (k / 256) * 32) + up(m * 4);
-}
+int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return lhs_planes(nullptr, lhs_dtype, m, k).bytes; }
 
 hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                             float* out, void* workspace, hipStream_t s) {
-    auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
-    char* ws = (char*)workspace;
-    _Float16* a16 = (_Float16*)ws;
-    ws += up(m * k * 2);
-    _Float16* a16_lo = nullptr;
-    if (lhs_dtype == QMM_F32) {
-        a16_lo = (_Float16*)ws;
-        ws += up(m * k * 2);
-    }
-    _Float16* asum = (_Float16*)ws;
-    ws += up(m * (k / 256) * 32);
-    float* inv = (float*)ws;
-    if (lhs_dtype == QMM_F32)
-        q4k_prep_lhs_kernel<float><<<dim3((unsigned)m), dim3(256), 0, s>>>((const float*)lhs, (int)k, a16, a16_lo, asum, inv);
-    else
-        q4k_prep_lhs_kernel<uint16_t><<<dim3((unsigned)m), dim3(256), 0, s>>>((const uint16_t*)lhs, (int)k, a16, nullptr, asum, inv);
-    hipError_t e = hipGetLastError();
+    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
+    hipError_t e = launch_prep_lhs<kLhsOrderQ4K>(lhs, lhs_dtype, m, k, p, s);
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + BM - 1) / BM), tiles_n = (int)((n + BN - 1) / BN);
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8;
     dim3 grid((unsigned)(per_xcd * 8)), block(512);
     if (lhs_dtype == QMM_F32)
-        gemm_q4_k_kernel<2><<<grid, block, 0, s>>>(w, a16, a16_lo, asum, inv, out, (int)m, (int)n, (int)k, tiles_m, tiles_n);
+        gemm_q4_k_kernel<2><<<grid, block, 0, s>>>(w, p.a16, p.a16_lo, p.asum, p.inv, out, (int)m, (int)n, (int)k, tiles_m, tiles_n);
     else
-        gemm_q4_k_kernel<1><<<grid, block, 0, s>>>(w, a16, nullptr, asum, inv, out, (int)m, (int)n, (int)k, tiles_m, tiles_n);
+        gemm_q4_k_kernel<1><<<grid, block, 0, s>>>(w, p.a16, nullptr, p.asum, p.inv, out, (int)m, (int)n, (int)k, tiles_m, tiles_n);
     return hipGetLastError();
 }
 

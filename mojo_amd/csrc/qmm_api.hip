@@ -149,11 +149,11 @@ int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int
 }
 
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    (void)lhs_dtype;
     (void)n;
     if (m <= 0 || k <= 0) return 0;
     if (encoding == QMM_Q4_0) return q8_planes(nullptr, m, k).bytes;
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, k);
+    if (encoding == QMM_GPTQ && m > 16 && k % 256 == 0) return qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k);
     return 0;
 }
 
@@ -183,6 +183,10 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         if (int rc = check_gptq(cfg, n, k)) return rc;
         for (int i = 0; i < 3; i++)
             if (!rhs[i] || !aligned(rhs[i], 4)) return fail(QMM_ERR_INVALID, "qmm_matmul: GPTQ rhs[%d] null or misaligned", i);
+        if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size))
+            return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
+                                                    (const uint32_t*)rhs[2], m, n, k, cfg->group_size, out, workspace, s),
+                              "qmm_matmul(GPTQ GEMM)");
         for (int64_t m0 = 0; m0 < m; m0 += 16) {
             int mt = (int)(m - m0 < 16 ? m - m0 : 16);
             hipError_t e = qmm::launch_gemv_gptq((const char*)lhs + m0 * k * esz, lhs_dtype, (const uint32_t*)rhs[0],

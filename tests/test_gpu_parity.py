@@ -205,3 +205,42 @@ def test_q4_k_gemm_wide_range_lhs():
     got = qmatmul(QE.Q4_K, None, gpu(a).to(torch.bfloat16), gpu(wq)).cpu().numpy()
     scale = np.abs(truth).max(axis=1, keepdims=True)
     assert np.all(np.abs(got - truth) <= 1e-4 * scale + 1e-3 * np.abs(truth))
+
+
+@pytest.mark.parametrize("m,n,k,group", [(128, 256, 256, 128), (17, 40, 512, 64), (200, 304, 1024, 128),
+                                         (256, 512, 4096, 128), (130, 64, 2048, 256), (40, 72, 768, 64)])
+def test_gptq_gemm_bf16_lhs(m, n, k, group):
+    """GPTQ prefill kernel, bf16 lhs: against the fp32 oracle and the fp64 truth."""
+    w, a = synth(21, n, k, m)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    want = O.matmul_gptq(a, qw, sc, qz, group)
+    truth = O.matmul_gptq(a, qw, sc, qz, group, f64=True)
+    cfg = QuantizationConfig(group_size=group)
+    got = qmatmul(QE.GPTQ, cfg, gpu(a).to(torch.bfloat16), gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, want, f"GPTQ GEMM {m}x{n}x{k} g{group} vs fp32 oracle")
+    assert_close(got, truth, f"GPTQ GEMM {m}x{n}x{k} g{group} vs fp64 truth")
+
+
+@pytest.mark.parametrize("m,n,k,group", [(64, 128, 512, 128), (33, 64, 256, 64), (48, 96, 512, 256)])
+def test_gptq_gemm_f32_lhs(m, n, k, group):
+    w, a = synth(22, n, k, m)
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    want = O.matmul_gptq(a, qw, sc, qz, group)
+    got = qmatmul(QE.GPTQ, QuantizationConfig(group_size=group), gpu(a), gpu(qw), gpu(sc.view(np.float16)), gpu(qz),
+                  gpu(gi))
+    assert_close(got, want, f"GPTQ GEMM fp32 lhs {m}x{n}x{k} g{group}")
+
+
+def test_gptq_gemm_arbitrary_zero_points():
+    """Stored zero points other than 7: the zero term takes scale*zero as an exact fp16 hi + lo pair."""
+    m, n, k, group = 64, 128, 1024, 128
+    w, a = synth(23, n, k, m)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    rng = np.random.Generator(np.random.PCG64(24))
+    qz = rng.integers(0, 2**32, size=qz.shape, dtype=np.uint64).astype(np.uint32).view(np.int32)
+    truth = O.matmul_gptq(a, qw, sc, qz, group, f64=True)
+    got = qmatmul(QE.GPTQ, QuantizationConfig(group_size=group), gpu(a).to(torch.bfloat16), gpu(qw),
+                  gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, truth, "GPTQ GEMM random zero points")
