@@ -171,6 +171,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill"), default="decode",
+                    help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill: the M=2048 GEMM of the "
+                         "same model's gate projection (second target, matrix-core roofline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip per-shape and secondary-config timings")
     args = ap.parse_args()
@@ -184,6 +187,8 @@ def main() -> int:
     torch.cuda.set_device(0)
     gen = torch.Generator(device="cuda:0")
     gen.manual_seed(3)
+    if args.workload != "decode":
+        return prefill_main(args, gen)
     m = args.m
     acts = {k: torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}
     layers = []
@@ -236,7 +241,7 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": None,
-            "kernel": "gemv_q4_k_kernel",
+            "kernel": "gemv_q4_k_stream_kernel",
             "bytes_per_launch": avg_launch_bytes,
             "launch_us": round(avg_launch_us, 3),
         },
@@ -247,6 +252,36 @@ def main() -> int:
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
+    return 0
+
+
+def prefill_main(args, gen) -> int:
+    """Second target: bf16 lhs [2048, 4096] x 4-bit weights [14336, 4096], one launch per step."""
+    mm, n, k = 2048, 14336, 4096
+    steps, warmup = min(args.steps, 50), min(args.warmup, 5)
+    ab = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
+    if args.workload == "prefill":
+        call, name, kern = Gemv(QE.Q4_K, make_weight(QE.Q4_K, n, k, gen), ab), "Q4_K", "gemm_q4_k_kernel"
+    else:
+        wg = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
+        call, name, kern = GptqMatmul(wg, ab), "GPTQ g128", "gemm_gptq_kernel"
+    g = capture([call])
+    dev_s, wall_s = time_graphs([g], steps, warmup)
+    us = dev_s * 1e6 / steps
+    flops = 2.0 * mm * n * k
+    tf = flops / us / 1e6
+    print(json.dumps({
+        "metric": f"{name} prefill GEMM TFLOP/s", "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(us / 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 products, f32 sums", "data": "synthetic",
+        "config": {"workload": f"{name} prefill GEMM, bf16 lhs [{mm}, {k}] x weights [{n}, {k}], fp32 out; one step = "
+                               f"lhs preparation + one GEMM launch", "m": mm, "n": n, "k": k},
+        "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": kern,
+                     "flops_per_launch": flops, "launch_us": round(us, 2),
+                     "note": "launch_us includes the lhs preparation kernel (a few microseconds)"},
+        "cpu_baseline": None,
+    }))
     return 0
 
 

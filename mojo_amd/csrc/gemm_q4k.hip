@@ -305,6 +305,12 @@ int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return 
 
 hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                             float* out, void* workspace, hipStream_t s) {
+    // QMM_Q4K_GEMM=w4 selects the 4-wavefront kernel; the default is this file's 8-wavefront one.
+    static const bool use_w4 = [] {
+        const char* v = getenv("QMM_Q4K_GEMM");
+        return v && v[0] == 'w' && v[1] == '4';
+    }();
+    if (use_w4) return launch_gemm_q4_k_w4(lhs, lhs_dtype, w, m, n, k, out, workspace, s);
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
     hipError_t e = launch_prep_lhs<kLhsOrderQ4K>(lhs, lhs_dtype, m, k, p, s);
     if (e != hipSuccess) return e;
