@@ -44,6 +44,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
                                                         int tiles_n) {
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][NPART][BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) _Float16 lds_s[BM * 16];
+    __shared__ __attribute__((aligned(16))) float lds_inv[BM];
     constexpr int SPG = 4 / GB;  // 64-wide steps per group
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -160,6 +161,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
     QMM_A_LOAD(ax1, 1);
     QMM_A_LOAD(ax0, 2);
     as_prefetch(1);
+    if (tid < BM) lds_inv[tid] = inv[min(m0 + tid, m - 1)];
     __syncthreads();
 
     float gscale[2][GB];
@@ -268,18 +270,24 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
 #undef QMM_A_STORE
 #undef QMM_Q_LOAD
 
+    // ---- epilogue: undo the row scale (inverse scales come from LDS, four rows per read: a dependent
+    // global load per output row cost a fifth of the tile time), store
+    const int ocol0 = n0 + wn * 64 + nl, ocol1 = ocol0 + 32;
+    const bool c0_ok = ocol0 < n, c1_ok = ocol1 < n;
 #pragma unroll
     for (int mi = 0; mi < 2; mi++) {
+        float4 iv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) iv[j] = *(const float4*)(&lds_inv[wm * 64 + mi * 32 + 8 * j + 4 * g]);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+            const float4 q = iv[r >> 2];
+            const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
             if (row < m) {
-                const float is = inv[row];
-#pragma unroll
-                for (int ni = 0; ni < 2; ni++) {
-                    const int col = n0 + wn * 64 + ni * 32 + nl;
-                    if (col < n) out[(int64_t)row * n + col] = acc[mi][ni][r] * is;
-                }
+                float* o = out + (int64_t)row * n;
+                if (c0_ok) o[ocol0] = acc[mi][0][r] * is;
+                if (c1_ok) o[ocol1] = acc[mi][1][r] * is;
             }
         }
     }

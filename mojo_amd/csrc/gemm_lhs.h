@@ -43,6 +43,19 @@ __device__ __forceinline__ uint32_t pk_fma(uint32_t x, uint32_t s, uint32_t c) {
     return r.u;
 }
 
+// acc += g * P, element by element, written as the two-operand multiply-add so that acc stays in its own
+// registers.  Left to the compiler, the three-operand form puts the result where P was; the 16-register
+// tuples of the matrix-core accumulators then swap roles and fragment the register file, and the
+// multiply-adds get sunk past the next group's matrix-core instructions.
+__device__ __forceinline__ void rescale_add(float16v& acc, float g, const float16v& P) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        float t = acc[r];
+        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(t) : "v"(g), "v"(P[r]));
+        acc[r] = t;
+    }
+}
+
 // Operand orders inside every 64-wide chunk of a row; position f*16 + g*8 + slot holds column
 //   kLhsOrderQ4K : 32*(f/2) + 16*g + 8*(f%2) + (0,2,1,3,4,6,5,7)[slot]
 //   kLhsOrderGPTQ: 16*f + 8*g + (0,4,1,5,2,6,3,7)[slot], odd columns pre-multiplied by 1/16

@@ -244,3 +244,17 @@ def test_gptq_gemm_arbitrary_zero_points():
     got = qmatmul(QE.GPTQ, QuantizationConfig(group_size=group), gpu(a).to(torch.bfloat16), gpu(qw),
                   gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
     assert_close(got, truth, "GPTQ GEMM random zero points")
+
+
+@pytest.mark.parametrize("lhs_bf16", [True, False])
+def test_q4_k_gemm_many_tiles(lhs_bf16):
+    """More tiles than the device holds at once, not a whole number of rounds: the leftover tiles are cut
+    along K and summed in the output, which must not change the result beyond fp32 rounding."""
+    m, n, k = 2048, 4352, 512
+    w, a = synth(31, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_K GEMM {m}x{n}x{k} bf16={lhs_bf16}")
