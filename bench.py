@@ -164,6 +164,15 @@ def cpu_baseline(layer_w, m: int, budget_s: float = 12.0):
                       f"{el:.1f} s, OpenMP over N, host has {os.cpu_count()} logical cpus"}
 
 
+def measured_traffic(key: str):
+    """HBM bytes per launch from the committed PMC summary (profiles/hbm_traffic.json), or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            return json.load(f)[key]["traffic_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,9 +180,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill"), default="decode",
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "calib"), default="decode",
                     help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill: the M=2048 GEMM of the "
-                         "same model's gate projection (second target, matrix-core roofline)")
+                         "same model's gate projection (second target, matrix-core roofline); calib: a plain "
+                         "read and a plain copy of 256 MiB, the yardsticks for the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip per-shape and secondary-config timings")
     args = ap.parse_args()
@@ -187,6 +197,8 @@ def main() -> int:
     torch.cuda.set_device(0)
     gen = torch.Generator(device="cuda:0")
     gen.manual_seed(3)
+    if args.workload == "calib":
+        return calib_main()
     if args.workload != "decode":
         return prefill_main(args, gen)
     m = args.m
@@ -240,7 +252,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": measured_traffic("decode_m1") if m == 1 and args.layers == 8 else None,
             "kernel": "gemv_q4_k_stream_kernel",
             "bytes_per_launch": avg_launch_bytes,
             "launch_us": round(avg_launch_us, 3),
@@ -252,6 +264,22 @@ def main() -> int:
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
+    return 0
+
+
+def calib_main() -> int:
+    """Known-size kernels for scaling the HBM counters: qmm_read_probe reads 256 MiB, a torch copy reads
+    and writes 256 MiB.  Each runs three times; buffers are larger than every cache."""
+    nbytes = 256 << 20
+    src = torch.empty((nbytes,), dtype=torch.uint8, device="cuda:0").random_(0, 255)
+    dst = torch.empty_like(src)
+    probe = ReadProbe(src)
+    s = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        probe.launch(s)
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"calibration": {"read_probe_bytes": probe.nbytes, "copy_bytes_each_way": nbytes}}))
     return 0
 
 
