@@ -331,6 +331,11 @@ hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m,
 
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
+    if (!getenv("QMM_Q6K_V1")) {
+        bool handled = false;
+        hipError_t e = launch_gemv_q6_k_rows(a, a_dtype, w, m, n, k, out, ldo, s, &handled);
+        if (e != hipSuccess || handled) return e;
+    }
     dim3 grid((unsigned)((n + 3) / 4)), block(256);
 #define CALL(MT)                                                                                          \
     if (a_dtype == QMM_F32)                                                                               \

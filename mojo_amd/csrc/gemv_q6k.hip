@@ -1,0 +1,393 @@
+// Q6_K decode kernel for m <= 4 lhs rows: weights streamed through LDS, decoded 16 per lane.
+//
+// A Q6_K super-block is 210 bytes (128 B low nibbles, 64 B high bit pairs, 16 int8 scales, fp16 d),
+// so blocks are only 2-byte aligned and no field can be loaded as an aligned vector straight from
+// memory.  A wavefront therefore copies a run of up to 16 blocks of its row into a private LDS
+// buffer with aligned 16-byte loads (the run starts at the 16-byte boundary below its first byte),
+// and the lanes pick their fields out of LDS as two aligned dwords joined by a byte alignment
+// (every field sits at a multiple of 4 from its block's start, so one shift per block suffices).
+//
+// Lane t of a 16-lane group owns, in half h = t / 8 of a block, the four ql bytes 4j..4j+3
+// (j = t % 8), the four bytes 32 further and the four qh bytes 4j..4j+3: sixteen weights, four
+// each at columns 128h + 4j + {0, 32, 64, 96}, each quartet with its own scale.  Four groups work
+// on four blocks at a time.  The -32 offset of the codes is applied through per-16-column sums of
+// the activations, computed once per workgroup:  sum_k a_k sc (q_k - 32) = sc (sum a_k q_k) -
+// 32 sc asum16, one 16-column group per lane.  Activations come through the vector cache (a
+// 16 KB row stays resident), which keeps the LDS pipe for the weights.
+#include <stdlib.h>
+
+#include "qmm_internal.h"
+
+namespace qmm {
+
+namespace {
+
+constexpr int kRunBlocks = 16;                                   // blocks per staged run
+constexpr int kRunBytes = (kRunBlocks * Q6_K_BPB + 14 + 4 + 15) / 16 * 16;  // 3392: lead-in + run + one dword of read-ahead, in 16-byte pieces
+
+template <typename AT>
+__device__ __forceinline__ float4 load4(const AT* __restrict__ a, int64_t i);
+template <>
+__device__ __forceinline__ float4 load4<float>(const float* __restrict__ a, int64_t i) {
+    return *(const float4*)(a + i);
+}
+template <>
+__device__ __forceinline__ float4 load4<uint16_t>(const uint16_t* __restrict__ a, int64_t i) {
+    const uint2 v = *(const uint2*)(a + i);
+    return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                       __uint_as_float(v.y & 0xffff0000u));
+}
+
+__device__ __forceinline__ float ubf0(uint32_t x) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float ubf1(uint32_t x) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float ubf2(uint32_t x) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float ubf3(uint32_t x) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(x)); return r; }
+__device__ __forceinline__ float dot4u(float4 x, uint32_t q) {
+    return fmaf(x.w, ubf3(q), fmaf(x.z, ubf2(q), fmaf(x.y, ubf1(q), x.x * ubf0(q))));
+}
+__device__ __forceinline__ float sbyte(uint32_t x, int shift) { return (float)((int)(x << (24 - shift)) >> 24); }
+
+}  // namespace
+
+template <int MT, typename AT>
+__global__ __launch_bounds__(256) void gemv_q6_k_rows_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                             float* __restrict__ out, int m, int n, int k, int64_t ldo) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nblk = k >> 8, ngrp = k >> 4;
+    float* asum16 = (float*)smem;  // [MT][k/16]
+    uint8_t* wbuf = smem + ((MT * ngrp * 4 + 15) & ~15) + wave * kRunBytes;
+
+    // per-16-column activation sums
+    for (int gidx = tid; gidx < MT * ngrp; gidx += 256) {
+        const int mi = gidx / ngrp, gi = gidx - mi * ngrp;
+        float s = 0.0f;
+        if (mi < m) {
+            const AT* ar = a + (int64_t)mi * k + gi * 16;
+            const float4 x0 = load4(ar, 0), x1 = load4(ar, 4), x2 = load4(ar, 8), x3 = load4(ar, 12);
+            s = ((x0.x + x0.y) + (x0.z + x0.w)) + ((x1.x + x1.y) + (x1.z + x1.w)) + ((x2.x + x2.y) + (x2.z + x2.w)) +
+                ((x3.x + x3.y) + (x3.z + x3.w));
+        }
+        asum16[gidx] = s;
+    }
+    __syncthreads();
+
+    const int total_waves = (int)gridDim.x * 4, gw = (int)blockIdx.x * 4 + wave;
+    const int nrun = (nblk + kRunBlocks - 1) / kRunBlocks;
+    const int64_t row_bytes = (int64_t)nblk * Q6_K_BPB;
+    const int bq = lane >> 4, t = lane & 15, h = t >> 3, j = t & 7;
+    const int f_ql = 64 * h + 4 * j, f_qh = 128 + 32 * h + 4 * j, f_sc = 192 + 8 * h;
+    const int sc_shift = 8 * (j >> 2);          // this lane's quartet scales: bytes jj, jj + 2 of each scale dword
+    const uint32_t* lds32 = (const uint32_t*)wbuf;
+
+    uint4 r0, r1, r2, r3;
+    int delta = 0;  // offset of the run's first byte inside its first 16-byte piece
+    // aligned 16-byte pieces covering run `c` of row `row`; pieces past the end repeat the last one
+    auto issue = [&](int row, int c, int& dl) {
+        const int nb = min(kRunBlocks, nblk - c * kRunBlocks);
+        const uint8_t* p = w + (int64_t)row * row_bytes + (int64_t)c * kRunBlocks * Q6_K_BPB;
+        const uintptr_t ad = (uintptr_t)p;
+        dl = (int)(ad & 15);
+        const uint4* base = (const uint4*)(ad - (uintptr_t)dl);
+        const int last = (dl + nb * Q6_K_BPB + 15) / 16 - 1;
+        r0 = base[min(lane, last)];
+        r1 = base[min(lane + 64, last)];
+        r2 = base[min(lane + 128, last)];
+        r3 = base[min(lane + 192, last)];
+    };
+
+    float acc[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
+
+    int row = gw, c = 0;
+    if (row < n) issue(row, 0, delta);
+    while (row < n) {
+        // registers -> LDS (the previous run's reads were issued before this point: LDS is in order per wavefront)
+        uint4* wb = (uint4*)wbuf;
+        wb[lane] = r0;
+        wb[lane + 64] = r1;
+        wb[lane + 128] = r2;
+        if (lane + 192 < kRunBytes / 16) wb[lane + 192] = r3;
+        const int cur_delta = delta, cur_c = c, cur_row = row;
+        // next run of this row, or the first run of this wavefront's next row
+        int nrow = row, nc = c + 1;
+        if (nc == nrun) {
+            nc = 0;
+            nrow = row + total_waves;
+        }
+        int ndelta = delta;
+        issue(min(nrow, n - 1), nrow < n ? nc : 0, ndelta);  // past the end: a harmless repeat, never used
+        __builtin_amdgcn_wave_barrier();
+
+        const int nb = min(kRunBlocks, nblk - cur_c * kRunBlocks);
+#pragma unroll
+        for (int it = 0; it < kRunBlocks / 4; it++) {
+            const int bl = 4 * it + bq;
+            const bool live = bl < nb;
+            const int boff = cur_delta + Q6_K_BPB * min(bl, nb - 1);
+            const int sh = boff & 3, w0 = boff >> 2;  // byte shift (0 or 2), first aligned dword
+            auto rd = [&](int field) {
+                const int i = w0 + (field >> 2);
+                return __builtin_amdgcn_alignbyte(lds32[i + 1], lds32[i], (uint32_t)sh);
+            };
+            const uint32_t A = rd(f_ql), B = rd(f_ql + 32), H = rd(f_qh);
+            const uint32_t s0 = rd(f_sc), s1 = rd(f_sc + 4);
+            const float d = live ? h2f((uint16_t)(rd(208) & 0xffffu)) : 0.0f;
+            const uint32_t q1 = (A & 0x0F0F0F0Fu) | ((H << 4) & 0x30303030u);
+            const uint32_t q2 = (B & 0x0F0F0F0Fu) | ((H << 2) & 0x30303030u);
+            const uint32_t q3 = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
+            const uint32_t q4 = ((B >> 4) & 0x0F0F0F0Fu) | ((H >> 2) & 0x30303030u);
+            const float e1 = d * sbyte(s0, sc_shift), e2 = d * sbyte(s0, sc_shift + 16);
+            const float e3 = d * sbyte(s1, sc_shift), e4 = d * sbyte(s1, sc_shift + 16);
+            // this lane's 16-column group for the offset term: scale byte t % 8 of half h
+            const float eo = -32.0f * d * sbyte(j < 4 ? s0 : s1, 8 * (j & 3));
+            const int blk = cur_c * kRunBlocks + min(bl, nb - 1);
+            const int kb = blk * 256 + 128 * h + 4 * j;
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                if (mi < m) {
+                    const AT* ar = a + (int64_t)mi * k + kb;
+                    const float4 x1 = load4(ar, 0), x2 = load4(ar, 32), x3 = load4(ar, 64), x4 = load4(ar, 96);
+                    float v = acc[mi];
+                    v = fmaf(e1, dot4u(x1, q1), v);
+                    v = fmaf(e2, dot4u(x2, q2), v);
+                    v = fmaf(e3, dot4u(x3, q3), v);
+                    v = fmaf(e4, dot4u(x4, q4), v);
+                    acc[mi] = fmaf(eo, asum16[mi * ngrp + blk * 16 + t], v);
+                }
+            }
+        }
+        if (cur_c == nrun - 1) {
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                const float v = wave_sum(acc[mi]);
+                if (lane == 0 && mi < m) out[(int64_t)mi * ldo + cur_row] = v;
+                acc[mi] = 0.0f;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        row = nrow;
+        c = nc;
+        delta = ndelta;
+    }
+}
+
+
+// Variant for one lhs row with the loops interchanged: the run index is the outer loop and the
+// wavefront's rows the inner one, so a lane's activations (64 floats per lhs row for its four
+// block slots of the run) and offset sums are loaded once per run and stay in registers while
+// the weights of all its rows stream through.  Per-row partial sums wait in LDS until the last
+// run (one slot per row of the wavefront, kParkRows at most).
+constexpr int kParkRows = 128;
+
+template <int MT, typename AT>
+__global__ __launch_bounds__(256) void gemv_q6_k_slab_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                             float* __restrict__ out, int m, int n, int k, int64_t ldo) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nblk = k >> 8;
+    uint8_t* wbuf = smem + wave * kRunBytes;
+    float* park = (float*)(smem + 4 * kRunBytes) + wave * MT * kParkRows;  // [MT][kParkRows]
+    const int total_waves = (int)gridDim.x * 4, gw = (int)blockIdx.x * 4 + wave;
+    const int nrows_w = gw < n ? (n - gw + total_waves - 1) / total_waves : 0;
+    const int nrun = (nblk + kRunBlocks - 1) / kRunBlocks;
+    const int64_t row_bytes = (int64_t)nblk * Q6_K_BPB;
+    const int bq = lane >> 4, t = lane & 15, h = t >> 3, j = t & 7;
+    const int f_ql = 64 * h + 4 * j, f_qh = 128 + 32 * h + 4 * j, f_sc = 192 + 8 * h;
+    const int sc_shift = 8 * (j >> 2);
+    const uint32_t* lds32 = (const uint32_t*)wbuf;
+    for (int i = lane; i < MT * kParkRows; i += 64) park[i] = 0.0f;
+
+    // two register sets: the loads of rows i + 1 and i + 2 are in flight while row i is decoded
+    uint4 ra0, ra1, ra2, ra3, rb0, rb1, rb2, rb3;
+    int delta_a = 0, delta_b = 0;
+#define QMM_Q6K_ISSUE(SET, ROW, C, DL)                                                               \
+    do {                                                                                             \
+        const int nb_ = min(kRunBlocks, nblk - (C) * kRunBlocks);                                    \
+        const uintptr_t ad_ = (uintptr_t)(w + (int64_t)(ROW) * row_bytes + (int64_t)(C) * kRunBlocks * Q6_K_BPB); \
+        DL = (int)(ad_ & 15);                                                                        \
+        const uint4* base_ = (const uint4*)(ad_ - (uintptr_t)(DL));                                  \
+        const int last_ = ((DL) + nb_ * Q6_K_BPB + 15) / 16 - 1;                                     \
+        SET##0 = base_[min(lane, last_)];                                                            \
+        SET##1 = base_[min(lane + 64, last_)];                                                       \
+        SET##2 = base_[min(lane + 128, last_)];                                                      \
+        SET##3 = base_[min(lane + 192, last_)];                                                      \
+    } while (0)
+#define QMM_Q6K_STAGE(SET)                                              \
+    do {                                                                \
+        uint4* wb_ = (uint4*)wbuf;                                      \
+        wb_[lane] = SET##0;                                             \
+        wb_[lane + 64] = SET##1;                                        \
+        wb_[lane + 128] = SET##2;                                       \
+        if (lane + 192 < kRunBytes / 16) wb_[lane + 192] = SET##3;      \
+    } while (0)
+
+    for (int c = 0; c < nrun; c++) {
+        const int nb = min(kRunBlocks, nblk - c * kRunBlocks);
+        // this lane's activations for the run: per block slot, four quartets; and its offset sums
+        float4 x[MT][4][4];
+        float os[MT][4], lv[4];
+        int boff0[4];
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int bl = 4 * it + bq;
+            lv[it] = bl < nb ? 1.0f : 0.0f;
+            const int blc = min(bl, nb - 1);
+            boff0[it] = Q6_K_BPB * blc;
+            const int blk = c * kRunBlocks + blc;
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                if (mi < m) {
+                    const AT* ar = a + (int64_t)mi * k + blk * 256;
+                    const AT* aq = ar + 128 * h + 4 * j;
+                    x[mi][it][0] = load4(aq, 0);
+                    x[mi][it][1] = load4(aq, 32);
+                    x[mi][it][2] = load4(aq, 64);
+                    x[mi][it][3] = load4(aq, 96);
+                    const AT* ag = ar + 16 * t;
+                    const float4 y0 = load4(ag, 0), y1 = load4(ag, 4), y2 = load4(ag, 8), y3 = load4(ag, 12);
+                    os[mi][it] = -32.0f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
+                                           ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
+                } else {
+                    x[mi][it][0] = x[mi][it][1] = x[mi][it][2] = x[mi][it][3] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    os[mi][it] = 0.0f;
+                }
+            }
+        }
+        auto row_of = [&](int i) { return min(gw + i * total_waves, n - 1); };  // past the last row: a harmless repeat
+        auto decode_row = [&](int i, int cur_delta) {
+            float v[MT];
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) v[mi] = 0.0f;
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                const int boff = cur_delta + boff0[it];
+                const int sh = boff & 3, w0 = boff >> 2;
+                auto rd = [&](int field) {
+                    const int q = w0 + (field >> 2);
+                    return __builtin_amdgcn_alignbyte(lds32[q + 1], lds32[q], (uint32_t)sh);
+                };
+                const uint32_t A = rd(f_ql), B = rd(f_ql + 32), H = rd(f_qh);
+                const uint32_t s0 = rd(f_sc), s1 = rd(f_sc + 4);
+                const float d = h2f((uint16_t)(rd(208) & 0xffffu)) * lv[it];
+                const uint32_t q1 = (A & 0x0F0F0F0Fu) | ((H << 4) & 0x30303030u);
+                const uint32_t q2 = (B & 0x0F0F0F0Fu) | ((H << 2) & 0x30303030u);
+                const uint32_t q3 = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
+                const uint32_t q4 = ((B >> 4) & 0x0F0F0F0Fu) | ((H >> 2) & 0x30303030u);
+                const float e1 = d * sbyte(s0, sc_shift), e2 = d * sbyte(s0, sc_shift + 16);
+                const float e3 = d * sbyte(s1, sc_shift), e4 = d * sbyte(s1, sc_shift + 16);
+                const float eo = d * sbyte(j < 4 ? s0 : s1, 8 * (j & 3));
+#pragma unroll
+                for (int mi = 0; mi < MT; mi++) {
+                    float u = v[mi];
+                    u = fmaf(e1, dot4u(x[mi][it][0], q1), u);
+                    u = fmaf(e2, dot4u(x[mi][it][1], q2), u);
+                    u = fmaf(e3, dot4u(x[mi][it][2], q3), u);
+                    u = fmaf(e4, dot4u(x[mi][it][3], q4), u);
+                    v[mi] = fmaf(eo, os[mi][it], u);
+                }
+            }
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                const float sum = wave_sum(v[mi]);
+                if (lane == 0) park[mi * kParkRows + i] += sum;
+            }
+        };
+        if (nrows_w > 0) {
+            QMM_Q6K_ISSUE(ra, row_of(0), c, delta_a);
+            QMM_Q6K_ISSUE(rb, row_of(1), c, delta_b);
+        }
+        for (int i = 0; i < nrows_w; i += 2) {
+            QMM_Q6K_STAGE(ra);
+            const int da = delta_a;
+            QMM_Q6K_ISSUE(ra, row_of(i + 2), c, delta_a);
+            __builtin_amdgcn_wave_barrier();
+            decode_row(i, da);
+            __builtin_amdgcn_wave_barrier();
+            if (i + 1 < nrows_w) {
+                QMM_Q6K_STAGE(rb);
+                const int db = delta_b;
+                QMM_Q6K_ISSUE(rb, row_of(i + 3), c, delta_b);
+                __builtin_amdgcn_wave_barrier();
+                decode_row(i + 1, db);
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    }
+#undef QMM_Q6K_ISSUE
+#undef QMM_Q6K_STAGE
+    __builtin_amdgcn_wave_barrier();
+    for (int i = lane; i < nrows_w; i += 64) {
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++)
+            if (mi < m) out[(int64_t)mi * ldo + gw + (int64_t)i * total_waves] = park[mi * kParkRows + i];
+    }
+}
+
+// LDS bytes of one workgroup; 0 if the shape does not fit (the caller then uses the generic kernel).
+static size_t q6k_rows_lds(int mt, int64_t k) {
+    const size_t b = ((size_t)mt * (k / 16) * 4 + 15) / 16 * 16 + 4 * (size_t)kRunBytes;
+    return b <= 96 * 1024 ? b : 0;
+}
+
+hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
+                                 float* out, int64_t ldo, hipStream_t s, bool* handled) {
+    *handled = false;
+    const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
+    if (m > 4 || ((uintptr_t)w & 1)) return hipSuccess;
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipGetLastError();
+        cus = prop.multiProcessorCount;
+    }
+    // One lhs row and enough weight rows per wavefront to amortise the per-run activation loads: the
+    // loop-interchanged kernel; otherwise the row-at-a-time kernel below.
+    static const int pc_env = getenv("QMM_Q6K_WG_PER_CU") ? atoi(getenv("QMM_Q6K_WG_PER_CU")) : 0;
+    const int pc = pc_env > 0 ? pc_env : 3;
+    if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !getenv("QMM_Q6K_ROWS")) {
+        const size_t lds2 = 4 * (size_t)kRunBytes + 4 * (size_t)kParkRows * 4;
+        // enough wavefronts that none has more rows than its LDS parking slots
+        const int64_t wgs = max((int64_t)cus * pc, (n + 4 * kParkRows - 1) / (4 * kParkRows));
+        dim3 grid2((unsigned)min(wgs, (n + 3) / 4)), block2(256);
+        if (a_dtype == QMM_F32)
+            gemv_q6_k_slab_kernel<1, float><<<grid2, block2, lds2, s>>>(w, (const float*)a, out, m, (int)n, (int)k, ldo);
+        else
+            gemv_q6_k_slab_kernel<1, uint16_t><<<grid2, block2, lds2, s>>>(w, (const uint16_t*)a, out, m, (int)n, (int)k, ldo);
+        *handled = true;
+        return hipGetLastError();
+    }
+    const size_t lds = q6k_rows_lds(mt, k);
+    if (!lds) return hipSuccess;
+    int per_cu = pc_env > 0 ? pc_env : (int)min((size_t)4, (size_t)(128 * 1024) / lds);
+    per_cu = max(per_cu, 1);
+    const int64_t wg_needed = (n + 3) / 4;
+    dim3 grid((unsigned)min((int64_t)cus * per_cu, wg_needed)), block(256);
+#define QMM_Q6K_GO(MT_)                                                                                              \
+    do {                                                                                                             \
+        if (a_dtype == QMM_F32) {                                                                                    \
+            if (lds > 64 * 1024)                                                                                     \
+                (void)hipFuncSetAttribute((const void*)gemv_q6_k_rows_kernel<MT_, float>,                            \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+            gemv_q6_k_rows_kernel<MT_, float><<<grid, block, lds, s>>>(w, (const float*)a, out, m, (int)n, (int)k, ldo); \
+        } else {                                                                                                     \
+            if (lds > 64 * 1024)                                                                                     \
+                (void)hipFuncSetAttribute((const void*)gemv_q6_k_rows_kernel<MT_, uint16_t>,                         \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+            gemv_q6_k_rows_kernel<MT_, uint16_t><<<grid, block, lds, s>>>(w, (const uint16_t*)a, out, m, (int)n,     \
+                                                                         (int)k, ldo);                               \
+        }                                                                                                            \
+    } while (0)
+    if (mt == 1) QMM_Q6K_GO(1);
+    else if (mt == 2) QMM_Q6K_GO(2);
+    else QMM_Q6K_GO(4);
+#undef QMM_Q6K_GO
+    *handled = true;
+    return hipGetLastError();
+}
+
+}  // namespace qmm

@@ -33,6 +33,8 @@ hipError_t launch_gemv_q4_k_mfma(const void* a, int a_dtype, const uint8_t* w, i
                                  float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s);
+hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
+                                 float* out, int64_t ldo, hipStream_t s, bool* handled);
 bool gemm_gptq_supported(int64_t k, int group);
 int64_t gemm_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
 hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales,

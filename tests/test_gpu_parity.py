@@ -258,3 +258,17 @@ def test_q4_k_gemm_many_tiles(lhs_bf16):
     want = O.matmul_f32(O.Q4_K, a, wq)
     got = qmatmul(QE.Q4_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
     assert_close(got, want, f"Q4_K GEMM {m}x{n}x{k} bf16={lhs_bf16}")
+
+
+@pytest.mark.parametrize("lhs_bf16", [False, True])
+def test_q6_k_decode_many_rows(lhs_bf16):
+    """One lhs row against many weight rows (the vocabulary-projection shape): runs of 16 blocks with a
+    partial last run, a row count that is not a multiple of the wavefront count."""
+    n, k = 12418, 4864
+    w, a = synth(41, n, k, 1)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q6_K, w)
+    want = O.matmul_f32(O.Q6_K, a, wq)
+    got = qmatmul(QE.Q6_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q6_K 1x{n}x{k} bf16={lhs_bf16}")
