@@ -302,22 +302,29 @@ __global__ __launch_bounds__(256) void gemv_gptq_kernel(const uint32_t* __restri
     else if (m <= 8) { CALL(8); } \
     else { CALL(16); }
 
-// Kernel choice for Q4_K decode shapes.  Measured on MI355X: with one or two lhs rows the
-// vector-ALU kernel below is faster on the Llama-3-8B projection shapes; from three rows on its
-// cost grows with m while the matrix-core kernel's does not.  QMM_Q4K_GEMV=valu|mfma overrides.
+// Kernel choice for Q4_K decode shapes.  Measured on MI355X: the vector-ALU streaming kernel (one or
+// two lhs rows per pass) is the fastest up to four lhs rows, with three and four rows done as two
+// passes over the weights; from five rows on the matrix-core kernel, whose cost does not grow with m,
+// wins.  QMM_Q4K_GEMV=valu|mfma overrides.
 static bool q4k_use_valu(int m) {
     static const int forced = [] {
         const char* e = getenv("QMM_Q4K_GEMV");
         return !e ? 0 : (e[0] == 'v' ? 1 : (e[0] == 'm' ? 2 : 0));
     }();
     if (forced) return forced == 1;
-    return m <= 2;
+    return m <= 4;
 }
 
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
     if (!q4k_use_valu(m)) return launch_gemv_q4_k_mfma(a, a_dtype, w, m, n, k, out, ldo, s);
     if (m <= 2 && !getenv("QMM_Q4K_V1")) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
+    if (m <= 4 && !getenv("QMM_Q4K_V1")) {
+        const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
+        hipError_t e = launch_gemv_q4_k_rows(a, a_dtype, w, 2, n, k, out, ldo, s);
+        if (e != hipSuccess) return e;
+        return launch_gemv_q4_k_rows((const char*)a + 2 * k * esz, a_dtype, w, m - 2, n, k, out + 2 * ldo, ldo, s);
+    }
     dim3 grid((unsigned)((n + 3) / 4)), block(256);
 #define CALL(MT)                                                                                          \
     if (a_dtype == QMM_F32)                                                                               \
