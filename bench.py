@@ -377,6 +377,12 @@ def extra_timings(layers, acts, gen):
         us = dev_s * 1e6 / (20 * copies)
         out[tag] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q4_0, mm, n, k) / us / 1e3, 1)}
         del cs
+    # Q4_0 prefill on the int8 matrix cores, same shape as cfg5
+    ab32 = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
+    g = capture([Gemv(QE.Q4_0, make_weight(QE.Q4_0, 14336, 4096, gen), ab32)])
+    dev_s, _ = time_graphs([g], 5, 1)
+    us = dev_s * 1e6 / 5
+    out["q4_0_prefill_m2048"] = {"us": round(us, 1), "TOP/s": round(2 * 2048 * 14336 * 4096 / us / 1e6, 1)}
     return out
 
 

@@ -1,0 +1,249 @@
+// Q4_0 weights x Q8_0-quantised activations on the int8 matrix cores, for m >= 5 lhs rows.
+//
+// The reference CPU kernel quantises the lhs to Q8_0 (32-wide blocks, fp16 scale) and forms, per
+// (lhs row, weight row, block), the integer dot of the codes times the product of the two block
+// scales.  Here one v_mfma_i32_16x16x32_i8 produces the 16 x 16 integer block dots of 16 lhs rows
+// against 16 weight rows for one block (K = 32 is exactly a block, so the integer sums are the
+// reference's, bit for bit), and the lanes apply  acc += float(isum - 8 asum) * (d_w * d_a)  as the
+// decode kernel does.
+//
+// lhs side: a pre-pass writes the Q8_0 codes in matrix-core operand order (for every 16-row tile and
+// block, 64 lanes x 8 bytes, so a wavefront's operand load is 512 contiguous bytes), and the block
+// scales and code sums transposed to [tile][block][16 rows] so that the four rows a lane scales are
+// one 16-byte load.  Rows beyond m are zero.
+//
+// Weight side: 18-byte blocks are only 2-byte aligned.  A wavefront owns 16 weight rows and a
+// share of K; it copies runs of 16 blocks of its 16 rows into private LDS with aligned 16-byte
+// loads (19 pieces per row and run), and each lane reads its 8 code bytes and the block scale as
+// aligned dwords joined by v_alignbyte_b32.  The nibbles stay unsigned (0..15); the -8 goes through
+// the activation code sums.  The 4 or 8 wavefronts of a workgroup add their K shares through LDS.
+// For m > 16 the grid's second dimension walks groups of four 16-row tiles, each group streaming the
+// weights again (this path is bound by the per-block fp32 scaling in the vector ALUs, not by the
+// matrix cores: 4 instructions per (lhs row, weight row, block)).
+#include <stdlib.h>
+
+#include "qmm_internal.h"
+
+namespace qmm {
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kRun = 16;                 // blocks per staged run
+constexpr int kRowPieces = 19;           // 16-byte pieces per row and run: 288 bytes + lead-in
+constexpr int kRowLds = kRowPieces * 16; // 304
+constexpr int kWaveLds = 16 * kRowLds + 16;  // one dword of read-ahead past the last row
+
+struct LhsQ8T {
+    int8_t* codes;   // [tiles][k/32][64][8]
+    float* scale;    // [tiles][k/32][16]
+    int32_t* sum;    // [tiles][k/32][16]
+    int64_t bytes;
+};
+inline LhsQ8T lhs_q8t(void* ws, int64_t m, int64_t k) {
+    auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
+    const int64_t tiles = (m + 15) / 16, nkb = k / 32;
+    LhsQ8T p;
+    char* b = (char*)ws;
+    p.codes = (int8_t*)b;
+    int64_t off = up(tiles * nkb * 512);
+    p.scale = (float*)(b + off);
+    off += up(tiles * nkb * 64);
+    p.sum = (int32_t*)(b + off);
+    off += up(tiles * nkb * 64);
+    p.bytes = off;
+    return p;
+}
+
+}  // namespace
+
+// One 32-lane group per (padded lhs row, block); same rounding rule as the Q8_0 quantiser:
+// d = amax / 127 stored as fp16, codes = round-half-away(x / d) with the fp32 d.
+template <typename InT>
+__global__ __launch_bounds__(256) void quantize_q8_0_operand_kernel(const InT* __restrict__ x, int m, int k, int64_t ngroups,
+                                                                    int8_t* __restrict__ codes, float* __restrict__ dscale,
+                                                                    int32_t* __restrict__ csum) {
+    const int64_t grp = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    const int l = threadIdx.x & 31;
+    if (grp >= ngroups) return;
+    const int nkb = k >> 5;
+    const int64_t row = grp / nkb;
+    const int kb = (int)(grp - row * nkb);
+    const float v = row < m ? load_f32(x, row * (int64_t)k + kb * 32 + l) : 0.0f;
+    float amax = fabsf(v);
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)roundf(v * id);
+    int sum = q;
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 32);
+    const int64_t tile = row >> 4;
+    const int mm = (int)(row & 15), g = l >> 3;
+    const int64_t tb = tile * nkb + kb;
+    codes[(tb * 64 + g * 16 + mm) * 8 + (l & 7)] = (int8_t)q;
+    if (l == 0) {
+        dscale[tb * 16 + mm] = h2f(f2h(d));
+        csum[tb * 16 + mm] = sum;
+    }
+}
+
+template <int MG>
+__global__ __launch_bounds__(512) void gemm_q4_0_kernel(const uint8_t* __restrict__ w, const int8_t* __restrict__ codes,
+                                                        const float* __restrict__ dscale, const int32_t* __restrict__ csum,
+                                                        float* __restrict__ out, int m, int n, int k) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nkb = k >> 5;
+    const int64_t row_bytes = (int64_t)nkb * Q4_0_BPB;
+    const int n0 = (int)blockIdx.x * 16;
+    const int tile0 = (int)blockIdx.y * MG;           // first 16-row lhs tile of this pass
+    const int tiles = (m + 15) >> 4;
+    const int nn = lane & 15, g = lane >> 4;
+    uint8_t* wbuf = smem + wave * kWaveLds;
+    const uint32_t* lds32 = (const uint32_t*)wbuf;
+
+    // this wavefront's share of K (4 or 8 wavefronts per workgroup)
+    const int nw = (int)(blockDim.x >> 6);
+    const int kb0 = wave * nkb / nw, kb1 = (wave + 1) * nkb / nw;
+
+    float acc[MG][4];
+#pragma unroll
+    for (int t = 0; t < MG; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+
+    // piece p = lane + 64 i of the run: row p / 19, 16-byte piece p % 19 of that row's run
+    int prow[5], pidx[5];
+#pragma unroll
+    for (int i = 0; i < 5; i++) {
+        const int p = min(lane + 64 * i, 16 * kRowPieces - 1);  // pieces 0..303; the last load is partial
+        prow[i] = p / kRowPieces;
+        pidx[i] = p - prow[i] * kRowPieces;
+    }
+    const uint8_t* my_row = w + (int64_t)min(n0 + nn, n - 1) * row_bytes;  // the row this lane decodes
+
+    for (int kb = kb0; kb < kb1; kb += kRun) {
+        const int nb = min(kRun, kb1 - kb);
+        // stage: aligned 16-byte pieces covering blocks kb .. kb + nb - 1 of each of the 16 rows
+        uint4 r0, r1, r2, r3, r4;
+#define QMM_STAGE_LOAD(I, R)                                                                                          \
+    do {                                                                                                              \
+        const uintptr_t ad_ = (uintptr_t)(w + (int64_t)min(n0 + prow[I], n - 1) * row_bytes + (int64_t)kb * Q4_0_BPB); \
+        const int dl_ = (int)(ad_ & 15);                                                                              \
+        const int last_ = (dl_ + nb * Q4_0_BPB + 15) / 16 - 1;                                                        \
+        R = ((const uint4*)(ad_ - (uintptr_t)dl_))[min(pidx[I], last_)];                                              \
+    } while (0)
+        QMM_STAGE_LOAD(0, r0);
+        QMM_STAGE_LOAD(1, r1);
+        QMM_STAGE_LOAD(2, r2);
+        QMM_STAGE_LOAD(3, r3);
+        QMM_STAGE_LOAD(4, r4);
+#undef QMM_STAGE_LOAD
+        __builtin_amdgcn_wave_barrier();  // the previous run's LDS reads are issued (LDS is in order per wavefront)
+        *(uint4*)(wbuf + prow[0] * kRowLds + pidx[0] * 16) = r0;
+        *(uint4*)(wbuf + prow[1] * kRowLds + pidx[1] * 16) = r1;
+        *(uint4*)(wbuf + prow[2] * kRowLds + pidx[2] * 16) = r2;
+        *(uint4*)(wbuf + prow[3] * kRowLds + pidx[3] * 16) = r3;
+        if (lane + 256 < 16 * kRowPieces) *(uint4*)(wbuf + prow[4] * kRowLds + pidx[4] * 16) = r4;
+        __builtin_amdgcn_wave_barrier();
+
+        const int delta = (int)((uintptr_t)(my_row + (int64_t)kb * Q4_0_BPB) & 15);
+        for (int b = 0; b < nb; b++) {
+            // weight operand: 8 code bytes of k-group g (low nibbles of bytes 8(g&1).., or their high nibbles)
+            const int boff = nn * kRowLds + delta + Q4_0_BPB * b;
+            const int qoff = boff + 2 + 8 * (g & 1);
+            const int wi = qoff >> 2;
+            const uint32_t sh = (uint32_t)(qoff & 3);
+            const uint32_t w0 = lds32[wi], w1 = lds32[wi + 1], w2 = lds32[wi + 2];
+            uint32_t lo = __builtin_amdgcn_alignbyte(w1, w0, sh), hi = __builtin_amdgcn_alignbyte(w2, w1, sh);
+            if (g & 2) {
+                lo >>= 4;
+                hi >>= 4;
+            }
+            lo &= 0x0F0F0F0Fu;
+            hi &= 0x0F0F0F0Fu;
+            const long bop = (long)(((uint64_t)hi << 32) | lo);
+            const uint32_t dw32 = lds32[boff >> 2] >> (8 * (boff & 3));
+            const float dw = h2f((uint16_t)(dw32 & 0xffffu));
+#pragma unroll
+            for (int t = 0; t < MG; t++) {
+                const int tile = min(tile0 + t, tiles - 1);
+                const int64_t tb = (int64_t)tile * nkb + kb + b;
+                const long aop = *(const long*)(codes + (tb * 64 + lane) * 8);
+                const float4 da = *(const float4*)(dscale + tb * 16 + 4 * g);
+                const int4v as = *(const int4v*)(csum + tb * 16 + 4 * g);
+                int4v z = {0, 0, 0, 0};
+                const int4v dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop, bop, z, 0, 0, 0);
+                acc[t][0] = fmaf((float)(dot[0] - 8 * as[0]), dw * da.x, acc[t][0]);
+                acc[t][1] = fmaf((float)(dot[1] - 8 * as[1]), dw * da.y, acc[t][1]);
+                acc[t][2] = fmaf((float)(dot[2] - 8 * as[2]), dw * da.z, acc[t][2]);
+                acc[t][3] = fmaf((float)(dot[3] - 8 * as[3]), dw * da.w, acc[t][3]);
+            }
+        }
+    }
+
+    // add the K shares: red[wave][MG*4][64]
+    __syncthreads();
+    float* red = (float*)smem;
+#pragma unroll
+    for (int t = 0; t < MG; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[(wave * MG * 4 + t * 4 + r) * 64 + lane] = acc[t][r];
+    __syncthreads();
+    if (wave == 0 && n0 + nn < n) {
+#pragma unroll
+        for (int t = 0; t < MG; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int row = (tile0 + t) * 16 + 4 * g + r;
+                if (row < m) {
+                    const int i = (t * 4 + r) * 64 + lane;
+                    float v = (red[i] + red[MG * 4 * 64 + i]) + (red[2 * MG * 4 * 64 + i] + red[3 * MG * 4 * 64 + i]);
+                    if (nw == 8)
+                        v += (red[4 * MG * 4 * 64 + i] + red[5 * MG * 4 * 64 + i]) +
+                             (red[6 * MG * 4 * 64 + i] + red[7 * MG * 4 * 64 + i]);
+                    out[(int64_t)row * n + n0 + nn] = v;
+                }
+            }
+        }
+    }
+}
+
+int64_t gemm_q4_0_workspace_bytes(int64_t m, int64_t k) { return lhs_q8t(nullptr, m, k).bytes; }
+
+hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                            float* out, void* workspace, hipStream_t s) {
+    const LhsQ8T p = lhs_q8t(workspace, m, k);
+    const int64_t tiles = (m + 15) / 16, ngroups = tiles * 16 * (k / 32);
+    dim3 qgrid((unsigned)((ngroups * 32 + 255) / 256)), qblock(256);
+    if (lhs_dtype == QMM_F32)
+        quantize_q8_0_operand_kernel<float><<<qgrid, qblock, 0, s>>>((const float*)lhs, (int)m, (int)k, ngroups, p.codes,
+                                                                     p.scale, p.sum);
+    else
+        quantize_q8_0_operand_kernel<uint16_t><<<qgrid, qblock, 0, s>>>((const uint16_t*)lhs, (int)m, (int)k, ngroups,
+                                                                        p.codes, p.scale, p.sum);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    // Few lhs rows: the weights are read once and the kernel lives on HBM latency, so K is cut eight
+    // ways for more wavefronts in flight; otherwise four.
+    const int nw = (tiles <= 2 && k >= 2048) ? 8 : 4;
+    const size_t lds = (size_t)nw * kWaveLds;  // also holds the nw x MG*4 x 64 floats of the final reduction
+    dim3 block(64 * nw);
+    if (tiles == 1) {
+        dim3 grid((unsigned)((n + 15) / 16), 1);
+        gemm_q4_0_kernel<1><<<grid, block, lds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n, (int)k);
+    } else if (tiles == 2) {
+        dim3 grid((unsigned)((n + 15) / 16), 1);
+        gemm_q4_0_kernel<2><<<grid, block, lds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n, (int)k);
+    } else {
+        dim3 grid((unsigned)((n + 15) / 16), (unsigned)((tiles + 3) / 4));
+        gemm_q4_0_kernel<4><<<grid, block, lds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n, (int)k);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace qmm

@@ -3,6 +3,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <stdlib.h>
+
 #include "qmm_internal.h"
 
 namespace {
@@ -151,7 +153,10 @@ int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     (void)n;
     if (m <= 0 || k <= 0) return 0;
-    if (encoding == QMM_Q4_0) return q8_planes(nullptr, m, k).bytes;
+    if (encoding == QMM_Q4_0) {
+        const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
+        return a > b ? a : b;
+    }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, k);
     if (encoding == QMM_GPTQ && m > 16 && k % 256 == 0) return qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k);
     return 0;
@@ -208,6 +213,8 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     if (encoding == QMM_Q4_K && !aligned(w, 16)) return fail(QMM_ERR_INVALID, "qmm_matmul: Q4_K rhs must be 16-byte aligned");
     if (!aligned(w, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: rhs must be 2-byte aligned");
 
+    if (encoding == QMM_Q4_0 && m >= 5 && !getenv("QMM_Q4_0_GEMV"))
+        return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0) {
         Q8Planes p = q8_planes(workspace, m, k);
         hipError_t e = qmm::launch_quantize_q8_0(lhs, lhs_dtype, m, k, nullptr, p.codes, p.scale, p.sum, s);

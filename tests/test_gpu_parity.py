@@ -272,3 +272,16 @@ def test_q6_k_decode_many_rows(lhs_bf16):
     want = O.matmul_f32(O.Q6_K, a, wq)
     got = qmatmul(QE.Q6_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
     assert_close(got, want, f"Q6_K 1x{n}x{k} bf16={lhs_bf16}")
+
+
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(200, 300, 1024, False), (64, 130, 4096, True), (17, 16, 96, False)])
+def test_q4_0_matmul_int8_matrix_cores(m, n, k, lhs_bf16):
+    """Q4_0 with many lhs rows: 16 x 16 integer block dots per matrix-core instruction, several passes of
+    64 lhs rows, ragged N and a K that does not split evenly over the four wavefronts."""
+    w, a = synth(51, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_0, w)
+    want = O.matmul_q4_0(a, wq)
+    got = qmatmul(QE.Q4_0, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_0 {m}x{n}x{k} bf16={lhs_bf16}")
