@@ -377,6 +377,15 @@ def extra_timings(layers, acts, gen):
         us = dev_s * 1e6 / (20 * copies)
         out[tag] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q4_0, mm, n, k) / us / 1e3, 1)}
         del cs
+    # GPTQ (group 128) decode on the gate shape
+    am1 = torch.randn((1, 4096), dtype=torch.float32, device="cuda:0", generator=gen)
+    cs = [GptqMatmul(quantize_gptq(torch.randn((14336, 4096), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02),
+                     am1) for _ in range(8)]
+    g = capture(cs)
+    dev_s, _ = time_graphs([g], 20, 3)
+    us = dev_s * 1e6 / (20 * 8)
+    out["gptq_g128_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round((14336 * 4096 * 0.5176 + 4096 * 4 + 14336 * 4) / us / 1e3, 1)}
+    del cs
     # Q4_0 prefill on the int8 matrix cores, same shape as cfg5
     ab32 = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
     g = capture([Gemv(QE.Q4_0, make_weight(QE.Q4_0, 14336, 4096, gen), ab32)])

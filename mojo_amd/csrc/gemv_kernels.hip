@@ -367,6 +367,17 @@ hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const i
 hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                             const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                             int64_t ldo, hipStream_t s) {
+    if (!getenv("QMM_GPTQ_V1")) {
+        // up to four lhs rows per pass of the column kernel; more rows take more passes over the weights
+        const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
+        bool handled = true;
+        for (int m0 = 0; m0 < m && handled; m0 += 4) {
+            hipError_t e = launch_gemv_gptq_cols((const char*)a + (int64_t)m0 * k * esz, a_dtype, qweight, scales, qzeros,
+                                                 min(4, m - m0), n, k, group, out + (int64_t)m0 * ldo, ldo, s, &handled);
+            if (e != hipSuccess) return e;
+        }
+        if (handled) return hipSuccess;
+    }
     dim3 grid((unsigned)((n + 63) / 64)), block(256);
 #define CALL(MT)                                                                                       \
     if (a_dtype == QMM_F32)                                                                            \
