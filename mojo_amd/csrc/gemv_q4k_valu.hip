@@ -276,17 +276,6 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void gemv_q4_k_stream_kernel(
     const int64_t row_bytes = (int64_t)nblk * Q4_K_BPB;
     const int sb = lane >> 3, u = lane & 7, c = u >> 1;
 
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++) {
-        const AT* ar = a + (int64_t)min(mi, m - 1) * k;
-        for (int pk = threadIdx.x; pk < nblk * 64; pk += blockDim.x) {
-            const int b = pk >> 6, p = pk & 63;
-            const int pc = p >> 4, r16 = p & 15;
-            const int pu = 2 * pc + ((r16 >> 2) & 1), pj = 4 * (r16 >> 3) + (r16 & 3);
-            lds_act[(size_t)mi * iters * 512 + (b >> 3) * 512 + pj * 64 + (b & 7) * 8 + pu] = load_a4(ar, 4 * pk);
-        }
-    }
-
     const int sh = 16 * (c & 1);
     const bool upper = c >= 2;
     const int gw = blockIdx.x * nwaves + wave, GW = gridDim.x * nwaves;
@@ -311,6 +300,18 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void gemv_q4_k_stream_kernel(
         ring[s].qs = make_uint4(0, 0, 0, 0);
         if (s < total) load_unit(ring[s], s);
     }
+    // The first ring of weight loads is already in flight: stage the activations under its latency.
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) {
+        const AT* ar = a + (int64_t)min(mi, m - 1) * k;
+        for (int pk = threadIdx.x; pk < nblk * 64; pk += blockDim.x) {
+            const int b = pk >> 6, p = pk & 63;
+            const int pc = p >> 4, r16 = p & 15;
+            const int pu = 2 * pc + ((r16 >> 2) & 1), pj = 4 * (r16 >> 3) + (r16 & 3);
+            lds_act[(size_t)mi * iters * 512 + (b >> 3) * 512 + pj * 64 + (b & 7) * 8 + pu] = load_a4(ar, 4 * pk);
+        }
+    }
+
     __syncthreads();  // staged activations visible
     // per (step, lane) sums of the 16 + 16 activations a lane multiplies: the same for every row
     float2* lds_asum = (float2*)(lds_act + (size_t)MT * iters * 512);
@@ -441,7 +442,8 @@ hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     const int r = r_env > 0 ? r_env : (n >= 8192 ? 4 : (n >= 4096 ? 2 : 1));
     const int nblk = (int)(k >> 8);
     // staged lhs rows, padded to 8 super-blocks, plus 512 bytes of lane sums per step, plus result slots
-    const size_t lds = (size_t)mt * ((nblk + 7) / 8) * (8192 + 512) + (size_t)8 * kStreamMaxRows * mt * 4;
+    const int wv_stream = (w_env == 4 || w_env == 8) ? w_env : 8;  // wavefronts per workgroup of the streaming kernel
+    const size_t lds = (size_t)mt * ((nblk + 7) / 8) * (8192 + 512) + (size_t)wv_stream * kStreamMaxRows * mt * 4;
     const bool ldsa = lds <= 64 * 1024 && !getenv("QMM_GEMV_NOLDS");
     const int waves = w_env > 0 ? w_env : (lds > 32 * 1024 ? 8 : 4);
     const int g = g_env > 0 ? g_env : 1;  // row groups per wavefront
@@ -452,7 +454,7 @@ hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, i
             if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev);
             return cu > 0 ? cu : 256;
         }();
-        const int wv = w_env > 0 ? w_env : 8;
+        const int wv = wv_stream;
         int64_t wgs = (int64_t)num_cu * (16 / wv) * (g_env > 0 ? g_env : 1);
         size_t per_cu = (size_t)160 * 1024 / lds;  // workgroups per CU that the staged activations allow
         if (per_cu < 1) per_cu = 1;
