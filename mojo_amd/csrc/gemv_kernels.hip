@@ -9,6 +9,19 @@
 
 namespace qmm {
 
+static bool env_flag_qmm_q4k_v1() {
+    static const bool v = getenv("QMM_Q4K_V1") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+static bool env_flag_qmm_q6k_v1() {
+    static const bool v = getenv("QMM_Q6K_V1") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+static bool env_flag_qmm_gptq_v1() {
+    static const bool v = getenv("QMM_GPTQ_V1") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+
 template <typename AT>
 __device__ __forceinline__ float4 load_a4(const AT* __restrict__ a, int64_t i) {
     if constexpr (sizeof(AT) == 4) {
@@ -318,8 +331,8 @@ static bool q4k_use_valu(int m) {
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
     if (!q4k_use_valu(m)) return launch_gemv_q4_k_mfma(a, a_dtype, w, m, n, k, out, ldo, s);
-    if (m <= 2 && !getenv("QMM_Q4K_V1")) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
-    if (m <= 4 && !getenv("QMM_Q4K_V1")) {
+    if (m <= 2 && !env_flag_qmm_q4k_v1()) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
+    if (m <= 4 && !env_flag_qmm_q4k_v1()) {
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
         hipError_t e = launch_gemv_q4_k_rows(a, a_dtype, w, 2, n, k, out, ldo, s);
         if (e != hipSuccess) return e;
@@ -338,7 +351,7 @@ hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m,
 
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
-    if (!getenv("QMM_Q6K_V1")) {
+    if (!env_flag_qmm_q6k_v1()) {
         bool handled = false;
         hipError_t e = launch_gemv_q6_k_rows(a, a_dtype, w, m, n, k, out, ldo, s, &handled);
         if (e != hipSuccess || handled) return e;
@@ -367,7 +380,7 @@ hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const i
 hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                             const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                             int64_t ldo, hipStream_t s) {
-    if (!getenv("QMM_GPTQ_V1")) {
+    if (!env_flag_qmm_gptq_v1()) {
         // up to four lhs rows per pass of the column kernel; more rows take more passes over the weights
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
         bool handled = true;

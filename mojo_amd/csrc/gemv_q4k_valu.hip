@@ -15,6 +15,15 @@
 
 namespace qmm {
 
+static bool env_flag_qmm_gemv_nolds() {
+    static const bool v = getenv("QMM_GEMV_NOLDS") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+static bool env_flag_qmm_gemv_rows() {
+    static const bool v = getenv("QMM_GEMV_ROWS") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+
 namespace {
 
 template <typename AT>
@@ -444,10 +453,10 @@ hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     // staged lhs rows, padded to 8 super-blocks, plus 512 bytes of lane sums per step, plus result slots
     const int wv_stream = (w_env == 4 || w_env == 8) ? w_env : 8;  // wavefronts per workgroup of the streaming kernel
     const size_t lds = (size_t)mt * ((nblk + 7) / 8) * (8192 + 512) + (size_t)wv_stream * kStreamMaxRows * mt * 4;
-    const bool ldsa = lds <= 64 * 1024 && !getenv("QMM_GEMV_NOLDS");
+    const bool ldsa = lds <= 64 * 1024 && !env_flag_qmm_gemv_nolds();
     const int waves = w_env > 0 ? w_env : (lds > 32 * 1024 ? 8 : 4);
     const int g = g_env > 0 ? g_env : 1;  // row groups per wavefront
-    if (ldsa && !getenv("QMM_GEMV_ROWS")) {
+    if (ldsa && !env_flag_qmm_gemv_rows()) {
         // streaming kernel: persistent workgroups, as many as fill the machine at 4 wavefronts per SIMD
         static const int num_cu = [] {
             int dev = 0, cu = 256;

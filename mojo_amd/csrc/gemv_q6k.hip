@@ -20,6 +20,11 @@
 
 namespace qmm {
 
+static bool env_flag_qmm_q6k_rows() {
+    static const bool v = getenv("QMM_Q6K_ROWS") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+
 namespace {
 
 constexpr int kRunBlocks = 16;                                   // blocks per staged run
@@ -349,7 +354,7 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     // loop-interchanged kernel; otherwise the row-at-a-time kernel below.
     static const int pc_env = getenv("QMM_Q6K_WG_PER_CU") ? atoi(getenv("QMM_Q6K_WG_PER_CU")) : 0;
     const int pc = pc_env > 0 ? pc_env : 3;
-    if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !getenv("QMM_Q6K_ROWS")) {
+    if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !env_flag_qmm_q6k_rows()) {
         const size_t lds2 = 4 * (size_t)kRunBytes + 4 * (size_t)kParkRows * 4;
         // enough wavefronts that none has more rows than its LDS parking slots
         const int64_t wgs = max((int64_t)cus * pc, (n + 4 * kParkRows - 1) / (4 * kParkRows));

@@ -7,6 +7,11 @@
 
 #include "qmm_internal.h"
 
+static bool env_flag_qmm_q4_0_gemv() {
+    static const bool v = getenv("QMM_Q4_0_GEMV") != nullptr;  // read once: tuning and fallback switch
+    return v;
+}
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -213,7 +218,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     if (encoding == QMM_Q4_K && !aligned(w, 16)) return fail(QMM_ERR_INVALID, "qmm_matmul: Q4_K rhs must be 16-byte aligned");
     if (!aligned(w, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: rhs must be 2-byte aligned");
 
-    if (encoding == QMM_Q4_0 && m >= 5 && !getenv("QMM_Q4_0_GEMV"))
+    if (encoding == QMM_Q4_0 && m >= 5 && !env_flag_qmm_q4_0_gemv())
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0) {
         Q8Planes p = q8_planes(workspace, m, k);
