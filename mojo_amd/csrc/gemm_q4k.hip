@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
                                                            const _Float16* __restrict__ asum,
                                                            const float* __restrict__ inv, float* __restrict__ out,
                                                            int m, int n, int k, int tiles_m, int tiles_n,
-                                                           int with_min, int accumulate) {
+                                                           int with_min, int accumulate, int ksplit) {
     constexpr int BM = 64 * WM;  // WM wavefront rows of 64 lhs rows each; 256 * WM threads
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) _Float16 lds_s[2][BM * 16];
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
     const int nl = lane & 31, g = lane >> 5;
     const int nblk = k >> 8;
     const int64_t row_bytes = (int64_t)nblk * Q4_K_BPB;
-    const int total = tiles_m * tiles_n;
+    const int total = tiles_m * tiles_n * ksplit;  // work units: (tile, share of K)
     const int per_xcd = (total + 7) / 8;
     const int a_row = tid >> 2, a_seg = tid & 3;
     _Float16* a_dst = &lds_a[0][a_row * A_STRIDE + a_seg * 8];
@@ -85,23 +85,26 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
     const _Float16* s_frag_base = &lds_s[0][(wm * 64 + nl) * 16 + g * 8];
     const int q_lane_off = 16 + 16 * g;
 
-    // Tiles of one XCD (workgroup ids congruent mod 8 share an XCD and its L2) form a contiguous
-    // range of an order that keeps two lhs tile rows fixed while walking N.
-    // Slot j of an XCD (workgroup ids congruent mod 8 share an XCD and its L2) takes tiles j, j + S, ...
-    // of the XCD's contiguous tile range.  (Cutting the leftover tiles of the last round along K to fill
-    // every slot was tried and lost: a workgroup that has its compute unit to itself runs its last tile
-    // about 1.6x faster, and the partial sums cost atomic traffic.)
+    // Units of one XCD (workgroup ids congruent mod 8 share an XCD and its L2) form a contiguous range of
+    // an order that keeps a few lhs tile rows fixed while walking N; slot j of an XCD takes units j, j + S, ...
+    // With ksplit > 1 (few lhs rows, hence few tiles) a unit is one tile's share of the super-blocks and
+    // writes its partial result to slice `ks` of `out`, which is then a [ksplit][m][n] buffer that a
+    // second kernel adds up in a fixed order.  (For large m, cutting only the leftover tiles of the last
+    // round along K was tried and lost: a workgroup that has its compute unit to itself runs its last tile
+    // about 1.6x faster, and the partial sums cost traffic.)
     for (int it = 0, tq = (int)(blockIdx.x >> 3); tq < per_xcd; it++, tq += (int)(gridDim.x >> 3)) {
-        const int nb = nblk, ns = nb * 4;
         const int o = (int)(blockIdx.x & 7) * per_xcd + tq;
         if (o >= total) break;
+        const int tile = o / ksplit, ks = o - tile * ksplit;
+        const int kb0 = ks * nblk / ksplit;
+        const int nb = (ks + 1) * nblk / ksplit - kb0, ns = nb * 4;
         int tile_m, tile_n;
-        tile_coords(o, tiles_m, tiles_n, 4 / WM, tile_m, tile_n);
+        tile_coords(tile, tiles_m, tiles_n, 4 / WM, tile_m, tile_n);
         const int m0 = tile_m * BM, n0 = tile_n * BN;
 
         // lhs chunk staging: 128 rows x 128 bytes per step, two 16-byte pieces per thread; two
         // register sets (parity of the step) keep two steps of loads in flight.
-        const uint4* a_src = (const uint4*)(a16 + (int64_t)min(m0 + a_row, m - 1) * k + a_seg * 8);
+        const uint4* a_src = (const uint4*)(a16 + (int64_t)min(m0 + a_row, m - 1) * k + kb0 * 256 + a_seg * 8);
         uint4 ax0_0, ax0_1, ax1_0, ax1_1;
 #define QMM_A_LOAD(SET, STEP)                          \
     do {                                               \
@@ -117,8 +120,8 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
     } while (0)
 
         // this lane's two weight columns
-        const uint8_t* wcol0 = w + (int64_t)min(n0 + wn * 64 + nl, n - 1) * row_bytes;
-        const uint8_t* wcol1 = w + (int64_t)min(n0 + wn * 64 + 32 + nl, n - 1) * row_bytes;
+        const uint8_t* wcol0 = w + (int64_t)min(n0 + wn * 64 + nl, n - 1) * row_bytes + kb0 * Q4_K_BPB;
+        const uint8_t* wcol1 = w + (int64_t)min(n0 + wn * 64 + 32 + nl, n - 1) * row_bytes + kb0 * Q4_K_BPB;
         uint4 qx0_c0, qx0_c1, qx1_c0, qx1_c1;
 #define QMM_Q_LOAD(SET, STEP)                                                 \
     do {                                                                      \
@@ -142,7 +145,7 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
 
         // block headers and sub-block sums are fetched one super-block ahead
         uint4 hdr_n0, hdr_n1, as_n = make_uint4(0, 0, 0, 0);
-        const uint4* as_src = (const uint4*)(asum + (int64_t)min(m0 + (tid >> 1), m - 1) * nblk * 16 + (tid & 1) * 8);
+        const uint4* as_src = (const uint4*)(asum + ((int64_t)min(m0 + (tid >> 1), m - 1) * nblk + kb0) * 16 + (tid & 1) * 8);
         auto hdr_prefetch = [&](int blk) {
             const int bc = min(blk, nb - 1);
             hdr_n0 = *(const uint4*)(wcol0 + bc * Q4_K_BPB);
@@ -337,7 +340,7 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
                     const float4 q = iv[r >> 2];
                     const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
                     if (row < m) {
-                        float* o = out + (int64_t)row * n;
+                        float* o = out + ((int64_t)ks * m + row) * n;
                         const float v0 = acc[mi][0][r] * is, v1 = acc[mi][1][r] * is;
                         if (accumulate) {
                             if (c0_ok) o[col0] += v0;
@@ -353,7 +356,33 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
     }
 }
 
-int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return lhs_planes(nullptr, lhs_dtype, m, k).bytes; }
+// out[i] (+)= part[0][i] + part[1][i] + ... in that order
+__global__ __launch_bounds__(256) void sum_k_shares_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                           int64_t count, int ksplit, int accumulate) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float v = accumulate ? out[i] : 0.0f;
+    for (int s = 0; s < ksplit; s++) v += part[(int64_t)s * count + i];
+    out[i] = v;
+}
+
+namespace {
+
+// Shares of K per tile: 1 when the tiles alone fill the machine, otherwise enough for about a thousand
+// work units, each at least two super-blocks long.  A function of the shape only.
+int k_shares(int64_t m, int64_t n, int64_t k, int bm) {
+    const int64_t tiles = ((m + bm - 1) / bm) * ((n + BN - 1) / BN), nblk = k / 256;
+    if (tiles >= 256) return 1;
+    const int64_t want = (1024 + tiles - 1) / tiles, cap = nblk / 2 > 1 ? nblk / 2 : 1;
+    return (int)(want < cap ? want : cap);
+}
+
+}  // namespace
+
+int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    const int ks = k_shares(m, n, k, 64);
+    return lhs_planes(nullptr, lhs_dtype, m, k).bytes + (ks > 1 ? (int64_t)ks * m * n * 4 : 0);
+}
 
 hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                float* out, void* workspace, hipStream_t s) {
@@ -362,10 +391,12 @@ hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, in
     if (e != hipSuccess) return e;
     // QMM_GEMM_WM=2 selects 8-wavefront workgroups on 128-row tiles (one per compute unit); the default
     // is 4-wavefront workgroups on 64-row tiles, two per compute unit, which run out of phase.
-    static const int wm_rows = getenv("QMM_GEMM_WM") && atoi(getenv("QMM_GEMM_WM")) == 2 ? 2 : 1;
+    static const int wm_env = getenv("QMM_GEMM_WM") && atoi(getenv("QMM_GEMM_WM")) == 2 ? 2 : 1;
+    const int ksplit = k_shares(m, n, k, 64);
+    const int wm_rows = ksplit > 1 ? 1 : wm_env;
     const int bm = 64 * wm_rows;
     const int tiles_m = (int)((m + bm - 1) / bm), tiles_n = (int)((n + BN - 1) / BN);
-    const int total = tiles_m * tiles_n;
+    const int total = tiles_m * tiles_n * ksplit;
     const int per_xcd = (total + 7) / 8;
     static int cus = 0;
     if (!cus) {
@@ -377,13 +408,20 @@ hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, in
     // persistent workgroups: as many as fit on the device at once (two per compute unit for the 4-wavefront shape)
     const int wg = 8 * min(per_xcd, max(1, cus / 8) * (2 / wm_rows));
     dim3 grid((unsigned)wg), block(256 * wm_rows);
-#define QMM_GEMM_GO(WM_)                                                                                             \
-    do {                                                                                                           \
-        gemm_q4_k_kernel<WM_><<<grid, block, 0, s>>>(w, p.a16, p.asum, p.inv, out, (int)m, (int)n, (int)k,     \
-                                                        tiles_m, tiles_n, 1, 0);                                   \
-        if (p.a16_lo) /* fp32 lhs: the residual plane, added on top */                                             \
-            gemm_q4_k_kernel<WM_><<<grid, block, 0, s>>>(w, p.a16_lo, p.asum, p.inv, out, (int)m, (int)n,      \
-                                                            (int)k, tiles_m, tiles_n, 0, 1);                       \
+    float* part = ksplit > 1 ? (float*)((char*)workspace + p.bytes) : nullptr;
+    float* dst = part ? part : out;
+    const int64_t count = m * n;
+    dim3 rgrid((unsigned)((count + 255) / 256)), rblock(256);
+#define QMM_GEMM_GO(WM_)                                                                                          \
+    do {                                                                                                          \
+        gemm_q4_k_kernel<WM_><<<grid, block, 0, s>>>(w, p.a16, p.asum, p.inv, dst, (int)m, (int)n, (int)k,       \
+                                                     tiles_m, tiles_n, 1, 0, ksplit);                             \
+        if (part) sum_k_shares_kernel<<<rgrid, rblock, 0, s>>>(part, out, count, ksplit, 0);                      \
+        if (p.a16_lo) { /* fp32 lhs: the residual plane, added on top */                                          \
+            gemm_q4_k_kernel<WM_><<<grid, block, 0, s>>>(w, p.a16_lo, p.asum, p.inv, dst, (int)m, (int)n,        \
+                                                         (int)k, tiles_m, tiles_n, 0, part ? 0 : 1, ksplit);      \
+            if (part) sum_k_shares_kernel<<<rgrid, rblock, 0, s>>>(part, out, count, ksplit, 1);                  \
+        }                                                                                                         \
     } while (0)
     if (wm_rows == 2)
         QMM_GEMM_GO(2);

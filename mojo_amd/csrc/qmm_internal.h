@@ -50,7 +50,7 @@ hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight,
                             const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                             int64_t ldo, hipStream_t s);
 // Prefill-shape kernels (m > 16).
-int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
+int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                             float* out, void* workspace, hipStream_t s);
 
