@@ -60,7 +60,9 @@ __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float1
 //   kLhsOrderQ4K : 32*(f/2) + 16*g + 8*(f%2) + (0,2,1,3,4,6,5,7)[slot]
 //   kLhsOrderGPTQ: 16*f + 8*g + (0,4,1,5,2,6,3,7)[slot], odd columns pre-multiplied by 1/16
 //                  (their codes are used in place in the high nibble position, 16*q)
-constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1;
+//   kLhsOrderQ4K16: 8*(pos/8) + (0,2,1,3,4,6,5,7)[slot]   (natural order, the two middle pairs of every 8 swapped:
+//                  the operand order of the 16x16x32 small-batch kernel)
+constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1, kLhsOrderQ4K16 = 2;
 
 template <typename AT, int ORDER>
 __global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
@@ -91,6 +93,10 @@ __global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a,
             const int hin = kl >> 5, gg = (kl >> 4) & 1, odd = (kl >> 3) & 1;
             const int pos = (2 * hin + odd) * 16 + gg * 8 + (kl & 4);
             const int64_t o = (int64_t)row * k + (i & ~63) + pos;
+            *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
+            if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
+        } else if constexpr (ORDER == kLhsOrderQ4K16) {
+            const int64_t o = (int64_t)row * k + i;
             *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
             if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
         } else {

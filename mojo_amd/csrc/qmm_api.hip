@@ -165,7 +165,8 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         return a > b ? a : b;
     }
-    if (encoding == QMM_Q4_K && m >= 9 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
+    if (encoding == QMM_Q4_K && m >= 3 && m <= 16 && k % 256 == 0) return qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);
+    if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     if (encoding == QMM_GPTQ && m > 16 && k % 256 == 0) return qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k);
     return 0;
 }
@@ -236,9 +237,10 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         return QMM_OK;
     }
 
-    // measured on the 14336 x 4096 shape: 5..8 lhs rows are faster through the matrix-core decode kernel
-    // (32 us), 9..16 through the prefill kernel with K cut into shares (49 us against 92 us)
-    if (encoding == QMM_Q4_K && m >= 9 && !env_flag_qmm_q4k_small_gemv())
+    // 3..16 lhs rows: the small-batch matrix-core kernel; more: the prefill kernel
+    if (encoding == QMM_Q4_K && m >= 3 && m <= 16 && !env_flag_qmm_q4k_small_gemv())
+        return hip_status(qmm::launch_gemv_q4_k_mm(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K small batch)");
+    if (encoding == QMM_Q4_K && m > 16)
         return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");
 
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
