@@ -1,29 +1,34 @@
-// Q4_K small-batch kernel (3 <= m <= 16 lhs rows): weight rows streamed through LDS, 16 x 16 x 32
+// Q4_K small-batch kernel (up to 16 lhs rows): weight rows streamed through LDS, 16 x 16 x 32
 // matrix-core products over exact integer codes.
 //
 // Arithmetic is that of the prefill kernel (gemm_q4k.hip): a masked nibble is the fp16 subnormal
 // q*2^-24, one packed fp16 multiply folds the 6-bit sub-block scale in, the lhs is narrowed to fp16
-// (hi, plus a residual plane for fp32 input) after an exact per-row power-of-two scaling, the fp32
-// super-block scale is applied in the lanes and the min term is one extra matrix product per
-// super-block (K = 32 slots hold  asum_hi x dmn_hi,  asum_lo x dmn_hi,  asum_hi x dmn_lo).
+// (hi, plus a residual plane) after an exact power-of-two scaling, the fp32 super-block scale is
+// applied in the lanes and the min term is one extra matrix product per super-block.
 //
 // Shape of the work: a workgroup of 8 wavefronts walks a list of up to 4 weight tiles of 16 rows.
-// Wavefront w owns the super-blocks [w nblk / 8, (w + 1) nblk / 8) of every row and goes through
-// them two at a time ("groups"); its lhs fragments for the two super-blocks of a group (16 lhs rows,
-// hi and residual planes) are loaded into registers once per group and reused for every tile of the
-// workgroup (loading them per tile made the lhs planes, not the weights, the bulk of the traffic).
-// The weights of a (group, tile) item, 288 contiguous bytes of each of the 16 rows, travel from
-// global memory straight into a wavefront-private ring of three LDS slots (global_load_lds_dwordx4:
-// no registers are held while they are in flight), two items ahead of the one being decoded; the
-// wavefront waits with a vmcnt that leaves the younger items in flight.  Each lane (row n =
-// lane % 16, k-group lane / 16) reads its 8 code bytes of a 64-wide chunk with one ds_read_b64 and
-// they serve two matrix-core instructions, the low nibbles (sub-block 2c) and the high nibbles
-// (sub-block 2c + 1).  A wavefront accumulates its partial result of a tile over the groups in a
-// private LDS slot; one barrier at the end, then the 8 partial results of a tile are added in a
-// fixed order.
+// The super-blocks of a row are dealt to the wavefronts in groups of 16, two per wavefront; a
+// wavefront's lhs fragments for its two super-blocks of a group are held in registers and reused
+// for every tile of the workgroup.  The weights of a (group, tile) item, 288 contiguous bytes of
+// each of the 16 rows, travel from global memory straight into a wavefront-private ring of three
+// LDS slots (global_load_lds_dwordx4: no registers are held while they are in flight), two items
+// ahead of the one being decoded; the wavefront waits with a vmcnt that leaves the younger items
+// in flight.  Lane (row n = lane % 16, chunk c = lane / 16) decodes the 32 code bytes of chunk c of
+// its row: sub-block 2c in the low nibbles, 2c + 1 in the high ones, so it needs only those two
+// scales and mins; 8 code bytes feed two matrix-core instructions.  A wavefront accumulates its
+// partial result of a tile over the groups in a private LDS slot; one barrier at the end, then the
+// 8 partial results of a tile are added in a fixed order.
+//
+// Two ways to the lhs fragments:
+//   m <= 8  the wavefront converts its own two super-blocks of every lhs row itself (scaled by a
+//           power of two per lhs row and super-block, hi part in operand rows 0..7, residual in
+//           rows 8..15, added at the end): one launch, no workspace;
+//   m > 8   a separate pass (gemm_lhs.h) has written fp16 planes scaled per lhs row; fp32 lhs costs
+//           a second matrix product per operand.
 #include <stdlib.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "gemm_lhs.h"
 #include "qmm_internal.h"
@@ -37,24 +42,29 @@ namespace {
 constexpr int kRunBlk = 2;                      // super-blocks per item
 constexpr int kRowBytes = kRunBlk * Q4_K_BPB;   // 288: bytes of a row in an item (18 pieces of 16 bytes)
 constexpr int kPieces = 16 * kRowBytes / 16;    // 288 pieces per item, piece p at LDS offset 16 p
-constexpr int kLoads = (kPieces + 63) / 64;     // 5 load instructions per item
-constexpr int kSlotBytes = kLoads * 1024;       // 5120: the last instruction's upper lanes land in the slot's unused tail
+constexpr int kLoads = (kPieces + 63) / 64;     // 5 load instructions per item, the last one by 32 lanes
+constexpr int kSlotBytes = kPieces * 16;        // 4608
 constexpr int kSlots = 3;                       // ring: one item being decoded, two in flight
 constexpr float kTwo24f = 16777216.0f;
 constexpr int kWaves = 8;                       // wavefronts per workgroup
 constexpr int kMaxTiles = 4;                    // tiles per workgroup (private LDS accumulators per wavefront)
+constexpr int kPlaneStride = 528;               // staged lhs plane of one super-block: 512 bytes + 16 (bank spread)
+constexpr int kStageBytes = 2 * kPlaneStride + 32;  // hi plane, residual plane, 8 sub-block sums (hi, lo)
 constexpr int kRingBytes = kWaves * kSlots * kSlotBytes;
-constexpr int kLdsBytes = kRingBytes + kWaves * kMaxTiles * 4 * 64 * 4;
+constexpr int kAccBytes = kWaves * kMaxTiles * 4 * 64 * 4;
+constexpr int kLdsBytes = kRingBytes + kAccBytes;
+static_assert(4 * kStageBytes + 16 <= kSlotBytes, "four staged lhs rows and their scales fit the free ring slot");
 
 typedef __attribute__((address_space(3))) void* lds_space_ptr;
 
 // 16 bytes per lane from global memory to LDS at lds_base + 16 * lane (lds_base uniform).  The
 // compiler is not told that this is a load: it keeps no count of it, and the caller waits with
 // wait_vmcnt before reading the slot.  (The builtin for this instruction makes the compiler wait
-// for all of them before every LDS read, which would leave nothing in flight.)  m0 is put back.
+// for all of them before every LDS read, which would leave nothing in flight.)  m0 is put back; the
+// s_nop is the wait state the hardware wants between a write of m0 and an LDS-direct load.
 __device__ __forceinline__ void load16_to_lds(const void* g, uint32_t lds_base) {
     uint32_t keep;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
                  : "=&s"(keep)
                  : "v"(g), "s"(lds_base)
                  : "memory");
@@ -66,12 +76,48 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));  // what the packed conversion builtin returns
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Plain global loads that the compiler is not told about either, for values that must arrive while
+// the loads into LDS above are in flight: a wait the compiler places itself counts those too and
+// would drain them.  The destination may only be used after wait_vmcnt and tie() on it.
+__device__ __forceinline__ void hidden_load(u32x4& d, const void* g) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(g) : "memory");
+}
+__device__ __forceinline__ void hidden_load(u32x2& d, const void* g) {
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(g) : "memory");
+}
+template <typename T>
+__device__ __forceinline__ void tie(T& d) {
+    asm volatile("" : "+v"(d));
+}
+// wait until at most 5 * items + extra loads are outstanding (items 0..2, extra 0 or NX)
+template <int NX>
+__device__ __forceinline__ void wait_items(int items, bool extra) {
+    if (extra) {
+        if (items >= 2) wait_vmcnt<2 * kLoads + NX>();
+        else if (items == 1) wait_vmcnt<kLoads + NX>();
+        else wait_vmcnt<NX>();
+    } else {
+        if (items >= 2) wait_vmcnt<2 * kLoads>();
+        else if (items == 1) wait_vmcnt<kLoads>();
+        else wait_vmcnt<0>();
+    }
+}
+
+__device__ __forceinline__ half8 zero_half8() { return pack4(0u, 0u, 0u, 0u); }
+
 }  // namespace
 
-// NPART: matrix products per weight operand (2: hi and residual lhs planes).  STACK (with NPART 1, m <= 8):
-// the residual plane of lhs row r rides in operand row r + 8 and the two results are added at the end.
-template <int NPART, bool STACK>
-__global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __restrict__ w, const _Float16* __restrict__ a16,
+// NPART: matrix products per weight operand (2: hi and residual planes from the workspace).
+// INLINE: lhs converted in the kernel (m <= 8, AT = float or bf16 bits); otherwise a16 / a16_lo / asum /
+// inv come from prep_lhs_kernel<.., kLhsOrderQ4K16>.
+// MROWS (INLINE): lhs rows converted, 1, 2, 4 or 8 (>= m; rows past m repeat the last one and their results are dropped).
+template <int NPART, bool INLINE, int MROWS, typename AT>
+__global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                           const _Float16* __restrict__ a16,
                                                            const _Float16* __restrict__ a16_lo,
                                                            const _Float16* __restrict__ asum, const float* __restrict__ inv,
                                                            float* __restrict__ out, int m, int n, int k) {
@@ -113,56 +159,191 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
         const int last_piece = max(cnt, 1) * 9 - 1;
         const uint8_t* base = w + (int64_t)bc * Q4_K_BPB;
 #pragma unroll
-        for (int i = 0; i < kLoads; i++)
-            load16_to_lds(base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * min(pidx[i], last_piece),
-                          ring_lds + slot * kSlotBytes + i * 1024);
+        for (int i = 0; i < kLoads; i++) {
+            const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * min(pidx[i], last_piece);
+            if (i < kLoads - 1 || lane < kPieces - 64 * (kLoads - 1))  // the last instruction: 32 lanes
+                load16_to_lds(src, ring_lds + slot * kSlotBytes + i * 1024);
+        }
     };
 
-    // lhs row whose fragments this lane holds (rows >= m repeat the last one)
-    const int mrow = min(STACK ? (nn & 7) : nn, m - 1);
-    const _Float16* a_hi = (STACK && nn >= 8 ? a16_lo : a16) + (int64_t)mrow * k + 8 * kg;
-    const _Float16* a_lo = NPART == 2 ? a16_lo + (int64_t)mrow * k + 8 * kg : nullptr;
-    const _Float16* as_row = asum + (int64_t)mrow * nblk * 16 + (kg & 1) * 8;
-    const uint32_t M1 = 0x000F000Fu, M2 = 0x00F000F0u;
-
+    int last_issued = -1;  // newest item whose loads into LDS have been issued
+    int x_after = -1;      // the item that was newest when the last load_x was issued
     // items in flight: it + 1 and it + 2
     int ig = 0, it_t = 0, islot = 0;  // next item to issue
     auto issue_next = [&]() {
         issue(ig, it_t, islot);
+        last_issued++;
         islot = islot == kSlots - 1 ? 0 : islot + 1;
         if (++it_t == my_tiles) { it_t = 0; ig++; }
     };
+    // INLINE: raw lhs values of the wavefront's two super-blocks of the next group to convert; lane holds
+    // columns 4 lane .. 4 lane + 3 of each.  Loaded a group ahead (the first ones before the first weights).
+    constexpr int RP = MROWS < 4 ? MROWS : 4;  // rows converted together (they share the free ring slot as staging)
+    constexpr int NX = INLINE ? kRunBlk * MROWS : 0;  // load instructions of one load_x
+    typedef typename std::conditional<sizeof(AT) == 4, u32x4, u32x2>::type xraw_t;
+    xraw_t xr[kRunBlk][MROWS];
+    auto load_x = [&](int g) {
+        int b0, cnt;
+        group_share(g, b0, cnt);
+#pragma unroll
+        for (int bb = 0; bb < kRunBlk; bb++) {
+            const int blk = min(b0 + bb, nblk - 1);
+#pragma unroll
+            for (int mi = 0; mi < MROWS; mi++)
+                hidden_load(xr[bb][mi], a + (int64_t)min(mi, m - 1) * k + (int64_t)blk * 256 + 4 * lane);
+        }
+        x_after = last_issued;
+    };
+    if constexpr (INLINE) {
+        if (total > 0) load_x(0);
+    }
+    // one item before the conversion: its loads keep the memory system busy while the lhs is converted, and
+    // the wavefront is not held up in the issue of more loads before it gets to the conversion
     if (total > 0) issue_next();
-    if (total > 1) issue_next();
+    if (!INLINE && total > 1) issue_next();
 
-    half8 fa[kRunBlk][8][NPART], fs[kRunBlk];
+    // lhs operand row of this lane: INLINE: row nn % 8, hi plane for nn < 8, residual for nn >= 8
+    const int mrow = min(INLINE ? (nn & 7) : nn, m - 1);
+    const uint32_t M1 = 0x000F000Fu, M2 = 0x00F000F0u;
+    const int sh = 16 * (kg & 1);  // byte pair (2c, 2c + 1) mod 4 inside a dword of the 6-bit fields
+    const bool upper = kg >= 2;    // sub-blocks 4..7 use the split encoding
+
+    half8 fa[kRunBlk][4][2][NPART], fs[kRunBlk];
+    float bs[kRunBlk][4];  // INLINE: inverse lhs scale of (super-block, accumulator register's lhs row)
+#pragma unroll
+    for (int bb = 0; bb < kRunBlk; bb++) {
+        fs[bb] = zero_half8();
+#pragma unroll
+        for (int r = 0; r < 4; r++) bs[bb][r] = 0.0f;
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int q = 0; q < NPART; q++) fa[bb][p][h][q] = zero_half8();
+    }
+
     int grp = 0, ti = 0, slot = 0;
     for (int it = 0; it < total; it++) {
         int gb0, nb;
         group_share(grp, gb0, nb);
         if (ti == 0) {
-            // lhs fragments and sub-block sums of the group's super-blocks: registers, reused for every tile
+            // lhs fragments of the group's super-blocks: registers, reused for every tile.
+            // Fragment (p, h) of chunk kg holds lhs columns 64 kg + 32 h + 8 p + (0,2,1,3,4,6,5,7).
+            if constexpr (INLINE) {
+                // The slot the next item will be loaded into is free: RP staged rows fit it.
+                uint8_t* stg = ring + islot * kSlotBytes;
+                const int rr = nn & 7;
+                // the raw lhs values: everything issued after them may stay in flight
+                wait_items<0>(last_issued - x_after, false);
 #pragma unroll
-            for (int bb = 0; bb < kRunBlk; bb++) {
-                const int blk = min(gb0 + bb, nblk - 1);
-                fs[bb] = *(const half8*)(as_row + (int64_t)blk * 16);
-                if (STACK && nn >= 8) fs[bb] = half8{0, 0, 0, 0, 0, 0, 0, 0};  // the min term belongs to the hi rows
+                for (int bb = 0; bb < kRunBlk; bb++)
 #pragma unroll
-                for (int sl = 0; sl < 8; sl++) {
-                    fa[bb][sl][0] = *(const half8*)(a_hi + (int64_t)blk * 256 + 32 * sl);
-                    if constexpr (NPART == 2) fa[bb][sl][1] = *(const half8*)(a_lo + (int64_t)blk * 256 + 32 * sl);
+                    for (int mi = 0; mi < MROWS; mi++) tie(xr[bb][mi]);
+                x_after = -2;  // none outstanding
+#pragma unroll
+                for (int ps = 0; ps < MROWS / RP; ps++) {
+                    uint32_t hp[kRunBlk][RP][2], lp[kRunBlk][RP][2], sp[kRunBlk][RP];
+                    float isc[kRunBlk][RP];
+#pragma unroll
+                    for (int bb = 0; bb < kRunBlk; bb++) {
+#pragma unroll
+                        for (int j = 0; j < RP; j++) {
+                            const xraw_t raw = xr[bb][ps * RP + j];
+                            float x0, x1, x2, x3;
+                            if constexpr (sizeof(AT) == 4) {
+                                x0 = __uint_as_float(raw.x); x1 = __uint_as_float(raw.y);
+                                x2 = __uint_as_float(raw.z); x3 = __uint_as_float(raw.w);
+                            } else {
+                                x0 = __uint_as_float(raw.x << 16); x1 = __uint_as_float(raw.x & 0xffff0000u);
+                                x2 = __uint_as_float(raw.y << 16); x3 = __uint_as_float(raw.y & 0xffff0000u);
+                            }
+                            const uint32_t mxb =
+                                wave_max_nonneg_bits(fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3))));
+                            int e = (int)((mxb >> 23) & 0xffu) - 127;
+                            if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite: leave unscaled
+                            const float sc = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
+                            isc[bb][j] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+                            x0 *= sc; x1 *= sc; x2 *= sc; x3 *= sc;
+                            // hi part: the value cut to fp16 (toward zero: one instruction converts and packs two);
+                            // the residual x - hi is exact in fp32 and is cut to fp16 the same way
+                            const fp16x2 c02 = __builtin_amdgcn_cvt_pkrtz(x0, x2), c13 = __builtin_amdgcn_cvt_pkrtz(x1, x3);
+                            const fp16x2 r02 = __builtin_amdgcn_cvt_pkrtz(x0 - (float)c02.x, x2 - (float)c02.y);
+                            const fp16x2 r13 = __builtin_amdgcn_cvt_pkrtz(x1 - (float)c13.x, x3 - (float)c13.y);
+                            const float sum = sum8((x0 + x1) + (x2 + x3));  // 8 consecutive lanes = one 32-wide sub-block
+                            const fp16x2 sm = __builtin_amdgcn_cvt_pkrtz(sum, 0.0f);
+                            hp[bb][j][0] = __builtin_bit_cast(uint32_t, c02); hp[bb][j][1] = __builtin_bit_cast(uint32_t, c13);
+                            lp[bb][j][0] = __builtin_bit_cast(uint32_t, r02); lp[bb][j][1] = __builtin_bit_cast(uint32_t, r13);
+                            sp[bb][j] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sum, sum - (float)sm.x));
+                        }
+                    }
+#pragma unroll
+                    for (int bb = 0; bb < kRunBlk; bb++) {
+                        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                        for (int j = 0; j < RP; j++) {
+                            uint8_t* st = stg + j * kStageBytes;
+                            *(uint2*)(st + 8 * lane) = make_uint2(hp[bb][j][0], hp[bb][j][1]);
+                            *(uint2*)(st + kPlaneStride + 8 * lane) = make_uint2(lp[bb][j][0], lp[bb][j][1]);
+                            if ((lane & 7) == 0) *(uint32_t*)(st + 2 * kPlaneStride + 4 * (lane >> 3)) = sp[bb][j];
+                            if (lane == 0) *(float*)(stg + RP * kStageBytes + 4 * j) = isc[bb][j];
+                        }
+                        __builtin_amdgcn_wave_barrier();
+                        if (rr >= ps * RP && rr < ps * RP + RP) {
+                            const uint8_t* st = stg + (rr - ps * RP) * kStageBytes;
+                            const uint8_t* pl = st + (nn >= 8 ? kPlaneStride : 0) + 128 * kg;
+#pragma unroll
+                            for (int p = 0; p < 4; p++) {
+                                fa[bb][p][0][0] = *(const half8*)(pl + 16 * p);
+                                fa[bb][p][1][0] = *(const half8*)(pl + 64 + 16 * p);
+                            }
+                            if (nn < 8) {
+                                // min-term operand: (ah0, al0, ah0, ah1, al1, ah1, 0, 0) for sub-blocks 2 kg, 2 kg + 1
+                                const uint2 s2 = *(const uint2*)(st + 2 * kPlaneStride + 8 * kg);
+                                fs[bb] = pack4(s2.x, (s2.x & 0xffffu) | (s2.y << 16), (s2.y >> 16) | (s2.y << 16), 0u);
+                            }
+                        }
+                        // inverse scales of the lhs rows of this lane's accumulator registers: rows (4 kg + r) % 8
+                        // (with fewer than 4 staged rows every lane takes them: rows past m are dropped at the end)
+                        if (RP < 4 || (kg & 1) == ps) {
+#pragma unroll
+                            for (int r = 0; r < RP; r++) bs[bb][r] = *(const float*)(stg + RP * kStageBytes + 4 * r);
+                        }
+                    }
+                }
+                // the staged rows are in registers before the next item's load may overwrite the slot
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (grp + 1 < ngrp) load_x(grp + 1);
+            } else {
+#pragma unroll
+                for (int bb = 0; bb < kRunBlk; bb++) {
+                    const int blk = min(gb0 + bb, nblk - 1);
+                    const _Float16* ah = a16 + (int64_t)mrow * k + (int64_t)blk * 256 + 64 * kg;
+#pragma unroll
+                    for (int p = 0; p < 4; p++) {
+                        fa[bb][p][0][0] = *(const half8*)(ah + 8 * p);
+                        fa[bb][p][1][0] = *(const half8*)(ah + 32 + 8 * p);
+                    }
+                    if constexpr (NPART == 2) {
+                        const _Float16* al = a16_lo + (int64_t)mrow * k + (int64_t)blk * 256 + 64 * kg;
+#pragma unroll
+                        for (int p = 0; p < 4; p++) {
+                            fa[bb][p][0][1] = *(const half8*)(al + 8 * p);
+                            fa[bb][p][1][1] = *(const half8*)(al + 32 + 8 * p);
+                        }
+                    }
+                    // asum: 8 hi parts then 8 lo parts per super-block
+                    const uint16_t* as = (const uint16_t*)asum + ((int64_t)mrow * nblk + blk) * 16 + 2 * kg;
+                    const uint32_t hi = *(const uint32_t*)as, lo = *(const uint32_t*)(as + 8);  // (ah0, ah1), (al0, al1)
+                    fs[bb] = pack4((hi & 0xffffu) | (lo << 16), hi, (lo >> 16) | (hi & 0xffff0000u), 0u);
                 }
             }
         }
         // the slot of item it - 1 is free: its reads fed matrix products whose results are already stored
-        if (it + 2 < total) {
-            issue_next();
-            wait_vmcnt<2 * kLoads>();
-        } else if (it + 1 < total) {
-            wait_vmcnt<kLoads>();
-        } else {
-            wait_vmcnt<0>();
-        }
+        while (last_issued < min(it + 2, total - 1)) issue_next();
+        // item `it` has landed when only the younger loads are outstanding: later items and, if it was
+        // issued after this item, the next group's raw lhs
+        wait_items<NX>(last_issued - it, INLINE && x_after >= it);
         const uint8_t* wbuf = ring + slot * kSlotBytes;
 
         float4v acc = {0.f, 0.f, 0.f, 0.f};
@@ -171,56 +352,46 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
             if (bb >= nb) break;
             const uint8_t* lb = wbuf + nn * kRowBytes + bb * Q4_K_BPB;
             const uint4 hdr = *(const uint4*)lb;
-            // 6-bit scales and mins of the 8 sub-blocks
-            const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
-            const uint32_t sc_lo = s0 & 0x3F3F3F3Fu, sc_hi = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
-            const uint32_t mn_lo = s1 & 0x3F3F3F3Fu, mn_hi = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
-            uint32_t sp[8];
-            {
-                const float e0 = (float)(sc_lo & 0xffu), e1 = 0.0625f * (float)((sc_lo >> 8) & 0xffu);
-                const float e2 = (float)((sc_lo >> 16) & 0xffu), e3 = 0.0625f * (float)(sc_lo >> 24);
-                const float e4 = (float)(sc_hi & 0xffu), e5 = 0.0625f * (float)((sc_hi >> 8) & 0xffu);
-                const float e6 = (float)((sc_hi >> 16) & 0xffu), e7 = 0.0625f * (float)(sc_hi >> 24);
-                sp[0] = pack_half2(e0, e0); sp[1] = pack_half2(e1, e1);
-                sp[2] = pack_half2(e2, e2); sp[3] = pack_half2(e3, e3);
-                sp[4] = pack_half2(e4, e4); sp[5] = pack_half2(e5, e5);
-                sp[6] = pack_half2(e6, e6); sp[7] = pack_half2(e7, e7);
-            }
-            // min term: B slots (k-group 0,1: hi parts, 2: lo parts) of -(dmin*mn_j), A slots asum hi / lo
+            const uint4 q0 = *(const uint4*)(lb + 16 + 32 * kg), q1 = *(const uint4*)(lb + 32 + 32 * kg);
+            // 6-bit scales and mins of sub-blocks 2 kg, 2 kg + 1
+            const uint32_t p0 = (hdr.y >> sh) & 0xffffu, p1 = (hdr.z >> sh) & 0xffffu, p2 = (hdr.w >> sh) & 0xffffu;
+            const uint32_t sc_pair = upper ? ((p2 & 0x0F0Fu) | ((p0 >> 2) & 0x3030u)) : (p0 & 0x3F3Fu);
+            const uint32_t mn_pair = upper ? (((p2 >> 4) & 0x0F0Fu) | ((p1 >> 2) & 0x3030u)) : (p1 & 0x3F3Fu);
+            const float e0 = (float)(sc_pair & 0xffu), e1 = 0.0625f * (float)(sc_pair >> 8);
+            const uint32_t sp_lo = pack_half2(e0, e0), sp_hi = pack_half2(e1, e1);
+            // min term: weight slots (bh0, bh0, bl0, bh1, bh1, bl1, 0, 0) of -(dmin * mn_j), hi and residual parts
+            float4v Bk = {0.f, 0.f, 0.f, 0.f};
             {
                 const uint32_t ndm = ((hdr.x >> 16) ^ 0x8000u) * 0x00010001u;  // (-dmin, -dmin)
-                const uint32_t mp[4] = {pack_half2((float)(mn_lo & 0xffu), (float)((mn_lo >> 8) & 0xffu)),
-                                        pack_half2((float)((mn_lo >> 16) & 0xffu), (float)(mn_lo >> 24)),
-                                        pack_half2((float)(mn_hi & 0xffu), (float)((mn_hi >> 8) & 0xffu)),
-                                        pack_half2((float)((mn_hi >> 16) & 0xffu), (float)(mn_hi >> 24))};
-                uint32_t v[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint32_t hi = pk_mul(ndm, mp[i]);
-                    const uint32_t lo = pk_fma(ndm, mp[i], hi ^ 0x80008000u);
-                    v[i] = kg < 2 ? hi : (kg == 2 ? lo : 0u);  // slots 24..31 (asum_lo x dmn_lo) are dropped
-                }
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(fs[bb], pack4(v[0], v[1], v[2], v[3]), acc, 0, 0, 0);
+                const uint32_t mp = pack_half2((float)(mn_pair & 0xffu), (float)(mn_pair >> 8));
+                const uint32_t hi = pk_mul(ndm, mp);
+                const uint32_t lo = pk_fma(ndm, mp, hi ^ 0x80008000u);
+                const half8 bmin = pack4((hi & 0xffffu) * 0x00010001u, (lo & 0xffffu) | (hi & 0xffff0000u),
+                                         (hi >> 16) | (lo & 0xffff0000u), 0u);
+                Bk = __builtin_amdgcn_mfma_f32_16x16x32_f16(fs[bb], bmin, Bk, 0, 0, 0);
             }
-            float4v P = {0.f, 0.f, 0.f, 0.f};
+            float4v P = {0.f, 0.f, 0.f, 0.f}, Q = {0.f, 0.f, 0.f, 0.f};  // two chains: low and high nibbles
+            const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const uint2 q = *(const uint2*)(lb + 16 + 32 * c + 8 * kg);
-                const uint32_t x0 = q.x, x1 = q.y, y0 = q.x >> 8, y1 = q.y >> 8;
-                const half8 blo = pack4(pk_mul(x0 & M1, sp[2 * c]), pk_mul(y0 & M1, sp[2 * c]),
-                                        pk_mul(x1 & M1, sp[2 * c]), pk_mul(y1 & M1, sp[2 * c]));
-                const half8 bhi = pack4(pk_mul(x0 & M2, sp[2 * c + 1]), pk_mul(y0 & M2, sp[2 * c + 1]),
-                                        pk_mul(x1 & M2, sp[2 * c + 1]), pk_mul(y1 & M2, sp[2 * c + 1]));
-                P = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][2 * c][0], blo, P, 0, 0, 0);
-                P = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][2 * c + 1][0], bhi, P, 0, 0, 0);
+            for (int p = 0; p < 4; p++) {
+                const uint32_t x0 = qd[2 * p], x1 = qd[2 * p + 1], y0 = x0 >> 8, y1 = x1 >> 8;
+                const half8 blo = pack4(pk_mul(x0 & M1, sp_lo), pk_mul(y0 & M1, sp_lo), pk_mul(x1 & M1, sp_lo),
+                                        pk_mul(y1 & M1, sp_lo));
+                const half8 bhi = pack4(pk_mul(x0 & M2, sp_hi), pk_mul(y0 & M2, sp_hi), pk_mul(x1 & M2, sp_hi),
+                                        pk_mul(y1 & M2, sp_hi));
+                P = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][p][0][0], blo, P, 0, 0, 0);
+                Q = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][p][1][0], bhi, Q, 0, 0, 0);
                 if constexpr (NPART == 2) {
-                    P = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][2 * c][1], blo, P, 0, 0, 0);
-                    P = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][2 * c + 1][1], bhi, P, 0, 0, 0);
+                    P = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][p][0][1], blo, P, 0, 0, 0);
+                    Q = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][p][1][1], bhi, Q, 0, 0, 0);
                 }
             }
             const float dsc = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo24f;
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[r] = fmaf(dsc, P[r], acc[r]);
+            for (int r = 0; r < 4; r++) {
+                const float v = fmaf(dsc, P[r] + Q[r], Bk[r]);
+                acc[r] = INLINE ? fmaf(bs[bb][r], v, acc[r]) : acc[r] + v;  // INLINE: undo the lhs scale of this super-block
+            }
         }
         // this wavefront's running sum of the tile over its groups
         float* mine = accs + ((wave * kMaxTiles + ti) * 4) * 64 + lane;
@@ -239,19 +410,18 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) {
             const float* slot_r = accs + ((ww * kMaxTiles + t) * 4 + r) * 64;
-            v += STACK ? slot_r[lane & 31] + slot_r[(lane & 31) + 32] : slot_r[lane];
+            v += INLINE ? slot_r[lane & 31] + slot_r[(lane & 31) + 32] : slot_r[lane];
         }
-        if (row < m && col < n) out[(int64_t)row * n + col] = v * inv[row];
+        if (row < m && col < n) out[(int64_t)row * n + col] = INLINE ? v : v * inv[row];
     }
 }
 
-int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return lhs_planes(nullptr, lhs_dtype, m, k).bytes; }
+int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) {
+    return m <= 8 ? 0 : lhs_planes(nullptr, lhs_dtype, m, k).bytes;
+}
 
 hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                float* out, void* workspace, hipStream_t s) {
-    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
-    hipError_t e = launch_prep_lhs<kLhsOrderQ4K16>(lhs, lhs_dtype, m, k, p, s);
-    if (e != hipSuccess) return e;
     static int cus = 0;
     if (!cus) {
         int dev = 0;
@@ -259,27 +429,51 @@ hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w,
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipGetLastError();
         cus = prop.multiProcessorCount;
     }
-    const int64_t ntiles = (n + 15) / 16;
-    // every workgroup gets the same number of tiles (at most kMaxTiles), one workgroup per compute unit when that fits
-    const int64_t per_wg = std::min<int64_t>(kMaxTiles, (ntiles + cus - 1) / cus);
-    const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
+    hipError_t e = hipSuccess;
     static bool lds_set = false;
     if (!lds_set) {
-        const void* fns[3] = {(const void*)gemv_q4_k_mm_kernel<1, false>, (const void*)gemv_q4_k_mm_kernel<1, true>,
-                              (const void*)gemv_q4_k_mm_kernel<2, false>};
+        const void* fns[10] = {(const void*)gemv_q4_k_mm_kernel<1, true, 1, float>, (const void*)gemv_q4_k_mm_kernel<1, true, 2, float>,
+                               (const void*)gemv_q4_k_mm_kernel<1, true, 4, float>, (const void*)gemv_q4_k_mm_kernel<1, true, 8, float>,
+                               (const void*)gemv_q4_k_mm_kernel<1, true, 1, uint16_t>, (const void*)gemv_q4_k_mm_kernel<1, true, 2, uint16_t>,
+                               (const void*)gemv_q4_k_mm_kernel<1, true, 4, uint16_t>, (const void*)gemv_q4_k_mm_kernel<1, true, 8, uint16_t>,
+                               (const void*)gemv_q4_k_mm_kernel<1, false, 1, float>, (const void*)gemv_q4_k_mm_kernel<2, false, 1, float>};
         for (const void* fn : fns) {
             e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
             if (e != hipSuccess) return e;
         }
         lds_set = true;
     }
+    const int64_t ntiles = (n + 15) / 16;
+    // every workgroup gets the same number of tiles (at most kMaxTiles), one workgroup per compute unit when that fits
+    const int64_t per_wg = std::min<int64_t>(kMaxTiles, (ntiles + cus - 1) / cus);
+    const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
     dim3 grid((unsigned)wgs), block(64 * kWaves);
+    if (m <= 8) {
+#define QMM_MM_INLINE(MR_)                                                                                            \
+    do {                                                                                                              \
+        if (lhs_dtype == QMM_F32)                                                                                     \
+            gemv_q4_k_mm_kernel<1, true, MR_, float><<<grid, block, kLdsBytes, s>>>(                                  \
+                w, (const float*)lhs, nullptr, nullptr, nullptr, nullptr, out, (int)m, (int)n, (int)k);               \
+        else                                                                                                          \
+            gemv_q4_k_mm_kernel<1, true, MR_, uint16_t><<<grid, block, kLdsBytes, s>>>(                               \
+                w, (const uint16_t*)lhs, nullptr, nullptr, nullptr, nullptr, out, (int)m, (int)n, (int)k);            \
+    } while (0)
+        if (m == 1) QMM_MM_INLINE(1);
+        else if (m == 2) QMM_MM_INLINE(2);
+        else if (m <= 4) QMM_MM_INLINE(4);
+        else QMM_MM_INLINE(8);
+#undef QMM_MM_INLINE
+        return hipGetLastError();
+    }
+    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
+    e = launch_prep_lhs<kLhsOrderQ4K16>(lhs, lhs_dtype, m, k, p, s);
+    if (e != hipSuccess) return e;
     if (!p.a16_lo)
-        gemv_q4_k_mm_kernel<1, false><<<grid, block, kLdsBytes, s>>>(w, p.a16, nullptr, p.asum, p.inv, out, (int)m, (int)n, (int)k);
-    else if (m <= 8)
-        gemv_q4_k_mm_kernel<1, true><<<grid, block, kLdsBytes, s>>>(w, p.a16, p.a16_lo, p.asum, p.inv, out, (int)m, (int)n, (int)k);
+        gemv_q4_k_mm_kernel<1, false, 1, float><<<grid, block, kLdsBytes, s>>>(w, nullptr, p.a16, nullptr, p.asum, p.inv, out, (int)m,
+                                                                           (int)n, (int)k);
     else
-        gemv_q4_k_mm_kernel<2, false><<<grid, block, kLdsBytes, s>>>(w, p.a16, p.a16_lo, p.asum, p.inv, out, (int)m, (int)n, (int)k);
+        gemv_q4_k_mm_kernel<2, false, 1, float><<<grid, block, kLdsBytes, s>>>(w, nullptr, p.a16, p.a16_lo, p.asum, p.inv, out, (int)m,
+                                                                           (int)n, (int)k);
     return hipGetLastError();
 }
 

@@ -270,6 +270,9 @@ __global__ __launch_bounds__(512, 4) void gemv_q4_k_rows_kernel(const uint8_t* _
 // walks its (row, 8-super-block step) units with a ring of four units of loads in flight, so the
 // loads of later units overlap the arithmetic of the current one; activations are read from LDS
 // (staged once per workgroup in lane order) one 16-byte piece at a time.
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ half2v as_half2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
+
 constexpr int kStreamMaxRows = 64;  // rows a wavefront may own in the streaming kernel (LDS result slots)
 
 template <int MT, typename AT>
@@ -349,30 +352,33 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void gemv_q4_k_stream_kernel(
         const uint32_t qd[4] = {x.qs.x, x.qs.y, x.qs.z, x.qs.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t lo = qd[i] & 0x0F0F0F0Fu, hi = (qd[i] >> 4) & 0x0F0F0F0Fu;
-            const float l0 = ub0(lo), l1 = ub1(lo), l2 = ub2(lo), l3 = ub3(lo);
-            const float h0 = ub0(hi), h1 = ub1(hi), h2 = ub2(hi), h3 = ub3(hi);
+            // A masked nibble in a 16-bit half is the fp16 subnormal q * 2^-24 (low nibbles) or 16 q * 2^-24
+            // (high nibbles, left in place); the fused multiply-add widens the half itself, so no
+            // conversion instruction is spent per code.  The powers of two go into d1 / d2 below.
+            const uint32_t y = qd[i] >> 8;
+            const half2v l02 = as_half2(qd[i] & 0x000F000Fu), l13 = as_half2(y & 0x000F000Fu);
+            const half2v h02 = as_half2(qd[i] & 0x00F000F0u), h13 = as_half2(y & 0x00F000F0u);
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) {
                 const float4* la = lds_act + (size_t)mi * iters * 512 + it * 512 + lane;
                 const float4 xa = la[i * 64], ya = la[(4 + i) * 64];
                 float t = slo[mi];
-                t = fmaf(xa.x, l0, t);
-                t = fmaf(xa.y, l1, t);
-                t = fmaf(xa.z, l2, t);
-                slo[mi] = fmaf(xa.w, l3, t);
+                t = fmaf(xa.x, (float)l02.x, t);
+                t = fmaf(xa.y, (float)l13.x, t);
+                t = fmaf(xa.z, (float)l02.y, t);
+                slo[mi] = fmaf(xa.w, (float)l13.y, t);
                 t = shi[mi];
-                t = fmaf(ya.x, h0, t);
-                t = fmaf(ya.y, h1, t);
-                t = fmaf(ya.z, h2, t);
-                shi[mi] = fmaf(ya.w, h3, t);
+                t = fmaf(ya.x, (float)h02.x, t);
+                t = fmaf(ya.y, (float)h13.x, t);
+                t = fmaf(ya.z, (float)h02.y, t);
+                shi[mi] = fmaf(ya.w, (float)h13.y, t);
             }
         }
         const float d = h2f((uint16_t)(x.hdr.x & 0xffffu)), dmin = h2f((uint16_t)(x.hdr.x >> 16));
         const uint32_t p0 = (x.hdr.y >> sh) & 0xffffu, p1 = (x.hdr.z >> sh) & 0xffffu, p2 = (x.hdr.w >> sh) & 0xffffu;
         const uint32_t sc_pair = upper ? ((p2 & 0x0F0Fu) | ((p0 >> 2) & 0x3030u)) : (p0 & 0x3F3Fu);
         const uint32_t mn_pair = upper ? (((p2 >> 4) & 0x0F0Fu) | ((p1 >> 2) & 0x3030u)) : (p1 & 0x3F3Fu);
-        const float d1 = d * ub0(sc_pair), d2 = d * ub1(sc_pair);
+        const float d1 = d * ub0(sc_pair) * 16777216.0f, d2 = d * ub1(sc_pair) * 1048576.0f;  // 2^24, 2^24 / 16
         const float m1 = dmin * ub0(mn_pair), m2 = dmin * ub1(mn_pair);
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {

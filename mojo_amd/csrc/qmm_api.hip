@@ -11,6 +11,10 @@ static bool env_flag_qmm_q4k_small_gemv() {
     static const bool v = getenv("QMM_Q4K_SMALL_GEMV") != nullptr;  // read once: 5..16 lhs rows through the decode kernels
     return v;
 }
+static int env_q4k_mm_min_m() {
+    static const int v = [] { const char* e = getenv("QMM_Q4K_MM_MIN_M"); return e ? atoi(e) : 2; }();  // read once: tuning switch
+    return v;
+}
 static bool env_flag_qmm_q4_0_gemv() {
     static const bool v = getenv("QMM_Q4_0_GEMV") != nullptr;  // read once: tuning and fallback switch
     return v;
@@ -165,7 +169,7 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         return a > b ? a : b;
     }
-    if (encoding == QMM_Q4_K && m >= 3 && m <= 16 && k % 256 == 0) return qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);
+    if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) return qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);  // 0 up to 8 rows
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     if (encoding == QMM_GPTQ && m > 16 && k % 256 == 0) return qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k);
     return 0;
@@ -238,7 +242,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     }
 
     // 3..16 lhs rows: the small-batch matrix-core kernel; more: the prefill kernel
-    if (encoding == QMM_Q4_K && m >= 3 && m <= 16 && !env_flag_qmm_q4k_small_gemv())
+    if (encoding == QMM_Q4_K && m >= env_q4k_mm_min_m() && m <= 16 && !env_flag_qmm_q4k_small_gemv())
         return hip_status(qmm::launch_gemv_q4_k_mm(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K small batch)");
     if (encoding == QMM_Q4_K && m > 16)
         return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");

@@ -70,7 +70,8 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.qmm_quantize(1, fake, 0, 256, fake, None) == -1
     assert lib.qmm_matmul_workspace_bytes(0, 0, 16, 4096, 4096) == 16 * 4096 + 2 * 16 * 128 * 4
     assert lib.qmm_matmul_workspace_bytes(1, 0, 2, 4096, 4096) == 0  # Q4_K decode reads the lhs as it is
-    assert lib.qmm_matmul_workspace_bytes(1, 0, 4, 4096, 4096) >= 2 * 4 * 4096 * 2  # fp16 hi and residual planes of the 4 rows
+    assert lib.qmm_matmul_workspace_bytes(1, 0, 8, 4096, 4096) == 0  # up to 8 rows the kernel narrows the lhs itself
+    assert lib.qmm_matmul_workspace_bytes(1, 0, 12, 4096, 4096) >= 2 * 12 * 4096 * 2  # fp16 hi and residual planes
     assert lib.qmm_matmul_workspace_bytes(1, 1, 2048, 14336, 4096) >= 2048 * 4096 * 2
 
 
