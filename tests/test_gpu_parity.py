@@ -172,6 +172,39 @@ def test_leading_dims_broadcast():
     assert_close(got, want, "leading dims")
 
 
+# ------------------------------------------------------------------ Q4_K small batch (2..16 lhs rows)
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(2, 9000, 1024, False), (4, 8200, 4608, False), (7, 4100, 2048, True),
+                                            (8, 6000, 4608, False), (5, 300, 256, False), (12, 5000, 1280, True),
+                                            (12, 5000, 1280, False), (16, 4500, 4608, False)])
+def test_q4_k_small_batch_many_tiles(m, n, k, lhs_bf16):
+    """Several 16-row tiles per workgroup, ragged last tile, groups of K with one or two super-blocks per wavefront."""
+    w, a = synth(21, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq)
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a)
+    got = qmatmul(QE.Q4_K, None, lhs, gpu(wq))
+    assert_close(got, want, f"Q4_K small batch {m}x{n}x{k} vs fp32 oracle")
+    assert_close(got, truth, f"Q4_K small batch {m}x{n}x{k} vs fp64 truth")
+
+
+@pytest.mark.parametrize("m", [3, 8])
+def test_q4_k_small_batch_wide_range_lhs(m):
+    """Rows and 256-column blocks of very different magnitude: the power-of-two scaling per row and block keeps the
+    fp16 operands in range, and what each block contributes keeps its relative precision."""
+    n, k = 200, 2048
+    w, a = synth(22, n, k, m)
+    a *= np.logspace(-5, 4, m, dtype=np.float32)[:, None]
+    a *= np.repeat(np.logspace(-3, 3, k // 256, dtype=np.float32), 256)[None, :]
+    wq = O.quantize(O.Q4_K, w)
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a), gpu(wq)).cpu().numpy()
+    scale = np.abs(truth).max(axis=1, keepdims=True)
+    assert np.all(np.abs(got - truth) <= 1e-4 * scale + 1e-3 * np.abs(truth))
+
+
 # ------------------------------------------------------------------ prefill shapes (m > 16)
 @pytest.mark.parametrize("m,n,k", [(128, 256, 256), (17, 40, 512), (200, 300, 1024), (256, 512, 4096), (130, 64, 2048)])
 def test_q4_k_gemm_bf16_lhs(m, n, k):
