@@ -315,22 +315,11 @@ __global__ __launch_bounds__(256) void gemv_gptq_kernel(const uint32_t* __restri
     else if (m <= 8) { CALL(8); } \
     else { CALL(16); }
 
-// Kernel choice for Q4_K decode shapes.  Measured on MI355X: the vector-ALU streaming kernel (one or
-// two lhs rows per pass) is the fastest up to four lhs rows, with three and four rows done as two
-// passes over the weights; from five rows on the matrix-core kernel, whose cost does not grow with m,
-// wins.  QMM_Q4K_GEMV=valu|mfma overrides.
-static bool q4k_use_valu(int m) {
-    static const int forced = [] {
-        const char* e = getenv("QMM_Q4K_GEMV");
-        return !e ? 0 : (e[0] == 'v' ? 1 : (e[0] == 'm' ? 2 : 0));
-    }();
-    if (forced) return forced == 1;
-    return m <= 4;
-}
-
+// Q4_K through the decode kernels: the streaming kernel for one or two lhs rows, three and four rows as two
+// passes over the weights, more rows through the generic kernel.  (qmm_matmul sends 2..16 rows to the
+// small-batch matrix-core kernel instead; this is what is left when that is switched off.)
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
-    if (!q4k_use_valu(m)) return launch_gemv_q4_k_mfma(a, a_dtype, w, m, n, k, out, ldo, s);
     if (m <= 2 && !env_flag_qmm_q4k_v1()) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
     if (m <= 4 && !env_flag_qmm_q4k_v1()) {
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;

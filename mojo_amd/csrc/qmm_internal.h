@@ -29,8 +29,6 @@ hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m,
                             float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s);
-hipError_t launch_gemv_q4_k_mfma(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
-                                 float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
