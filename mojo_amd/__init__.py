@@ -14,6 +14,7 @@ from .ops import (
     quantize,
     quantize_gptq,
 )
+from .weights import GGUFWeights, load_gptq_config, load_gptq_linear
 
 __all__ = [
     "BlockParameters",
@@ -24,4 +25,7 @@ __all__ = [
     "quantize",
     "quantize_gptq",
     "block_dots_q4_0",
+    "GGUFWeights",
+    "load_gptq_config",
+    "load_gptq_linear",
 ]
