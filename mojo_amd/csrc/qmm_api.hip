@@ -5,6 +5,8 @@
 
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include "qmm_internal.h"
 
 static bool env_flag_qmm_q4k_small_gemv() {
@@ -228,6 +230,13 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
 
     if (encoding == QMM_Q4_0 && m >= 5 && !env_flag_qmm_q4_0_gemv())
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
+    if (encoding == QMM_Q4_0 && m <= 4) {
+        // decode: the kernel that quantises the lhs itself (takes K <= 8192)
+        bool handled = false;
+        hipError_t e = qmm::launch_gemv_q4_0_stream(lhs, lhs_dtype, w, (int)m, n, k, out, n, s, &handled);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_0 decode)");
+        if (handled) return QMM_OK;
+    }
     if (encoding == QMM_Q4_0) {
         Q8Planes p = q8_planes(workspace, m, k);
         hipError_t e = qmm::launch_quantize_q8_0(lhs, lhs_dtype, m, k, nullptr, p.codes, p.scale, p.sum, s);

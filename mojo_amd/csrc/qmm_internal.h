@@ -22,6 +22,8 @@ hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group,
                                 void* scales, void* qzeros, void* g_idx, hipStream_t s);
 
 // Decode-shape kernels (m <= 16 rows of lhs per launch).
+hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                   int64_t ldo, hipStream_t s, bool* handled);
 hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const int32_t* a_sum,
                             const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
                             hipStream_t s);

@@ -130,6 +130,21 @@ def test_q4_0_matmul(m, n, k):
     assert_close(got, want, f"Q4_0 {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(2, 1000, 8192, False), (4, 300, 4096, True), (1, 5001, 2048, False),
+                                            (1, 70000, 256, False), (3, 9, 4128, False), (2, 64, 8224, True),
+                                            (4, 33, 8192, False)])
+def test_q4_0_decode_shapes(m, n, k, lhs_bf16):
+    """Q4_0 decode: rows at every 2-byte alignment, K up to 8192 in the kernel that quantises the lhs itself
+    (K past that and 4 rows at K = 8192 through the Q8_0 planes), many rows per wavefront, bf16 lhs."""
+    w, a = synth(52, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_0, w)
+    want = O.matmul_q4_0(a, wq)
+    got = qmatmul(QE.Q4_0, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_0 decode {m}x{n}x{k} bf16={lhs_bf16}")
+
+
 # ------------------------------------------------------------------ Q4_K / Q6_K with fp32 activations
 @pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K])
 @pytest.mark.parametrize("m,n,k", [(1, 1024, 4096), (4, 512, 4096), (16, 256, 2048), (3, 5, 256), (2, 66, 14336),
