@@ -20,8 +20,19 @@
 // For m > 16 the grid's second dimension walks groups of four 16-row tiles, each group streaming the
 // weights again (this path is bound by the per-block fp32 scaling in the vector ALUs, not by the
 // matrix cores: 4 instructions per (lhs row, weight row, block)).
+//
+// Up to 16 lhs rows with K a multiple of 256 take gemm_q4_0_small_kernel instead: the schedule of the
+// Q4_K small-batch kernel (gemv_q4k_mm.hip).  A workgroup of 8 wavefronts walks up to 4 tiles of 16
+// weight rows; wavefront w owns 8 blocks (144 bytes of every row, 16-byte aligned) of each group of 64
+// blocks and keeps the lhs operands of those 8 blocks in registers for all the tiles; the 16 x 144
+// bytes of a (group, tile) item go global -> LDS directly into a private 3-slot ring, two items
+// ahead.  Inside the 144 bytes the block offsets 18 j are compile-time, so the byte alignment of
+// every field is too.
 #include <stdlib.h>
 
+#include <algorithm>
+
+#include "lds_stream.h"
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -213,6 +224,151 @@ __global__ __launch_bounds__(512) void gemm_q4_0_kernel(const uint8_t* __restric
     }
 }
 
+namespace {
+constexpr int kSWaves = 8;                          // wavefronts per workgroup
+constexpr int kSBlk = 8;                            // blocks per wavefront and group: 144 bytes of a row
+constexpr int kSRow = kSBlk * Q4_0_BPB;             // 144
+constexpr int kSPieces = 16 * kSRow / 16;           // 144 pieces of 16 bytes per item
+constexpr int kSLoads = (kSPieces + 63) / 64;       // 3 load instructions per item, the last one by 16 lanes
+constexpr int kSSlot = kSPieces * 16 + 16;          // 2320: one dword of read-ahead past the last row
+constexpr int kSSlots = 3;
+constexpr int kSMaxTiles = 4;
+constexpr int kSRing = kSWaves * kSSlots * kSSlot;
+constexpr int kSLds = kSRing + kSWaves * kSMaxTiles * 4 * 64 * 4;
+}  // namespace
+
+__global__ __launch_bounds__(64 * kSWaves) void gemm_q4_0_small_kernel(const uint8_t* __restrict__ w,
+                                                                      const int8_t* __restrict__ codes,
+                                                                      const float* __restrict__ dscale,
+                                                                      const int32_t* __restrict__ csum,
+                                                                      float* __restrict__ out, int m, int n, int k) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nkb = k >> 5;                       // a multiple of 8
+    const int64_t row_bytes = (int64_t)nkb * Q4_0_BPB;
+    const int nn = lane & 15, g = lane >> 4;
+    uint8_t* ring = smem + wave * (kSSlots * kSSlot);
+    const uint32_t ring_lds = lds_address(ring);
+    float* accs = (float*)(smem + kSRing);        // [kSWaves][kSMaxTiles][4][64]
+    const int ntiles = (n + 15) >> 4;
+    const int my_tiles = min(kSMaxTiles, (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
+    const int ngrp = (nkb + kSWaves * kSBlk - 1) / (kSWaves * kSBlk);
+    const int total = ngrp * my_tiles;
+    // group gi: blocks [64 gi + 8 wave, + 8) when they exist (K is a multiple of 256, so a share is whole or absent)
+    auto share = [&](int gi, int& first, bool& have) {
+        first = kSWaves * kSBlk * gi + kSBlk * wave;
+        have = first < nkb;
+        first = min(first, nkb - kSBlk);  // (absent: a valid address, the data is not used)
+    };
+    int prow[kSLoads], pidx[kSLoads];
+#pragma unroll
+    for (int i = 0; i < kSLoads; i++) {
+        const int p = min(lane + 64 * i, kSPieces - 1);
+        prow[i] = p / 9;
+        pidx[i] = p - prow[i] * 9;
+    }
+    auto issue = [&](int gi, int t, int slot) {
+        const int n0 = ((int)blockIdx.x + t * (int)gridDim.x) * 16;
+        int kb;
+        bool have;
+        share(gi, kb, have);
+        const uint8_t* base = w + (int64_t)kb * Q4_0_BPB;
+#pragma unroll
+        for (int i = 0; i < kSLoads; i++) {
+            const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * pidx[i];
+            if (i < kSLoads - 1 || lane < kSPieces - 64 * (kSLoads - 1))
+                load16_to_lds(src, ring_lds + slot * kSSlot + i * 1024);
+        }
+    };
+    int last_issued = -1, ig = 0, it_t = 0, islot = 0;
+    auto issue_next = [&]() {
+        issue(ig, it_t, islot);
+        last_issued++;
+        islot = islot == kSSlots - 1 ? 0 : islot + 1;
+        if (++it_t == my_tiles) { it_t = 0; ig++; }
+    };
+
+    // lhs operands of the wavefront's 8 blocks of the current group
+    long aop[kSBlk];
+    float4 da[kSBlk], da8[kSBlk];  // block scales of lhs rows 4 g .. 4 g + 3, and -8 * code sum * scale
+
+    int grp = 0, ti = 0, slot = 0;
+    for (int it = 0; it < total; it++) {
+        int kb0;
+        bool have;
+        share(grp, kb0, have);
+        if (ti == 0) {
+            // (ordinary loads: the compiler's waits for them also wait for the items in flight, once per group)
+#pragma unroll
+            for (int j = 0; j < kSBlk; j++) {
+                const int64_t tb = kb0 + j;  // one 16-row lhs tile
+                aop[j] = *(const long*)(codes + (tb * 64 + lane) * 8);
+                da[j] = *(const float4*)(dscale + tb * 16 + 4 * g);
+                const int4v as = *(const int4v*)(csum + tb * 16 + 4 * g);
+                da8[j] = make_float4(-8.0f * (float)as[0] * da[j].x, -8.0f * (float)as[1] * da[j].y,
+                                     -8.0f * (float)as[2] * da[j].z, -8.0f * (float)as[3] * da[j].w);
+            }
+        }
+        while (last_issued < min(it + 2, total - 1)) issue_next();
+        wait_items<kSLoads, 0>(last_issued - it, false);
+        const uint8_t* wrow = ring + slot * kSSlot + nn * kSRow;
+        const uint32_t* l32 = (const uint32_t*)wrow;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        if (have) {
+#pragma unroll
+            for (int j = 0; j < kSBlk; j++) {
+                // block j at byte 18 j of the row's 144: d, then 16 nibble bytes; this lane's 8 code bytes are the low
+                // nibbles of bytes 8 (g & 1) .. + 7 (g < 2) or their high nibbles
+                constexpr int kUnused = 0;
+                (void)kUnused;
+                const int qoff = Q4_0_BPB * j + 2 + 8 * (g & 1);
+                const int wi = qoff >> 2;                                  // (18 j + 2) / 4 + 2 (g & 1)
+                const uint32_t sh = (uint32_t)((Q4_0_BPB * j + 2) & 3);    // compile-time: 2, 0, 2, 0, ...
+                uint32_t lo, hi;
+                if (sh == 0) {
+                    lo = l32[wi];
+                    hi = l32[wi + 1];
+                } else {
+                    const uint32_t w0 = l32[wi], w1 = l32[wi + 1], w2 = l32[wi + 2];
+                    lo = __builtin_amdgcn_alignbyte(w1, w0, sh);
+                    hi = __builtin_amdgcn_alignbyte(w2, w1, sh);
+                }
+                if (g & 2) {
+                    lo >>= 4;
+                    hi >>= 4;
+                }
+                lo &= 0x0F0F0F0Fu;
+                hi &= 0x0F0F0F0Fu;
+                const long bop = (long)(((uint64_t)hi << 32) | lo);
+                const uint32_t dwv = l32[(Q4_0_BPB * j) >> 2] >> (8 * ((Q4_0_BPB * j) & 3));
+                const float dw = h2f((uint16_t)(dwv & 0xffffu));
+                int4v z = {0, 0, 0, 0};
+                const int4v dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[j], bop, z, 0, 0, 0);
+                // float(dot - 8 asum) * (dw * da), with the -8 asum da part formed once per group
+                acc[0] = fmaf(dw, fmaf((float)dot[0], da[j].x, da8[j].x), acc[0]);
+                acc[1] = fmaf(dw, fmaf((float)dot[1], da[j].y, da8[j].y), acc[1]);
+                acc[2] = fmaf(dw, fmaf((float)dot[2], da[j].z, da8[j].z), acc[2]);
+                acc[3] = fmaf(dw, fmaf((float)dot[3], da[j].w, da8[j].w), acc[3]);
+            }
+        }
+        float* mine = accs + ((wave * kSMaxTiles + ti) * 4) * 64 + lane;
+#pragma unroll
+        for (int r = 0; r < 4; r++) mine[r * 64] = grp == 0 ? acc[r] : mine[r * 64] + acc[r];
+        slot = slot == kSSlots - 1 ? 0 : slot + 1;
+        if (++ti == my_tiles) { ti = 0; grp++; }
+    }
+    __syncthreads();
+    for (int pr = wave; pr < my_tiles * 4; pr += kSWaves) {
+        const int t = pr >> 2, r = pr & 3;
+        const int col = ((int)blockIdx.x + t * (int)gridDim.x) * 16 + nn, row = 4 * g + r;
+        float v = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < kSWaves; ww++) v += accs[((ww * kSMaxTiles + t) * 4 + r) * 64 + lane];
+        if (row < m && col < n) out[(int64_t)row * n + col] = v;
+    }
+}
+
 int64_t gemm_q4_0_workspace_bytes(int64_t m, int64_t k) { return lhs_q8t(nullptr, m, k).bytes; }
 
 hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
@@ -230,6 +386,28 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
     if (e != hipSuccess) return e;
     // Few lhs rows: the weights are read once and the kernel lives on HBM latency, so K is cut eight
     // ways for more wavefronts in flight; otherwise four.
+    static const bool small_off = getenv("QMM_Q4_0_SMALL_V1") != nullptr;  // read once: fallback switch
+    if (tiles == 1 && k % 256 == 0 && !small_off) {
+        static int cus = 0;
+        if (!cus) {
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+                cus = 256;
+        }
+        static bool lds_set = false;
+        if (!lds_set) {
+            hipError_t e = hipFuncSetAttribute((const void*)gemm_q4_0_small_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kSLds);
+            if (e != hipSuccess) return e;
+            lds_set = true;
+        }
+        const int64_t ntiles = (n + 15) / 16;
+        const int64_t per_wg = std::min<int64_t>(kSMaxTiles, (ntiles + cus - 1) / cus);
+        const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
+        gemm_q4_0_small_kernel<<<dim3((unsigned)wgs), dim3(64 * kSWaves), kSLds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n,
+                                                                                   (int)k);
+        return hipGetLastError();
+    }
     const int nw = (tiles <= 2 && k >= 2048) ? 8 : 4;
     const size_t lds = (size_t)nw * kWaveLds;  // also holds the nw x MG*4 x 64 floats of the final reduction
     dim3 block(64 * nw);

@@ -19,6 +19,7 @@
 
 #include <algorithm>
 
+#include "lds_stream.h"
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -27,31 +28,6 @@ namespace {
 
 constexpr int kWaves = 8;        // wavefronts per workgroup
 constexpr int kMaxRows = 64;     // rows a wavefront may own (LDS result slots)
-
-typedef __attribute__((address_space(3))) void* lds_space_ptr;
-
-__device__ __forceinline__ void load16_to_lds(const void* g, uint32_t lds_base) {
-    uint32_t keep;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
-                 : "=&s"(keep)
-                 : "v"(g), "s"(lds_base)
-                 : "memory");
-}
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// A plain 16-byte global load the compiler is not told about either (a wait it places itself would count the
-// loads into LDS too and drain them).  The destination may only be used after wait_vmcnt and tie() on it.
-__device__ __forceinline__ void hidden_load(u32x4& d, const void* g) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(g) : "memory");
-}
-__device__ __forceinline__ void tie(u32x4& d) { asm volatile("" : "+v"(d)); }
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt has six bits");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
 
 // wait until at most `rows` rows (L load instructions each) are outstanding
 template <int L>
@@ -90,7 +66,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
     const int nblk = k >> 5;
     const int64_t row_bytes = (int64_t)nblk * Q4_0_BPB;
     uint8_t* ring = smem + wave * (RING * kSlot);
-    const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_space_ptr)ring);
+    const uint32_t ring_lds = lds_address(ring);
     float* res = (float*)(smem + kWaves * RING * kSlot) + wave * kMaxRows * MT;
     const int gw = (int)blockIdx.x * kWaves + wave, GW = (int)gridDim.x * kWaves;
     const int my_rows = gw < n ? (n - gw + GW - 1) / GW : 0;

@@ -31,6 +31,7 @@
 #include <type_traits>
 
 #include "gemm_lhs.h"
+#include "lds_stream.h"
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -55,57 +56,7 @@ constexpr int kAccBytes = kWaves * kMaxTiles * 4 * 64 * 4;
 constexpr int kLdsBytes = kRingBytes + kAccBytes;
 static_assert(4 * kStageBytes + 16 <= kSlotBytes, "four staged lhs rows and their scales fit the free ring slot");
 
-typedef __attribute__((address_space(3))) void* lds_space_ptr;
-
-// 16 bytes per lane from global memory to LDS at lds_base + 16 * lane (lds_base uniform).  The
-// compiler is not told that this is a load: it keeps no count of it, and the caller waits with
-// wait_vmcnt before reading the slot.  (The builtin for this instruction makes the compiler wait
-// for all of them before every LDS read, which would leave nothing in flight.)  m0 is put back; the
-// s_nop is the wait state the hardware wants between a write of m0 and an LDS-direct load.
-__device__ __forceinline__ void load16_to_lds(const void* g, uint32_t lds_base) {
-    uint32_t keep;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
-                 : "=&s"(keep)
-                 : "v"(g), "s"(lds_base)
-                 : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt has six bits");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
 typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));  // what the packed conversion builtin returns
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-// Plain global loads that the compiler is not told about either, for values that must arrive while
-// the loads into LDS above are in flight: a wait the compiler places itself counts those too and
-// would drain them.  The destination may only be used after wait_vmcnt and tie() on it.
-__device__ __forceinline__ void hidden_load(u32x4& d, const void* g) {
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(g) : "memory");
-}
-__device__ __forceinline__ void hidden_load(u32x2& d, const void* g) {
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(d) : "v"(g) : "memory");
-}
-template <typename T>
-__device__ __forceinline__ void tie(T& d) {
-    asm volatile("" : "+v"(d));
-}
-// wait until at most 5 * items + extra loads are outstanding (items 0..2, extra 0 or NX)
-template <int NX>
-__device__ __forceinline__ void wait_items(int items, bool extra) {
-    if (extra) {
-        if (items >= 2) wait_vmcnt<2 * kLoads + NX>();
-        else if (items == 1) wait_vmcnt<kLoads + NX>();
-        else wait_vmcnt<NX>();
-    } else {
-        if (items >= 2) wait_vmcnt<2 * kLoads>();
-        else if (items == 1) wait_vmcnt<kLoads>();
-        else wait_vmcnt<0>();
-    }
-}
 
 __device__ __forceinline__ half8 zero_half8() { return pack4(0u, 0u, 0u, 0u); }
 
@@ -128,7 +79,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
     const int64_t row_bytes = (int64_t)nblk * Q4_K_BPB;
     const int nn = lane & 15, kg = lane >> 4;
     uint8_t* ring = smem + wave * (kSlots * kSlotBytes);
-    const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_space_ptr)ring);
+    const uint32_t ring_lds = lds_address(ring);
     float* accs = (float*)(smem + kRingBytes);  // [kWaves][kMaxTiles][4][64]
     const int ntiles = (n + 15) >> 4;
     const int my_tiles = min(kMaxTiles, (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
@@ -235,7 +186,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
                 uint8_t* stg = ring + islot * kSlotBytes;
                 const int rr = nn & 7;
                 // the raw lhs values: everything issued after them may stay in flight
-                wait_items<0>(last_issued - x_after, false);
+                wait_items<kLoads, 0>(last_issued - x_after, false);
 #pragma unroll
                 for (int bb = 0; bb < kRunBlk; bb++)
 #pragma unroll
@@ -343,7 +294,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
         while (last_issued < min(it + 2, total - 1)) issue_next();
         // item `it` has landed when only the younger loads are outstanding: later items and, if it was
         // issued after this item, the next group's raw lhs
-        wait_items<NX>(last_issued - it, INLINE && x_after >= it);
+        wait_items<kLoads, NX>(last_issued - it, INLINE && x_after >= it);
         const uint8_t* wbuf = ring + slot * kSlotBytes;
 
         float4v acc = {0.f, 0.f, 0.f, 0.f};

@@ -145,6 +145,20 @@ def test_q4_0_decode_shapes(m, n, k, lhs_bf16):
     assert_close(got, want, f"Q4_0 decode {m}x{n}x{k} bf16={lhs_bf16}")
 
 
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(16, 5000, 4096, False), (9, 300, 512, False), (12, 64, 14336, True),
+                                            (5, 4100, 256, False), (16, 16400, 2048, True)])
+def test_q4_0_small_batch(m, n, k, lhs_bf16):
+    """5..16 lhs rows, K a multiple of 256: several 16-row tiles per workgroup, ragged last tile, groups of K in
+    which only some wavefronts have a share."""
+    w, a = synth(53, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_0, w)
+    want = O.matmul_q4_0(a, wq)
+    got = qmatmul(QE.Q4_0, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_0 small batch {m}x{n}x{k} bf16={lhs_bf16}")
+
+
 # ------------------------------------------------------------------ Q4_K / Q6_K with fp32 activations
 @pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K])
 @pytest.mark.parametrize("m,n,k", [(1, 1024, 4096), (4, 512, 4096), (16, 256, 2048), (3, 5, 256), (2, 66, 14336),
