@@ -253,7 +253,7 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": measured_traffic("decode_m1") if m == 1 and args.layers == 8 else None,
-            "kernel": "gemv_q4_k_stream_kernel",
+            "kernel": "gemv_q4_k_lanes_kernel",
             "bytes_per_launch": avg_launch_bytes,
             "launch_us": round(avg_launch_us, 3),
         },

@@ -320,7 +320,12 @@ __global__ __launch_bounds__(256) void gemv_gptq_kernel(const uint32_t* __restri
 // small-batch matrix-core kernel instead; this is what is left when that is switched off.)
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
-    if (m <= 2 && !env_flag_qmm_q4k_v1()) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
+    if (m <= 2 && !env_flag_qmm_q4k_v1()) {
+        bool handled = false;
+        hipError_t e = launch_gemv_q4_k_lanes(a, a_dtype, w, m, n, k, out, ldo, s, &handled);
+        if (e != hipSuccess || handled) return e;
+        return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
+    }
     if (m <= 4 && !env_flag_qmm_q4k_v1()) {
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
         hipError_t e = launch_gemv_q4_k_rows(a, a_dtype, w, 2, n, k, out, ldo, s);

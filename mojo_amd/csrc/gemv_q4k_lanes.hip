@@ -1,0 +1,293 @@
+// Q4_K decode kernel for one or two lhs rows: every lane owns one fixed 64-column chunk of K, so its
+// activations never leave its registers; weight rows travel global -> LDS directly.
+//
+// A wavefront covers up to 16 super-blocks of a row (4096 columns): lane l owns chunk l % 4 of
+// super-block l / 4, i.e. 32 code bytes whose low nibbles are sub-block 2c and whose high nibbles are
+// sub-block 2c + 1, and needs only those two scales and mins.  Longer rows are cut into 2 or 4
+// parts, one wavefront each (K = 14336: 4 parts of 14 super-blocks), and the partial sums of a row
+// are added through LDS at the end.  The 64 activations of the lane's chunk (and their two sums, for
+// the min term) are read once, from a copy of the lhs that the workgroup stages in LDS at the start.
+//
+// A wavefront walks its rows (persistent); a row part goes as 16-byte pieces straight into a
+// private ring of four LDS slots (global_load_lds_dwordx4, up to three rows ahead, hidden from the
+// compiler and waited for with exact vmcnt counts: lds_stream.h).  Per row a lane issues three
+// 16-byte LDS reads (header, 32 code bytes), masks the nibbles in place into fp16 subnormals
+// (q * 2^-24, or 16 q * 2^-24 for the high ones) and multiplies them by its fp32 activations with
+// v_fma_mix_f32; d * sc and dmin * mn are applied once per chunk.  Against the streaming kernel
+// (8 lanes per super-block, activations from LDS) this is about 150 instead of 235 vector
+// instructions per 2304-byte row, which is what bounds both.
+#include <stdlib.h>
+
+#include <algorithm>
+
+#include "lds_stream.h"
+#include "qmm_internal.h"
+
+namespace qmm {
+
+namespace {
+
+constexpr int kWaves = 8;     // wavefronts per workgroup
+constexpr int kMaxRows = 64;  // rows a wavefront may own (LDS result slots)
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ half2v as_half2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
+
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);  // every lane of a 16-lane row holds the row sum
+    const int b = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ float ubyte0(uint32_t v) { float f; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v)); return f; }
+
+}  // namespace
+
+// WPR: wavefronts (parts of K) per row.  L: load instructions per row part (64 pieces of 16 bytes each).
+// ring: LDS slots per wavefront (2..4): one row part being decoded, the others in flight.
+template <int MT, int WPR, int L, typename AT>
+__global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                                        float* __restrict__ out, int m, int n, int k,
+                                                                        int64_t ldo, int ring_slots) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nblk = k >> 8;
+    const int64_t row_bytes = (int64_t)nblk * Q4_K_BPB;
+    const int part = wave % WPR;
+    const int bpw = (nblk + WPR - 1) / WPR;                       // super-blocks per part (<= 16)
+    const int blk0 = min(part * bpw, nblk - 1);
+    const int nb = max(0, min(bpw, nblk - part * bpw));           // super-blocks of this part
+    const int kRing = ring_slots;
+    const int pieces = bpw * 9;       // 16-byte pieces of a full row part
+    const int kSlot = pieces * 16;    // bytes of a slot
+    uint8_t* ring = smem + wave * (kRing * kSlot);
+    const uint32_t ring_lds = lds_address(ring);
+    float* res = (float*)(smem + kWaves * kRing * kSlot) + wave * kMaxRows * MT;
+    const int gs = (int)blockIdx.x * (kWaves / WPR) + wave / WPR, GS = (int)gridDim.x * (kWaves / WPR);
+    const int my_rows = gs < n ? (n - gs + GS - 1) / GS : 0;
+
+    // a row part into a slot.  Every one of the L instructions has a live lane in every wavefront (the mask
+    // follows the full part length, a shorter last part repeats its last piece), so the wait counts stay exact.
+    const int last_piece = max(nb, 1) * 9 - 1;
+    auto issue = [&](int ri, int slot) {
+        const uint8_t* base = w + (int64_t)(gs + (int64_t)ri * GS) * row_bytes + (int64_t)blk0 * Q4_K_BPB;
+#pragma unroll
+        for (int i = 0; i < L; i++)
+            if (lane + 64 * i < pieces)
+                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
+    };
+
+    // --- the lane's chunk: super-block blk0 + lane / 4 (clamped: lanes past the part get zero activations),
+    //     chunk c = lane % 4.  The lhs rows are staged once per workgroup: coalesced 16-byte pieces straight
+    //     into LDS, laid out as one record per 64-column chunk (its pieces plus one piece of padding, so that
+    //     the lanes' 16-byte reads of their own records spread over the banks), issued before the first weight
+    //     rows and waited for together with them.
+    const int lb = min(lane >> 2, max(nb, 1) - 1), c = lane & 3;
+    const bool live = (lane >> 2) < nb;
+    constexpr int kCp = sizeof(AT) == 4 ? 16 : 8;  // 16-byte pieces of a chunk's 64 activations
+    uint8_t* act = smem + kWaves * kRing * kSlot + kWaves * kMaxRows * MT * 4;
+    const int nchunk = k >> 6, npos = nchunk * (kCp + 1);  // records, and their pieces (padding included)
+    const int nposp = (npos + 63) & ~63;                   // per lhs row, rounded up to whole load instructions
+    {
+        const uint32_t act_lds = lds_address(act);
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            const uint8_t* ar = (const uint8_t*)(a + (int64_t)min(mi, m - 1) * k);
+            for (int q0 = wave * 64; q0 < npos; q0 += 64 * kWaves) {
+                const int q = min(q0 + lane, npos - 1);
+                const int owner = q / (kCp + 1), slot = q - owner * (kCp + 1);
+                load16_to_lds(ar + 16 * (owner * kCp + min(slot, kCp - 1)), act_lds + (mi * nposp + q0) * 16);
+            }
+        }
+    }
+    int issued = 0;
+    int islot = 0;  // slot of the next row to issue
+    for (; issued < min(kRing - 1, my_rows); issued++) {
+        issue(issued, islot);
+        islot = islot + 1 == kRing ? 0 : islot + 1;
+    }
+    wait_items<L, 0>(issued, false);  // the activation loads are older than these rows
+    __syncthreads();                  // every wavefront's share of the activations has landed
+    float alo[MT][32], ahi[MT][32], slo_a[MT], shi_a[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) {
+        float v[64];
+        const uint4* rec = (const uint4*)(act + ((size_t)mi * nposp + (size_t)((blk0 + lb) * 4 + c) * (kCp + 1)) * 16);
+#pragma unroll
+        for (int i = 0; i < kCp; i++) {
+            const uint4 r = rec[i];
+            if constexpr (sizeof(AT) == 4) {
+                v[4 * i] = __uint_as_float(r.x); v[4 * i + 1] = __uint_as_float(r.y);
+                v[4 * i + 2] = __uint_as_float(r.z); v[4 * i + 3] = __uint_as_float(r.w);
+            } else {
+                v[8 * i] = __uint_as_float(r.x << 16); v[8 * i + 1] = __uint_as_float(r.x & 0xffff0000u);
+                v[8 * i + 2] = __uint_as_float(r.y << 16); v[8 * i + 3] = __uint_as_float(r.y & 0xffff0000u);
+                v[8 * i + 4] = __uint_as_float(r.z << 16); v[8 * i + 5] = __uint_as_float(r.z & 0xffff0000u);
+                v[8 * i + 6] = __uint_as_float(r.w << 16); v[8 * i + 7] = __uint_as_float(r.w & 0xffff0000u);
+            }
+        }
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            alo[mi][i] = live ? v[i] : 0.0f;
+            ahi[mi][i] = live ? v[32 + i] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < 32; i += 4) {
+            s0 += (alo[mi][i] + alo[mi][i + 1]) + (alo[mi][i + 2] + alo[mi][i + 3]);
+            s1 += (ahi[mi][i] + ahi[mi][i + 1]) + (ahi[mi][i + 2] + ahi[mi][i + 3]);
+        }
+        slo_a[mi] = s0;
+        shi_a[mi] = s1;
+    }
+    const int sh = 16 * (c & 1);  // byte pair (2c, 2c + 1) mod 4 inside a dword of the 6-bit fields
+    const bool upper = c >= 2;    // sub-blocks 4..7 use the split encoding
+
+    int cslot = 0;  // slot of the row being decoded
+    for (int ri = 0; ri < my_rows; ri++) {
+        // the slot of row ri - 1 is free (its reads fed the sum that was parked): refill it
+        if (issued < my_rows) {
+            issue(issued, islot);
+            islot = islot + 1 == kRing ? 0 : islot + 1;
+            issued++;
+        }
+        wait_items<L, 0>(issued - 1 - ri, false);
+        const uint8_t* blk = ring + cslot * kSlot + lb * Q4_K_BPB;
+        cslot = cslot + 1 == kRing ? 0 : cslot + 1;
+        const uint4 hdr = *(const uint4*)blk;
+        const uint4 q0 = *(const uint4*)(blk + 16 + 32 * c), q1 = *(const uint4*)(blk + 32 + 32 * c);
+        const uint32_t qd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        float slo[MT], shi[MT];
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) slo[mi] = shi[mi] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            // a masked nibble in a 16-bit half is the fp16 subnormal q * 2^-24 (low nibbles) or 16 q * 2^-24 (high
+            // nibbles, left in place); the fused multiply-add widens the half itself
+            const uint32_t y = qd[i] >> 8;
+            const half2v l02 = as_half2(qd[i] & 0x000F000Fu), l13 = as_half2(y & 0x000F000Fu);
+            const half2v h02 = as_half2(qd[i] & 0x00F000F0u), h13 = as_half2(y & 0x00F000F0u);
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                float t = slo[mi];
+                t = fmaf(alo[mi][4 * i], (float)l02.x, t);
+                t = fmaf(alo[mi][4 * i + 1], (float)l13.x, t);
+                t = fmaf(alo[mi][4 * i + 2], (float)l02.y, t);
+                slo[mi] = fmaf(alo[mi][4 * i + 3], (float)l13.y, t);
+                t = shi[mi];
+                t = fmaf(ahi[mi][4 * i], (float)h02.x, t);
+                t = fmaf(ahi[mi][4 * i + 1], (float)h13.x, t);
+                t = fmaf(ahi[mi][4 * i + 2], (float)h02.y, t);
+                shi[mi] = fmaf(ahi[mi][4 * i + 3], (float)h13.y, t);
+            }
+        }
+        const float d = h2f((uint16_t)(hdr.x & 0xffffu)), dmin = h2f((uint16_t)(hdr.x >> 16));
+        const uint32_t p0 = (hdr.y >> sh) & 0xffffu, p1 = (hdr.z >> sh) & 0xffffu, p2 = (hdr.w >> sh) & 0xffffu;
+        const uint32_t sc_pair = upper ? ((p2 & 0x0F0Fu) | ((p0 >> 2) & 0x3030u)) : (p0 & 0x3F3Fu);
+        const uint32_t mn_pair = upper ? (((p2 >> 4) & 0x0F0Fu) | ((p1 >> 2) & 0x3030u)) : (p1 & 0x3F3Fu);
+        const float d1 = d * ubyte0(sc_pair) * 16777216.0f, d2 = d * ubyte1(sc_pair) * 1048576.0f;  // 2^24, 2^24 / 16
+        const float m1 = dmin * ubyte0(mn_pair), m2 = dmin * ubyte1(mn_pair);
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            float t = d1 * slo[mi];
+            t = fmaf(-m1, slo_a[mi], t);
+            t = fmaf(d2, shi[mi], t);
+            t = fmaf(-m2, shi_a[mi], t);
+            const float v = wave_sum_dpp(t);
+            if (lane == 0) res[ri * MT + mi] = v;
+        }
+    }
+    if constexpr (WPR == 1) {
+        for (int idx = lane; idx < my_rows * MT; idx += 64) {
+            const int r = idx / MT, mi = idx - r * MT;
+            if (mi < m) out[(int64_t)mi * ldo + gs + (int64_t)r * GS] = res[idx];
+        }
+    } else {
+        __syncthreads();
+        if (part == 0) {
+            for (int idx = lane; idx < my_rows * MT; idx += 64) {
+                const int r = idx / MT, mi = idx - r * MT;
+                float v = res[idx];
+#pragma unroll
+                for (int q = 1; q < WPR; q++) v += res[q * kMaxRows * MT + idx];
+                if (mi < m) out[(int64_t)mi * ldo + gs + (int64_t)r * GS] = v;
+            }
+        }
+    }
+}
+
+// Takes K <= 16384 and m = 1 (reports other shapes through *handled = false).
+hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                  int64_t ldo, hipStream_t s, bool* handled) {
+    *handled = false;
+    static const bool off = getenv("QMM_Q4K_LANES_OFF") != nullptr;  // read once: fallback switch
+    const int nblk = (int)(k / 256);
+    if (off || m > 1 || nblk > 64) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
+    const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
+    const int bpw = (nblk + wpr - 1) / wpr;
+    const int l = (bpw * 9 + 63) / 64;  // 1..3
+    const int mt = m <= 1 ? 1 : 2;
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
+    // staged lhs rows: one padded record per chunk, each row rounded up to whole load instructions (1 KB)
+    const size_t act_bytes = (size_t)mt * (((size_t)(k / 64) * (64 * esz + 16) + 1023) / 1024 * 1024);
+    static const int ring_env = [] { const char* e = getenv("QMM_Q4K_LANES_RING"); return e ? atoi(e) : 0; }();   // read once: tuning
+    static const int percu_env = [] { const char* e = getenv("QMM_Q4K_LANES_WGS"); return e ? atoi(e) : 0; }();  // read once: tuning
+    const size_t fixed = (size_t)kWaves * kMaxRows * mt * 4 + act_bytes, slot = (size_t)bpw * Q4_K_BPB;
+    // three slots (two row parts in flight per wavefront), one workgroup per compute unit: measured best over
+    // (2..4 slots) x (1..3 workgroups per compute unit) on the Llama-3-8B shapes
+    int ring = ring_env >= 2 && ring_env <= 4 ? ring_env : 3;
+    const int per_cu = percu_env > 0 ? percu_env : 1;
+    if (!ring_env && (size_t)kWaves * ring * slot + fixed > 160 * 1024) ring = 2;
+    const size_t lds = (size_t)kWaves * ring * slot + fixed;
+    if (lds > 160 * 1024) return hipSuccess;
+    const int streams = kWaves / wpr;  // rows in progress per workgroup
+    int64_t wgs = (int64_t)cus * per_cu;
+    if (wgs * streams > n) wgs = (n + streams - 1) / streams;
+    const int64_t min_wgs = (n + (int64_t)streams * kMaxRows - 1) / ((int64_t)streams * kMaxRows);
+    if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots
+    dim3 grid((unsigned)wgs), block(64 * kWaves);
+#define QMM_GO3(MT_, WPR_, L_, AT_)                                                                                   \
+    do {                                                                                                              \
+        hipError_t e_ = hipFuncSetAttribute((const void*)gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_>,                  \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                    \
+        if (e_ != hipSuccess) return e_;                                                                              \
+        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(w, (const AT_*)a, out, m, (int)n, (int)k, ldo, ring); \
+    } while (0)
+#define QMM_GO2(MT_, WPR_, L_)                            \
+    do {                                                  \
+        if (a_dtype == QMM_F32) QMM_GO3(MT_, WPR_, L_, float); \
+        else QMM_GO3(MT_, WPR_, L_, uint16_t);            \
+    } while (0)
+#define QMM_GO1(WPR_, L_) QMM_GO2(1, WPR_, L_)
+#define QMM_GO0(WPR_)               \
+    do {                            \
+        if (l == 1) QMM_GO1(WPR_, 1); \
+        else if (l == 2) QMM_GO1(WPR_, 2); \
+        else QMM_GO1(WPR_, 3);      \
+    } while (0)
+    if (wpr == 1) QMM_GO0(1);
+    else if (wpr == 2) QMM_GO0(2);
+    else QMM_GO0(4);
+#undef QMM_GO0
+#undef QMM_GO1
+#undef QMM_GO2
+#undef QMM_GO3
+    *handled = true;
+    return hipGetLastError();
+}
+
+}  // namespace qmm

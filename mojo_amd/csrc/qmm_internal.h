@@ -29,6 +29,8 @@ hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const i
                             hipStream_t s);
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s);
+hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                  int64_t ldo, hipStream_t s, bool* handled);
 hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
