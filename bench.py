@@ -69,6 +69,30 @@ class Gemv:
         _lib.check(rc, "qmm_matmul")
 
 
+class GroupedGemv:
+    """One preallocated qmm_matmul_grouped call: several weight matrices, one lhs."""
+
+    def __init__(self, enc: QE, ws, a: torch.Tensor):
+        self.lib = _lib.load()
+        self.enc, self.ws_t, self.a = enc, list(ws), a
+        self.m, self.k = a.shape
+        self.outs = [torch.empty((self.m, w.shape[0]), dtype=torch.float32, device=a.device) for w in self.ws_t]
+        self.dt = _lib.QMM_F32 if a.dtype == torch.float32 else _lib.QMM_BF16
+        self.need = max(self.lib.qmm_matmul_workspace_bytes(enc.code, self.dt, self.m, w.shape[0], self.k) for w in self.ws_t)
+        self.ws = torch.empty((max(self.need, 1),), dtype=torch.uint8, device=a.device)
+        cnt = len(self.ws_t)
+        self.cnt = cnt
+        self.rhs_p = (C.c_void_p * cnt)(*[w.data_ptr() for w in self.ws_t])
+        self.out_p = (C.c_void_p * cnt)(*[o.data_ptr() for o in self.outs])
+        self.n_p = (C.c_int64 * cnt)(*[w.shape[0] for w in self.ws_t])
+
+    def launch(self, stream_ptr: int) -> None:
+        rc = self.lib.qmm_matmul_grouped(self.enc.code, C.c_void_p(self.a.data_ptr()), self.dt, self.m, self.k, self.cnt,
+                                         self.rhs_p, self.n_p, self.out_p, C.c_void_p(self.ws.data_ptr()), self.need,
+                                         C.c_void_p(stream_ptr))
+        _lib.check(rc, "qmm_matmul_grouped")
+
+
 class GptqMatmul:
     """One preallocated GPTQ qmm_matmul call on (qweight, scales, qzeros)."""
 
@@ -342,6 +366,13 @@ def extra_timings(layers, acts, gen):
     dev_s, _ = time_graphs(graphs, 100, 10)
     wbytes = sum(n * QE.Q4_K.packed_row_bytes(k) for _, n, k in PROJ)
     out["plain_read_same_set"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(wbytes * 100 / dev_s / 1e9, 1)}
+    # the same step with the projections that share their lhs in one launch each: q|k|v, o, gate|up, down
+    if m == 1:
+        graphs = [capture([GroupedGemv(QE.Q4_K, lw[0:3], acts[4096]), Gemv(QE.Q4_K, lw[3], acts[4096]),
+                           GroupedGemv(QE.Q4_K, lw[4:6], acts[4096]), Gemv(QE.Q4_K, lw[6], acts[14336])]) for lw in layers]
+        dev_s, _ = time_graphs(graphs, 100, 10)
+        sb = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
+        out["q4_k_m1_grouped_4_launches"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sb * 100 / dev_s / 1e9, 1)}
     # M=4 over the same set
     if m == 1:
         acts4 = {k: torch.randn((4, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}

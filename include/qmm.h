@@ -124,6 +124,20 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
                void* workspace, int64_t workspace_bytes, int flags, void* stream);
 
 /*
+ * Several GGUF weight matrices applied to one lhs, as the callers of ops.qmatmul in a transformer
+ * block do (q | k | v, and gate | up, take the same activations):
+ *   out[j] fp32[m, n[j]] = lhs[m, k] . dequant(rhs[j])^T,  j < count, all rhs of `encoding` and of row length k.
+ * Where a kernel takes the whole group (Q4_K, m = 1, count <= 4, k <= 16384) this is one launch that
+ * numbers the rows of the matrices through; otherwise it is one qmm_matmul per matrix, in order
+ * (workspace: the largest any of them needs).  The reference exposes the per-matrix op only; fusing
+ * its calls is its graph compiler's job, for which this is the kernel-side counterpart.
+ * rhs, n and out are host arrays.
+ */
+int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, int count,
+                       const void* const* rhs, const int64_t* n, float* const* out, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+
+/*
  * Test hook for the bit-exact integer check: raw int32 block sums
  * out[m, n, k/32] = sum_32 (q4 - 8) * q8 of Q8_0 lhs blocks (uint8[m, k/32*34])
  * against Q4_0 rhs blocks.

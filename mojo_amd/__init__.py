@@ -11,6 +11,7 @@ from .ops import (
     block_dots_q4_0,
     dequantize,
     qmatmul,
+    qmatmul_grouped,
     quantize,
     quantize_gptq,
 )
@@ -21,6 +22,7 @@ __all__ = [
     "QuantizationConfig",
     "QuantizationEncoding",
     "qmatmul",
+    "qmatmul_grouped",
     "dequantize",
     "quantize",
     "quantize_gptq",

@@ -51,10 +51,12 @@ __device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ub
 
 // WPR: wavefronts (parts of K) per row.  L: load instructions per row part (64 pieces of 16 bytes each).
 // ring: LDS slots per wavefront (2..4): one row part being decoded, the others in flight.
+// mats: up to kLanesMaxMats weight matrices that share the lhs and K; their rows are numbered through
+// (matrix j owns rows [end[j - 1], end[j])), so one launch serves q|k|v or gate|up.
 template <int MT, int WPR, int L, typename AT>
-__global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
-                                                                        float* __restrict__ out, int m, int n, int k,
-                                                                        int64_t ldo, int ring_slots) {
+__global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const LanesMats mats, const AT* __restrict__ a,
+                                                                        int m, int k, int64_t ldo, int ring_slots) {
+    const int n = mats.end[mats.count - 1];
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -77,7 +79,11 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     // follows the full part length, a shorter last part repeats its last piece), so the wait counts stay exact.
     const int last_piece = max(nb, 1) * 9 - 1;
     auto issue = [&](int ri, int slot) {
-        const uint8_t* base = w + (int64_t)(gs + (int64_t)ri * GS) * row_bytes + (int64_t)blk0 * Q4_K_BPB;
+        const int row = gs + ri * GS;
+        int j = 0;
+        while (j + 1 < mats.count && row >= mats.end[j]) j++;  // (uniform: a few scalar compares)
+        const int local = row - (j ? mats.end[j - 1] : 0);
+        const uint8_t* base = mats.w[j] + (int64_t)local * row_bytes + (int64_t)blk0 * Q4_K_BPB;
 #pragma unroll
         for (int i = 0; i < L; i++)
             if (lane + 64 * i < pieces)
@@ -204,10 +210,17 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             if (lane == 0) res[ri * MT + mi] = v;
         }
     }
+    auto store_row = [&](int mi, int row, float v) {
+        int j = 0;
+        while (j + 1 < mats.count && row >= mats.end[j]) j++;
+        const int local = row - (j ? mats.end[j - 1] : 0);
+        const int nj = mats.end[j] - (j ? mats.end[j - 1] : 0);
+        mats.out[j][(int64_t)mi * (ldo ? ldo : nj) + local] = v;
+    };
     if constexpr (WPR == 1) {
         for (int idx = lane; idx < my_rows * MT; idx += 64) {
             const int r = idx / MT, mi = idx - r * MT;
-            if (mi < m) out[(int64_t)mi * ldo + gs + (int64_t)r * GS] = res[idx];
+            if (mi < m) store_row(mi, gs + r * GS, res[idx]);
         }
     } else {
         __syncthreads();
@@ -217,19 +230,31 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
                 float v = res[idx];
 #pragma unroll
                 for (int q = 1; q < WPR; q++) v += res[q * kMaxRows * MT + idx];
-                if (mi < m) out[(int64_t)mi * ldo + gs + (int64_t)r * GS] = v;
+                if (mi < m) store_row(mi, gs + r * GS, v);
             }
         }
     }
 }
 
-// Takes K <= 16384 and m = 1 (reports other shapes through *handled = false).
-hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
-                                  int64_t ldo, hipStream_t s, bool* handled) {
+// Takes K <= 16384 and m = 1 (reports other shapes through *handled = false).  count matrices [n[j], k] share the
+// lhs; out[j] is fp32 [m, n[j]] (ldo = 0: dense; a single matrix may give its own leading dimension).
+hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
+                                          float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled) {
     *handled = false;
     static const bool off = getenv("QMM_Q4K_LANES_OFF") != nullptr;  // read once: fallback switch
     const int nblk = (int)(k / 256);
-    if (off || m > 1 || nblk > 64) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
+    if (off || m > 1 || nblk > 64 || count < 1 || count > kLanesMaxMats) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
+    LanesMats mats;
+    int64_t n = 0;
+    for (int j = 0; j < kLanesMaxMats; j++) {
+        const int jj = j < count ? j : count - 1;
+        if (j < count) n += ns[j];
+        mats.w[j] = ws[jj];
+        mats.out[j] = outs[jj];
+        mats.end[j] = (int)n;
+    }
+    mats.count = count;
+    if (n > 0x7fffffff) return hipSuccess;
     const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
     const int bpw = (nblk + wpr - 1) / wpr;
     const int l = (bpw * 9 + 63) / 64;  // 1..3
@@ -265,7 +290,7 @@ hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, 
         hipError_t e_ = hipFuncSetAttribute((const void*)gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_>,                  \
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                    \
         if (e_ != hipSuccess) return e_;                                                                              \
-        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(w, (const AT_*)a, out, m, (int)n, (int)k, ldo, ring); \
+        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring); \
     } while (0)
 #define QMM_GO2(MT_, WPR_, L_)                            \
     do {                                                  \
@@ -288,6 +313,11 @@ hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, 
 #undef QMM_GO3
     *handled = true;
     return hipGetLastError();
+}
+
+hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                  int64_t ldo, hipStream_t s, bool* handled) {
+    return launch_gemv_q4_k_lanes_grouped(a, a_dtype, 1, &w, &n, &out, m, k, ldo, s, handled);
 }
 
 }  // namespace qmm

@@ -266,6 +266,41 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     return QMM_OK;
 }
 
+int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, int count,
+                       const void* const* rhs, const int64_t* n, float* const* out, void* workspace,
+                       int64_t workspace_bytes, void* stream) {
+    if (!lhs || !rhs || !n || !out) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: null pointer");
+    if (count < 1 || count > 64) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: count %d out of range (1..64)", count);
+    int64_t epb, bpb;
+    if (encoding == QMM_Q8_0 || encoding == QMM_GPTQ || !block_params(encoding, epb, bpb))
+        return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: encoding %d is not a GGUF weight encoding", encoding);
+    for (int j = 0; j < count; j++)
+        if (!rhs[j] || !out[j] || n[j] <= 0) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: matrix %d: null pointer or N <= 0", j);
+    if (encoding == QMM_Q4_K && m == 1 && k > 0 && k % 256 == 0 && count <= qmm::kLanesMaxMats &&
+        (lhs_dtype == QMM_F32 || lhs_dtype == QMM_BF16) && aligned(lhs, 16)) {
+        bool ok = true;
+        int64_t total = 0;
+        const uint8_t* ws[qmm::kLanesMaxMats];
+        for (int j = 0; j < count; j++) {
+            ok = ok && aligned(rhs[j], 16) && aligned(out[j], 4);
+            total += n[j];
+            ws[j] = (const uint8_t*)rhs[j];
+        }
+        if (ok && total <= INT32_MAX) {
+            bool handled = false;
+            hipError_t e = qmm::launch_gemv_q4_k_lanes_grouped(lhs, lhs_dtype, count, ws, n, out, 1, k, 0, (hipStream_t)stream, &handled);
+            if (e != hipSuccess) return hip_status(e, "qmm_matmul_grouped(Q4_K decode)");
+            if (handled) return QMM_OK;
+        }
+    }
+    for (int j = 0; j < count; j++) {
+        const void* one[1] = {rhs[j]};
+        if (int rc = qmm_matmul(encoding, nullptr, lhs, lhs_dtype, m, k, one, 1, n[j], out[j], workspace, workspace_bytes, 0, stream))
+            return rc;
+    }
+    return QMM_OK;
+}
+
 int qmm_block_dots_q4_0(const void* lhs_q8_0, const void* rhs_q4_0, int64_t m, int64_t n, int64_t k, int32_t* out,
                         void* stream) {
     if (!lhs_q8_0 || !rhs_q4_0 || !out) return fail(QMM_ERR_INVALID, "qmm_block_dots_q4_0: null pointer");

@@ -29,6 +29,16 @@ hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const i
                             hipStream_t s);
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s);
+// Weight matrices that share one lhs, for the grouped decode launch.
+constexpr int kLanesMaxMats = 4;
+struct LanesMats {
+    const uint8_t* w[kLanesMaxMats];
+    float* out[kLanesMaxMats];
+    int end[kLanesMaxMats];  // running row count: matrix j owns rows [end[j - 1], end[j])
+    int count;
+};
+hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
+                                          float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled);
 hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
                                   int64_t ldo, hipStream_t s, bool* handled);
 hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,

@@ -6,7 +6,7 @@ number is produced by the HIP kernels in ``libqmm.so``.
 from __future__ import annotations
 
 import ctypes as C
-from typing import Optional, Sequence
+from typing import List, Optional, Sequence
 
 import torch
 
@@ -110,6 +110,48 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
                         need, _lib.QMM_FLAG_W_BF16 if w_bf16 else 0, _stream(lhs))
     _lib.check(rc, "qmatmul")
     return out.reshape(*lead, n)
+
+
+def qmatmul_grouped(encoding: QuantizationEncoding, lhs: torch.Tensor, rhs: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+    """``[lhs @ dequantize(w)^T for w in rhs]`` for GGUF weight matrices that share ``lhs`` (q | k | v, gate | up).
+
+    One launch where a kernel takes the whole group (Q4_K, a single lhs row, up to four matrices); otherwise
+    the library runs one matmul per matrix.  Results are those of ``qmatmul`` on each matrix.
+    """
+    if not isinstance(encoding, QuantizationEncoding) or not encoding.is_gguf:
+        raise TypeError("qmatmul_grouped takes a GGUF weight encoding")
+    rhs = list(rhs)
+    if not rhs:
+        raise ValueError("qmatmul_grouped needs at least one rhs tensor")
+    _require_gpu(lhs, "lhs")
+    if lhs.dtype not in _DTYPES:
+        raise TypeError(f"lhs must be float32 or bfloat16, got {lhs.dtype}")
+    k = lhs.shape[-1]
+    lead = lhs.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    if m == 0:
+        raise ValueError("qmatmul of an empty tensor")
+    for w in rhs:
+        _require_gpu(w, "rhs")
+        if w.dtype != torch.uint8 or w.dim() != 2 or w.shape[0] == 0:
+            raise TypeError("every rhs must be a non-empty rank-2 uint8 tensor of packed blocks")
+        if w.shape[1] != encoding.packed_row_bytes(k):
+            raise ValueError(
+                f"rhs rows hold {w.shape[1]} bytes; K={k} in {encoding.name} needs {encoding.packed_row_bytes(k)}")
+    lib = _lib.load()
+    lhs_dt = _DTYPES[lhs.dtype]
+    outs = [torch.empty((m, w.shape[0]), dtype=torch.float32, device=lhs.device) for w in rhs]
+    need = max(lib.qmm_matmul_workspace_bytes(encoding.code, lhs_dt, m, w.shape[0], k) for w in rhs)
+    ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
+    count = len(rhs)
+    rhs_p = (C.c_void_p * count)(*[w.data_ptr() for w in rhs])
+    out_p = (C.c_void_p * count)(*[o.data_ptr() for o in outs])
+    n_p = (C.c_int64 * count)(*[w.shape[0] for w in rhs])
+    rc = lib.qmm_matmul_grouped(encoding.code, _ptr(lhs), lhs_dt, m, k, count, rhs_p, n_p, out_p, _ptr(ws), need, _stream(lhs))
+    _lib.check(rc, "qmatmul_grouped")
+    return [o.reshape(*lead, o.shape[1]) for o in outs]
 
 
 def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Optional[int] = None,

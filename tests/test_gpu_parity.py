@@ -11,7 +11,7 @@ import torch
 import oracle as O
 from conftest import synth
 from mojo_amd import QuantizationConfig, QuantizationEncoding as QE
-from mojo_amd import block_dots_q4_0, dequantize, qmatmul, quantize, quantize_gptq
+from mojo_amd import block_dots_q4_0, dequantize, qmatmul, qmatmul_grouped, quantize, quantize_gptq
 
 pytestmark = pytest.mark.gpu
 
@@ -232,6 +232,31 @@ def test_q4_k_small_batch_wide_range_lhs(m):
     got = qmatmul(QE.Q4_K, None, gpu(a), gpu(wq)).cpu().numpy()
     scale = np.abs(truth).max(axis=1, keepdims=True)
     assert np.all(np.abs(got - truth) <= 1e-4 * scale + 1e-3 * np.abs(truth))
+
+
+# ------------------------------------------------------------------ matrices that share their lhs
+@pytest.mark.parametrize("enc,m,k,ns,lhs_bf16", [(QE.Q4_K, 1, 4096, (512, 130, 130), False), (QE.Q4_K, 1, 14336, (300, 77), True),
+                                                 (QE.Q4_K, 1, 512, (9000, 1, 17, 4100), False),
+                                                 (QE.Q4_K, 3, 1024, (64, 200), False), (QE.Q6_K, 1, 1024, (96, 40), False),
+                                                 (QE.Q4_0, 2, 256, (33, 64, 5), False), (QE.Q4_K, 1, 256, (8, 8, 8, 8, 8), False)])
+def test_grouped_matmul_equals_separate_calls(enc, m, k, ns, lhs_bf16):
+    """q | k | v and gate | up style groups: the one-launch path (Q4_K, one lhs row, up to four matrices) and the
+    per-matrix path give what qmatmul gives on each matrix, bit for bit, and agree with the oracle."""
+    ws, a = [], None
+    for j, n in enumerate(ns):
+        w, a = synth(60 + j, n, k, m)
+        ws.append(O.quantize(ENC[enc], w))
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    lhs = gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a)
+    rhs = [gpu(w) for w in ws]
+    got = qmatmul_grouped(enc, lhs, rhs)
+    assert [tuple(g.shape) for g in got] == [(m, n) for n in ns]
+    for j, n in enumerate(ns):
+        one = qmatmul(enc, None, lhs, rhs[j])
+        assert torch.equal(got[j], one), f"matrix {j} differs from the separate call"
+        want = O.matmul_q4_0(a, ws[j]) if enc is QE.Q4_0 else O.matmul_f32(ENC[enc], a, ws[j])
+        assert_close(got[j], want, f"grouped {enc.name} matrix {j} ({m}x{n}x{k})")
 
 
 # ------------------------------------------------------------------ prefill shapes (m > 16)
