@@ -38,17 +38,6 @@ __device__ __forceinline__ void wait_rows(int rows) {
     else wait_vmcnt<0>();
 }
 
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    v += dpp_move<0x140>(v);  // every lane of a 16-lane row holds the row sum
-    const int b = __float_as_int(v);
-    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
-    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
-    return (r0 + r1) + (r2 + r3);
-}
-
 }  // namespace
 
 // BPL: blocks per lane (k <= 2048 * BPL).  L = load instructions per row = pieces of 16 bytes / 64, for the
@@ -248,14 +237,12 @@ hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w,
     do {                                                                                                              \
         hipError_t e_;                                                                                                \
         if (a_dtype == QMM_F32) {                                                                                     \
-            e_ = hipFuncSetAttribute((const void*)gemv_q4_0_stream_kernel<MT_, BPL_, RING_, float>,                   \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                           \
+            e_ = allow_full_lds<gemv_q4_0_stream_kernel<MT_, BPL_, RING_, float>>();                                  \
             if (e_ != hipSuccess) return e_;                                                                          \
             gemv_q4_0_stream_kernel<MT_, BPL_, RING_, float><<<grid, block, lds, s>>>(w, (const float*)a, out, m, (int)n, \
                                                                                      (int)k, ldo);                   \
         } else {                                                                                                      \
-            e_ = hipFuncSetAttribute((const void*)gemv_q4_0_stream_kernel<MT_, BPL_, RING_, uint16_t>,                \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                           \
+            e_ = allow_full_lds<gemv_q4_0_stream_kernel<MT_, BPL_, RING_, uint16_t>>();                               \
             if (e_ != hipSuccess) return e_;                                                                          \
             gemv_q4_0_stream_kernel<MT_, BPL_, RING_, uint16_t><<<grid, block, lds, s>>>(w, (const uint16_t*)a, out, m, \
                                                                                         (int)n, (int)k, ldo);        \

@@ -33,17 +33,6 @@ constexpr int kMaxRows = 64;  // rows a wavefront may own (LDS result slots)
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ half2v as_half2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
 
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    v += dpp_move<0x140>(v);  // every lane of a 16-lane row holds the row sum
-    const int b = __float_as_int(v);
-    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
-    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
-    return (r0 + r1) + (r2 + r3);
-}
-
 __device__ __forceinline__ float ubyte0(uint32_t v) { float f; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v)); return f; }
 __device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v)); return f; }
 
@@ -278,7 +267,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     const int per_cu = percu_env > 0 ? percu_env : 1;
     if (!ring_env && (size_t)kWaves * ring * slot + fixed > 160 * 1024) ring = 2;
     const size_t lds = (size_t)kWaves * ring * slot + fixed;
-    if (lds > 160 * 1024) return hipSuccess;
+    if (lds > (size_t)kLdsPerCu) return hipSuccess;
     const int streams = kWaves / wpr;  // rows in progress per workgroup
     int64_t wgs = (int64_t)cus * per_cu;
     if (wgs * streams > n) wgs = (n + streams - 1) / streams;
@@ -287,8 +276,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     dim3 grid((unsigned)wgs), block(64 * kWaves);
 #define QMM_GO3(MT_, WPR_, L_, AT_)                                                                                   \
     do {                                                                                                              \
-        hipError_t e_ = hipFuncSetAttribute((const void*)gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_>,                  \
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                    \
+        hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_>>();                                \
         if (e_ != hipSuccess) return e_;                                                                              \
         gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring); \
     } while (0)

@@ -44,18 +44,6 @@ __device__ __forceinline__ float ub1(uint32_t v) { float f; asm("v_cvt_f32_ubyte
 __device__ __forceinline__ float ub2(uint32_t v) { float f; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v)); return f; }
 __device__ __forceinline__ float ub3(uint32_t v) { float f; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v)); return f; }
 
-// Sum over the 64 lanes through DPP; the total is returned in every lane.
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    v += dpp_move<0x140>(v);  // every lane of a 16-lane row holds the row sum
-    const int b = __float_as_int(v);
-    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
-    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
-    return (r0 + r1) + (r2 + r3);
-}
-
 }  // namespace
 
 // LDSA: the lhs rows are staged once per workgroup in LDS, 16-byte pieces stored in the order the

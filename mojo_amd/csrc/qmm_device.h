@@ -77,6 +77,18 @@ __device__ __forceinline__ float sum8(float v) {
     return v;
 }
 
+// Sum over the 64 lanes through DPP; the total is returned in every lane.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);  // every lane of a 16-lane row holds the row sum
+    const int b = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0)), r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32)), r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
 // Largest value of a non-negative float over the 64 lanes, as its bit pattern (wave-uniform).
 __device__ __forceinline__ uint32_t wave_max_nonneg_bits(float v) {
     v = fmaxf(v, dpp_move<0xB1>(v));

@@ -29,6 +29,15 @@ hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const i
                             hipStream_t s);
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s);
+// Kernels that use more than 64 KB of dynamic LDS must say so once before their first launch: this raises the
+// kernel's limit to the 160 KB of a gfx950 compute unit, the first time it is called for the kernel.
+constexpr int kLdsPerCu = 160 * 1024;
+template <auto Kernel>
+inline hipError_t allow_full_lds() {
+    static const hipError_t st = hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsPerCu);
+    return st;
+}
+
 // Weight matrices that share one lhs, for the grouped decode launch.
 constexpr int kLanesMaxMats = 4;
 struct LanesMats {
