@@ -201,6 +201,24 @@ def test_leading_dims_broadcast():
     assert_close(got, want, "leading dims")
 
 
+# ------------------------------------------------------------------ Q4_K decode (one lhs row)
+@pytest.mark.parametrize("n,k,lhs_bf16", [(1, 256, False), (7, 512, True), (70000, 256, False), (129, 4096, False),
+                                          (300, 4352, True), (50, 8192, False), (33, 9984, False), (40, 16384, True),
+                                          (12, 16640, False), (5000, 3840, False)])
+def test_q4_k_decode_shapes(n, k, lhs_bf16):
+    """One lhs row: rows cut into 1, 2 or 4 parts (K up to 16384; longer rows take the streaming kernel), parts that
+    do not fill a wavefront, fewer rows than wavefronts, many rows per wavefront."""
+    w, a = synth(23, n, k, 1)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq)
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q4_K decode 1x{n}x{k} vs fp32 oracle")
+    assert_close(got, truth, f"Q4_K decode 1x{n}x{k} vs fp64 truth")
+
+
 # ------------------------------------------------------------------ Q4_K small batch (2..16 lhs rows)
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(2, 9000, 1024, False), (4, 8200, 4608, False), (7, 4100, 2048, True),
                                             (8, 6000, 4608, False), (5, 300, 256, False), (12, 5000, 1280, True),
