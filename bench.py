@@ -49,9 +49,9 @@ def alg_bytes(enc: QE, m: int, n: int, k: int) -> int:
 class Gemv:
     """One preallocated qmm_matmul call (no Python-side allocation when launched)."""
 
-    def __init__(self, enc: QE, w: torch.Tensor, a: torch.Tensor):
+    def __init__(self, enc: QE, w: torch.Tensor, a: torch.Tensor, flags: int = 0):
         self.lib = _lib.load()
-        self.enc, self.w, self.a = enc, w, a
+        self.enc, self.w, self.a, self.flags = enc, w, a, flags
         self.m, self.k = a.shape
         self.n = w.shape[0]
         self.out = torch.empty((self.m, self.n), dtype=torch.float32, device=a.device)
@@ -65,7 +65,7 @@ class Gemv:
     def launch(self, stream_ptr: int) -> None:
         rc = self.lib.qmm_matmul(self.enc.code, None, C.c_void_p(self.a.data_ptr()), self.dt, self.m, self.k,
                                  self.ptrs, 1, self.n, C.c_void_p(self.out.data_ptr()),
-                                 C.c_void_p(self.ws.data_ptr()), self.need, 0, C.c_void_p(stream_ptr))
+                                 C.c_void_p(self.ws.data_ptr()), self.need, self.flags, C.c_void_p(stream_ptr))
         _lib.check(rc, "qmm_matmul")
 
 
@@ -373,6 +373,13 @@ def extra_timings(layers, acts, gen):
         dev_s, _ = time_graphs(graphs, 100, 10)
         sb = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
         out["q4_k_m1_grouped_4_launches"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sb * 100 / dev_s / 1e9, 1)}
+    # the optional integer-activation treatment (lhs -> Q8_K in the kernel, integer sub-block dots), M = 1 and 4
+    for mm in (1, 4):
+        a8 = {kk: torch.randn((mm, kk), dtype=torch.float32, device="cuda:0", generator=gen) for kk in (4096, 14336)}
+        graphs = [capture([Gemv(QE.Q4_K, w, a8[kk], _lib.QMM_FLAG_ACT_Q8K) for w, (_, nn, kk) in zip(lw, PROJ)]) for lw in layers]
+        dev_s, _ = time_graphs(graphs, 100, 10)
+        sb = sum(alg_bytes(QE.Q4_K, mm, nn, kk) for _, nn, kk in PROJ)
+        out[f"q4_k_act_q8k_m{mm}"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sb * 100 / dev_s / 1e9, 1)}
     # M=4 over the same set
     if m == 1:
         acts4 = {k: torch.randn((4, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}

@@ -39,7 +39,8 @@ enum qmm_encoding {
     QMM_Q4_K = 1, /* 256 weights / 144 bytes: f16 d, dmin, 12 B 6-bit, 128 B */
     QMM_Q6_K = 2, /* 256 weights / 210 bytes: ql[128] qh[64] i8 sc[16] f16 d */
     QMM_GPTQ = 3, /* AutoGPTQ v1 tensors: qweight, scales, qzeros[, g_idx]   */
-    QMM_Q8_0 = 8  /* 32 values / 34 bytes  : f16 d, 32 x i8 (activations)    */
+    QMM_Q8_0 = 8, /* 32 values / 34 bytes  : f16 d, 32 x i8 (activations)    */
+    QMM_Q8_K = 9  /* 256 values / 292 bytes: f32 d, 256 x i8, 16 x i16 sums (activations) */
 };
 
 enum qmm_dtype { QMM_F32 = 0, QMM_BF16 = 1, QMM_F16 = 2 };
@@ -95,7 +96,7 @@ int qmm_dequantize_gptq(const qmm_gptq_config* cfg, const void* qweight, const v
 
 /*
  * Quantisers.  x fp32[rows, k] -> packed blocks uint8[rows, k/epb*bpb].
- * QMM_Q4_0 and QMM_Q8_0 follow the GGUF reference quantisers; QMM_Q4_K and
+ * QMM_Q4_0, QMM_Q8_0 and QMM_Q8_K follow the GGUF reference quantisers; QMM_Q4_K and
  * QMM_Q6_K use a direct (non-iterative) min/max fit.
  */
 int qmm_quantize(int encoding, const float* x, int64_t rows, int64_t k, void* out, void* stream);
@@ -115,10 +116,14 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
  *   lhs_dtype QMM_F32 or QMM_BF16.  Q4_0 quantises lhs rows to Q8_0 and takes
  *   integer block dots (the reference CPU path); the others keep lhs as given.
  *   flags: bit 0 (QMM_FLAG_W_BF16) rounds dequantised weights to bf16 before
- *   the product in the M > 16 kernels.
+ *   the product in the M > 16 kernels.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K only: the
+ *   lhs is quantised to Q8_K blocks (256 wide, fp32 scale) and the product is the
+ *   integer sub-block dot of the ggml-lineage CPU kernels instead of the default
+ *   floating-point one; K <= 16384, any m (passes of four rows).
  * rhs is a host array of device pointers.
  */
 #define QMM_FLAG_W_BF16 1
+#define QMM_FLAG_ACT_Q8K 2
 int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m,
                int64_t k, const void* const* rhs, int n_rhs, int64_t n, float* out,
                void* workspace, int64_t workspace_bytes, int flags, void* stream);

@@ -9,6 +9,7 @@ LIB_PATH = os.path.join(HERE, "libqmm.so")
 
 QMM_F32, QMM_BF16, QMM_F16 = 0, 1, 2
 QMM_FLAG_W_BF16 = 1
+QMM_FLAG_ACT_Q8K = 2
 
 
 class GptqConfig(C.Structure):

@@ -45,6 +45,7 @@ bool block_params(int enc, int64_t& epb, int64_t& bpb) {
     switch (enc) {
         case QMM_Q4_0: epb = 32; bpb = 18; return true;
         case QMM_Q8_0: epb = 32; bpb = 34; return true;
+        case QMM_Q8_K: epb = 256; bpb = 292; return true;
         case QMM_Q4_K: epb = 256; bpb = 144; return true;
         case QMM_Q6_K: epb = 256; bpb = 210; return true;
         default: return false;
@@ -119,7 +120,7 @@ int qmm_read_probe(const void* buf, int64_t bytes, void* stream) {
 
 int qmm_dequantize(int encoding, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype, void* stream) {
     int64_t epb, bpb;
-    if (encoding == QMM_Q8_0 || !block_params(encoding, epb, bpb))
+    if (encoding == QMM_Q8_0 || encoding == QMM_Q8_K || !block_params(encoding, epb, bpb))
         return fail(QMM_ERR_INVALID, "qmm_dequantize: encoding %d is not a GGUF weight encoding", encoding);
     if (!rhs || !out) return fail(QMM_ERR_INVALID, "qmm_dequantize: null pointer");
     if (n <= 0 || k <= 0 || k % epb)
@@ -152,6 +153,8 @@ int qmm_quantize(int encoding, const float* x, int64_t rows, int64_t k, void* ou
     if (rows <= 0 || k <= 0 || k % epb)
         return fail(QMM_ERR_INVALID, "qmm_quantize: rows=%lld, K=%lld; K must be a positive multiple of %lld",
                     (long long)rows, (long long)k, (long long)epb);
+    if (encoding == QMM_Q8_K)
+        return hip_status(qmm::launch_quantize_q8_k(x, QMM_F32, rows, k, out, (hipStream_t)stream), "qmm_quantize(Q8_K)");
     return hip_status(qmm::launch_quantize(encoding, x, rows, k, out, (hipStream_t)stream), "qmm_quantize");
 }
 
@@ -180,9 +183,9 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
 int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
                int flags, void* stream) {
-    (void)flags;
     hipStream_t s = (hipStream_t)stream;
     if (!lhs || !rhs || !out) return fail(QMM_ERR_INVALID, "qmm_matmul: null pointer");
+    if (flags & ~(QMM_FLAG_W_BF16 | QMM_FLAG_ACT_Q8K)) return fail(QMM_ERR_INVALID, "qmm_matmul: unknown flag bits 0x%x", flags);
     if (m <= 0 || n <= 0 || k <= 0)
         return fail(QMM_ERR_INVALID, "qmm_matmul: M=%lld N=%lld K=%lld must all be positive", (long long)m,
                     (long long)n, (long long)k);
@@ -218,7 +221,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     }
 
     int64_t epb, bpb;
-    if (encoding == QMM_Q8_0 || !block_params(encoding, epb, bpb))
+    if (encoding == QMM_Q8_0 || encoding == QMM_Q8_K || !block_params(encoding, epb, bpb))
         return fail(QMM_ERR_INVALID, "qmm_matmul: unknown encoding %d", encoding);
     if (n_rhs != 1 || !rhs[0]) return fail(QMM_ERR_INVALID, "qmm_matmul: GGUF encodings take exactly one rhs tensor");
     if (k % epb)
@@ -228,6 +231,17 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     if (encoding == QMM_Q4_K && !aligned(w, 16)) return fail(QMM_ERR_INVALID, "qmm_matmul: Q4_K rhs must be 16-byte aligned");
     if (!aligned(w, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: rhs must be 2-byte aligned");
 
+    if (flags & QMM_FLAG_ACT_Q8K) {
+        if (encoding != QMM_Q4_K) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations are implemented for Q4_K weights only");
+        for (int64_t m0 = 0; m0 < m; m0 += 4) {
+            bool handled = false;
+            hipError_t e = qmm::launch_gemv_q4_k_q8k((const char*)lhs + m0 * k * esz, lhs_dtype, w, (int)std::min<int64_t>(4, m - m0), n, k,
+                                                     out + m0 * n, n, s, &handled);
+            if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K x Q8_K)");
+            if (!handled) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations need K <= 16384 (K = %lld)", (long long)k);
+        }
+        return QMM_OK;
+    }
     if (encoding == QMM_Q4_0 && m >= 5 && !env_flag_qmm_q4_0_gemv())
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0 && m <= 4) {
@@ -272,7 +286,7 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
     if (!lhs || !rhs || !n || !out) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: null pointer");
     if (count < 1 || count > 64) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: count %d out of range (1..64)", count);
     int64_t epb, bpb;
-    if (encoding == QMM_Q8_0 || encoding == QMM_GPTQ || !block_params(encoding, epb, bpb))
+    if (encoding == QMM_Q8_0 || encoding == QMM_Q8_K || encoding == QMM_GPTQ || !block_params(encoding, epb, bpb))
         return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: encoding %d is not a GGUF weight encoding", encoding);
     for (int j = 0; j < count; j++)
         if (!rhs[j] || !out[j] || n[j] <= 0) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: matrix %d: null pointer or N <= 0", j);

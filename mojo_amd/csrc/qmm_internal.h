@@ -18,6 +18,7 @@ hipError_t launch_dequant_gptq(const void* qweight, const void* scales, const vo
 hipError_t launch_quantize(int enc, const float* x, int64_t rows, int64_t k, void* out, hipStream_t s);
 hipError_t launch_quantize_q8_0(const void* x, int x_dtype, int64_t rows, int64_t k, void* blocks,
                                 void* codes, void* dscale, void* csum, hipStream_t s);
+hipError_t launch_quantize_q8_k(const void* x, int x_dtype, int64_t rows, int64_t k, void* out, hipStream_t s);
 hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group, void* qweight,
                                 void* scales, void* qzeros, void* g_idx, hipStream_t s);
 
@@ -37,6 +38,10 @@ inline hipError_t allow_full_lds() {
     static const hipError_t st = hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsPerCu);
     return st;
 }
+
+// Q4_K with Q8_K-quantised activations (integer dots), m <= 4.
+hipError_t launch_gemv_q4_k_q8k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                int64_t ldo, hipStream_t s, bool* handled);
 
 // Weight matrices that share one lhs, for the grouped decode launch.
 constexpr int kLanesMaxMats = 4;

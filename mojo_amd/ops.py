@@ -42,14 +42,15 @@ def _gptq_cfg(config: Optional[QuantizationConfig]) -> _lib.GptqConfig:
 
 
 def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], lhs: torch.Tensor,
-            *rhs: torch.Tensor, w_bf16: bool = False) -> torch.Tensor:
+            *rhs: torch.Tensor, w_bf16: bool = False, act_q8k: bool = False) -> torch.Tensor:
     """``out[..., N] = lhs[..., K] @ dequantize(rhs)^T`` in fp32.
 
     GGUF encodings take one ``uint8[N, K/epb*bpb]`` tensor of packed blocks (the
     transposed, quantised weight).  GPTQ takes the AutoGPTQ tensors
     ``(qweight int32[K/8, N], scales float16[K/g, N], qzeros int32[K/g, N/8][, g_idx int32[K]])``.
     ``lhs`` is float32 or bfloat16.  Q4_0 quantises ``lhs`` to Q8_0 blocks and
-    takes integer block dots; the other encodings use ``lhs`` as given.
+    takes integer block dots; the other encodings use ``lhs`` as given.  ``act_q8k=True`` (Q4_K only)
+    quantises ``lhs`` to Q8_K blocks and takes the integer sub-block dots of the ggml-lineage CPU kernels instead.
     """
     if not isinstance(encoding, QuantizationEncoding):
         raise TypeError("encoding must be a QuantizationEncoding")
@@ -107,7 +108,8 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
     ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
     ptrs = (C.c_void_p * len(rhs))(*[t.data_ptr() for t in rhs])
     rc = lib.qmm_matmul(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), _ptr(ws),
-                        need, _lib.QMM_FLAG_W_BF16 if w_bf16 else 0, _stream(lhs))
+                        need, (_lib.QMM_FLAG_W_BF16 if w_bf16 else 0) | (_lib.QMM_FLAG_ACT_Q8K if act_q8k else 0),
+                        _stream(lhs))
     _lib.check(rc, "qmatmul")
     return out.reshape(*lead, n)
 
@@ -196,7 +198,7 @@ def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Opti
 
 
 def quantize(encoding: QuantizationEncoding, x: torch.Tensor) -> torch.Tensor:
-    """fp32 ``[rows, K]`` -> packed ``uint8[rows, K/epb*bpb]`` (Q4_0, Q8_0, Q4_K, Q6_K)."""
+    """fp32 ``[rows, K]`` -> packed ``uint8[rows, K/epb*bpb]`` (Q4_0, Q8_0, Q8_K, Q4_K, Q6_K)."""
     _require_gpu(x, "x")
     if x.dtype != torch.float32 or x.dim() != 2:
         raise TypeError("x must be a rank-2 float32 tensor")

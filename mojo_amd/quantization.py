@@ -24,6 +24,8 @@ class QuantizationEncoding(enum.Enum):
     GPTQ = "GPTQ"
     # activation-side block format of the Q4_0 path; not a weight encoding of qmatmul
     Q8_0 = "Q8_0"
+    # activation-side block format of the optional integer Q4_K path (``qmatmul(..., act_q8k=True)``)
+    Q8_K = "Q8_K"
 
     @property
     def code(self) -> int:
@@ -53,10 +55,12 @@ _CODES = {
     QuantizationEncoding.Q6_K: 2,
     QuantizationEncoding.GPTQ: 3,
     QuantizationEncoding.Q8_0: 8,
+    QuantizationEncoding.Q8_K: 9,
 }
 _BLOCKS = {
     QuantizationEncoding.Q4_0: BlockParameters(32, 18),
     QuantizationEncoding.Q8_0: BlockParameters(32, 34),
+    QuantizationEncoding.Q8_K: BlockParameters(256, 292),
     QuantizationEncoding.Q4_K: BlockParameters(256, 144),
     QuantizationEncoding.Q6_K: BlockParameters(256, 210),
 }

@@ -185,6 +185,42 @@ def matmul_q4_0_q8_0(a_q8, w_q4, k: int) -> np.ndarray:
     return out
 
 
+def quantize_q8_k(x) -> np.ndarray:
+    """fp32 [rows, K] -> Q8_K blocks uint8 [rows, K/256*292] (float d, 256 int8 codes, 16 int16 sums of 16)."""
+    x, rows, k = _rows_k(x)
+    assert k % 256 == 0
+    out = np.empty((rows, k // 256 * 292), np.uint8)
+    lib().qo_quantize_q8_k(_p(x), _i64(rows), _i64(k), _p(out))
+    return out
+
+
+def block_sums_q4_k_q8_k(a_q8k, w, k: int):
+    """(isum, msum) int32 [M, N, K/256]: the integer parts of the Q4_K x Q8_K dot, block by block."""
+    a_q8k, w = _c(a_q8k, np.uint8), _c(w, np.uint8)
+    m, n = a_q8k.shape[0], w.shape[0]
+    isum, msum = np.empty((m, n, k // 256), np.int32), np.empty((m, n, k // 256), np.int32)
+    lib().qo_block_sums_q4_k_q8_k(_p(a_q8k), _p(w), _i64(m), _i64(n), _i64(k), _p(isum), _p(msum))
+    return isum, msum
+
+
+def matmul_q4_k_q8_k(a_q8k, w, k: int) -> np.ndarray:
+    a_q8k, w = _c(a_q8k, np.uint8), _c(w, np.uint8)
+    m, n = a_q8k.shape[0], w.shape[0]
+    out = np.empty((m, n), np.float32)
+    lib().qo_matmul_q4_k_q8_k(_p(a_q8k), _p(w), _i64(m), _i64(n), _i64(k), _p(out))
+    return out
+
+
+def matmul_q4_k_act_q8_k(a, w) -> np.ndarray:
+    """The integer-activation Q4_K path: fp32 activations -> Q8_K, integer sub-block dots."""
+    a, m, k = _rows_k(a)
+    w = _c(w, np.uint8)
+    n = w.shape[0]
+    out = np.empty((m, n), np.float32)
+    lib().qo_matmul_q4_k_act_q8_k(_p(a), _p(w), _i64(m), _i64(n), _i64(k), _p(out))
+    return out
+
+
 def matmul_f32(enc: int, a, w, w_bf16: bool = False) -> np.ndarray:
     a, m, k = _rows_k(a)
     w = _c(w, np.uint8)

@@ -48,6 +48,17 @@
  *   activation treatment for Q4_K/Q6_K (fp32 activations, no Q8_K step)
  *                                     PARITY UNPINNED: taken from the workload
  *                                     description, not from reference source.
+ *   qo_quantize_q8_k, qo_block_sums_q4_k_q8_k, qo_matmul_q4_k_q8_k
+ *                                     the alternative ggml-lineage CPU kernels
+ *                                     compute (activations -> Q8_K, integer
+ *                                     sub-block dots): integer sums pinned by
+ *                                     brute force vs int64 and by the identity
+ *                                     with the fp32 path on exactly
+ *                                     representable activations; the quantiser
+ *                                     by its properties (largest element ->
+ *                                     -127, round-half-even, bsums).  Which of
+ *                                     the two treatments the reference uses is
+ *                                     PARITY UNPINNED (see the line above).
  */
 #include <math.h>
 #include <stdint.h>
@@ -529,6 +540,127 @@ void qo_matmul_q4_0(const float* a, const uint8_t* w_q4, int64_t m, int64_t n, i
     uint8_t* aq = (uint8_t*)malloc((size_t)(m * (k / 32) * 34));
     qo_quantize_q8_0(a, m, k, aq);
     qo_matmul_q4_0_q8_0(aq, w_q4, m, n, k, out);
+    free(aq);
+}
+
+/* ------------------------------------------------------------------ */
+/* Q8_K activations and the integer Q4_K dot (ggml block_q8_K:         */
+/* float d; int8 qs[256]; int16 bsums[16]: 292 bytes)                  */
+/* ------------------------------------------------------------------ */
+
+/* round to nearest, ties to even, through the fp32 adder (ggml nearest_int) */
+static inline int nearest_int(float f) {
+    float v = f + 12582912.f;
+    int i;
+    memcpy(&i, &v, 4);
+    return (i & 0x007fffff) - 0x00400000;
+}
+
+/* ggml quantize_row_q8_K_ref: max = the first element of largest magnitude (signed), iscale = -127 / max,
+ * q = min(127, nearest_int(iscale * x)), d = 1 / iscale, bsums = sums of 16 codes.  An all-zero block has
+ * d = 0, codes 0, bsums 0. */
+void qo_quantize_q8_k(const float* x, int64_t rows, int64_t k, uint8_t* out) {
+    int64_t nb = k / 256;
+    for (int64_t r = 0; r < rows; r++) {
+        for (int64_t b = 0; b < nb; b++) {
+            const float* xb = x + r * k + b * 256;
+            uint8_t* ob = out + (r * nb + b) * 292;
+            int8_t* qs = (int8_t*)(ob + 4);
+            float max = 0.0f, amax = 0.0f;
+            for (int j = 0; j < 256; j++) {
+                float ax = fabsf(xb[j]);
+                if (ax > amax) {
+                    amax = ax;
+                    max = xb[j];
+                }
+            }
+            float d = 0.0f;
+            if (amax == 0.0f) {
+                memset(qs, 0, 256);
+            } else {
+                const float iscale = -127.f / max;
+                for (int j = 0; j < 256; j++) {
+                    int v = nearest_int(iscale * xb[j]);
+                    qs[j] = (int8_t)(v > 127 ? 127 : v);
+                }
+                d = 1.0f / iscale;
+            }
+            memcpy(ob, &d, 4);
+            for (int j = 0; j < 16; j++) {
+                int sum = 0;
+                for (int i = 0; i < 16; i++) sum += qs[j * 16 + i];
+                int16_t s16 = (int16_t)sum;
+                memcpy(ob + 260 + 2 * j, &s16, 2);
+            }
+        }
+    }
+}
+
+/* integer sums of one Q4_K block against one Q8_K block:
+ *   isum = sum_sub sc_sub * sum_32 q4 * q8,   msum = sum_sub mn_sub * (bsums[2 sub] + bsums[2 sub + 1]) */
+static void block_sums_q4_k_q8_k(const uint8_t* wb, const uint8_t* ab, int32_t* isum, int32_t* msum) {
+    uint8_t sc[8], mn[8];
+    qo_unpack_scales_q4_k(wb + 4, sc, mn);
+    const int8_t* q8 = (const int8_t*)(ab + 4);
+    const uint8_t* qs = wb + 16;
+    int32_t is = 0, ms = 0;
+    for (int c = 0; c < 4; c++) {
+        int32_t lo = 0, hi = 0;
+        for (int t = 0; t < 32; t++) {
+            lo += (int)(qs[32 * c + t] & 0xF) * (int)q8[64 * c + t];
+            hi += (int)(qs[32 * c + t] >> 4) * (int)q8[64 * c + 32 + t];
+        }
+        is += (int32_t)sc[2 * c] * lo + (int32_t)sc[2 * c + 1] * hi;
+    }
+    for (int sub = 0; sub < 8; sub++) {
+        int16_t b0, b1;
+        memcpy(&b0, ab + 260 + 4 * sub, 2);
+        memcpy(&b1, ab + 262 + 4 * sub, 2);
+        ms += (int32_t)mn[sub] * ((int32_t)b0 + (int32_t)b1);
+    }
+    *isum = is;
+    *msum = ms;
+}
+
+/* out int32[M, N, K/256] each */
+void qo_block_sums_q4_k_q8_k(const uint8_t* a_q8k, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                             int32_t* isum, int32_t* msum) {
+    int64_t nb = k / 256;
+#pragma omp parallel for schedule(static)
+    for (int64_t j = 0; j < n; j++)
+        for (int64_t i = 0; i < m; i++)
+            for (int64_t b = 0; b < nb; b++)
+                block_sums_q4_k_q8_k(w + (j * nb + b) * 144, a_q8k + (i * nb + b) * 292,
+                                     isum + (i * n + j) * nb + b, msum + (i * n + j) * nb + b);
+}
+
+/* out[m, n] = sum_b (d8 * f32(d)) * isum - (d8 * f32(dmin)) * msum, blocks in ascending order */
+void qo_matmul_q4_k_q8_k(const uint8_t* a_q8k, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out) {
+    int64_t nb = k / 256;
+#pragma omp parallel for schedule(static)
+    for (int64_t j = 0; j < n; j++) {
+        for (int64_t i = 0; i < m; i++) {
+            float acc = 0.0f;
+            for (int64_t b = 0; b < nb; b++) {
+                const uint8_t* wb = w + (j * nb + b) * 144;
+                const uint8_t* ab = a_q8k + (i * nb + b) * 292;
+                int32_t is, ms;
+                block_sums_q4_k_q8_k(wb, ab, &is, &ms);
+                float d8;
+                memcpy(&d8, ab, 4);
+                acc += (d8 * rd_f16(wb)) * (float)is;
+                acc -= (d8 * rd_f16(wb + 2)) * (float)ms;
+            }
+            out[i * n + j] = acc;
+        }
+    }
+}
+
+/* fp32 activations in, quantised to Q8_K on the way */
+void qo_matmul_q4_k_act_q8_k(const float* a, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out) {
+    uint8_t* aq = (uint8_t*)malloc((size_t)(m * (k / 256) * 292));
+    qo_quantize_q8_k(a, m, k, aq);
+    qo_matmul_q4_k_q8_k(aq, w, m, n, k, out);
     free(aq);
 }
 

@@ -252,6 +252,42 @@ def test_q4_k_small_batch_wide_range_lhs(m):
     assert np.all(np.abs(got - truth) <= 1e-4 * scale + 1e-3 * np.abs(truth))
 
 
+# ------------------------------------------------------------------ Q4_K with Q8_K-quantised activations
+def test_quantize_q8_k_bytes_match_oracle():
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((9, 1024)) * rng.uniform(1e-3, 40.0, (9, 1))).astype(np.float32)
+    x[1, 256:512] = 0.0
+    x[2, 3], x[2, 200] = -55.0, 55.0
+    x[2, :256] = np.clip(x[2, :256], -55, 55)
+    x[3, 0], x[3, 1:7] = 127.0, [0.5, 1.5, 2.5, -0.5, -1.5, -2.5]
+    x[3, 7:256] = np.clip(x[3, 7:256], -100, 100)
+    assert np.array_equal(bits(quantize(QE.Q8_K, gpu(x))), O.quantize_q8_k(x))
+
+
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(1, 1000, 4096, False), (4, 300, 4096, False), (2, 129, 14336, True),
+                                            (3, 5000, 512, False), (1, 70, 16384, False), (7, 64, 1024, False),
+                                            (4, 40, 8192, True), (1, 3, 256, False)])
+def test_q4_k_matmul_with_q8_k_activations(m, n, k, lhs_bf16):
+    """The integer-activation treatment against its own oracle, at a tolerance ten times tighter than the parity bar
+    (only fp32 summation order differs); and it is not the floating-point treatment."""
+    w, a = synth(71, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_q4_k_act_q8_k(a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a)
+    got = qmatmul(QE.Q4_K, None, lhs, gpu(wq), act_q8k=True).cpu().numpy()
+    assert O.isclose(got, want, 1e-4, 1e-5).all(), f"max abs err {np.abs(got - want).max()}"
+    if n * m >= 64 and k >= 1024:
+        assert not O.isclose(got, O.matmul_f32(O.Q4_K, a, wq), 1e-4, 1e-5).all()
+
+
+def test_q8_k_activations_only_for_q4_k():
+    w, a = synth(72, 8, 256, 1)
+    with pytest.raises(NotImplementedError):
+        qmatmul(QE.Q6_K, None, gpu(a), gpu(O.quantize(O.Q6_K, w)), act_q8k=True)
+
+
 # ------------------------------------------------------------------ matrices that share their lhs
 @pytest.mark.parametrize("enc,m,k,ns,lhs_bf16", [(QE.Q4_K, 1, 4096, (512, 130, 130), False), (QE.Q4_K, 1, 14336, (300, 77), True),
                                                  (QE.Q4_K, 1, 512, (9000, 1, 17, 4100), False),
