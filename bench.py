@@ -380,6 +380,13 @@ def extra_timings(layers, acts, gen):
         dev_s, _ = time_graphs(graphs, 100, 10)
         sb = sum(alg_bytes(QE.Q4_K, mm, nn, kk) for _, nn, kk in PROJ)
         out[f"q4_k_act_q8k_m{mm}"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sb * 100 / dev_s / 1e9, 1)}
+    # M = 4 with the shared-lhs projections grouped, as above
+    a4g = {kk: torch.randn((4, kk), dtype=torch.float32, device="cuda:0", generator=gen) for kk in (4096, 14336)}
+    graphs = [capture([GroupedGemv(QE.Q4_K, lw[0:3], a4g[4096]), Gemv(QE.Q4_K, lw[3], a4g[4096]),
+                       GroupedGemv(QE.Q4_K, lw[4:6], a4g[4096]), Gemv(QE.Q4_K, lw[6], a4g[14336])]) for lw in layers]
+    dev_s, _ = time_graphs(graphs, 100, 10)
+    sb4 = sum(alg_bytes(QE.Q4_K, 4, nn, kk) for _, nn, kk in PROJ)
+    out["q4_k_m4_grouped_4_launches"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sb4 * 100 / dev_s / 1e9, 1)}
     # M=4 over the same set
     if m == 1:
         acts4 = {k: torch.randn((4, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}

@@ -132,8 +132,8 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
  * Several GGUF weight matrices applied to one lhs, as the callers of ops.qmatmul in a transformer
  * block do (q | k | v, and gate | up, take the same activations):
  *   out[j] fp32[m, n[j]] = lhs[m, k] . dequant(rhs[j])^T,  j < count, all rhs of `encoding` and of row length k.
- * Where a kernel takes the whole group (Q4_K, m = 1, count <= 4, k <= 16384) this is one launch that
- * numbers the rows of the matrices through; otherwise it is one qmm_matmul per matrix, in order
+ * Where a kernel takes the whole group (Q4_K, count <= 4: m = 1 with k <= 16384, or 2 <= m <= 16) this is one
+ * launch that numbers the rows of the matrices through (the lhs is staged or narrowed once for all of them); otherwise it is one qmm_matmul per matrix, in order
  * (workspace: the largest any of them needs).  The reference exposes the per-matrix op only; fusing
  * its calls is its graph compiler's job, for which this is the kernel-side counterpart.
  * rhs, n and out are host arrays.

@@ -67,11 +67,11 @@ __device__ __forceinline__ half8 zero_half8() { return pack4(0u, 0u, 0u, 0u); }
 // inv come from prep_lhs_kernel<.., kLhsOrderQ4K16>.
 // MROWS (INLINE): lhs rows converted, 1, 2, 4 or 8 (>= m; rows past m repeat the last one and their results are dropped).
 template <int NPART, bool INLINE, int MROWS, typename AT>
-__global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+__global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, const AT* __restrict__ a,
                                                            const _Float16* __restrict__ a16,
                                                            const _Float16* __restrict__ a16_lo,
                                                            const _Float16* __restrict__ asum, const float* __restrict__ inv,
-                                                           float* __restrict__ out, int m, int n, int k) {
+                                                           int m, int k) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
     uint8_t* ring = smem + wave * (kSlots * kSlotBytes);
     const uint32_t ring_lds = lds_address(ring);
     float* accs = (float*)(smem + kRingBytes);  // [kWaves][kMaxTiles][4][64]
-    const int ntiles = (n + 15) >> 4;
+    const int ntiles = mats.tile_end[mats.count - 1];  // 16-row tiles, numbered through the matrices
     const int my_tiles = min(kMaxTiles, (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
     // group g is super-blocks [16 g, 16 g + 16): two per wavefront, or, when 8 or fewer are left, one
     const int ngrp = (nblk + kRunBlk * kWaves - 1) / (kRunBlk * kWaves);
@@ -104,11 +104,14 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
     }
     // item (group g, tile index t) -> ring slot `slot`
     auto issue = [&](int g, int t, int slot) {
-        const int n0 = ((int)blockIdx.x + t * (int)gridDim.x) * 16;
+        const int tile = (int)blockIdx.x + t * (int)gridDim.x;
+        int j = 0;
+        while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;  // (uniform: a few scalar compares)
+        const int n0 = (tile - (j ? mats.tile_end[j - 1] : 0)) * 16, n = mats.n[j];
         int bc, cnt;
         group_share(g, bc, cnt);
         const int last_piece = max(cnt, 1) * 9 - 1;
-        const uint8_t* base = w + (int64_t)bc * Q4_K_BPB;
+        const uint8_t* base = mats.w[j] + (int64_t)bc * Q4_K_BPB;
 #pragma unroll
         for (int i = 0; i < kLoads; i++) {
             const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * min(pidx[i], last_piece);
@@ -356,7 +359,12 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const uint8_t* __rest
     // lane holds lhs rows 4 kg + r of weight row 16 tile + nn; (tile, r) pairs are dealt to the wavefronts
     for (int pr = wave; pr < my_tiles * 4; pr += kWaves) {
         const int t = pr >> 2, r = pr & 3;
-        const int col = ((int)blockIdx.x + t * (int)gridDim.x) * 16 + nn, row = 4 * kg + r;
+        const int tile = (int)blockIdx.x + t * (int)gridDim.x;
+        int j = 0;
+        while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;
+        const int n = mats.n[j];
+        float* out = mats.out[j];
+        const int col = (tile - (j ? mats.tile_end[j - 1] : 0)) * 16 + nn, row = 4 * kg + r;
         float v = 0.0f;
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) {
@@ -371,8 +379,21 @@ int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) {
     return m <= 8 ? 0 : lhs_planes(nullptr, lhs_dtype, m, k).bytes;
 }
 
-hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
-                               float* out, void* workspace, hipStream_t s) {
+// count matrices [ns[j], k] that share the lhs (count = 1: the plain call); out[j] is fp32 [m, ns[j]], dense.
+hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
+                                       float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s) {
+    if (count < 1 || count > kLanesMaxMats) return hipErrorInvalidValue;
+    MmMats mats;
+    int64_t ntiles = 0;
+    for (int j = 0; j < kLanesMaxMats; j++) {
+        const int jj = j < count ? j : count - 1;
+        if (j < count) ntiles += (ns[j] + 15) / 16;
+        mats.w[j] = ws[jj];
+        mats.out[j] = outs[jj];
+        mats.n[j] = (int)ns[jj];
+        mats.tile_end[j] = (int)ntiles;
+    }
+    mats.count = count;
     static int cus = 0;
     if (!cus) {
         int dev = 0;
@@ -394,7 +415,6 @@ hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w,
         }
         lds_set = true;
     }
-    const int64_t ntiles = (n + 15) / 16;
     // every workgroup gets the same number of tiles (at most kMaxTiles), one workgroup per compute unit when that fits
     const int64_t per_wg = std::min<int64_t>(kMaxTiles, (ntiles + cus - 1) / cus);
     const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
@@ -404,10 +424,10 @@ hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w,
     do {                                                                                                              \
         if (lhs_dtype == QMM_F32)                                                                                     \
             gemv_q4_k_mm_kernel<1, true, MR_, float><<<grid, block, kLdsBytes, s>>>(                                  \
-                w, (const float*)lhs, nullptr, nullptr, nullptr, nullptr, out, (int)m, (int)n, (int)k);               \
+                mats, (const float*)lhs, nullptr, nullptr, nullptr, nullptr, (int)m, (int)k);                         \
         else                                                                                                          \
             gemv_q4_k_mm_kernel<1, true, MR_, uint16_t><<<grid, block, kLdsBytes, s>>>(                               \
-                w, (const uint16_t*)lhs, nullptr, nullptr, nullptr, nullptr, out, (int)m, (int)n, (int)k);            \
+                mats, (const uint16_t*)lhs, nullptr, nullptr, nullptr, nullptr, (int)m, (int)k);                      \
     } while (0)
         if (m == 1) QMM_MM_INLINE(1);
         else if (m == 2) QMM_MM_INLINE(2);
@@ -420,12 +440,15 @@ hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w,
     e = launch_prep_lhs<kLhsOrderQ4K16>(lhs, lhs_dtype, m, k, p, s);
     if (e != hipSuccess) return e;
     if (!p.a16_lo)
-        gemv_q4_k_mm_kernel<1, false, 1, float><<<grid, block, kLdsBytes, s>>>(w, nullptr, p.a16, nullptr, p.asum, p.inv, out, (int)m,
-                                                                           (int)n, (int)k);
+        gemv_q4_k_mm_kernel<1, false, 1, float><<<grid, block, kLdsBytes, s>>>(mats, nullptr, p.a16, nullptr, p.asum, p.inv, (int)m, (int)k);
     else
-        gemv_q4_k_mm_kernel<2, false, 1, float><<<grid, block, kLdsBytes, s>>>(w, nullptr, p.a16, p.a16_lo, p.asum, p.inv, out, (int)m,
-                                                                           (int)n, (int)k);
+        gemv_q4_k_mm_kernel<2, false, 1, float><<<grid, block, kLdsBytes, s>>>(mats, nullptr, p.a16, p.a16_lo, p.asum, p.inv, (int)m, (int)k);
     return hipGetLastError();
+}
+
+hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                               float* out, void* workspace, hipStream_t s) {
+    return launch_gemv_q4_k_mm_grouped(lhs, lhs_dtype, 1, &w, &n, &out, m, k, workspace, s);
 }
 
 }  // namespace qmm

@@ -290,7 +290,7 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
         return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: encoding %d is not a GGUF weight encoding", encoding);
     for (int j = 0; j < count; j++)
         if (!rhs[j] || !out[j] || n[j] <= 0) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: matrix %d: null pointer or N <= 0", j);
-    if (encoding == QMM_Q4_K && m == 1 && k > 0 && k % 256 == 0 && count <= qmm::kLanesMaxMats &&
+    if (encoding == QMM_Q4_K && m >= 1 && m <= 16 && k > 0 && k % 256 == 0 && count <= qmm::kLanesMaxMats &&
         (lhs_dtype == QMM_F32 || lhs_dtype == QMM_BF16) && aligned(lhs, 16)) {
         bool ok = true;
         int64_t total = 0;
@@ -300,11 +300,21 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
             total += n[j];
             ws[j] = (const uint8_t*)rhs[j];
         }
-        if (ok && total <= INT32_MAX) {
+        if (ok && total <= INT32_MAX && m == 1) {
             bool handled = false;
             hipError_t e = qmm::launch_gemv_q4_k_lanes_grouped(lhs, lhs_dtype, count, ws, n, out, 1, k, 0, (hipStream_t)stream, &handled);
             if (e != hipSuccess) return hip_status(e, "qmm_matmul_grouped(Q4_K decode)");
             if (handled) return QMM_OK;
+        }
+        if (ok && total <= INT32_MAX && m >= env_q4k_mm_min_m() && !env_flag_qmm_q4k_small_gemv()) {
+            // the lhs is narrowed once (in the kernel up to 8 rows, by the separate pass beyond) for all the matrices
+            const int64_t need = qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);
+            if (need > 0 && (!workspace || workspace_bytes < need))
+                return fail(QMM_ERR_WORKSPACE, "qmm_matmul_grouped: workspace of %lld bytes required, %lld given", (long long)need,
+                            (long long)workspace_bytes);
+            if (need > 0 && !aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_grouped: workspace must be 256-byte aligned");
+            return hip_status(qmm::launch_gemv_q4_k_mm_grouped(lhs, lhs_dtype, count, ws, n, out, m, k, workspace, (hipStream_t)stream),
+                              "qmm_matmul_grouped(Q4_K small batch)");
         }
     }
     for (int j = 0; j < count; j++) {

@@ -51,6 +51,16 @@ struct LanesMats {
     int end[kLanesMaxMats];  // running row count: matrix j owns rows [end[j - 1], end[j])
     int count;
 };
+// The same for the small-batch matrix-core kernel: 16-row tiles are numbered through the matrices.
+struct MmMats {
+    const uint8_t* w[kLanesMaxMats];
+    float* out[kLanesMaxMats];
+    int tile_end[kLanesMaxMats];  // running tile count: matrix j owns tiles [tile_end[j - 1], tile_end[j])
+    int n[kLanesMaxMats];
+    int count;
+};
+hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
+                                       float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s);
 hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
                                           float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled);
 hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,

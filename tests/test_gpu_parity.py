@@ -291,10 +291,12 @@ def test_q8_k_activations_only_for_q4_k():
 # ------------------------------------------------------------------ matrices that share their lhs
 @pytest.mark.parametrize("enc,m,k,ns,lhs_bf16", [(QE.Q4_K, 1, 4096, (512, 130, 130), False), (QE.Q4_K, 1, 14336, (300, 77), True),
                                                  (QE.Q4_K, 1, 512, (9000, 1, 17, 4100), False),
-                                                 (QE.Q4_K, 3, 1024, (64, 200), False), (QE.Q6_K, 1, 1024, (96, 40), False),
+                                                 (QE.Q4_K, 3, 1024, (64, 200), False), (QE.Q4_K, 4, 4096, (4100, 130, 130), False),
+                                                 (QE.Q4_K, 8, 2304, (20, 33, 7, 50), True), (QE.Q4_K, 12, 512, (300, 17), False),
+                                                 (QE.Q6_K, 1, 1024, (96, 40), False),
                                                  (QE.Q4_0, 2, 256, (33, 64, 5), False), (QE.Q4_K, 1, 256, (8, 8, 8, 8, 8), False)])
 def test_grouped_matmul_equals_separate_calls(enc, m, k, ns, lhs_bf16):
-    """q | k | v and gate | up style groups: the one-launch path (Q4_K, one lhs row, up to four matrices) and the
+    """q | k | v and gate | up style groups: the one-launch paths (Q4_K, up to four matrices, 1..16 lhs rows) and the
     per-matrix path give what qmatmul gives on each matrix, bit for bit, and agree with the oracle."""
     ws, a = [], None
     for j, n in enumerate(ns):
