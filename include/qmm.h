@@ -58,7 +58,7 @@ typedef struct qmm_gptq_config {
     int32_t bits;       /* 4                                      */
     int32_t group_size; /* 128 (any multiple of 32 dividing K)    */
     int32_t desc_act;   /* 0: g_idx[k] = k / group_size           */
-    int32_t sym;        /* 1: stored zero-point 7 (true zero 8)   */
+    int32_t sym;        /* 1: stored zero-point 7 (true zero 8); 0: any stored zero-point (true zero = stored + 1) */
 } qmm_gptq_config;
 
 int qmm_version(void);

@@ -54,11 +54,13 @@ bool block_params(int enc, int64_t& epb, int64_t& bpb) {
 
 int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
-int check_gptq(const qmm_gptq_config* cfg, int64_t n, int64_t k) {
+// sym = 0 (asymmetric checkpoints: zero points other than 8) is read like sym = 1: every kernel takes the zero
+// point from qzeros (stored value + 1, the AutoGPTQ v1 convention); only the quantiser here is symmetric.
+int check_gptq(const qmm_gptq_config* cfg, int64_t n, int64_t k, bool quantiser = false) {
     if (!cfg) return fail(QMM_ERR_INVALID, "GPTQ requires a config");
     if (cfg->bits != 4) return fail(QMM_ERR_UNSUPPORTED, "GPTQ bits=%d: only 4-bit is supported", cfg->bits);
     if (cfg->desc_act) return fail(QMM_ERR_UNSUPPORTED, "GPTQ desc_act=True is not supported");
-    if (!cfg->sym) return fail(QMM_ERR_UNSUPPORTED, "GPTQ sym=False is not supported");
+    if (!cfg->sym && quantiser) return fail(QMM_ERR_UNSUPPORTED, "GPTQ sym=False: the quantiser here is symmetric only");
     if (cfg->group_size <= 0 || cfg->group_size % 32 || k % cfg->group_size)
         return fail(QMM_ERR_INVALID, "GPTQ group_size=%d must be a multiple of 32 dividing K=%lld", cfg->group_size,
                     (long long)k);
@@ -162,7 +164,7 @@ int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int
                       void* qzeros, void* g_idx, void* stream) {
     if (!w || !qweight || !scales || !qzeros || !g_idx) return fail(QMM_ERR_INVALID, "qmm_quantize_gptq: null pointer");
     if (n <= 0 || k <= 0) return fail(QMM_ERR_INVALID, "qmm_quantize_gptq: empty shape");
-    if (int rc = check_gptq(cfg, n, k)) return rc;
+    if (int rc = check_gptq(cfg, n, k, true)) return rc;
     return hip_status(
         qmm::launch_quantize_gptq(w, n, k, cfg->group_size, qweight, scales, qzeros, g_idx, (hipStream_t)stream),
         "qmm_quantize_gptq");

@@ -101,6 +101,24 @@ def test_dequantize_gptq_bit_exact():
     assert np.array_equal(bits(got), want.view(np.uint8).reshape(128, -1))
 
 
+@pytest.mark.parametrize("m", [1, 4, 64])
+def test_gptq_asymmetric_checkpoint(m):
+    """sym=False: zero points other than 8 in qzeros (stored value + 1), through dequantize and every matmul kernel."""
+    n, k, group = 128, 1024, 128
+    w, a = synth(25, n, k, m)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    rng = np.random.Generator(np.random.PCG64(26))
+    qz = rng.integers(0, 2**32, size=qz.shape, dtype=np.uint64).astype(np.uint32).view(np.int32)
+    cfg = QuantizationConfig(group_size=group, sym=False)
+    want_w = O.dequantize_gptq(qw, sc, qz, group)
+    got_w = dequantize(QE.GPTQ, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), config=cfg)
+    assert np.array_equal(bits(got_w), want_w.view(np.uint8).reshape(n, -1))
+    truth = O.matmul_gptq(a, qw, sc, qz, group, f64=True)
+    got = qmatmul(QE.GPTQ, cfg, gpu(a), gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, truth, f"asymmetric GPTQ m={m}")
+
+
 # ------------------------------------------------------------------ Q4_0: integer dots and matmul
 def test_block_dots_bit_exact():
     w, a = synth(0, 256, 1024, 4)
