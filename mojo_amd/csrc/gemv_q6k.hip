@@ -16,6 +16,7 @@
 // 16 KB row stays resident), which keeps the LDS pipe for the weights.
 #include <stdlib.h>
 
+#include "lds_stream.h"
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -338,6 +339,112 @@ static size_t q6k_rows_lds(int mt, int64_t k) {
     return b <= 96 * 1024 ? b : 0;
 }
 
+// One lhs row, rows of 8 or 16 super-blocks (K = 2048 or 4096: then every row is 16-byte aligned): the
+// decode of the slab kernel above with the alignment worked out at compile time and the rows delivered
+// global -> LDS directly.  Group bq = lane / 16 takes super-blocks 4 bq + it, it = 0..3, so a super-block
+// starts at 840 bq + 210 it bytes of the row: 4-byte aligned for even `it` (fields are plain dword reads),
+// 2 bytes off for odd `it` (two dwords joined at a fixed byte offset).  A wavefront walks its rows
+// (persistent) with a private ring of three LDS slots, two rows in flight (global_load_lds_dwordx4, hidden
+// from the compiler, exact vmcnt waits: lds_stream.h); no registers are spent on staging.
+// L: load instructions per row (64 pieces of 16 bytes each): 4 for 16 super-blocks, 2 for 8.
+template <int L, typename AT>
+__global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                              float* __restrict__ out, int n, int k, int ring_slots) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nblk = k >> 8;                       // 8 or 16
+    const int64_t row_bytes = (int64_t)nblk * Q6_K_BPB;
+    const int pieces = (int)(row_bytes / 16);      // 105 or 210
+    const int kSlot = pieces * 16 + 16;            // one dword of read-ahead past the last block
+    uint8_t* ring = smem + wave * (ring_slots * kSlot);
+    const uint32_t ring_lds = lds_address(ring);
+    float* park = (float*)(smem + 4 * ring_slots * kSlot) + wave * kParkRows;
+    const int total_waves = (int)gridDim.x * 4, gw = (int)blockIdx.x * 4 + wave;
+    const int my_rows = gw < n ? (n - gw + total_waves - 1) / total_waves : 0;
+    const int bq = lane >> 4, t = lane & 15, h = t >> 3, j = t & 7;
+    const int sc_shift = 8 * (j >> 2);
+
+    // this lane's activations: per super-block slot `it`, four quartets at columns 128 h + 4 j + {0, 32, 64, 96};
+    // and -32 times the sum of one 16-column group per lane (group t of the super-block)
+    float4 x[4][4];
+    float os[4], lv[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int bl = 4 * bq + it;
+        lv[it] = bl < nblk ? 1.0f : 0.0f;
+        const int blc = min(bl, nblk - 1);
+        const AT* ar = a + blc * 256;
+        const AT* aq = ar + 128 * h + 4 * j;
+        x[it][0] = load4(aq, 0);
+        x[it][1] = load4(aq, 32);
+        x[it][2] = load4(aq, 64);
+        x[it][3] = load4(aq, 96);
+        const AT* ag = ar + 16 * t;
+        const float4 y0 = load4(ag, 0), y1 = load4(ag, 4), y2 = load4(ag, 8), y3 = load4(ag, 12);
+        os[it] = -32.0f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
+                           ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
+    }
+    // (the loads above are ordinary ones, finished before the first hidden load is issued: the sums depend on them)
+    float keep = os[0] + os[1] + os[2] + os[3];
+    asm volatile("" : "+v"(keep));
+
+    auto issue = [&](int ri, int slot) {
+        const uint8_t* base = w + (int64_t)(gw + (int64_t)ri * total_waves) * row_bytes;
+#pragma unroll
+        for (int i = 0; i < L; i++)
+            if (lane + 64 * i < pieces) load16_to_lds(base + 16 * (lane + 64 * i), ring_lds + slot * kSlot + i * 1024);
+    };
+    int issued = 0, islot = 0, cslot = 0;
+    for (; issued < min(ring_slots - 1, my_rows); issued++) {
+        issue(issued, islot);
+        islot = islot + 1 == ring_slots ? 0 : islot + 1;
+    }
+    // dword offsets of this lane's fields inside a super-block
+    const int o_ql = 16 * h + j, o_qh = 32 + 8 * h + j, o_sc = 48 + 2 * h;
+    for (int ri = 0; ri < my_rows; ri++) {
+        if (issued < my_rows) {
+            issue(issued, islot);
+            islot = islot + 1 == ring_slots ? 0 : islot + 1;
+            issued++;
+        }
+        wait_items<L, 0>(issued - 1 - ri, false);
+        // super-block 4 bq: byte 840 bq (groups past the row read the last group's blocks again; their lv is 0)
+        const uint32_t* l32 = (const uint32_t*)(ring + cslot * kSlot) + 210 * min(bq, nblk / 4 - 1);
+        cslot = cslot + 1 == ring_slots ? 0 : cslot + 1;
+        float v = 0.0f;
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            constexpr int kDummy = 0;
+            (void)kDummy;
+            const int q0 = (Q6_K_BPB * it) >> 2;              // dword of the super-block's first (aligned) byte
+            const bool odd = ((Q6_K_BPB * it) & 3) != 0;      // compile-time: it = 1, 3 start 2 bytes into that dword
+            auto rd = [&](int dw) {
+                return odd ? __builtin_amdgcn_alignbyte(l32[q0 + dw + 1], l32[q0 + dw], 2u) : l32[q0 + dw];
+            };
+            const uint32_t A = rd(o_ql), B = rd(o_ql + 8), H = rd(o_qh);
+            const uint32_t s0 = rd(o_sc), s1 = rd(o_sc + 1);
+            const uint32_t dv = odd ? l32[q0 + 52] >> 16 : l32[q0 + 52] & 0xffffu;
+            const float d = h2f((uint16_t)dv) * lv[it];
+            const uint32_t q1 = (A & 0x0F0F0F0Fu) | ((H << 4) & 0x30303030u);
+            const uint32_t q2 = (B & 0x0F0F0F0Fu) | ((H << 2) & 0x30303030u);
+            const uint32_t q3 = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
+            const uint32_t q4 = ((B >> 4) & 0x0F0F0F0Fu) | ((H >> 2) & 0x30303030u);
+            // the int8 scales of the four quartets and of this lane's 16-column group; d once at the end
+            float u = sbyte(s0, sc_shift) * dot4u(x[it][0], q1);
+            u = fmaf(sbyte(s0, sc_shift + 16), dot4u(x[it][1], q2), u);
+            u = fmaf(sbyte(s1, sc_shift), dot4u(x[it][2], q3), u);
+            u = fmaf(sbyte(s1, sc_shift + 16), dot4u(x[it][3], q4), u);
+            u = fmaf(sbyte(j < 4 ? s0 : s1, 8 * (j & 3)), os[it], u);
+            v = fmaf(d, u, v);
+        }
+        const float sum = wave_sum_dpp(v);
+        if (lane == 0) park[ri] = sum;
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int i = lane; i < my_rows; i += 64) out[gw + (int64_t)i * total_waves] = park[i];
+}
+
 hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s, bool* handled) {
     *handled = false;
@@ -354,6 +461,27 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     // loop-interchanged kernel; otherwise the row-at-a-time kernel below.
     static const int pc_env = getenv("QMM_Q6K_WG_PER_CU") ? atoi(getenv("QMM_Q6K_WG_PER_CU")) : 0;
     const int pc = pc_env > 0 ? pc_env : 3;
+    static const bool lanes_off = getenv("QMM_Q6K_LANES_OFF") != nullptr;  // read once: fallback switch
+    if (m == 1 && (k == 2048 || k == 4096) && !((uintptr_t)w & 15) && n >= (int64_t)cus * pc * 4 * 4 && !lanes_off &&
+        !env_flag_qmm_q6k_rows()) {
+        const int ring = 3;
+        const size_t slot = (size_t)(k / 256) * Q6_K_BPB + 16;
+        const size_t lds3 = 4 * ring * slot + 4 * (size_t)kParkRows * 4;
+        const int64_t wgs = max((int64_t)cus * pc, (n + 4 * kParkRows - 1) / (4 * kParkRows));
+        dim3 grid3((unsigned)min(wgs, (n + 3) / 4)), block3(256);
+#define QMM_Q6K_LANES(L_)                                                                                             \
+    do {                                                                                                              \
+        if (a_dtype == QMM_F32)                                                                                       \
+            gemv_q6_k_lanes_kernel<L_, float><<<grid3, block3, lds3, s>>>(w, (const float*)a, out, (int)n, (int)k, ring); \
+        else                                                                                                          \
+            gemv_q6_k_lanes_kernel<L_, uint16_t><<<grid3, block3, lds3, s>>>(w, (const uint16_t*)a, out, (int)n, (int)k, ring); \
+    } while (0)
+        if (k == 4096) QMM_Q6K_LANES(4);
+        else QMM_Q6K_LANES(2);
+#undef QMM_Q6K_LANES
+        *handled = true;
+        return hipGetLastError();
+    }
     if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !env_flag_qmm_q6k_rows()) {
         const size_t lds2 = 4 * (size_t)kRunBytes + 4 * (size_t)kParkRows * 4;
         // enough wavefronts that none has more rows than its LDS parking slots
