@@ -365,6 +365,18 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
     const int bq = lane >> 4, t = lane & 15, h = t >> 3, j = t & 7;
     const int sc_shift = 8 * (j >> 2);
 
+    // the first rows are requested before the activations, so that their latencies overlap
+    auto issue = [&](int ri, int slot) {
+        const uint8_t* base = w + (int64_t)(gw + (int64_t)ri * total_waves) * row_bytes;
+#pragma unroll
+        for (int i = 0; i < L; i++)
+            if (lane + 64 * i < pieces) load16_to_lds(base + 16 * (lane + 64 * i), ring_lds + slot * kSlot + i * 1024);
+    };
+    int issued = 0, islot = 0, cslot = 0;
+    for (; issued < min(ring_slots - 1, my_rows); issued++) {
+        issue(issued, islot);
+        islot = islot + 1 == ring_slots ? 0 : islot + 1;
+    }
     // this lane's activations: per super-block slot `it`, four quartets at columns 128 h + 4 j + {0, 32, 64, 96};
     // and -32 times the sum of one 16-column group per lane (group t of the super-block)
     float4 x[4][4];
@@ -385,21 +397,11 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
         os[it] = -32.0f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
                            ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
     }
-    // (the loads above are ordinary ones, finished before the first hidden load is issued: the sums depend on them)
+    // (ordinary loads, younger than the rows requested above: the wait for them also covers those rows, and it
+    // is forced here, before the loop, so that no wait of the compiler's lands between the counted ones)
     float keep = os[0] + os[1] + os[2] + os[3];
     asm volatile("" : "+v"(keep));
 
-    auto issue = [&](int ri, int slot) {
-        const uint8_t* base = w + (int64_t)(gw + (int64_t)ri * total_waves) * row_bytes;
-#pragma unroll
-        for (int i = 0; i < L; i++)
-            if (lane + 64 * i < pieces) load16_to_lds(base + 16 * (lane + 64 * i), ring_lds + slot * kSlot + i * 1024);
-    };
-    int issued = 0, islot = 0, cslot = 0;
-    for (; issued < min(ring_slots - 1, my_rows); issued++) {
-        issue(issued, islot);
-        islot = islot + 1 == ring_slots ? 0 : islot + 1;
-    }
     // dword offsets of this lane's fields inside a super-block
     const int o_ql = 16 * h + j, o_qh = 32 + 8 * h + j, o_sc = 48 + 2 * h;
     for (int ri = 0; ri < my_rows; ri++) {
@@ -415,8 +417,6 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
         float v = 0.0f;
 #pragma unroll
         for (int it = 0; it < 4; it++) {
-            constexpr int kDummy = 0;
-            (void)kDummy;
             const int q0 = (Q6_K_BPB * it) >> 2;              // dword of the super-block's first (aligned) byte
             const bool odd = ((Q6_K_BPB * it) & 3) != 0;      // compile-time: it = 1, 3 start 2 bytes into that dword
             auto rd = [&](int dw) {
