@@ -361,6 +361,11 @@ def extra_timings(layers, acts, gen):
         b = alg_bytes(QE.Q4_K, m, n, k)
         per_shape[f"{name}_{n}x{k}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1)}
     out["q4_k_per_shape"] = per_shape
+    # warm cache, labelled as such: one layer (123 MB, inside the 256 MB last-level cache) replayed by itself
+    g = capture([Gemv(QE.Q4_K, w, acts[k]) for w, (_, n, k) in zip(layers[0], PROJ)])
+    dev_s, _ = time_graphs([g], 100, 10)
+    sbw = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
+    out["q4_k_warm_cache_one_layer"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sbw * 100 / dev_s / 1e9, 1)}
     # the same seven weight tensors per layer, only read (no arithmetic): what the memory system gives
     graphs = [capture([ReadProbe(w) for w in lw]) for lw in layers]
     dev_s, _ = time_graphs(graphs, 100, 10)

@@ -57,7 +57,8 @@ enum qmm_status {
 typedef struct qmm_gptq_config {
     int32_t bits;       /* 4                                      */
     int32_t group_size; /* 128 (any multiple of 32 dividing K)    */
-    int32_t desc_act;   /* 0: g_idx[k] = k / group_size           */
+    int32_t desc_act;   /* 0: the group of k is k / group_size (g_idx is not read); 1: act-order checkpoint, the
+                           group of k is g_idx[k] (required; any order, values in [0, K / group_size))       */
     int32_t sym;        /* 1: stored zero-point 7 (true zero 8); 0: any stored zero-point (true zero = stored + 1) */
 } qmm_gptq_config;
 
@@ -89,7 +90,7 @@ int qmm_read_probe(const void* buf, int64_t bytes, void* stream);
 int qmm_dequantize(int encoding, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
                    void* stream);
 
-/* GPTQ tensors -> out[n, k] (the transposed, GGUF-like orientation). */
+/* GPTQ tensors -> out[n, k] (the transposed, GGUF-like orientation).  g_idx may be null when cfg->desc_act is 0. */
 int qmm_dequantize_gptq(const qmm_gptq_config* cfg, const void* qweight, const void* scales,
                         const void* qzeros, const void* g_idx, int64_t n, int64_t k, void* out,
                         int out_dtype, void* stream);
@@ -113,6 +114,8 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
  *   encoding Q4_0/Q4_K/Q6_K: n_rhs = 1, rhs[0] = uint8[n, k/epb*bpb];
  *   encoding GPTQ: cfg required, n_rhs = 3 or 4,
  *     rhs = {qweight i32[k/8, n], scales f16[k/g, n], qzeros i32[k/g, n/8], g_idx i32[k]}.
+ *     cfg->desc_act = 1 (n_rhs = 4) goes through a decode-shaped kernel for every m, four lhs rows per
+ *     pass over the weights; the matrix-core kernel takes plain groups only.
  *   lhs_dtype QMM_F32 or QMM_BF16.  Q4_0 quantises lhs rows to Q8_0 and takes
  *   integer block dots (the reference CPU path); the others keep lhs as given.
  *   flags: bit 0 (QMM_FLAG_W_BF16) rounds dequantised weights to bf16 before

@@ -146,4 +146,113 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Act-order checkpoints (desc_act = True): g_idx[k] names the group of every k, in no particular order,
+// so the scale and the zero point change from one k to the next.  Same lane-per-column shape as above;
+// the 64 columns' (scale, -scale * zero) pairs of every group sit in LDS (TABLE; read from global memory
+// when they do not fit), g_idx and the activations are read with wave-uniform addresses, and a weight
+// is fma(scale, q, -scale * zero): both products and their difference are exact in fp32.
+// Group indices outside [0, K / group) are clamped (the result is then meaningless, nothing is read
+// out of bounds).
+// ---------------------------------------------------------------------------
+template <int MT, bool TABLE, typename AT>
+__global__ __launch_bounds__(64 * kWaves) void gemv_gptq_act_order_kernel(
+    const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
+    const int32_t* __restrict__ g_idx, const AT* __restrict__ a, float* __restrict__ out, int m, int n, int k, int group,
+    int64_t ldo) {
+    extern __shared__ __attribute__((aligned(16))) float gsm[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ngroups = k / group;
+    float2* table = (float2*)gsm;                          // [ngroups][64]
+    float* red = gsm + (TABLE ? 2 * 64 * ngroups : 0);     // [kWaves][MT][64]
+    const int col = (int)blockIdx.x * 64 + lane;
+    const int ccol = min(col, n - 1);
+    const int zshift = 4 * (ccol & 7);
+    auto pair_of = [&](int g) {
+        const float sc = h2f(scales[(int64_t)g * n + ccol]);
+        const float z = (float)(((qzeros[(int64_t)g * (n >> 3) + (ccol >> 3)] >> zshift) & 0xFu) + 1u);
+        return make_float2(sc, -sc * z);
+    };
+    if constexpr (TABLE) {
+        for (int g = wave; g < ngroups; g += kWaves) table[g * 64 + lane] = pair_of(g);
+        __syncthreads();
+    }
+    float acc[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
+    // wavefront w walks the k8 rows [w * per, (w + 1) * per), four rows of loads at a time (K / 8 is a multiple of 4)
+    constexpr int U = 4;
+    const int rows = k >> 3;
+    const int per = ((rows + kWaves - 1) / kWaves + U - 1) / U * U;
+    const int r_end = min(rows, (wave + 1) * per);
+    for (int r = wave * per; r < r_end; r += U) {
+        uint32_t x[U];
+#pragma unroll
+        for (int j = 0; j < U; j++) x[j] = (qweight + (int64_t)(r + j) * n)[ccol];
+#pragma unroll
+        for (int j = 0; j < U; j++) {
+            const int k0 = (r + j) * 8;
+            const uint32_t qe = x[j] & 0x0F0F0F0Fu, qo = (x[j] >> 4) & 0x0F0F0F0Fu;  // k 0,2,4,6 / k 1,3,5,7
+            const float q[8] = {gub0(qe), gub0(qo), gub1(qe), gub1(qo), gub2(qe), gub2(qo), gub3(qe), gub3(qo)};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int g = min(max(g_idx[k0 + i], 0), ngroups - 1);  // wave-uniform
+                const float2 sz = TABLE ? table[g * 64 + lane] : pair_of(g);
+                const float w = fmaf(sz.x, q[i], sz.y);
+#pragma unroll
+                for (int mi = 0; mi < MT; mi++)
+                    acc[mi] = fmaf(w, act(a + (int64_t)(mi < m ? mi : 0) * k, k0 + i), acc[mi]);
+            }
+        }
+    }
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) red[(wave * MT + mi) * 64 + lane] = acc[mi];
+    __syncthreads();
+    if (wave == 0 && col < n) {
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            if (mi < m) {
+                float v = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; w++) v += red[(w * MT + mi) * 64 + lane];
+                out[(int64_t)mi * ldo + col] = v;
+            }
+        }
+    }
+}
+
+// m <= 4 lhs rows; K % 32 == 0 and N % 8 == 0 are the caller's checks.
+hipError_t launch_gemv_gptq_act_order(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
+                                      const uint32_t* qzeros, const int32_t* g_idx, int m, int64_t n, int64_t k, int group,
+                                      float* out, int64_t ldo, hipStream_t s) {
+    if (m < 1 || m > 4 || (k & 31)) return hipErrorInvalidValue;
+    const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
+    const size_t red_bytes = (size_t)kWaves * mt * 64 * 4;
+    const size_t table_bytes = (size_t)(k / group) * 64 * 8;
+    const bool table = table_bytes + red_bytes <= 64 * 1024;
+    const size_t lds = red_bytes + (table ? table_bytes : 0);
+    dim3 grid((unsigned)((n + 63) / 64)), block(64 * kWaves);
+#define QMM_GPTQ_AO(MT_, TB_)                                                                                          \
+    do {                                                                                                              \
+        if (a_dtype == QMM_F32)                                                                                       \
+            gemv_gptq_act_order_kernel<MT_, TB_, float><<<grid, block, lds, s>>>(                                     \
+                qweight, scales, qzeros, g_idx, (const float*)a, out, m, (int)n, (int)k, group, ldo);                 \
+        else                                                                                                          \
+            gemv_gptq_act_order_kernel<MT_, TB_, uint16_t><<<grid, block, lds, s>>>(                                  \
+                qweight, scales, qzeros, g_idx, (const uint16_t*)a, out, m, (int)n, (int)k, group, ldo);              \
+    } while (0)
+#define QMM_GPTQ_AO_MT(TB_)                        \
+    do {                                           \
+        if (mt == 1) QMM_GPTQ_AO(1, TB_);          \
+        else if (mt == 2) QMM_GPTQ_AO(2, TB_);     \
+        else QMM_GPTQ_AO(4, TB_);                  \
+    } while (0)
+    if (table) QMM_GPTQ_AO_MT(true);
+    else QMM_GPTQ_AO_MT(false);
+#undef QMM_GPTQ_AO_MT
+#undef QMM_GPTQ_AO
+    return hipGetLastError();
+}
+
 }  // namespace qmm

@@ -59,7 +59,7 @@ int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 int check_gptq(const qmm_gptq_config* cfg, int64_t n, int64_t k, bool quantiser = false) {
     if (!cfg) return fail(QMM_ERR_INVALID, "GPTQ requires a config");
     if (cfg->bits != 4) return fail(QMM_ERR_UNSUPPORTED, "GPTQ bits=%d: only 4-bit is supported", cfg->bits);
-    if (cfg->desc_act) return fail(QMM_ERR_UNSUPPORTED, "GPTQ desc_act=True is not supported");
+    if (cfg->desc_act && quantiser) return fail(QMM_ERR_UNSUPPORTED, "GPTQ desc_act=True: the quantiser here writes plain groups only");
     if (!cfg->sym && quantiser) return fail(QMM_ERR_UNSUPPORTED, "GPTQ sym=False: the quantiser here is symmetric only");
     if (cfg->group_size <= 0 || cfg->group_size % 32 || k % cfg->group_size)
         return fail(QMM_ERR_INVALID, "GPTQ group_size=%d must be a multiple of 32 dividing K=%lld", cfg->group_size,
@@ -141,9 +141,11 @@ int qmm_dequantize_gptq(const qmm_gptq_config* cfg, const void* qweight, const v
     if (!qweight || !scales || !qzeros || !out) return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: null pointer");
     if (n <= 0 || k <= 0) return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: empty shape");
     if (int rc = check_gptq(cfg, n, k)) return rc;
+    if (cfg->desc_act && !g_idx) return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: desc_act=True needs g_idx");
     if (out_dtype != QMM_F32 && out_dtype != QMM_BF16)
         return fail(QMM_ERR_INVALID, "qmm_dequantize_gptq: out_dtype must be f32 or bf16");
-    return hip_status(qmm::launch_dequant_gptq(qweight, scales, qzeros, g_idx, n, k, cfg->group_size, out, out_dtype,
+    // desc_act = 0: the groups are k / group_size whatever g_idx says (it is not read)
+    return hip_status(qmm::launch_dequant_gptq(qweight, scales, qzeros, cfg->desc_act ? g_idx : nullptr, n, k, cfg->group_size, out, out_dtype,
                                                (hipStream_t)stream),
                       "qmm_dequantize_gptq");
 }
@@ -208,6 +210,19 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         if (int rc = check_gptq(cfg, n, k)) return rc;
         for (int i = 0; i < 3; i++)
             if (!rhs[i] || !aligned(rhs[i], 4)) return fail(QMM_ERR_INVALID, "qmm_matmul: GPTQ rhs[%d] null or misaligned", i);
+        if (cfg->desc_act) {
+            // act-order checkpoints: the decode kernel that looks the group of every k up, four lhs rows per pass
+            if (n_rhs != 4 || !rhs[3] || !aligned(rhs[3], 4))
+                return fail(QMM_ERR_INVALID, "qmm_matmul: GPTQ desc_act=True needs rhs[3] = g_idx int32[K]");
+            for (int64_t m0 = 0; m0 < m; m0 += 4) {
+                hipError_t e = qmm::launch_gemv_gptq_act_order((const char*)lhs + m0 * k * esz, lhs_dtype, (const uint32_t*)rhs[0],
+                                                               (const uint16_t*)rhs[1], (const uint32_t*)rhs[2],
+                                                               (const int32_t*)rhs[3], (int)std::min<int64_t>(4, m - m0), n, k,
+                                                               cfg->group_size, out + m0 * n, n, s);
+                if (e != hipSuccess) return hip_status(e, "qmm_matmul(GPTQ act-order)");
+            }
+            return QMM_OK;
+        }
         if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size))
             return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
                                                     (const uint32_t*)rhs[2], m, n, k, cfg->group_size, out, workspace, s),

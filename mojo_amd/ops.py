@@ -85,6 +85,8 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
             _require_gpu(rhs[3], "g_idx")
             if rhs[3].dtype != torch.int32 or tuple(rhs[3].shape) != (k,):
                 raise TypeError("g_idx must be int32[K]")
+        elif cfg.desc_act:
+            raise TypeError("GPTQ with desc_act=True needs g_idx as the fourth rhs tensor")
         cfg_p = C.byref(cfg)
     elif encoding.is_gguf:
         if len(rhs) != 1:
@@ -171,6 +173,10 @@ def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Opti
         g_idx = quantized[3] if len(quantized) == 4 else None
         cfg = _gptq_cfg(config)
         kk, n = qweight.shape[0] * 8, qweight.shape[1]
+        if g_idx is not None and (g_idx.dtype != torch.int32 or tuple(g_idx.shape) != (kk,)):
+            raise TypeError("g_idx must be int32[K]")
+        if g_idx is None and cfg.desc_act:
+            raise TypeError("GPTQ with desc_act=True needs g_idx")
         out = torch.empty((n, kk), dtype=dtype, device=qweight.device)
         rc = lib.qmm_dequantize_gptq(C.byref(cfg), _ptr(qweight), _ptr(scales), _ptr(qzeros), _ptr(g_idx), n, kk,
                                      _ptr(out), _DTYPES[dtype], _stream(qweight))

@@ -149,12 +149,15 @@ def dequantize(enc: int, w, k: int) -> np.ndarray:
     return out
 
 
-def dequantize_gptq(qweight, scales, qzeros, group: int = 128) -> np.ndarray:
-    """-> fp32 [N, K]"""
+def dequantize_gptq(qweight, scales, qzeros, group: int = 128, g_idx=None) -> np.ndarray:
+    """-> fp32 [N, K].  g_idx int32[K] (act-order checkpoints) names the group of every k; None: k // group."""
     qweight, scales, qzeros = _c(qweight, np.int32), _c(scales, np.uint16), _c(qzeros, np.int32)
     k, n = qweight.shape[0] * 8, qweight.shape[1]
+    gi = None if g_idx is None else _c(g_idx, np.int32)
+    assert gi is None or gi.shape == (k,)
     out = np.empty((n, k), np.float32)
-    lib().qo_dequantize_gptq(_p(qweight), _p(scales), _p(qzeros), _i64(n), _i64(k), _i64(group), _p(out))
+    lib().qo_dequantize_gptq(_p(qweight), _p(scales), _p(qzeros), None if gi is None else _p(gi), _i64(n), _i64(k),
+                             _i64(group), _p(out))
     return out
 
 
@@ -241,13 +244,16 @@ def matmul_f64(enc: int, a, w, w_bf16: bool = False) -> np.ndarray:
     return out
 
 
-def matmul_gptq(a, qweight, scales, qzeros, group: int = 128, w_bf16: bool = False, f64: bool = False):
+def matmul_gptq(a, qweight, scales, qzeros, group: int = 128, w_bf16: bool = False, f64: bool = False, g_idx=None):
     a, m, k = _rows_k(a)
     qweight, scales, qzeros = _c(qweight, np.int32), _c(scales, np.uint16), _c(qzeros, np.int32)
     n = qweight.shape[1]
+    gi = None if g_idx is None else _c(g_idx, np.int32)
+    assert gi is None or gi.shape == (k,)
     out = np.empty((m, n), np.float64 if f64 else np.float32)
     lib().qo_matmul_gptq_f32(
-        _p(a), _p(qweight), _p(scales), _p(qzeros), _i64(m), _i64(n), _i64(k), _i64(group), C.c_int(int(w_bf16)),
+        _p(a), _p(qweight), _p(scales), _p(qzeros), None if gi is None else _p(gi), _i64(m), _i64(n), _i64(k),
+        _i64(group), C.c_int(int(w_bf16)),
         None if f64 else _p(out), _p(out) if f64 else None)
     return out
 

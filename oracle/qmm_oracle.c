@@ -479,11 +479,11 @@ int qo_dequantize(int enc, const uint8_t* w, int64_t rows, int64_t k, float* out
 
 /* out fp32[N, K] (transposed orientation, like the GGUF rhs after dequant) */
 void qo_dequantize_gptq(const int32_t* qweight, const uint16_t* scales, const int32_t* qzeros,
-                        int64_t n, int64_t k, int64_t group, float* out) {
+                        const int32_t* g_idx, int64_t n, int64_t k, int64_t group, float* out) {
 #pragma omp parallel for schedule(static)
     for (int64_t col = 0; col < n; col++) {
         for (int64_t kk = 0; kk < k; kk++) {
-            int64_t g = kk / group;
+            int64_t g = g_idx ? g_idx[kk] : kk / group; /* act-order checkpoints: any group per k */
             int q = (int)(((uint32_t)qweight[(kk / 8) * n + col] >> (4 * (kk % 8))) & 0xF);
             int z = (int)(((uint32_t)qzeros[g * (n / 8) + col / 8] >> (4 * (col % 8))) & 0xF) + 1;
             out[col * k + kk] = qo_f16_to_f32(scales[g * n + col]) * (float)(q - z);
@@ -729,15 +729,15 @@ int qo_matmul_f64(int enc, const float* a, const uint8_t* w, int64_t m, int64_t 
 
 /* GPTQ: weights dequantised to fp32[N, K] per output column on the fly. */
 void qo_matmul_gptq_f32(const float* a, const int32_t* qweight, const uint16_t* scales,
-                        const int32_t* qzeros, int64_t m, int64_t n, int64_t k, int64_t group,
-                        int w_bf16, float* out, double* out64) {
+                        const int32_t* qzeros, const int32_t* g_idx, int64_t m, int64_t n, int64_t k,
+                        int64_t group, int w_bf16, float* out, double* out64) {
 #pragma omp parallel
     {
         float* wrow = (float*)malloc(sizeof(float) * (size_t)k);
 #pragma omp for schedule(static)
         for (int64_t col = 0; col < n; col++) {
             for (int64_t kk = 0; kk < k; kk++) {
-                int64_t g = kk / group;
+                int64_t g = g_idx ? g_idx[kk] : kk / group;
                 int q = (int)(((uint32_t)qweight[(kk / 8) * n + col] >> (4 * (kk % 8))) & 0xF);
                 int z = (int)(((uint32_t)qzeros[g * (n / 8) + col / 8] >> (4 * (col % 8))) & 0xF) + 1;
                 wrow[kk] = maybe_bf16(qo_f16_to_f32(scales[g * n + col]) * (float)(q - z), w_bf16);

@@ -62,7 +62,7 @@ def dequant_q6_k(packed: np.ndarray, k: int) -> np.ndarray:
     return w.astype(np.float32).reshape(n, k)
 
 
-def dequant_gptq(qweight, scales_u16, qzeros, group=128) -> np.ndarray:
+def dequant_gptq(qweight, scales_u16, qzeros, group=128, g_idx=None) -> np.ndarray:
     """-> [N, K] float32"""
     k8, n = qweight.shape
     k = k8 * 8
@@ -70,9 +70,31 @@ def dequant_gptq(qweight, scales_u16, qzeros, group=128) -> np.ndarray:
     q = ((qweight.view(np.uint32)[:, None, :] >> shifts[None, :, None]) & 15).reshape(k, n).astype(np.int32)
     z = ((qzeros.view(np.uint32)[:, :, None] >> shifts[None, None, :]) & 15).reshape(qzeros.shape[0], n).astype(np.int32) + 1
     s = scales_u16.view(np.float16).astype(np.float32)
-    g = np.arange(k) // group
+    g = np.arange(k) // group if g_idx is None else np.asarray(g_idx, np.int64)
     w = s[g, :] * (q - z[g, :]).astype(np.float32)
     return np.ascontiguousarray(w.T.astype(np.float32))
+
+
+def gptq_act_order(qweight_sorted, perm, group=128):
+    """An act-order (desc_act=True) checkpoint from tensors quantised in sorted order.
+
+    `qweight_sorted` packs the weight whose input columns were taken in the order `perm` (sorted position p
+    holds original column perm[p]), quantised with plain groups of `group` sorted positions.  AutoGPTQ stores
+    such a layer with the rows of qweight back in the original order and `g_idx[perm[p]] = p // group`;
+    scales and qzeros stay as they are.  Returns (qweight int32[K/8, N], g_idx int32[K]).
+    """
+    k8, n = qweight_sorted.shape
+    k = k8 * 8
+    perm = np.asarray(perm, np.int64)
+    assert sorted(perm.tolist()) == list(range(k))
+    shifts = 4 * np.arange(8, dtype=np.uint32)
+    nib = ((qweight_sorted.view(np.uint32)[:, None, :] >> shifts[None, :, None]) & 15).reshape(k, n)
+    orig = np.empty_like(nib)
+    orig[perm] = nib
+    packed = (orig.reshape(k8, 8, n).astype(np.uint32) << shifts[None, :, None]).sum(axis=1, dtype=np.uint64).astype(np.uint32)
+    g_idx = np.empty(k, np.int32)
+    g_idx[perm] = (np.arange(k) // group).astype(np.int32)
+    return np.ascontiguousarray(packed).view(np.int32), g_idx
 
 
 def quantize_q4_0(x: np.ndarray) -> np.ndarray:

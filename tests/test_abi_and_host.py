@@ -62,7 +62,10 @@ def test_argument_validation_happens_before_any_launch():
     bad = _lib.GptqConfig(8, 128, 0, 1)
     rhs3 = (C.c_void_p * 3)(0x2000, 0x3000, 0x4000)
     assert matmul(3, 1, 4096, 8, cfg=C.byref(bad), n_rhs=3, rhs_arr=rhs3) == -2
-    assert matmul(3, 1, 4096, 8, cfg=C.byref(_lib.GptqConfig(4, 128, 1, 1)), n_rhs=3, rhs_arr=rhs3) == -2  # desc_act
+    assert matmul(3, 1, 4096, 8, cfg=C.byref(_lib.GptqConfig(4, 128, 1, 1)), n_rhs=3, rhs_arr=rhs3) == -1  # desc_act without g_idx
+    assert b"g_idx" in lib.qmm_last_error()
+    assert lib.qmm_quantize_gptq(C.byref(_lib.GptqConfig(4, 128, 1, 1)), fake, 8, 256, fake, fake, fake, fake, None) == -2  # desc_act
+    assert lib.qmm_dequantize_gptq(C.byref(_lib.GptqConfig(4, 128, 1, 1)), fake, fake, fake, None, 8, 256, fake, 0, None) == -1
     assert lib.qmm_quantize_gptq(C.byref(_lib.GptqConfig(4, 128, 0, 0)), fake, 8, 256, fake, fake, fake, fake, None) == -2  # sym=False
     assert matmul(3, 1, 4096, 8, cfg=C.byref(_lib.GptqConfig(4, 100, 0, 1)), n_rhs=3, rhs_arr=rhs3) == -1
     assert lib.qmm_dequantize(1, fake, 4, 100, fake, 0, None) == -1

@@ -119,6 +119,34 @@ def test_gptq_asymmetric_checkpoint(m):
     assert_close(got, truth, f"asymmetric GPTQ m={m}")
 
 
+@pytest.mark.parametrize("m,n,k,group,bf16", [(1, 200, 1024, 128, False), (3, 72, 512, 64, True), (5, 136, 1024, 128, False),
+                                               (20, 64, 512, 32, False), (2, 72, 4096, 32, False)])
+def test_gptq_act_order_checkpoint(m, n, k, group, bf16):
+    """desc_act=True: g_idx names the group of every k in no particular order; through dequantize (bit-exact) and
+    the matmul (the last shape has too many groups for the kernel's LDS table and reads scales from memory)."""
+    import np_formats as NF
+
+    w, a = synth(27, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    rng = np.random.Generator(np.random.PCG64(28))
+    perm = rng.permutation(k)
+    qs, sc, qz, _ = O.quantize_gptq(np.ascontiguousarray(w[:, perm]), group)
+    qz = rng.integers(0, 2**32, size=qz.shape, dtype=np.uint64).astype(np.uint32).view(np.int32)
+    qw, gi = NF.gptq_act_order(qs, perm, group)
+    cfg = QuantizationConfig(group_size=group, desc_act=True, sym=False)
+    want_w = O.dequantize_gptq(qw, sc, qz, group, g_idx=gi)
+    got_w = dequantize(QE.GPTQ, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi), config=cfg)
+    assert np.array_equal(bits(got_w), want_w.view(np.uint8).reshape(n, -1))
+    truth = O.matmul_gptq(a, qw, sc, qz, group, f64=True, g_idx=gi)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.GPTQ, cfg, lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, truth, f"act-order GPTQ m={m} n={n} k={k} group={group}")
+    assert_close(got, O.matmul_gptq(a, qw, sc, qz, group, g_idx=gi), "act-order GPTQ against the fp32 oracle")
+    with pytest.raises(TypeError):
+        qmatmul(QE.GPTQ, cfg, lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz))
+
+
 # ------------------------------------------------------------------ Q4_0: integer dots and matmul
 def test_block_dots_bit_exact():
     w, a = synth(0, 256, 1024, 4)

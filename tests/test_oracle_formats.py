@@ -247,6 +247,35 @@ def test_dequant_gptq_matches_vectorised_restatement():
     assert np.array_equal(O.dequantize_gptq(qw, sc, qz), NF.dequant_gptq(qw, sc, qz))
 
 
+def test_gptq_act_order_group_index():
+    """g_idx: (1) the plain index k // group changes nothing; (2) an act-order checkpoint dequantises to the
+    sorted-order weight with its columns put back (an independent route: pack in sorted order, then permute
+    the dequantised columns); (3) the vectorised restatement agrees on arbitrary bits and arbitrary group indices."""
+    n, k, group = 24, 512, 64
+    w, _ = synth(31, n, k, 1)
+    rng = np.random.default_rng(32)
+    perm = rng.permutation(k)
+    qs, sc, qz, gi0 = O.quantize_gptq(np.ascontiguousarray(w[:, perm]), group)
+    qz = rng.integers(-2**31, 2**31, qz.shape, dtype=np.int64).astype(np.int32)  # every zero point 1..16
+    assert np.array_equal(O.dequantize_gptq(qs, sc, qz, group, g_idx=gi0), O.dequantize_gptq(qs, sc, qz, group))
+    qw, gi = NF.gptq_act_order(qs, perm, group)
+    assert np.array_equal(np.bincount(gi, minlength=k // group), np.full(k // group, group))
+    sorted_w = O.dequantize_gptq(qs, sc, qz, group)          # [N, K] in sorted order
+    want = np.empty_like(sorted_w)
+    want[:, perm] = sorted_w
+    got = O.dequantize_gptq(qw, sc, qz, group, g_idx=gi)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert not np.array_equal(got, O.dequantize_gptq(qw, sc, qz, group))  # the index matters
+    anyg = rng.integers(0, k // group, k).astype(np.int32)
+    qr = rng.integers(-2**31, 2**31, qw.shape, dtype=np.int64).astype(np.int32)
+    assert np.array_equal(O.dequantize_gptq(qr, sc, qz, group, g_idx=anyg), NF.dequant_gptq(qr, sc, qz, group, g_idx=anyg))
+    # matmul: fp64 sums over the dequantised weight
+    a = rng.standard_normal((3, k)).astype(np.float32)
+    truth = a.astype(np.float64) @ got.astype(np.float64).T
+    assert np.abs(O.matmul_gptq(a, qw, sc, qz, group, f64=True, g_idx=gi) - truth).max() < 1e-12
+    assert O.isclose(O.matmul_gptq(a, qw, sc, qz, group, g_idx=gi), truth, 1e-5, 2e-6).all()
+
+
 def test_non_finite_and_zero_scales_propagate():
     blk = np.zeros((1, 18), np.uint8)
     blk[0, 2:] = 0x5A
