@@ -39,6 +39,7 @@ enum qmm_encoding {
     QMM_Q4_K = 1, /* 256 weights / 144 bytes: f16 d, dmin, 12 B 6-bit, 128 B */
     QMM_Q6_K = 2, /* 256 weights / 210 bytes: ql[128] qh[64] i8 sc[16] f16 d */
     QMM_GPTQ = 3, /* AutoGPTQ v1 tensors: qweight, scales, qzeros[, g_idx]   */
+    QMM_Q5_K = 4, /* 256 weights / 176 bytes: the Q4_K header, qh[32] fifth bits, 128 B nibbles */
     QMM_Q8_0 = 8, /* 32 values / 34 bytes  : f16 d, 32 x i8 (activations)    */
     QMM_Q8_K = 9  /* 256 values / 292 bytes: f32 d, 256 x i8, 16 x i16 sums (activations) */
 };

@@ -48,6 +48,7 @@ bool block_params(int enc, int64_t& epb, int64_t& bpb) {
         case QMM_Q8_K: epb = 256; bpb = 292; return true;
         case QMM_Q4_K: epb = 256; bpb = 144; return true;
         case QMM_Q6_K: epb = 256; bpb = 210; return true;
+        case QMM_Q5_K: epb = 256; bpb = 176; return true;
         default: return false;
     }
 }
@@ -130,8 +131,8 @@ int qmm_dequantize(int encoding, const void* rhs, int64_t n, int64_t k, void* ou
                     (long long)n, (long long)k, (long long)epb);
     if (out_dtype != QMM_F32 && out_dtype != QMM_BF16)
         return fail(QMM_ERR_INVALID, "qmm_dequantize: out_dtype must be f32 or bf16");
-    if (encoding == QMM_Q4_K && !aligned(rhs, 16))
-        return fail(QMM_ERR_INVALID, "qmm_dequantize: Q4_K rhs must be 16-byte aligned");
+    if ((encoding == QMM_Q4_K || encoding == QMM_Q5_K) && !aligned(rhs, 16))
+        return fail(QMM_ERR_INVALID, "qmm_dequantize: Q4_K / Q5_K rhs must be 16-byte aligned");
     return hip_status(qmm::launch_dequant(encoding, rhs, n, k, out, out_dtype, (hipStream_t)stream),
                       "qmm_dequantize");
 }
@@ -245,7 +246,8 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         return fail(QMM_ERR_INVALID, "qmm_matmul: K=%lld is not a multiple of the block size %lld", (long long)k,
                     (long long)epb);
     const uint8_t* w = (const uint8_t*)rhs[0];
-    if (encoding == QMM_Q4_K && !aligned(w, 16)) return fail(QMM_ERR_INVALID, "qmm_matmul: Q4_K rhs must be 16-byte aligned");
+    if ((encoding == QMM_Q4_K || encoding == QMM_Q5_K) && !aligned(w, 16))
+        return fail(QMM_ERR_INVALID, "qmm_matmul: Q4_K / Q5_K rhs must be 16-byte aligned");
     if (!aligned(w, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: rhs must be 2-byte aligned");
 
     if (flags & QMM_FLAG_ACT_Q8K) {
@@ -256,6 +258,20 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
                                                      out + m0 * n, n, s, &handled);
             if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K x Q8_K)");
             if (!handled) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations need K <= 16384 (K = %lld)", (long long)k);
+        }
+        return QMM_OK;
+    }
+    if (encoding == QMM_Q5_K) {
+        // one decode-shaped kernel for every m; a pass takes as many lhs rows as fit its LDS copy of the lhs
+        const int64_t ngroups = (k / 256 + 15) / 16;
+        const int64_t pass = ngroups <= 2 ? 4 : ngroups <= 4 ? 2 : 1;
+        if (ngroups > 8) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q5_K takes K <= 32768 (K = %lld)", (long long)k);
+        for (int64_t m0 = 0; m0 < m; m0 += pass) {
+            bool handled = false;
+            hipError_t e = qmm::launch_gemv_q5_k((const char*)lhs + m0 * k * esz, lhs_dtype, w, (int)std::min<int64_t>(pass, m - m0), n, k,
+                                                 out + m0 * n, n, s, &handled);
+            if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q5_K)");
+            if (!handled) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q5_K shape not taken (M=%lld K=%lld)", (long long)m, (long long)k);
         }
         return QMM_OK;
     }

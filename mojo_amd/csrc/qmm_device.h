@@ -12,6 +12,7 @@ constexpr int Q4_0_EPB = 32, Q4_0_BPB = 18;
 constexpr int Q8_0_EPB = 32, Q8_0_BPB = 34;
 constexpr int Q4_K_EPB = 256, Q4_K_BPB = 144;
 constexpr int Q6_K_EPB = 256, Q6_K_BPB = 210;
+constexpr int Q5_K_EPB = 256, Q5_K_BPB = 176;
 
 __device__ __forceinline__ float h2f(uint16_t h) {
     union { uint16_t u; _Float16 f; } v;

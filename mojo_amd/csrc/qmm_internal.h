@@ -39,6 +39,10 @@ inline hipError_t allow_full_lds() {
     return st;
 }
 
+// Q5_K decode kernel, m <= 4 (fewer when K is long: the lhs copy in LDS takes 16 KB per row and 4096 columns).
+hipError_t launch_gemv_q5_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                            int64_t ldo, hipStream_t s, bool* handled);
+
 // Q4_K with Q8_K-quantised activations (integer dots), m <= 4.
 hipError_t launch_gemv_q4_k_q8k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
                                 int64_t ldo, hipStream_t s, bool* handled);

@@ -32,6 +32,20 @@ __device__ __forceinline__ float dequant_q4_k_elem(const uint8_t* b, int pos) {
     return (d * (float)sc) * (float)q - (dmin * (float)mn);
 }
 
+// Q5_K: the Q4_K header, then qh[32] (bit j of qh[l]: fifth bit of position l of sub-block j) and qs[128]
+__device__ __forceinline__ float dequant_q5_k_elem(const uint8_t* b, int pos) {
+    const uint32_t* w = (const uint32_t*)b;  // blocks are 16-byte aligned
+    uint32_t hdr = w[0];
+    float d = h2f((uint16_t)(hdr & 0xffffu)), dmin = h2f((uint16_t)(hdr >> 16));
+    uint32_t s[3] = {w[1], w[2], w[3]};
+    int j = pos >> 5, c = pos >> 6, l = pos & 31;
+    uint32_t sc, mn;
+    q4k_scale_min(j, s, sc, mn);
+    uint32_t byte = b[48 + 32 * c + l];
+    uint32_t q = ((j & 1) ? (byte >> 4) : (byte & 15u)) | ((((uint32_t)b[16 + l] >> j) & 1u) << 4);
+    return (d * (float)sc) * (float)q - (dmin * (float)mn);
+}
+
 __device__ __forceinline__ float dequant_q6_k_elem(const uint8_t* b, int pos) {
     int h = pos >> 7, r = pos & 127, quarter = r >> 5, l = r & 31;
     const uint8_t* ql = b + 64 * h;
@@ -49,7 +63,7 @@ template <int ENC, typename OutT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, int64_t total,
                                                       OutT* __restrict__ out) {
     constexpr int EPB = ENC == QMM_Q4_0 ? Q4_0_EPB : 256;
-    constexpr int BPB = ENC == QMM_Q4_0 ? Q4_0_BPB : (ENC == QMM_Q4_K ? Q4_K_BPB : Q6_K_BPB);
+    constexpr int BPB = ENC == QMM_Q4_0 ? Q4_0_BPB : (ENC == QMM_Q4_K ? Q4_K_BPB : (ENC == QMM_Q5_K ? Q5_K_BPB : Q6_K_BPB));
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
         int64_t blk = e / EPB;
@@ -58,6 +72,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         float v;
         if (ENC == QMM_Q4_0) v = dequant_q4_0_elem(b, pos);
         else if (ENC == QMM_Q4_K) v = dequant_q4_k_elem(b, pos);
+        else if (ENC == QMM_Q5_K) v = dequant_q5_k_elem(b, pos);
         else v = dequant_q6_k_elem(b, pos);
         if constexpr (sizeof(OutT) == 4) out[e] = v;
         else out[e] = f2bf(v);
@@ -126,6 +141,7 @@ hipError_t launch_dequant(int enc, const void* rhs, int64_t n, int64_t k, void* 
     else dequant_kernel<E, uint16_t><<<grid, block, 0, s>>>(w, total, (uint16_t*)out)
     if (enc == QMM_Q4_0) { QMM_DQ(QMM_Q4_0); }
     else if (enc == QMM_Q4_K) { QMM_DQ(QMM_Q4_K); }
+    else if (enc == QMM_Q5_K) { QMM_DQ(QMM_Q5_K); }
     else { QMM_DQ(QMM_Q6_K); }
 #undef QMM_DQ
     return hipGetLastError();
@@ -232,12 +248,15 @@ __global__ __launch_bounds__(256) void quantize_q4_0_kernel(const float* __restr
 
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
+// BITS = 4: Q4_K (codes at byte 16); BITS = 5: Q5_K (fifth bits in qh at byte 16, nibbles at byte 48)
+template <int BITS>
 __global__ __launch_bounds__(64) void quantize_q4_k_kernel(const float* __restrict__ x, int64_t nblocks,
                                                            uint8_t* __restrict__ out) {
+    constexpr int kQmax = (1 << BITS) - 1;
     int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (blk >= nblocks) return;
     const float* xb = x + blk * 256;
-    uint8_t* ob = out + blk * Q4_K_BPB;
+    uint8_t* ob = out + blk * (BITS == 4 ? Q4_K_BPB : Q5_K_BPB);
     float scale[8], minv[8];
     float max_scale = 0.0f, max_min = 0.0f;
     for (int j = 0; j < 8; j++) {
@@ -247,7 +266,7 @@ __global__ __launch_bounds__(64) void quantize_q4_k_kernel(const float* __restri
             if (v < lo) lo = v;
             if (v > hi) hi = v;
         }
-        scale[j] = (hi - lo) / 15.0f;
+        scale[j] = (hi - lo) / (float)kQmax;
         minv[j] = -lo;
         if (scale[j] > max_scale) max_scale = scale[j];
         if (minv[j] > max_min) max_min = minv[j];
@@ -278,15 +297,23 @@ __global__ __launch_bounds__(64) void quantize_q4_k_kernel(const float* __restri
     ob[3] = (uint8_t)(mh >> 8);
     for (int j = 0; j < 12; j++) ob[4 + j] = s[j];
     float d = h2f(dh), dmin = h2f(mh);
-    for (int c = 0; c < 4; c++) {
-        float d1 = d * (float)sc[2 * c], m1 = dmin * (float)mn[2 * c];
-        float d2 = d * (float)sc[2 * c + 1], m2 = dmin * (float)mn[2 * c + 1];
-        for (int l = 0; l < 32; l++) {
+    float dl[8], ml[8];
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+        dl[jj] = d * (float)sc[jj];
+        ml[jj] = dmin * (float)mn[jj];
+    }
+    for (int l = 0; l < 32; l++) {
+        uint32_t fifth = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
             int q1 = 0, q2 = 0;
-            if (d1 != 0.0f) q1 = clampi((int)rintf((xb[64 * c + l] + m1) / d1), 0, 15);
-            if (d2 != 0.0f) q2 = clampi((int)rintf((xb[64 * c + 32 + l] + m2) / d2), 0, 15);
-            ob[16 + 32 * c + l] = (uint8_t)(q1 | (q2 << 4));
+            if (dl[2 * c] != 0.0f) q1 = clampi((int)rintf((xb[64 * c + l] + ml[2 * c]) / dl[2 * c]), 0, kQmax);
+            if (dl[2 * c + 1] != 0.0f) q2 = clampi((int)rintf((xb[64 * c + 32 + l] + ml[2 * c + 1]) / dl[2 * c + 1]), 0, kQmax);
+            ob[(BITS == 4 ? 16 : 48) + 32 * c + l] = (uint8_t)((q1 & 15) | ((q2 & 15) << 4));
+            fifth |= (uint32_t)(((q1 >> 4) << (2 * c)) | ((q2 >> 4) << (2 * c + 1)));
         }
+        if constexpr (BITS == 5) ob[16 + l] = (uint8_t)fifth;
     }
 }
 
@@ -397,7 +424,8 @@ hipError_t launch_quantize(int enc, const float* x, int64_t rows, int64_t k, voi
     } else {
         int64_t nblocks = rows * (k / 256);
         dim3 grid((unsigned)((nblocks + 63) / 64)), block(64);
-        if (enc == QMM_Q4_K) quantize_q4_k_kernel<<<grid, block, 0, s>>>(x, nblocks, (uint8_t*)out);
+        if (enc == QMM_Q4_K) quantize_q4_k_kernel<4><<<grid, block, 0, s>>>(x, nblocks, (uint8_t*)out);
+        else if (enc == QMM_Q5_K) quantize_q4_k_kernel<5><<<grid, block, 0, s>>>(x, nblocks, (uint8_t*)out);
         else quantize_q6_k_kernel<<<grid, block, 0, s>>>(x, nblocks, (uint8_t*)out);
     }
     return hipGetLastError();

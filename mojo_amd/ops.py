@@ -204,7 +204,7 @@ def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Opti
 
 
 def quantize(encoding: QuantizationEncoding, x: torch.Tensor) -> torch.Tensor:
-    """fp32 ``[rows, K]`` -> packed ``uint8[rows, K/epb*bpb]`` (Q4_0, Q8_0, Q8_K, Q4_K, Q6_K)."""
+    """fp32 ``[rows, K]`` -> packed ``uint8[rows, K/epb*bpb]`` (Q4_0, Q8_0, Q8_K, Q4_K, Q5_K, Q6_K)."""
     _require_gpu(x, "x")
     if x.dtype != torch.float32 or x.dim() != 2:
         raise TypeError("x must be a rank-2 float32 tensor")

@@ -20,6 +20,7 @@ class BlockParameters:
 class QuantizationEncoding(enum.Enum):
     Q4_0 = "Q4_0"
     Q4_K = "Q4_K"
+    Q5_K = "Q5_K"
     Q6_K = "Q6_K"
     GPTQ = "GPTQ"
     # activation-side block format of the Q4_0 path; not a weight encoding of qmatmul
@@ -34,7 +35,8 @@ class QuantizationEncoding(enum.Enum):
 
     @property
     def is_gguf(self) -> bool:
-        return self in (QuantizationEncoding.Q4_0, QuantizationEncoding.Q4_K, QuantizationEncoding.Q6_K)
+        return self in (QuantizationEncoding.Q4_0, QuantizationEncoding.Q4_K, QuantizationEncoding.Q5_K,
+                        QuantizationEncoding.Q6_K)
 
     @property
     def block_parameters(self) -> BlockParameters:
@@ -54,6 +56,7 @@ _CODES = {
     QuantizationEncoding.Q4_K: 1,
     QuantizationEncoding.Q6_K: 2,
     QuantizationEncoding.GPTQ: 3,
+    QuantizationEncoding.Q5_K: 4,
     QuantizationEncoding.Q8_0: 8,
     QuantizationEncoding.Q8_K: 9,
 }
@@ -63,6 +66,7 @@ _BLOCKS = {
     QuantizationEncoding.Q8_K: BlockParameters(256, 292),
     QuantizationEncoding.Q4_K: BlockParameters(256, 144),
     QuantizationEncoding.Q6_K: BlockParameters(256, 210),
+    QuantizationEncoding.Q5_K: BlockParameters(256, 176),
 }
 
 

@@ -45,7 +45,8 @@ GGML_TYPES: Dict[int, Tuple[str, int, int]] = {
     28: ("F64", 1, 8),
     30: ("BF16", 1, 2),
 }
-_ENCODINGS = {"Q4_0": QuantizationEncoding.Q4_0, "Q4_K": QuantizationEncoding.Q4_K, "Q6_K": QuantizationEncoding.Q6_K}
+_ENCODINGS = {"Q4_0": QuantizationEncoding.Q4_0, "Q4_K": QuantizationEncoding.Q4_K, "Q5_K": QuantizationEncoding.Q5_K,
+              "Q6_K": QuantizationEncoding.Q6_K}
 _PLAIN_DTYPES = {"F32": np.float32, "F16": np.float16, "I8": np.int8, "I16": np.int16, "I32": np.int32,
                  "I64": np.int64, "F64": np.float64, "BF16": np.uint16}
 

@@ -18,8 +18,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libqmm_oracle.so")
 
-Q4_0, Q4_K, Q6_K, GPTQ = 0, 1, 2, 3
-BLOCK = {Q4_0: (32, 18), Q4_K: (256, 144), Q6_K: (256, 210)}
+Q4_0, Q4_K, Q6_K, GPTQ, Q5_K = 0, 1, 2, 3, 4
+BLOCK = {Q4_0: (32, 18), Q4_K: (256, 144), Q6_K: (256, 210), Q5_K: (256, 176)}
 
 
 def build(force: bool = False) -> str:
@@ -93,12 +93,13 @@ def _rows_k(x):
 
 
 def quantize(enc: int, x) -> np.ndarray:
-    """fp32 [rows, K] -> uint8 [rows, K/epb*bpb] (Q4_0 / Q4_K / Q6_K)."""
+    """fp32 [rows, K] -> uint8 [rows, K/epb*bpb] (Q4_0 / Q4_K / Q5_K / Q6_K)."""
     x, rows, k = _rows_k(x)
     epb, bpb = BLOCK[enc]
     assert k % epb == 0
     out = np.empty((rows, k // epb * bpb), np.uint8)
-    fn = {Q4_0: lib().qo_quantize_q4_0, Q4_K: lib().qo_quantize_q4_k, Q6_K: lib().qo_quantize_q6_k}[enc]
+    fn = {Q4_0: lib().qo_quantize_q4_0, Q4_K: lib().qo_quantize_q4_k, Q6_K: lib().qo_quantize_q6_k,
+          Q5_K: lib().qo_quantize_q5_k}[enc]
     fn(_p(x), _i64(rows), _i64(k), _p(out))
     return out
 

@@ -25,10 +25,13 @@
  *   qo_f32_to_bf16                    pinned: reference rule above + torch
  *   qo_unpack_scales_q4_k             pinned: pack/unpack round trip over all
  *                                     8 positions x 64 x 64 values + hand KAT
- *   qo_dequantize (Q4_0/Q4_K/Q6_K), qo_dequantize_gptq
+ *   qo_dequantize (Q4_0/Q4_K/Q5_K/Q6_K), qo_dequantize_gptq
  *                                     pinned: hand-worked known-answer blocks,
  *                                     exactness lemma brute force, independent
- *                                     vectorised restatement
+ *                                     vectorised restatement; the g_idx (act-
+ *                                     order) route: identity with k / group,
+ *                                     and equality with the sorted-order weight
+ *                                     whose columns are put back
  *   qo_block_dots_q4_0_q8_0           pinned: integer arithmetic, brute force vs
  *                                     int64, extreme vectors
  *   qo_matmul_* outputs               pinned: fp64 truth, closed-form special
@@ -39,7 +42,7 @@
  *                                     the choice of rounding rule itself
  *                                     (roundf, fp16 scale) is PARITY UNPINNED:
  *                                     nothing in the reference fixes it.
- *   qo_quantize_q4_k / qo_quantize_q6_k / qo_quantize_gptq
+ *   qo_quantize_q4_k / qo_quantize_q5_k / qo_quantize_q6_k / qo_quantize_gptq
  *                                     PARITY UNPINNED: these are this build's
  *                                     own simple packers (ggml's iterative
  *                                     search is not restated); they exist to
@@ -73,6 +76,7 @@
 #define QO_Q4_K 1
 #define QO_Q6_K 2
 #define QO_GPTQ 3
+#define QO_Q5_K 4
 
 /* ------------------------------------------------------------------ */
 /* scalar conversions                                                  */
@@ -174,6 +178,7 @@ int qo_block_params(int enc, int64_t* epb, int64_t* bpb) {
         case QO_Q4_0: *epb = 32; *bpb = 18; return 0;
         case QO_Q4_K: *epb = 256; *bpb = 144; return 0;
         case QO_Q6_K: *epb = 256; *bpb = 210; return 0;
+        case QO_Q5_K: *epb = 256; *bpb = 176; return 0;
         default: return -1;
     }
 }
@@ -316,6 +321,64 @@ void qo_quantize_q4_k(const float* x, int64_t rows, int64_t k, uint8_t* out) {
     }
 }
 
+/* Q5_K: the Q4_K fit with 5-bit codes.  Block: f16 d, f16 dmin, 12 B scales (as Q4_K), qh[32], qs[128];
+ * code j of chunk c (64 weights) has its low four bits in the low (j < 32) or high (j >= 32) nibble of
+ * qs[32 c + j % 32] and its fifth bit in bit 2 c + j / 32 of qh[j % 32]. */
+void qo_quantize_q5_k(const float* x, int64_t rows, int64_t k, uint8_t* out) {
+    int64_t nb = k / 256;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+        for (int64_t b = 0; b < nb; b++) {
+            const float* xb = x + r * k + b * 256;
+            uint8_t* ob = out + (r * nb + b) * 176;
+            float scale[8], minv[8];
+            float max_scale = 0.0f, max_min = 0.0f;
+            for (int j = 0; j < 8; j++) {
+                float lo = 0.0f, hi = 0.0f;
+                for (int l = 0; l < 32; l++) {
+                    float v = xb[j * 32 + l];
+                    if (v < lo) lo = v;
+                    if (v > hi) hi = v;
+                }
+                scale[j] = (hi - lo) / 31.0f;
+                minv[j] = -lo;
+                if (scale[j] > max_scale) max_scale = scale[j];
+                if (minv[j] > max_min) max_min = minv[j];
+            }
+            float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+            float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+            uint8_t sc[8], mn[8];
+            for (int j = 0; j < 8; j++) {
+                sc[j] = (uint8_t)clampi((int)rintf(inv_scale * scale[j]), 0, 63);
+                mn[j] = (uint8_t)clampi((int)rintf(inv_min * minv[j]), 0, 63);
+            }
+            wr_f16(ob, max_scale / 63.0f);
+            wr_f16(ob + 2, max_min / 63.0f);
+            qo_pack_scales_q4_k(sc, mn, ob + 4);
+            float d = rd_f16(ob), dmin = rd_f16(ob + 2);
+            uint8_t q[256];
+            for (int j = 0; j < 8; j++) {
+                float dl = d * (float)sc[j];
+                float ml = dmin * (float)mn[j];
+                for (int l = 0; l < 32; l++) {
+                    int v = 0;
+                    if (dl != 0.0f) v = clampi((int)rintf((xb[j * 32 + l] + ml) / dl), 0, 31);
+                    q[j * 32 + l] = (uint8_t)v;
+                }
+            }
+            uint8_t* qh = ob + 16;
+            uint8_t* qs = ob + 48;
+            memset(qh, 0, 32);
+            for (int c = 0; c < 4; c++)
+                for (int l = 0; l < 32; l++) {
+                    uint8_t a = q[c * 64 + l], bb = q[c * 64 + 32 + l];
+                    qs[c * 32 + l] = (uint8_t)((a & 0xF) | ((bb & 0xF) << 4));
+                    qh[l] |= (uint8_t)(((a >> 4) << (2 * c)) | ((bb >> 4) << (2 * c + 1)));
+                }
+        }
+    }
+}
+
 void qo_quantize_q6_k(const float* x, int64_t rows, int64_t k, uint8_t* out) {
     int64_t nb = k / 256;
 #pragma omp parallel for schedule(static)
@@ -438,6 +501,24 @@ static void dequant_block_q4_k(const uint8_t* b, float* y) {
     }
 }
 
+static void dequant_block_q5_k(const uint8_t* b, float* y) {
+    float d = rd_f16(b), dmin = rd_f16(b + 2);
+    uint8_t sc[8], mn[8];
+    qo_unpack_scales_q4_k(b + 4, sc, mn);
+    const uint8_t* qh = b + 16;
+    const uint8_t* qs = b + 48;
+    for (int c = 0; c < 4; c++) {
+        float d1 = d * (float)sc[2 * c], m1 = dmin * (float)mn[2 * c];
+        float d2 = d * (float)sc[2 * c + 1], m2 = dmin * (float)mn[2 * c + 1];
+        for (int l = 0; l < 32; l++) {
+            int q1 = (qs[32 * c + l] & 0xF) + (((qh[l] >> (2 * c)) & 1) << 4);
+            int q2 = (qs[32 * c + l] >> 4) + (((qh[l] >> (2 * c + 1)) & 1) << 4);
+            y[64 * c + l] = d1 * (float)q1 - m1;
+            y[64 * c + 32 + l] = d2 * (float)q2 - m2;
+        }
+    }
+}
+
 static void dequant_block_q6_k(const uint8_t* b, float* y) {
     float d = rd_f16(b + 208);
     for (int h = 0; h < 2; h++) {
@@ -462,6 +543,7 @@ static void dequant_block_q6_k(const uint8_t* b, float* y) {
 static void dequant_block(int enc, const uint8_t* b, float* y) {
     if (enc == QO_Q4_0) dequant_block_q4_0(b, y);
     else if (enc == QO_Q4_K) dequant_block_q4_k(b, y);
+    else if (enc == QO_Q5_K) dequant_block_q5_k(b, y);
     else dequant_block_q6_k(b, y);
 }
 

@@ -45,6 +45,24 @@ def dequant_q4_k(packed: np.ndarray, k: int) -> np.ndarray:
     return w.astype(np.float32).reshape(n, k)
 
 
+def dequant_q5_k(packed: np.ndarray, k: int) -> np.ndarray:
+    """176-byte blocks: f16 d, f16 dmin, 12 B scales (as Q4_K), qh[32], qs[128]; the fifth bit of sub-block j's
+    codes is bit j of the qh byte at the code's position in the sub-block."""
+    n = packed.shape[0]
+    b = packed.reshape(n, k // 256, 176)
+    d, dmin = f16(b[:, :, 0:2]), f16(b[:, :, 2:4])
+    sc, mn = unpack_scales_q4_k(b[:, :, 4:16])
+    qh = b[:, :, 16:48].astype(np.int32)                                   # [n, nb, 32]
+    qs = b[:, :, 48:].reshape(n, k // 256, 4, 32).astype(np.int32)
+    low = np.stack([qs & 15, qs >> 4], axis=3).reshape(n, k // 256, 8, 32)  # sub-block 2c low nibbles, 2c+1 high
+    fifth = (qh[:, :, None, :] >> np.arange(8)[None, None, :, None]) & 1    # [n, nb, 8, 32]
+    q = low + 16 * fifth
+    dl = (d[:, :, None] * sc.astype(np.float32)).astype(np.float32)
+    ml = (dmin[:, :, None] * mn.astype(np.float32)).astype(np.float32)
+    w = (dl[..., None] * q.astype(np.float32)).astype(np.float32) - ml[..., None]
+    return w.astype(np.float32).reshape(n, k)
+
+
 def dequant_q6_k(packed: np.ndarray, k: int) -> np.ndarray:
     n = packed.shape[0]
     b = packed.reshape(n, k // 256, 210)

@@ -81,6 +81,7 @@ def test_argument_validation_happens_before_any_launch():
 def test_quantization_encoding_metadata():
     assert QE.Q4_0.block_parameters == mojo_amd.BlockParameters(32, 18)
     assert QE.Q4_K.block_parameters.block_size == 144 and QE.Q6_K.block_parameters.block_size == 210
+    assert QE.Q5_K.block_parameters == mojo_amd.BlockParameters(256, 176) and QE.Q5_K.is_gguf and QE.Q5_K.code == 4
     assert QE.Q4_K.is_gguf and QE.Q6_K.is_gguf and QE.Q4_0.is_gguf and not QE.GPTQ.is_gguf
     assert QE.Q4_K.name == "Q4_K" and QE.GPTQ.code == 3
     assert QE.Q4_K.packed_row_bytes(4096) == 2304 and QE.Q6_K.packed_row_bytes(4096) == 3360

@@ -16,7 +16,7 @@ from mojo_amd import block_dots_q4_0, dequantize, qmatmul, qmatmul_grouped, quan
 pytestmark = pytest.mark.gpu
 
 RTOL, ATOL = 1e-3, 1e-4
-ENC = {QE.Q4_0: O.Q4_0, QE.Q4_K: O.Q4_K, QE.Q6_K: O.Q6_K}
+ENC = {QE.Q4_0: O.Q4_0, QE.Q4_K: O.Q4_K, QE.Q6_K: O.Q6_K, QE.Q5_K: O.Q5_K}
 DEV = "cuda:0"
 
 
@@ -40,7 +40,7 @@ def bits(x):
 
 
 # ------------------------------------------------------------------ quantisers
-@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q6_K])
+@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q6_K, QE.Q5_K])
 def test_quantize_bytes_match_oracle(enc):
     w, _ = synth(3, 96, 1024, 1)
     w[5, 256:512] = 0.0  # an all-zero super-block
@@ -68,7 +68,7 @@ def test_quantize_gptq_matches_oracle():
 
 
 # ------------------------------------------------------------------ dequantisers (bit-exact)
-@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q6_K])
+@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q6_K, QE.Q5_K])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_dequantize_bit_exact(enc, dtype):
     w, _ = synth(6, 128, 2048, 1)
@@ -78,7 +78,7 @@ def test_dequantize_bit_exact(enc, dtype):
     noisy = packed.copy()
     epb, bpb = O.BLOCK[ENC[enc]]
     blocks = noisy.reshape(-1, bpb)
-    keep = {O.Q4_0: slice(0, 2), O.Q4_K: slice(0, 4), O.Q6_K: slice(208, 210)}[ENC[enc]]
+    keep = {O.Q4_0: slice(0, 2), O.Q4_K: slice(0, 4), O.Q6_K: slice(208, 210), O.Q5_K: slice(0, 4)}[ENC[enc]]
     rnd = rng.integers(0, 256, blocks.shape, dtype=np.uint8)
     rnd[:, keep] = blocks[:, keep]
     blocks[64:] = rnd[64:]
@@ -206,7 +206,7 @@ def test_q4_0_small_batch(m, n, k, lhs_bf16):
 
 
 # ------------------------------------------------------------------ Q4_K / Q6_K with fp32 activations
-@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K])
+@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K, QE.Q5_K])
 @pytest.mark.parametrize("m,n,k", [(1, 1024, 4096), (4, 512, 4096), (16, 256, 2048), (3, 5, 256), (2, 66, 14336),
                                    (20, 64, 512)])
 def test_kquant_matmul_f32(enc, m, n, k):
@@ -219,7 +219,7 @@ def test_kquant_matmul_f32(enc, m, n, k):
     assert_close(got, truth, f"{enc.name} {m}x{n}x{k} vs fp64 truth")
 
 
-@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K])
+@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q6_K, QE.Q5_K])
 def test_kquant_matmul_bf16_lhs(enc):
     w, a = synth(5, 256, 1024, 4)
     a = O.bf16_to_f32(O.f32_to_bf16(a))
@@ -227,6 +227,27 @@ def test_kquant_matmul_bf16_lhs(enc):
     want = O.matmul_f32(ENC[enc], a, wq)
     got = qmatmul(enc, None, gpu(a).to(torch.bfloat16), gpu(wq))
     assert_close(got, want, f"{enc.name} bf16 lhs")
+
+
+@pytest.mark.parametrize("m,n,k,bf16", [(1, 4099, 4096, False), (1, 1030, 4096, True), (3, 777, 14336, False), (1, 130, 32768, False),
+                                        (4, 2050, 1280, True), (7, 300, 8192, False)])
+def test_q5_k_decode_shapes(m, n, k, bf16):
+    """Q5_K through its kernel's variants: activations in registers (one row, K <= 4096), from the LDS copy,
+    several groups of 16 super-blocks with a partial last one, row counts that leave wavefronts unequal work,
+    and the random bit patterns of the dequantiser test (every fifth-bit / nibble combination)."""
+    w, a = synth(41, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q5_K, w)
+    rng = np.random.default_rng(42)
+    blocks = wq.reshape(-1, 176)
+    rnd = rng.integers(0, 256, blocks.shape, dtype=np.uint8)
+    rnd[:, 0:4] = blocks[:, 0:4]
+    blocks[::3] = rnd[::3]
+    truth = O.matmul_f64(O.Q5_K, a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.Q5_K, None, lhs, gpu(wq))
+    assert_close(got, truth, f"Q5_K {m}x{n}x{k} bf16={bf16}")
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256)])

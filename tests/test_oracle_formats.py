@@ -71,8 +71,8 @@ def test_bf16_rule_matches_torch_and_reference_formula():
 
 # ------------------------------------------------------------------ block parameters
 def test_block_sizes_and_bits_per_weight():
-    assert O.BLOCK == {O.Q4_0: (32, 18), O.Q4_K: (256, 144), O.Q6_K: (256, 210)}
-    assert [8 * b / e for e, b in O.BLOCK.values()] == [4.5, 4.5, 6.5625]
+    assert O.BLOCK == {O.Q4_0: (32, 18), O.Q4_K: (256, 144), O.Q6_K: (256, 210), O.Q5_K: (256, 176)}
+    assert [8 * b / e for e, b in O.BLOCK.values()] == [4.5, 4.5, 6.5625, 5.5]
     assert O.quantize_q8_0(np.zeros((1, 32), np.float32)).shape == (1, 34)
 
 
@@ -112,6 +112,51 @@ def test_q4_k_known_block():
             want[64 * c + l] = 2.0 * sc[2 * c] * ((l + c) % 16) - 0.25 * mn[2 * c]
             want[64 * c + 32 + l] = 2.0 * sc[2 * c + 1] * ((3 * l + c) % 16) - 0.25 * mn[2 * c + 1]
     assert np.array_equal(got, want)
+
+
+def test_q5_k_known_block():
+    # d = 2.0, dmin = 0.25, the scale / min fields of the Q4_K block above; code of (sub-block j, position l) =
+    # (5 l + 3 j) % 32: low four bits in the nibble planes, fifth bit in bit j of qh[l]
+    sc = np.array([1, 63, 32, 5, 17, 48, 63, 33], np.uint8)
+    mn = np.array([0, 2, 63, 31, 16, 63, 1, 47], np.uint8)
+    blk = np.zeros(176, np.uint8)
+    blk[0:4] = [0x00, 0x40, 0x00, 0x34]
+    blk[4:16] = O.pack_scales_q4_k(sc, mn)
+    code = lambda j, l: (5 * l + 3 * j) % 32
+    for l in range(32):
+        blk[16 + l] = sum(((code(j, l) >> 4) & 1) << j for j in range(8))
+    for c in range(4):
+        for l in range(32):
+            blk[48 + 32 * c + l] = (code(2 * c, l) & 15) | ((code(2 * c + 1, l) & 15) << 4)
+    got = O.dequantize(O.Q5_K, blk[None, :], 256)[0]
+    want = np.array([2.0 * sc[j] * code(j, l) - 0.25 * mn[j] for j in range(8) for l in range(32)], np.float32)
+    assert np.array_equal(got, want)
+    assert {code(j, l) for j in range(8) for l in range(32)} == set(range(32))  # every code value occurs
+
+
+def test_q5_k_single_rounding_and_packer():
+    """d * sc * q is exact for 5-bit codes as well (11 + 6 + 5 bits); the packer's blocks decode to within half
+    a step of the input and use the fifth bit."""
+    rng = np.random.default_rng(14)
+    d = rng.integers(0x0400, 0x5000, 40).astype(np.uint16).view(np.float16).astype(np.float64)
+    dlq = d[:, None, None] * np.arange(64)[None, :, None] * np.arange(32)[None, None, :]
+    assert np.array_equal(dlq.astype(np.float32).astype(np.float64), dlq)
+    w, _ = synth(15, 16, 1024, 1)
+    packed = O.quantize(O.Q5_K, w)
+    assert packed.shape == (16, 4 * 176)
+    back = O.dequantize(O.Q5_K, packed, 1024)
+    b = packed.reshape(16, 4, 176)
+    dsc = NF.f16(b[:, :, 0:2])[:, :, None] * NF.unpack_scales_q4_k(b[:, :, 4:16])[0]        # step of every sub-block
+    dmn = NF.f16(b[:, :, 2:4])[:, :, None] * NF.unpack_scales_q4_k(b[:, :, 4:16])[1]
+    err = np.abs(back - w).reshape(16, 4, 8, 32)
+    # a code is the nearest one to (x + min) / step, so the error is half a step unless the 6-bit min or scale
+    # clipped the range; allow those the rounding of the two 6-bit fields
+    lim = 0.5 * dsc + np.abs(dmn - (-np.minimum(w.reshape(16, 4, 8, 32).min(axis=3), 0))) + 31 * np.abs(
+        dsc - (w.reshape(16, 4, 8, 32).max(axis=3).clip(0) - w.reshape(16, 4, 8, 32).min(axis=3).clip(None, 0)) / 31)
+    assert (err <= lim[..., None] + 1e-7).all()
+    rms = lambda e: float(np.sqrt(np.mean(e.astype(np.float64) ** 2)))
+    assert rms(back - w) < 0.75 * rms(O.dequantize(O.Q4_K, O.quantize(O.Q4_K, w), 1024) - w)  # one more bit of code
+    assert b[:, :, 16:48].any() and (b[:, :, 16:48] != 0xFF).any()
 
 
 def test_q6_k_known_block():
@@ -222,14 +267,15 @@ def test_q4_k_single_rounding():
 
 
 # ------------------------------------------------------------------ independent restatement on random bytes
-@pytest.mark.parametrize("enc,fn", [(O.Q4_0, NF.dequant_q4_0), (O.Q4_K, NF.dequant_q4_k), (O.Q6_K, NF.dequant_q6_k)])
+@pytest.mark.parametrize("enc,fn", [(O.Q4_0, NF.dequant_q4_0), (O.Q4_K, NF.dequant_q4_k), (O.Q6_K, NF.dequant_q6_k),
+                                    (O.Q5_K, NF.dequant_q5_k)])
 def test_dequant_matches_vectorised_restatement(enc, fn):
     w, _ = synth(20 + enc, 32, 1024, 1)
     packed = O.quantize(enc, w)
     rng = np.random.default_rng(5)
     epb, bpb = O.BLOCK[enc]
     blocks = packed.reshape(-1, bpb)
-    keep = {O.Q4_0: slice(0, 2), O.Q4_K: slice(0, 4), O.Q6_K: slice(208, 210)}[enc]
+    keep = {O.Q4_0: slice(0, 2), O.Q4_K: slice(0, 4), O.Q6_K: slice(208, 210), O.Q5_K: slice(0, 4)}[enc]
     rnd = rng.integers(0, 256, blocks.shape, dtype=np.uint8)
     rnd[:, keep] = blocks[:, keep]
     blocks[blocks.shape[0] // 2:] = rnd[blocks.shape[0] // 2:]  # half quantised data, half arbitrary bit patterns

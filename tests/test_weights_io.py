@@ -12,7 +12,7 @@ from gguf_writer import (T_ARR, T_BOOL, T_F32, T_I32, T_STR, T_U32, T_U64, write
 from mojo_amd import QuantizationEncoding as QE
 from mojo_amd.weights import GGUFWeights, load_gptq_config, load_gptq_linear
 
-GGML_F32, GGML_Q4_0, GGML_Q4_K, GGML_Q6_K, GGML_BF16 = 0, 2, 12, 14, 30
+GGML_F32, GGML_Q4_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_BF16 = 0, 2, 12, 13, 14, 30
 
 
 def _model_file(tmp_path, alignment=None, version=3):
@@ -20,6 +20,7 @@ def _model_file(tmp_path, alignment=None, version=3):
     f32 = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
     bf = (np.arange(10, dtype=np.uint16) * 257).reshape(2, 5)
     q4k, q6k, q40 = O.quantize(O.Q4_K, w), O.quantize(O.Q6_K, w), O.quantize(O.Q4_0, w[:, :96])
+    q5k = O.quantize(O.Q5_K, w)
     meta = [("general.architecture", T_STR, "llama"), ("llama.block_count", T_U32, 32),
             ("llama.rope.freq_base", T_F32, 500000.0), ("general.file_type", T_U64, 15), ("flag", T_BOOL, True),
             ("tokenizer.ggml.tokens", T_ARR, (T_STR, ["<s>", "</s>", "hé"])),
@@ -28,9 +29,10 @@ def _model_file(tmp_path, alignment=None, version=3):
                ("blk.0.attn_q.weight", [512, 48], GGML_Q4_K, q4k.tobytes()),
                ("output.weight", [512, 48], GGML_Q6_K, q6k.tobytes()),
                ("blk.0.ffn_up.weight", [96, 48], GGML_Q4_0, q40.tobytes()),
-               ("rope.bf16", [5, 2], GGML_BF16, bf.tobytes())]
+               ("rope.bf16", [5, 2], GGML_BF16, bf.tobytes()),
+               ("blk.0.attn_v.weight", [512, 48], GGML_Q5_K, q5k.tobytes())]
     path = write_gguf(os.path.join(tmp_path, "m.gguf"), meta, tensors, version=version, alignment=alignment)
-    return path, dict(w=w, f32=f32, bf=bf, q4k=q4k, q6k=q6k, q40=q40)
+    return path, dict(w=w, f32=f32, bf=bf, q4k=q4k, q6k=q6k, q40=q40, q5k=q5k)
 
 
 @pytest.mark.parametrize("alignment,version", [(None, 3), (64, 3), (32, 2)])
@@ -42,7 +44,9 @@ def test_gguf_metadata_and_tensor_views(tmp_path, alignment, version):
     assert g.metadata["llama.rope.freq_base"] == np.float32(500000.0) and g.metadata["flag"] is True
     assert g.metadata["tokenizer.ggml.tokens"] == ["<s>", "</s>", "hé"]
     assert g.metadata["tokenizer.ggml.token_type"].tolist() == [1, 2, -3]
-    assert list(g) == ["norm.weight", "blk.0.attn_q.weight", "output.weight", "blk.0.ffn_up.weight", "rope.bf16"]
+    assert list(g) == ["norm.weight", "blk.0.attn_q.weight", "output.weight", "blk.0.ffn_up.weight", "rope.bf16",
+                       "blk.0.attn_v.weight"]
+    assert g.encoding("blk.0.attn_v.weight") is QE.Q5_K and g.tensors["blk.0.attn_v.weight"].nbytes == 48 * 2 * 176
     q = g.tensors["blk.0.attn_q.weight"]
     assert q.shape == (48, 512) and q.ggml_type == "Q4_K" and q.encoding is QE.Q4_K and q.nbytes == 48 * 2 * 144
     assert (q.offset - g.data_offset) % g.alignment == 0
@@ -50,7 +54,8 @@ def test_gguf_metadata_and_tensor_views(tmp_path, alignment, version):
     assert g.encoding("norm.weight") is None
     np.testing.assert_array_equal(g.raw("norm.weight"), ref["f32"])
     np.testing.assert_array_equal(g.raw("rope.bf16"), ref["bf"])
-    for name, key in (("blk.0.attn_q.weight", "q4k"), ("output.weight", "q6k"), ("blk.0.ffn_up.weight", "q40")):
+    for name, key in (("blk.0.attn_q.weight", "q4k"), ("output.weight", "q6k"), ("blk.0.ffn_up.weight", "q40"),
+                      ("blk.0.attn_v.weight", "q5k")):
         raw = g.raw(name)
         assert raw.dtype == np.uint8 and raw.shape == ref[key].shape
         np.testing.assert_array_equal(raw, ref[key])
