@@ -96,21 +96,22 @@ class GroupedGemv:
 class GptqMatmul:
     """One preallocated GPTQ qmm_matmul call on (qweight, scales, qzeros)."""
 
-    def __init__(self, tensors, a: torch.Tensor, group: int = 128):
+    def __init__(self, tensors, a: torch.Tensor, group: int = 128, g_idx=None):
         self.lib = _lib.load()
-        self.t, self.a = tensors, a
+        self.t, self.a, self.g_idx = tensors, a, g_idx
         self.m, self.k = a.shape
         self.n = tensors[0].shape[1]
         self.out = torch.empty((self.m, self.n), dtype=torch.float32, device=a.device)
         self.dt = _lib.QMM_F32 if a.dtype == torch.float32 else _lib.QMM_BF16
         self.need = self.lib.qmm_matmul_workspace_bytes(QE.GPTQ.code, self.dt, self.m, self.n, self.k)
         self.ws = torch.empty((max(self.need, 1),), dtype=torch.uint8, device=a.device)
-        self.cfg = _lib.GptqConfig(4, group, 0, 1)
-        self.ptrs = (C.c_void_p * 3)(*[t.data_ptr() for t in tensors[:3]])
+        self.cfg = _lib.GptqConfig(4, group, 0 if g_idx is None else 1, 1)  # g_idx given: an act-order checkpoint
+        ptrs = [t.data_ptr() for t in tensors[:3]] + ([] if g_idx is None else [g_idx.data_ptr()])
+        self.ptrs = (C.c_void_p * len(ptrs))(*ptrs)
 
     def launch(self, stream_ptr: int) -> None:
         rc = self.lib.qmm_matmul(QE.GPTQ.code, C.byref(self.cfg), C.c_void_p(self.a.data_ptr()), self.dt, self.m,
-                                 self.k, self.ptrs, 3, self.n, C.c_void_p(self.out.data_ptr()),
+                                 self.k, self.ptrs, len(self.ptrs), self.n, C.c_void_p(self.out.data_ptr()),
                                  C.c_void_p(self.ws.data_ptr()), self.need, 0, C.c_void_p(stream_ptr))
         _lib.check(rc, "qmm_matmul")
 
@@ -441,6 +442,19 @@ def extra_timings(layers, acts, gen):
     dev_s, _ = time_graphs([g], 20, 3)
     us = dev_s * 1e6 / (20 * 8)
     out["gptq_g128_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round((14336 * 4096 * 0.5176 + 4096 * 4 + 14336 * 4) / us / 1e3, 1)}
+    # the same tensors read as an act-order checkpoint (desc_act=True): a random group for every k
+    gi = torch.arange(4096, dtype=torch.int32, device="cuda:0")[torch.randperm(4096, device="cuda:0", generator=gen)] // 128
+    g = capture([GptqMatmul(c.t, am1, g_idx=gi.to(torch.int32).contiguous()) for c in cs])
+    dev_s, _ = time_graphs([g], 20, 3)
+    us = dev_s * 1e6 / (20 * 8)
+    out["gptq_g128_act_order_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round((14336 * 4096 * 0.5176 + 4096 * 8 + 14336 * 4) / us / 1e3, 1)}
+    del cs
+    # Q5_K decode on the gate shape
+    cs = [Gemv(QE.Q5_K, make_weight(QE.Q5_K, 14336, 4096, gen), am1) for _ in range(8)]
+    g = capture(cs)
+    dev_s, _ = time_graphs([g], 20, 3)
+    us = dev_s * 1e6 / (20 * 8)
+    out["q5_k_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q5_K, 1, 14336, 4096) / us / 1e3, 1)}
     del cs
     # Q4_0 prefill on the int8 matrix cores, same shape as cfg5
     ab32 = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
