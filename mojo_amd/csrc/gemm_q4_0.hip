@@ -369,6 +369,144 @@ __global__ __launch_bounds__(64 * kSWaves) void gemm_q4_0_small_kernel(const uin
     }
 }
 
+// Many lhs rows (prefill).  Same operands and the same staging of the weight rows as gemm_q4_0_kernel, with the
+// work cut so that the vector cache is not the bound: the weights are the A operand of the matrix-core
+// instruction, so a lane holds the block dots of four weight rows (4 g + r) against ONE lhs row (lane % 16) and
+// needs one activation scale and one code sum per instruction (16 bytes per lane with the codes, against 40 the
+// other way round); a wavefront owns 32 weight rows for all of K and 8 lhs tiles per pass, so an activation
+// operand serves two matrix-core instructions and a weight operand eight; the 8 wavefronts of a workgroup take
+// neighbouring weight rows (no sum across wavefronts) and read the same activation operands (vector-cache hits).
+// Per (lhs row, weight row, block):  acc += d_w * (float(dot) * d_a - 8 asum d_a)  (convert, two fused
+// multiply-adds).
+namespace {
+constexpr int kWNT = 2;      // 16-row weight tiles per wavefront
+constexpr int kWMG = 8;      // 16-row lhs tiles per pass
+constexpr int kWWaves = 8;   // wavefronts per workgroup
+}  // namespace
+
+__global__ __launch_bounds__(64 * kWWaves) void gemm_q4_0_wide_kernel(const uint8_t* __restrict__ w, const int8_t* __restrict__ codes,
+                                                                     const float* __restrict__ dscale, const int32_t* __restrict__ csum,
+                                                                     float* __restrict__ out, int m, int n, int k) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nkb = k >> 5;
+    const int64_t row_bytes = (int64_t)nkb * Q4_0_BPB;
+    const int n0 = ((int)blockIdx.x * kWWaves + wave) * 16 * kWNT;  // first weight row of this wavefront
+    if (n0 >= n) return;                                            // (no workgroup-wide barrier below)
+    const int tile0 = (int)blockIdx.y * kWMG;
+    const int tiles = (m + 15) >> 4;
+    const int nn = lane & 15, g = lane >> 4;
+    uint8_t* wbuf = smem + wave * (kWNT * kWaveLds);
+
+    float acc[kWNT][kWMG][4];
+#pragma unroll
+    for (int nt = 0; nt < kWNT; nt++)
+#pragma unroll
+        for (int t = 0; t < kWMG; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[nt][t][r] = 0.0f;
+
+    // piece p = lane + 64 i of a tile's run: row p / 19, 16-byte piece p % 19 of that row's run
+    int prow[5], pidx[5];
+#pragma unroll
+    for (int i = 0; i < 5; i++) {
+        const int p = min(lane + 64 * i, 16 * kRowPieces - 1);
+        prow[i] = p / kRowPieces;
+        pidx[i] = p - prow[i] * kRowPieces;
+    }
+    const uint32_t lane8 = 8u * (uint32_t)lane, nn4 = 4u * (uint32_t)nn;
+    const uint8_t* my_row[kWNT];  // the row whose codes this lane turns into operands
+#pragma unroll
+    for (int nt = 0; nt < kWNT; nt++) my_row[nt] = w + (int64_t)min(n0 + 16 * nt + nn, n - 1) * row_bytes;
+
+    for (int kb = 0; kb < nkb; kb += kRun) {
+        const int nb = min(kRun, nkb - kb);
+        __builtin_amdgcn_wave_barrier();  // the previous run's LDS reads are issued (LDS is in order per wavefront)
+#pragma unroll
+        for (int nt = 0; nt < kWNT; nt++) {
+            uint4 rr[5];
+#pragma unroll
+            for (int i = 0; i < 5; i++) {
+                const uintptr_t ad = (uintptr_t)(w + (int64_t)min(n0 + 16 * nt + prow[i], n - 1) * row_bytes + (int64_t)kb * Q4_0_BPB);
+                const int dl = (int)(ad & 15);
+                const int last = (dl + nb * Q4_0_BPB + 15) / 16 - 1;
+                rr[i] = ((const uint4*)(ad - (uintptr_t)dl))[min(pidx[i], last)];
+            }
+            uint8_t* dst = wbuf + nt * kWaveLds;
+#pragma unroll
+            for (int i = 0; i < 4; i++) *(uint4*)(dst + prow[i] * kRowLds + pidx[i] * 16) = rr[i];
+            if (lane + 256 < 16 * kRowPieces) *(uint4*)(dst + prow[4] * kRowLds + pidx[4] * 16) = rr[4];
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        int delta[kWNT];
+#pragma unroll
+        for (int nt = 0; nt < kWNT; nt++) delta[nt] = (int)((uintptr_t)(my_row[nt] + (int64_t)kb * Q4_0_BPB) & 15);
+        for (int b = 0; b < nb; b++) {
+            long wop[kWNT];
+            float dw4[kWNT][4];
+#pragma unroll
+            for (int nt = 0; nt < kWNT; nt++) {
+                const uint32_t* lds32 = (const uint32_t*)(wbuf + nt * kWaveLds);
+                // 8 code bytes of k-group g (low nibbles of bytes 8 (g & 1) .., or their high nibbles)
+                const int boff = nn * kRowLds + delta[nt] + Q4_0_BPB * b;
+                const int qoff = boff + 2 + 8 * (g & 1);
+                const int wi = qoff >> 2;
+                const uint32_t sh = (uint32_t)(qoff & 3);
+                const uint32_t w0 = lds32[wi], w1 = lds32[wi + 1], w2 = lds32[wi + 2];
+                uint32_t lo = __builtin_amdgcn_alignbyte(w1, w0, sh), hi = __builtin_amdgcn_alignbyte(w2, w1, sh);
+                if (g & 2) {
+                    lo >>= 4;
+                    hi >>= 4;
+                }
+                lo &= 0x0F0F0F0Fu;
+                hi &= 0x0F0F0F0Fu;
+                wop[nt] = (long)(((uint64_t)hi << 32) | lo);
+                const uint32_t dw32 = lds32[boff >> 2] >> (8 * (boff & 3));
+                const float dw = h2f((uint16_t)(dw32 & 0xffffu));  // scale of row nn; the lane needs rows 4 g + r
+#pragma unroll
+                for (int r = 0; r < 4; r++) dw4[nt][r] = __shfl(dw, 4 * g + r, 64);
+            }
+#pragma unroll
+            for (int t = 0; t < kWMG; t++) {
+                const int tile = min(tile0 + t, tiles - 1);
+                const int64_t tb = (int64_t)tile * nkb + kb + b;
+                const long aop = *(const long*)((const char*)(codes + tb * 512) + lane8);
+                const float da = *(const float*)((const char*)(dscale + tb * 16) + nn4);
+                const float ts = -8.0f * (float)*(const int32_t*)((const char*)(csum + tb * 16) + nn4) * da;
+#pragma unroll
+                for (int nt = 0; nt < kWNT; nt++) {
+                    int4v z = {0, 0, 0, 0};
+                    const int4v dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(wop[nt], aop, z, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[nt][t][r] = fmaf(dw4[nt][r], fmaf((float)dot[r], da, ts), acc[nt][t][r]);
+                }
+            }
+        }
+    }
+
+    // lane holds out[16 (tile0 + t) + nn][n0 + 16 nt + 4 g + r]
+    const bool vec = (n & 3) == 0;
+#pragma unroll
+    for (int t = 0; t < kWMG; t++) {
+        const int row = (tile0 + t) * 16 + nn;
+        if (tile0 + t >= tiles || row >= m) continue;
+#pragma unroll
+        for (int nt = 0; nt < kWNT; nt++) {
+            const int col = n0 + 16 * nt + 4 * g;
+            float* o = out + (int64_t)row * n + col;
+            if (vec && col + 3 < n) {
+                *(float4*)o = make_float4(acc[nt][t][0], acc[nt][t][1], acc[nt][t][2], acc[nt][t][3]);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (col + r < n) o[r] = acc[nt][t][r];
+            }
+        }
+    }
+}
+
 int64_t gemm_q4_0_workspace_bytes(int64_t m, int64_t k) { return lhs_q8t(nullptr, m, k).bytes; }
 
 hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
@@ -406,6 +544,19 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
         const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
         gemm_q4_0_small_kernel<<<dim3((unsigned)wgs), dim3(64 * kSWaves), kSLds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n,
                                                                                    (int)k);
+        return hipGetLastError();
+    }
+    static const bool wide_off = getenv("QMM_Q4_0_WIDE_OFF") != nullptr;  // read once: fallback switch
+    if (tiles > 4 && !wide_off) {
+        const size_t wlds = (size_t)kWWaves * kWNT * kWaveLds;
+        static bool wide_set = false;
+        if (!wide_set) {
+            hipError_t e2 = hipFuncSetAttribute((const void*)gemm_q4_0_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
+            if (e2 != hipSuccess) return e2;
+            wide_set = true;
+        }
+        dim3 grid((unsigned)((n + 16 * kWNT * kWWaves - 1) / (16 * kWNT * kWWaves)), (unsigned)((tiles + kWMG - 1) / kWMG));
+        gemm_q4_0_wide_kernel<<<grid, dim3(64 * kWWaves), wlds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n, (int)k);
         return hipGetLastError();
     }
     const int nw = (tiles <= 2 && k >= 2048) ? 8 : 4;

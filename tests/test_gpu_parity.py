@@ -499,10 +499,13 @@ def test_q6_k_decode_vocabulary_shapes(n, k, lhs_bf16):
     assert_close(got, truth, f"Q6_K 1x{n}x{k} bf16={lhs_bf16} vs fp64 truth")
 
 
-@pytest.mark.parametrize("m,n,k,lhs_bf16", [(200, 300, 1024, False), (64, 130, 4096, True), (17, 16, 96, False)])
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(200, 300, 1024, False), (64, 130, 4096, True), (17, 16, 96, False),
+                                            (65, 33, 32, False), (130, 515, 608, True), (300, 258, 2048, False)])
 def test_q4_0_matmul_int8_matrix_cores(m, n, k, lhs_bf16):
     """Q4_0 with many lhs rows: 16 x 16 integer block dots per matrix-core instruction, several passes of
-    64 lhs rows, ragged N and a K that does not split evenly over the four wavefronts."""
+    64 lhs rows, ragged N and a K that does not split evenly over the four wavefronts; from 65 lhs rows on the
+    kernel with the weights as the first operand (N not a multiple of 4, 32 or 256, K of one block and of a
+    partial last run, a last lhs tile with one row)."""
     w, a = synth(51, n, k, m)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
