@@ -195,8 +195,8 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             t = fmaf(-m1, slo_a[mi], t);
             t = fmaf(d2, shi[mi], t);
             t = fmaf(-m2, shi_a[mi], t);
-            const float v = wave_sum_dpp(t);
-            if (lane == 0) res[ri * MT + mi] = v;
+            const float v = wave_sum_dpp_lane63(t);
+            if (lane == 63) res[ri * MT + mi] = v;
         }
     }
     auto store_row = [&](int mi, int row, float v) {

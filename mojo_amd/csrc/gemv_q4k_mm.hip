@@ -199,21 +199,33 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
                 for (int ps = 0; ps < MROWS / RP; ps++) {
                     uint32_t hp[kRunBlk][RP][2], lp[kRunBlk][RP][2], sp[kRunBlk][RP];
                     float isc[kRunBlk][RP];
+                    auto widen = [&](const xraw_t raw, float& x0, float& x1, float& x2, float& x3) {
+                        if constexpr (sizeof(AT) == 4) {
+                            x0 = __uint_as_float(raw.x); x1 = __uint_as_float(raw.y);
+                            x2 = __uint_as_float(raw.z); x3 = __uint_as_float(raw.w);
+                        } else {
+                            x0 = __uint_as_float(raw.x << 16); x1 = __uint_as_float(raw.x & 0xffff0000u);
+                            x2 = __uint_as_float(raw.y << 16); x3 = __uint_as_float(raw.y & 0xffff0000u);
+                        }
+                    };
+                    // largest magnitude of every (super-block, row) over the wavefront, all of them in one go
+                    uint32_t mxs[kRunBlk * RP];
+#pragma unroll
+                    for (int bb = 0; bb < kRunBlk; bb++)
+#pragma unroll
+                        for (int j = 0; j < RP; j++) {
+                            float x0, x1, x2, x3;
+                            widen(xr[bb][ps * RP + j], x0, x1, x2, x3);
+                            mxs[bb * RP + j] = max_abs_bits(x0, x1, x2, x3);
+                        }
+                    wave_umax_many(mxs);
 #pragma unroll
                     for (int bb = 0; bb < kRunBlk; bb++) {
 #pragma unroll
                         for (int j = 0; j < RP; j++) {
-                            const xraw_t raw = xr[bb][ps * RP + j];
                             float x0, x1, x2, x3;
-                            if constexpr (sizeof(AT) == 4) {
-                                x0 = __uint_as_float(raw.x); x1 = __uint_as_float(raw.y);
-                                x2 = __uint_as_float(raw.z); x3 = __uint_as_float(raw.w);
-                            } else {
-                                x0 = __uint_as_float(raw.x << 16); x1 = __uint_as_float(raw.x & 0xffff0000u);
-                                x2 = __uint_as_float(raw.y << 16); x3 = __uint_as_float(raw.y & 0xffff0000u);
-                            }
-                            const uint32_t mxb =
-                                wave_max_nonneg_bits(fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3))));
+                            widen(xr[bb][ps * RP + j], x0, x1, x2, x3);
+                            const uint32_t mxb = mxs[bb * RP + j];
                             int e = (int)((mxb >> 23) & 0xffu) - 127;
                             if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite: leave unscaled
                             const float sc = __uint_as_float((uint32_t)(127 + 9 - e) << 23);

@@ -438,8 +438,8 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             u = fmaf(sbyte(j < 4 ? s0 : s1, 8 * (j & 3)), os[it], u);
             v = fmaf(d, u, v);
         }
-        const float sum = wave_sum_dpp(v);
-        if (lane == 0) park[ri] = sum;
+        const float sum = wave_sum_dpp_lane63(v);
+        if (lane == 63) park[ri] = sum;
     }
     __builtin_amdgcn_wave_barrier();
     for (int i = lane; i < my_rows; i += 64) out[gw + (int64_t)i * total_waves] = park[i];

@@ -90,6 +90,63 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// The same sum, delivered in lane 63 only (the other lanes hold partial sums): after the four steps inside the
+// 16-lane rows, row_bcast15 adds row 0's total into row 1 and row 2's into row 3, row_bcast31 adds row 1's
+// into row 3.  Same association as wave_sum_dpp, (r0 + r1) + (r2 + r3), so the value is bit-identical.
+__device__ __forceinline__ float wave_sum_dpp_lane63(float v) {
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    v += dpp_move<0x140>(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xa, 0xf, false));  // row_bcast15 -> rows 1, 3
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xc, 0xf, false));  // row_bcast31 -> rows 2, 3
+    return v;
+}
+
+// Maxima over the 64 lanes of N unsigned values per lane at once (N = 2, 4 or 8); the results are wave-uniform.
+// Used on the bit patterns of float magnitudes: with the sign cleared the unsigned order is the numeric order
+// (NaN patterns sort above infinity).  Every step is one v_max_u32 with a DPP operand per value (the compiler keeps
+// the lane permutation and the maximum apart and pads them with wait states); the N values of a step are
+// independent, so only the first instruction of a step waits (s_nop 1: a DPP operand may be read two wait states
+// after the instruction that wrote it).  Steps: swap lane pairs, swap pairs of a quad, mirror 8, mirror 16, then
+// row_bcast15 into rows 1 and 3 and row_bcast31 into row 3: lane 63 holds the maximum.
+#define QMM_UMAX1(CTRL, A) "v_max_u32_dpp " A ", " A ", " A " " CTRL " bank_mask:0xf\n\t"
+#define QMM_UMAX_STEPS(M)                                                                                         \
+    M("quad_perm:[1,0,3,2] row_mask:0xf") M("quad_perm:[2,3,0,1] row_mask:0xf") M("row_half_mirror row_mask:0xf") \
+    M("row_mirror row_mask:0xf") M("row_bcast:15 row_mask:0xa") M("row_bcast:31 row_mask:0xc")
+template <int N>
+__device__ __forceinline__ void wave_umax_many(uint32_t (&v)[N]) {
+    static_assert(N == 2 || N == 4 || N == 8, "2, 4 or 8 values");
+    if constexpr (N == 2) {
+#define QMM_STEP(C) asm volatile("s_nop 1\n\t" QMM_UMAX1(C, "%0") "s_nop 0\n\t" QMM_UMAX1(C, "%1") : "+v"(v[0]), "+v"(v[1]));
+        QMM_UMAX_STEPS(QMM_STEP)
+#undef QMM_STEP
+    } else if constexpr (N == 4) {
+#define QMM_STEP(C)                                                                                         \
+    asm volatile("s_nop 1\n\t" QMM_UMAX1(C, "%0") QMM_UMAX1(C, "%1") QMM_UMAX1(C, "%2") QMM_UMAX1(C, "%3") \
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+        QMM_UMAX_STEPS(QMM_STEP)
+#undef QMM_STEP
+    } else {
+#define QMM_STEP(C)                                                                                         \
+    asm volatile("s_nop 1\n\t" QMM_UMAX1(C, "%0") QMM_UMAX1(C, "%1") QMM_UMAX1(C, "%2") QMM_UMAX1(C, "%3") \
+                     QMM_UMAX1(C, "%4") QMM_UMAX1(C, "%5") QMM_UMAX1(C, "%6") QMM_UMAX1(C, "%7")             \
+                 : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]));
+        QMM_UMAX_STEPS(QMM_STEP)
+#undef QMM_STEP
+    }
+    asm volatile("s_nop 1");  // (the readlanes below are the compiler's: it does not see what the block above wrote last)
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = (uint32_t)__builtin_amdgcn_readlane((int)v[i], 63);
+}
+#undef QMM_UMAX_STEPS
+// the magnitude bits of the largest of four floats (lane-local)
+__device__ __forceinline__ uint32_t max_abs_bits(float x0, float x1, float x2, float x3) {
+    const uint32_t a0 = __float_as_uint(x0) & 0x7fffffffu, a1 = __float_as_uint(x1) & 0x7fffffffu;
+    const uint32_t a2 = __float_as_uint(x2) & 0x7fffffffu, a3 = __float_as_uint(x3) & 0x7fffffffu;
+    return max(max(a0, a1), max(a2, a3));
+}
+
 // Largest value of a non-negative float over the 64 lanes, as its bit pattern (wave-uniform).
 __device__ __forceinline__ uint32_t wave_max_nonneg_bits(float v) {
     v = fmaxf(v, dpp_move<0xB1>(v));
