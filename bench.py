@@ -93,6 +93,27 @@ class GroupedGemv:
         _lib.check(rc, "qmm_matmul_grouped")
 
 
+class SwigluGemv:
+    """One preallocated qmm_matmul_swiglu call: silu(lhs . gate^T) * (lhs . up^T)."""
+
+    def __init__(self, enc: QE, gate: torch.Tensor, up: torch.Tensor, a: torch.Tensor):
+        self.lib = _lib.load()
+        self.enc, self.gate, self.up, self.a = enc, gate, up, a
+        self.m, self.k = a.shape
+        self.n = gate.shape[0]
+        self.out = torch.empty((self.m, self.n), dtype=torch.float32, device=a.device)
+        self.dt = _lib.QMM_F32 if a.dtype == torch.float32 else _lib.QMM_BF16
+        self.need = self.lib.qmm_matmul_swiglu_workspace_bytes(enc.code, self.dt, self.m, self.n, self.k)
+        self.ws = torch.empty((max(self.need, 1),), dtype=torch.uint8, device=a.device)
+
+    def launch(self, stream_ptr: int) -> None:
+        rc = self.lib.qmm_matmul_swiglu(self.enc.code, C.c_void_p(self.a.data_ptr()), self.dt, self.m, self.k,
+                                        C.c_void_p(self.gate.data_ptr()), C.c_void_p(self.up.data_ptr()), self.n,
+                                        C.c_void_p(self.out.data_ptr()), C.c_void_p(self.ws.data_ptr()), self.need,
+                                        C.c_void_p(stream_ptr))
+        _lib.check(rc, "qmm_matmul_swiglu")
+
+
 class GptqMatmul:
     """One preallocated GPTQ qmm_matmul call on (qweight, scales, qzeros)."""
 
@@ -379,6 +400,12 @@ def extra_timings(layers, acts, gen):
         dev_s, _ = time_graphs(graphs, 100, 10)
         sb = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
         out["q4_k_m1_grouped_4_launches"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(sb * 100 / dev_s / 1e9, 1)}
+        # ... and with the gate | up launch also applying silu(gate) * up (one output of 14336 instead of two)
+        graphs = [capture([GroupedGemv(QE.Q4_K, lw[0:3], acts[4096]), Gemv(QE.Q4_K, lw[3], acts[4096]),
+                           SwigluGemv(QE.Q4_K, lw[4], lw[5], acts[4096]), Gemv(QE.Q4_K, lw[6], acts[14336])]) for lw in layers]
+        dev_s, _ = time_graphs(graphs, 100, 10)
+        out["q4_k_m1_grouped_gated_4_launches"] = {"us_per_step": round(dev_s * 1e6 / 100, 2),
+                                                   "GB/s": round((sb - 4 * 14336) * 100 / dev_s / 1e9, 1)}
     # the optional integer-activation treatment (lhs -> Q8_K in the kernel, integer sub-block dots), M = 1 and 4
     for mm in (1, 4):
         a8 = {kk: torch.randn((mm, kk), dtype=torch.float32, device="cuda:0", generator=gen) for kk in (4096, 14336)}

@@ -147,6 +147,18 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
                        int64_t workspace_bytes, void* stream);
 
 /*
+ * The gated-MLP step either side of ops.qmatmul in a Llama block (no counterpart in the reference's op set: there the
+ * graph holds two qmatmul nodes, a SiLU and a multiply):
+ *     out fp32[m, n] = silu(lhs . dequant(gate)^T) * (lhs . dequant(up)^T),   silu(x) = x / (1 + exp(-x)).
+ * gate and up are two tensors of one GGUF encoding, uint8[n, k/epb*bpb] each.  Q4_K with one lhs row (K <= 16384) runs
+ * as ONE launch of the decode kernel with the combination as its epilogue and needs no workspace; every other shape is
+ * two qmm_matmul launches into the workspace and a combining launch.
+ */
+int64_t qmm_matmul_swiglu_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
+int qmm_matmul_swiglu(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, const void* gate, const void* up,
+                      int64_t n, float* out, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Test hook for the bit-exact integer check: raw int32 block sums
  * out[m, n, k/32] = sum_32 (q4 - 8) * q8 of Q8_0 lhs blocks (uint8[m, k/32*34])
  * against Q4_0 rhs blocks.

@@ -12,6 +12,7 @@ from .ops import (
     dequantize,
     qmatmul,
     qmatmul_grouped,
+    qmatmul_swiglu,
     quantize,
     quantize_gptq,
 )
@@ -23,6 +24,7 @@ __all__ = [
     "QuantizationEncoding",
     "qmatmul",
     "qmatmul_grouped",
+    "qmatmul_swiglu",
     "dequantize",
     "quantize",
     "quantize_gptq",

@@ -34,6 +34,8 @@ SIGNATURES = {
                           _i64, _int, _vp]),
     "qmm_matmul_grouped": (_int, [_int, _vp, _int, _i64, _i64, _int, C.POINTER(_vp), C.POINTER(_i64), C.POINTER(_vp), _vp,
                                   _i64, _vp]),
+    "qmm_matmul_swiglu_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64]),
+    "qmm_matmul_swiglu": (_int, [_int, _vp, _int, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _vp]),
     "qmm_block_dots_q4_0": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
 }
 

@@ -62,13 +62,18 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     const uint32_t ring_lds = lds_address(ring);
     float* res = (float*)(smem + kWaves * kRing * kSlot) + wave * kMaxRows * MT;
     const int gs = (int)blockIdx.x * (kWaves / WPR) + wave / WPR, GS = (int)gridDim.x * (kWaves / WPR);
-    const int my_rows = gs < n ? (n - gs + GS - 1) / GS : 0;
+    // Rows of this row stream.  Plain: gs, gs + GS, ...  Gated pair (mats.swiglu): the stream owns the row PAIRS
+    // gs, gs + GS, ... and walks gate row, up row, gate row, ...: both results of a pair end up in its own slots.
+    const bool paired = mats.swiglu != 0;
+    const int np = paired ? mats.end[0] : n;
+    const int my_rows = gs < np ? ((np - gs + GS - 1) / GS) * (paired ? 2 : 1) : 0;
+    auto row_of = [&](int ri) { return paired ? (ri & 1) * np + gs + (ri >> 1) * GS : gs + ri * GS; };
 
     // a row part into a slot.  Every one of the L instructions has a live lane in every wavefront (the mask
     // follows the full part length, a shorter last part repeats its last piece), so the wait counts stay exact.
     const int last_piece = max(nb, 1) * 9 - 1;
     auto issue = [&](int ri, int slot) {
-        const int row = gs + ri * GS;
+        const int row = row_of(ri);
         int j = 0;
         while (j + 1 < mats.count && row >= mats.end[j]) j++;  // (uniform: a few scalar compares)
         const int local = row - (j ? mats.end[j - 1] : 0);
@@ -206,20 +211,25 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
         const int nj = mats.end[j] - (j ? mats.end[j - 1] : 0);
         mats.out[j][(int64_t)mi * (ldo ? ldo : nj) + local] = v;
     };
-    if constexpr (WPR == 1) {
-        for (int idx = lane; idx < my_rows * MT; idx += 64) {
-            const int r = idx / MT, mi = idx - r * MT;
-            if (mi < m) store_row(mi, gs + r * GS, res[idx]);
-        }
-    } else {
-        __syncthreads();
-        if (part == 0) {
+    // result slot idx of this stream, the K parts added
+    auto result = [&](int idx) {
+        float v = res[idx];
+#pragma unroll
+        for (int q = 1; q < WPR; q++) v += res[q * kMaxRows * MT + idx];
+        return v;
+    };
+    if constexpr (WPR > 1) __syncthreads();
+    if (WPR == 1 || part == 0) {
+        if (paired) {
+            // (one lhs row) out[pair] = silu(gate) * up, silu(x) = x / (1 + exp(-x))
+            for (int idx = lane; idx < my_rows / 2; idx += 64) {
+                const float g = result(2 * idx), u = result(2 * idx + 1);
+                mats.out[0][gs + idx * GS] = g / (1.0f + expf(-g)) * u;
+            }
+        } else {
             for (int idx = lane; idx < my_rows * MT; idx += 64) {
                 const int r = idx / MT, mi = idx - r * MT;
-                float v = res[idx];
-#pragma unroll
-                for (int q = 1; q < WPR; q++) v += res[q * kMaxRows * MT + idx];
-                if (mi < m) store_row(mi, gs + r * GS, v);
+                if (mi < m) store_row(mi, gs + r * GS, result(idx));
             }
         }
     }
@@ -228,8 +238,10 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
 // Takes K <= 16384 and m = 1 (reports other shapes through *handled = false).  count matrices [n[j], k] share the
 // lhs; out[j] is fp32 [m, n[j]] (ldo = 0: dense; a single matrix may give its own leading dimension).
 hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
-                                          float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled) {
+                                          float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled,
+                                          bool swiglu) {
     *handled = false;
+    if (swiglu && (count != 2 || ns[0] != ns[1] || m != 1)) return hipSuccess;
     static const bool off = getenv("QMM_Q4K_LANES_OFF") != nullptr;  // read once: fallback switch
     const int nblk = (int)(k / 256);
     if (off || m > 1 || nblk > 64 || count < 1 || count > kLanesMaxMats) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
@@ -243,6 +255,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
         mats.end[j] = (int)n;
     }
     mats.count = count;
+    mats.swiglu = swiglu ? 1 : 0;
     if (n > 0x7fffffff) return hipSuccess;
     const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
     const int bpw = (nblk + wpr - 1) / wpr;
@@ -270,7 +283,8 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     if (lds > (size_t)kLdsPerCu) return hipSuccess;
     const int streams = kWaves / wpr;  // rows in progress per workgroup
     int64_t wgs = (int64_t)cus * per_cu;
-    if (wgs * streams > n) wgs = (n + streams - 1) / streams;
+    const int64_t units = swiglu ? n / 2 : n;  // rows, or gate / up row pairs, to deal to the streams
+    if (wgs * streams > units) wgs = (units + streams - 1) / streams;
     const int64_t min_wgs = (n + (int64_t)streams * kMaxRows - 1) / ((int64_t)streams * kMaxRows);
     if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots
     dim3 grid((unsigned)wgs), block(64 * kWaves);
@@ -303,9 +317,25 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     return hipGetLastError();
 }
 
+// The gated-MLP combination as a kernel of its own, for the shapes the fused epilogue above does not take.
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                     float* __restrict__ out, int64_t count) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+        const float g = gate[i];
+        out[i] = g / (1.0f + expf(-g)) * up[i];
+    }
+}
+
+hipError_t launch_swiglu(const float* gate, const float* up, float* out, int64_t count, hipStream_t s) {
+    const int64_t blocks = std::min<int64_t>((count + 255) / 256, 4096);
+    swiglu_kernel<<<dim3((unsigned)std::max<int64_t>(blocks, 1)), dim3(256), 0, s>>>(gate, up, out, count);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
                                   int64_t ldo, hipStream_t s, bool* handled) {
-    return launch_gemv_q4_k_lanes_grouped(a, a_dtype, 1, &w, &n, &out, m, k, ldo, s, handled);
+    return launch_gemv_q4_k_lanes_grouped(a, a_dtype, 1, &w, &n, &out, m, k, ldo, s, handled, false);
 }
 
 }  // namespace qmm

@@ -358,6 +358,47 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
     return QMM_OK;
 }
 
+int64_t qmm_matmul_swiglu_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    // one lhs row of Q4_K goes through the decode kernel with the combination as its epilogue: nothing to keep
+    if (encoding == QMM_Q4_K && m == 1 && k % 256 == 0 && k <= 16384) return 0;
+    return align_up(qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k), 256) + 2 * align_up(m * n * 4, 256);
+}
+
+int qmm_matmul_swiglu(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, const void* gate, const void* up,
+                      int64_t n, float* out, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (!lhs || !gate || !up || !out) return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: null pointer");
+    int64_t epb, bpb;
+    if (encoding == QMM_Q8_0 || encoding == QMM_Q8_K || encoding == QMM_GPTQ || !block_params(encoding, epb, bpb))
+        return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: encoding %d is not a GGUF weight encoding", encoding);
+    if (m <= 0 || n <= 0 || k <= 0 || k % epb || m > INT32_MAX || n > INT32_MAX / 2 || k > INT32_MAX)
+        return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: M=%lld N=%lld K=%lld (K a positive multiple of %lld)", (long long)m,
+                    (long long)n, (long long)k, (long long)epb);
+    if (lhs_dtype != QMM_F32 && lhs_dtype != QMM_BF16) return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: lhs dtype must be f32 or bf16");
+    if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: lhs must be 16-byte aligned");
+    if (encoding == QMM_Q4_K && m == 1 && k % 256 == 0 && aligned(gate, 16) && aligned(up, 16)) {
+        const uint8_t* ws[2] = {(const uint8_t*)gate, (const uint8_t*)up};
+        const int64_t ns[2] = {n, n};
+        float* outs[2] = {out, out};
+        bool handled = false;
+        hipError_t e = qmm::launch_gemv_q4_k_lanes_grouped(lhs, lhs_dtype, 2, ws, ns, outs, 1, k, 0, (hipStream_t)stream, &handled, true);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul_swiglu(Q4_K decode)");
+        if (handled) return QMM_OK;
+    }
+    // two products into the workspace, then the combination
+    const int64_t mm_ws = align_up(qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k), 256), plane = align_up(m * n * 4, 256);
+    if (!workspace || workspace_bytes < mm_ws + 2 * plane)
+        return fail(QMM_ERR_WORKSPACE, "qmm_matmul_swiglu: workspace of %lld bytes required, %lld given", (long long)(mm_ws + 2 * plane),
+                    (long long)workspace_bytes);
+    if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: workspace must be 256-byte aligned");
+    float* g = (float*)((char*)workspace + mm_ws);
+    float* u = (float*)((char*)workspace + mm_ws + plane);
+    const void* one[1] = {gate};
+    if (int rc = qmm_matmul(encoding, nullptr, lhs, lhs_dtype, m, k, one, 1, n, g, workspace, mm_ws, 0, stream)) return rc;
+    one[0] = up;
+    if (int rc = qmm_matmul(encoding, nullptr, lhs, lhs_dtype, m, k, one, 1, n, u, workspace, mm_ws, 0, stream)) return rc;
+    return hip_status(qmm::launch_swiglu(g, u, out, m * n, (hipStream_t)stream), "qmm_matmul_swiglu(combine)");
+}
+
 int qmm_block_dots_q4_0(const void* lhs_q8_0, const void* rhs_q4_0, int64_t m, int64_t n, int64_t k, int32_t* out,
                         void* stream) {
     if (!lhs_q8_0 || !rhs_q4_0 || !out) return fail(QMM_ERR_INVALID, "qmm_block_dots_q4_0: null pointer");

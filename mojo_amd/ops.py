@@ -158,6 +158,46 @@ def qmatmul_grouped(encoding: QuantizationEncoding, lhs: torch.Tensor, rhs: Sequ
     return [o.reshape(*lead, o.shape[1]) for o in outs]
 
 
+def qmatmul_swiglu(encoding: QuantizationEncoding, lhs: torch.Tensor, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(lhs @ dequantize(gate)^T) * (lhs @ dequantize(up)^T)``: the gated-MLP step around two ``qmatmul`` calls.
+
+    ``gate`` and ``up`` are packed GGUF tensors ``uint8[N, K/epb*bpb]`` of one encoding.  Q4_K with a single lhs row
+    runs as one launch (the combination is the decode kernel's epilogue); other shapes run two matmuls and a
+    combining kernel inside the library.
+    """
+    if not isinstance(encoding, QuantizationEncoding) or not encoding.is_gguf:
+        raise TypeError("qmatmul_swiglu takes a GGUF weight encoding")
+    _require_gpu(lhs, "lhs")
+    if lhs.dtype not in _DTYPES:
+        raise TypeError(f"lhs must be float32 or bfloat16, got {lhs.dtype}")
+    k = lhs.shape[-1]
+    lead = lhs.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    if m == 0:
+        raise ValueError("qmatmul of an empty tensor")
+    for w, name in ((gate, "gate"), (up, "up")):
+        _require_gpu(w, name)
+        if w.dtype != torch.uint8 or w.dim() != 2 or w.shape[0] == 0:
+            raise TypeError(f"{name} must be a non-empty rank-2 uint8 tensor of packed blocks")
+        if w.shape[1] != encoding.packed_row_bytes(k):
+            raise ValueError(
+                f"{name} rows hold {w.shape[1]} bytes; K={k} in {encoding.name} needs {encoding.packed_row_bytes(k)}")
+    if gate.shape != up.shape:
+        raise ValueError(f"gate {tuple(gate.shape)} and up {tuple(up.shape)} must have the same shape")
+    n = gate.shape[0]
+    lib = _lib.load()
+    lhs_dt = _DTYPES[lhs.dtype]
+    out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+    need = lib.qmm_matmul_swiglu_workspace_bytes(encoding.code, lhs_dt, m, n, k)
+    ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
+    rc = lib.qmm_matmul_swiglu(encoding.code, _ptr(lhs), lhs_dt, m, k, _ptr(gate), _ptr(up), n, _ptr(out), _ptr(ws), need,
+                               _stream(lhs))
+    _lib.check(rc, "qmatmul_swiglu")
+    return out.reshape(*lead, n)
+
+
 def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Optional[int] = None,
                config: Optional[QuantizationConfig] = None, dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """Unpack ``uint8[N, K/epb*bpb]`` blocks (or GPTQ tensors) to ``dtype[N, K]``."""

@@ -259,6 +259,13 @@ def matmul_gptq(a, qweight, scales, qzeros, group: int = 128, w_bf16: bool = Fal
     return out
 
 
+def swiglu(gate, up) -> np.ndarray:
+    """silu(gate) * up in fp64, silu(x) = x / (1 + exp(-x)): the gated-MLP combination of two matmul results."""
+    g = np.asarray(gate, np.float64)
+    with np.errstate(over="ignore"):
+        return g / (1.0 + np.exp(-g)) * np.asarray(up, np.float64)
+
+
 def num_threads() -> int:
     return int(lib().qo_num_threads())
 

@@ -11,7 +11,7 @@ import torch
 import oracle as O
 from conftest import synth
 from mojo_amd import QuantizationConfig, QuantizationEncoding as QE
-from mojo_amd import block_dots_q4_0, dequantize, qmatmul, qmatmul_grouped, quantize, quantize_gptq
+from mojo_amd import block_dots_q4_0, dequantize, qmatmul, qmatmul_grouped, qmatmul_swiglu, quantize, quantize_gptq
 
 pytestmark = pytest.mark.gpu
 
@@ -380,6 +380,32 @@ def test_grouped_matmul_equals_separate_calls(enc, m, k, ns, lhs_bf16):
         assert torch.equal(got[j], one), f"matrix {j} differs from the separate call"
         want = O.matmul_q4_0(a, ws[j]) if enc is QE.Q4_0 else O.matmul_f32(ENC[enc], a, ws[j])
         assert_close(got[j], want, f"grouped {enc.name} matrix {j} ({m}x{n}x{k})")
+
+
+@pytest.mark.parametrize("enc,m,n,k,bf16", [(QE.Q4_K, 1, 14336, 4096, False), (QE.Q4_K, 1, 777, 2048, True), (QE.Q4_K, 1, 130, 14336, False),
+                                            (QE.Q4_K, 1, 5, 256, False), (QE.Q4_K, 3, 200, 1024, False), (QE.Q6_K, 1, 300, 1024, False),
+                                            (QE.Q4_0, 2, 96, 512, True), (QE.Q4_K, 40, 64, 512, True)])
+def test_gated_pair_matches_two_matmuls(enc, m, n, k, bf16):
+    """silu(lhs . gate^T) * (lhs . up^T): the fused epilogue of the decode kernel (Q4_K, one lhs row: one K part, several,
+    a row count below the number of row streams) and the two-matmuls-and-combine route of every other shape, against
+    the oracle's fp64 products combined in fp64, and against the library's own separate matmuls."""
+    w, a = synth(61, 2 * n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    a_eff = a
+    if enc == QE.Q4_0:  # the Q4_0 path multiplies with the Q8_0 round trip of the lhs
+        blocks = O.quantize_q8_0(a).reshape(m, -1, 34)
+        d = O.f16_to_f32(np.ascontiguousarray(blocks[:, :, 0:2]).view(np.uint16)[..., 0])
+        a_eff = (d[..., None] * blocks[:, :, 2:].view(np.int8).astype(np.float32)).reshape(m, k)
+    wq = O.quantize(ENC[enc], w)
+    gate, up = wq[:n], wq[n:]
+    truth = O.swiglu(O.matmul_f64(ENC[enc], a_eff, gate), O.matmul_f64(ENC[enc], a_eff, up))
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul_swiglu(enc, lhs, gpu(gate), gpu(up))
+    assert got.shape == (m, n)
+    assert_close(got, truth, f"gated pair {enc.name} {m}x{n}x{k} bf16={bf16}")
+    g, u = qmatmul(enc, None, lhs, gpu(gate)).double(), qmatmul(enc, None, lhs, gpu(up)).double()
+    assert_close(got, (g / (1.0 + torch.exp(-g)) * u).cpu().numpy(), "gated pair against the separate matmuls")
 
 
 # ------------------------------------------------------------------ prefill shapes (m > 16)

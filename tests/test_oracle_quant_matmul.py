@@ -169,3 +169,19 @@ def test_isclose_is_the_reference_rule():
     assert O.isclose(0.0, 9e-5, 1e-3, 1e-4) and not O.isclose(0.0, 2e-4, 1e-3, 1e-4)
     assert O.isclose(np.inf, np.inf) and not O.isclose(np.inf, -np.inf) and not O.isclose(np.nan, np.nan)
     assert O.isclose(1000.0, 1000.9, 1e-3, 1e-4) == O.isclose(1000.9, 1000.0, 1e-3, 1e-4)
+
+
+def test_swiglu_closed_forms():
+    """silu(x) * u: zero at zero, x for large x, the reflection identity silu(x) - silu(-x) = x, the slope 1/2 at the
+    origin, the minimum -0.27846 at x = -1.27846, and no overflow at either end of the fp32 range."""
+    x = np.array([0.0, 1.0, -1.0, 30.0, -30.0, 1e30, -1e30], np.float32)
+    one = np.ones_like(x)
+    s = O.swiglu(x, one)
+    assert s[0] == 0.0 and abs(s[1] - 1.0 / (1.0 + np.exp(-1.0))) < 1e-15
+    assert np.allclose(O.swiglu(x, one) - O.swiglu(-x, one), x.astype(np.float64), rtol=1e-12)
+    assert abs(s[3] - 30.0) < 1e-11 and abs(s[4]) < 1e-11 and s[5] == np.float64(np.float32(1e30)) and s[6] == 0.0
+    assert abs(O.swiglu(np.float32(1e-6), 1.0) / 1e-6 - 0.5) < 1e-6
+    xm = -1.2784645
+    assert abs(O.swiglu(xm, 1.0) + 0.2784645) < 1e-6 and O.swiglu(xm - 0.01, 1.0) > O.swiglu(xm, 1.0) < O.swiglu(xm + 0.01, 1.0)
+    assert np.array_equal(O.swiglu(x, 3.0 * one), 3.0 * s)
+
