@@ -9,13 +9,17 @@
 // the min term) are read once, from a copy of the lhs that the workgroup stages in LDS at the start.
 //
 // A wavefront walks its rows (persistent); a row part goes as 16-byte pieces straight into a
-// private ring of four LDS slots (global_load_lds_dwordx4, up to three rows ahead, hidden from the
+// private ring of three LDS slots (global_load_lds_dwordx4, two rows ahead, hidden from the
 // compiler and waited for with exact vmcnt counts: lds_stream.h).  Per row a lane issues three
 // 16-byte LDS reads (header, 32 code bytes), masks the nibbles in place into fp16 subnormals
 // (q * 2^-24, or 16 q * 2^-24 for the high ones) and multiplies them by its fp32 activations with
 // v_fma_mix_f32; d * sc and dmin * mn are applied once per chunk.  Against the streaming kernel
 // (8 lanes per super-block, activations from LDS) this is about 150 instead of 235 vector
 // instructions per 2304-byte row, which is what bounds both.
+//
+// Up to four matrices that share the lhs go through one launch (rows numbered through the matrices).  In
+// the gated-pair mode (two matrices of equal size: gate, up) a row stream walks gate row r, up row r, gate
+// row r + GS, ... and the epilogue stores silu(gate) * up, one output row per pair.
 #include <stdlib.h>
 
 #include <algorithm>

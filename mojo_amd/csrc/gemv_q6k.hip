@@ -14,6 +14,12 @@
 // the activations, computed once per workgroup:  sum_k a_k sc (q_k - 32) = sc (sum a_k q_k) -
 // 32 sc asum16, one 16-column group per lane.  Activations come through the vector cache (a
 // 16 KB row stays resident), which keeps the LDS pipe for the weights.
+//
+// The vocabulary projection (one lhs row, K = 2048 or 4096, a 16-byte aligned tensor, many rows) takes
+// gemv_q6_k_lanes_kernel instead: a row of 8 or 16 super-blocks is a multiple of 16 bytes, so whole rows go
+// global -> LDS directly into a private ring, two rows ahead; the super-blocks of a row are dealt four to a
+// 16-lane group (block = 4 group + round), which makes the 2-byte misalignment of every field a compile-time
+// constant per round; a lane keeps the 64 activations of its four blocks in registers for the whole kernel.
 #include <stdlib.h>
 
 #include "lds_stream.h"
