@@ -118,3 +118,35 @@ def test_prefill_configuration_full_size(kind):
     ok = O.isclose(got[:, tidx].cpu().numpy(), truth, RTOL, ATOL)
     assert ok.all(), f"{kind} prefill: {(~ok).sum()}/{ok.size} sampled outputs differ from the oracle"
     check_all(got, a.double(), w32, f"{kind} prefill {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("enc,m,k,period,reps", [
+    (QE.Q4_K, 1, 4096, 9600, 100),    # 960 000 rows x 2304 B = 2.2 GB: the decode kernel's row offsets pass 2^31
+    (QE.Q4_K, 4, 4096, 9600, 100),    # the small-batch kernel
+    (QE.Q6_K, 1, 4096, 8000, 85),     # 680 000 rows x 3360 B = 2.3 GB: the vocabulary kernel
+    (QE.Q4_0, 1, 4096, 9600, 100),
+    (QE.Q4_0, 8, 4096, 9600, 100),
+])
+def test_row_offsets_beyond_two_gib(enc, m, k, period, reps):
+    """A weight tensor larger than 2^31 bytes, made of `reps` copies of the same `period` rows: every copy must
+    produce the same outputs, bit for bit (a row's arithmetic does not depend on where the row lies), and the first
+    copy must match the oracle on sampled rows.  A byte offset computed in 32 bits anywhere fails this."""
+    w, gen = weights(17, period, k)
+    base = quantize(enc, w)
+    packed = base.repeat(reps, 1)
+    assert packed.numel() > 2**31
+    a = torch.randn((m, k), dtype=torch.float32, device=DEV, generator=gen)
+    got = qmatmul(enc, None, a, packed)
+    assert got.shape == (m, period * reps)
+    first = got[:, :period]
+    assert torch.equal(got.view(m, reps, period), first.unsqueeze(1).expand(m, reps, period))
+    idx = np.sort(np.random.default_rng(3).choice(period, 32, replace=False))
+    tidx = torch.from_numpy(idx).to(DEV)
+    a_np = a.cpu().numpy()
+    a_eff = q8_0_round_trip(a_np) if enc == QE.Q4_0 else a_np
+    truth = O.matmul_f64(ENC[enc], a_eff, base[tidx].cpu().numpy())
+    assert O.isclose(first[:, tidx].cpu().numpy(), truth, RTOL, ATOL).all()
+    # the unpacker over the same tensor: the last copy equals the first
+    if m == 1:
+        deq = dequantize(enc, packed[-period:])
+        assert torch.equal(deq, dequantize(enc, base))
