@@ -259,6 +259,29 @@ def test_gptq_matmul(m, n, k):
     assert_close(got, want, f"GPTQ {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q5_K, QE.Q6_K])
+@pytest.mark.parametrize("m", [1, 4, 40])
+def test_non_finite_lhs_values_stay_in_their_row(enc, m):
+    """A NaN in the lhs gives the oracle's outputs, NaN for NaN (Q4_0: the Q8_0 quantiser's maximum search drops it on
+    both sides).  An infinity makes its whole output row non-finite on both sides; the kind may differ: the K-quant
+    kernels add the offset / min terms as separate sums, so they report NaN (inf - inf) where the element-wise
+    oracle reports +-inf.  Rows without such a value are not touched by it."""
+    w, a = synth(5, 64, 1024, m)
+    wq = O.quantize(ENC[enc], w)
+    for val in (np.nan, np.inf, -np.inf):
+        a2 = a.copy()
+        a2[0, 300] = val
+        want = O.matmul_q4_0(a2, wq) if enc == QE.Q4_0 else O.matmul_f32(ENC[enc], a2, wq)
+        got = qmatmul(enc, None, gpu(a2), gpu(wq)).cpu().numpy()
+        assert np.array_equal(np.isfinite(got[0]), np.isfinite(want[0])), f"{enc.name} m={m} {val}: finiteness of the row differs"
+        if np.isnan(val):
+            assert np.array_equal(np.isnan(got[0]), np.isnan(want[0]))
+        fin = np.isfinite(want[0])
+        assert O.isclose(got[0][fin], want[0][fin], RTOL, ATOL).all()
+        if m > 1:
+            assert_close(got[1:], want[1:], f"{enc.name} m={m}: rows next to a non-finite one")
+
+
 def test_leading_dims_broadcast():
     w, a = synth(8, 64, 512, 6)
     wq = O.quantize(O.Q4_K, w)
