@@ -353,9 +353,11 @@ static size_t q6k_rows_lds(int mt, int64_t k) {
 // (persistent) with a private ring of three LDS slots, two rows in flight (global_load_lds_dwordx4, hidden
 // from the compiler, exact vmcnt waits: lds_stream.h); no registers are spent on staging.
 // L: load instructions per row (64 pieces of 16 bytes each): 4 for 16 super-blocks, 2 for 8.
-template <int L, typename AT>
+// MT: lhs rows (1 or 2; the decode of a weight row is shared, the activations of both rows stay in registers).
+template <int MT, int L, typename AT>
 __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
-                                                              float* __restrict__ out, int n, int k, int ring_slots) {
+                                                              float* __restrict__ out, int n, int k, int ring_slots,
+                                                              int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -365,7 +367,7 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
     const int kSlot = pieces * 16 + 16;            // one dword of read-ahead past the last block
     uint8_t* ring = smem + wave * (ring_slots * kSlot);
     const uint32_t ring_lds = lds_address(ring);
-    float* park = (float*)(smem + 4 * ring_slots * kSlot) + wave * kParkRows;
+    float* park = (float*)(smem + 4 * ring_slots * kSlot) + wave * MT * kParkRows;  // [row][MT]
     const int total_waves = (int)gridDim.x * 4, gw = (int)blockIdx.x * 4 + wave;
     const int my_rows = gw < n ? (n - gw + total_waves - 1) / total_waves : 0;
     const int bq = lane >> 4, t = lane & 15, h = t >> 3, j = t & 7;
@@ -385,27 +387,31 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
     }
     // this lane's activations: per super-block slot `it`, four quartets at columns 128 h + 4 j + {0, 32, 64, 96};
     // and -32 times the sum of one 16-column group per lane (group t of the super-block)
-    float4 x[4][4];
-    float os[4], lv[4];
+    float4 x[MT][4][4];
+    float os[MT][4], lv[4];
+    float keep = 0.0f;
 #pragma unroll
     for (int it = 0; it < 4; it++) {
         const int bl = 4 * bq + it;
         lv[it] = bl < nblk ? 1.0f : 0.0f;
         const int blc = min(bl, nblk - 1);
-        const AT* ar = a + blc * 256;
-        const AT* aq = ar + 128 * h + 4 * j;
-        x[it][0] = load4(aq, 0);
-        x[it][1] = load4(aq, 32);
-        x[it][2] = load4(aq, 64);
-        x[it][3] = load4(aq, 96);
-        const AT* ag = ar + 16 * t;
-        const float4 y0 = load4(ag, 0), y1 = load4(ag, 4), y2 = load4(ag, 8), y3 = load4(ag, 12);
-        os[it] = -32.0f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
-                           ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            const AT* ar = a + (int64_t)mi * k + blc * 256;
+            const AT* aq = ar + 128 * h + 4 * j;
+            x[mi][it][0] = load4(aq, 0);
+            x[mi][it][1] = load4(aq, 32);
+            x[mi][it][2] = load4(aq, 64);
+            x[mi][it][3] = load4(aq, 96);
+            const AT* ag = ar + 16 * t;
+            const float4 y0 = load4(ag, 0), y1 = load4(ag, 4), y2 = load4(ag, 8), y3 = load4(ag, 12);
+            os[mi][it] = -32.0f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
+                                   ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
+            keep += os[mi][it];
+        }
     }
     // (ordinary loads, younger than the rows requested above: the wait for them also covers those rows, and it
     // is forced here, before the loop, so that no wait of the compiler's lands between the counted ones)
-    float keep = os[0] + os[1] + os[2] + os[3];
     asm volatile("" : "+v"(keep));
 
     // dword offsets of this lane's fields inside a super-block
@@ -420,7 +426,9 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
         // super-block 4 bq: byte 840 bq (groups past the row read the last group's blocks again; their lv is 0)
         const uint32_t* l32 = (const uint32_t*)(ring + cslot * kSlot) + 210 * min(bq, nblk / 4 - 1);
         cslot = cslot + 1 == ring_slots ? 0 : cslot + 1;
-        float v = 0.0f;
+        float v[MT];
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) v[mi] = 0.0f;
 #pragma unroll
         for (int it = 0; it < 4; it++) {
             const int q0 = (Q6_K_BPB * it) >> 2;              // dword of the super-block's first (aligned) byte
@@ -437,25 +445,36 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             const uint32_t q3 = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
             const uint32_t q4 = ((B >> 4) & 0x0F0F0F0Fu) | ((H >> 2) & 0x30303030u);
             // the int8 scales of the four quartets and of this lane's 16-column group; d once at the end
-            float u = sbyte(s0, sc_shift) * dot4u(x[it][0], q1);
-            u = fmaf(sbyte(s0, sc_shift + 16), dot4u(x[it][1], q2), u);
-            u = fmaf(sbyte(s1, sc_shift), dot4u(x[it][2], q3), u);
-            u = fmaf(sbyte(s1, sc_shift + 16), dot4u(x[it][3], q4), u);
-            u = fmaf(sbyte(j < 4 ? s0 : s1, 8 * (j & 3)), os[it], u);
-            v = fmaf(d, u, v);
+            const float c1 = sbyte(s0, sc_shift), c2 = sbyte(s0, sc_shift + 16), c3 = sbyte(s1, sc_shift), c4 = sbyte(s1, sc_shift + 16);
+            const float cg = sbyte(j < 4 ? s0 : s1, 8 * (j & 3));
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                float u = c1 * dot4u(x[mi][it][0], q1);
+                u = fmaf(c2, dot4u(x[mi][it][1], q2), u);
+                u = fmaf(c3, dot4u(x[mi][it][2], q3), u);
+                u = fmaf(c4, dot4u(x[mi][it][3], q4), u);
+                u = fmaf(cg, os[mi][it], u);
+                v[mi] = fmaf(d, u, v[mi]);
+            }
         }
-        const float sum = wave_sum_dpp_lane63(v);
-        if (lane == 63) park[ri] = sum;
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            const float sum = wave_sum_dpp_lane63(v[mi]);
+            if (lane == 63) park[ri * MT + mi] = sum;
+        }
     }
     __builtin_amdgcn_wave_barrier();
-    for (int i = lane; i < my_rows; i += 64) out[gw + (int64_t)i * total_waves] = park[i];
+    for (int i = lane; i < my_rows * MT; i += 64) {
+        const int r = i / MT, mi = i - r * MT;
+        out[(int64_t)mi * ldo + gw + (int64_t)r * total_waves] = park[i];
+    }
 }
 
 hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s, bool* handled) {
     *handled = false;
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
-    if (m > 4 || ((uintptr_t)w & 1)) return hipSuccess;
+    if (m < 1 || m > 16 || ((uintptr_t)w & 1)) return hipSuccess;
     static int cus = 0;
     if (!cus) {
         int dev = 0;
@@ -463,31 +482,45 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipGetLastError();
         cus = prop.multiProcessorCount;
     }
-    // One lhs row and enough weight rows per wavefront to amortise the per-run activation loads: the
-    // loop-interchanged kernel; otherwise the row-at-a-time kernel below.
     static const int pc_env = getenv("QMM_Q6K_WG_PER_CU") ? atoi(getenv("QMM_Q6K_WG_PER_CU")) : 0;
     const int pc = pc_env > 0 ? pc_env : 3;
     static const bool lanes_off = getenv("QMM_Q6K_LANES_OFF") != nullptr;  // read once: fallback switch
-    if (m == 1 && (k == 2048 || k == 4096) && !((uintptr_t)w & 15) && n >= (int64_t)cus * pc * 4 * 4 && !lanes_off &&
-        !env_flag_qmm_q6k_rows()) {
+    // The vocabulary shape: the kernel with whole rows global -> LDS and the activations in registers, one or two
+    // lhs rows per pass over the weights (up to 16 rows: passes of two).
+    if ((k == 2048 || k == 4096) && !((uintptr_t)w & 15) && n >= (int64_t)cus * pc * 4 * 4 && !lanes_off && !env_flag_qmm_q6k_rows()) {
         const int ring = 3;
         const size_t slot = (size_t)(k / 256) * Q6_K_BPB + 16;
-        const size_t lds3 = 4 * ring * slot + 4 * (size_t)kParkRows * 4;
-        const int64_t wgs = max((int64_t)cus * pc, (n + 4 * kParkRows - 1) / (4 * kParkRows));
-        dim3 grid3((unsigned)min(wgs, (n + 3) / 4)), block3(256);
-#define QMM_Q6K_LANES(L_)                                                                                             \
+        const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
+        for (int m0 = 0; m0 < m; m0 += 2) {
+            const int rows = min(2, m - m0);
+            const int pcl = rows == 1 ? pc : min(pc, 2);  // two lhs rows: twice the registers, two wavefronts per SIMD
+            const size_t lds3 = 4 * ring * slot + 4 * (size_t)rows * kParkRows * 4;
+            const int64_t wgs = max((int64_t)cus * pcl, (n + 4 * kParkRows - 1) / (4 * kParkRows));
+            dim3 grid3((unsigned)min(wgs, (n + 3) / 4)), block3(256);
+            const void* am = (const char*)a + (int64_t)m0 * k * esz;
+            float* om = out + (int64_t)m0 * ldo;
+#define QMM_Q6K_LANES(MT_, L_)                                                                                        \
     do {                                                                                                              \
         if (a_dtype == QMM_F32)                                                                                       \
-            gemv_q6_k_lanes_kernel<L_, float><<<grid3, block3, lds3, s>>>(w, (const float*)a, out, (int)n, (int)k, ring); \
+            gemv_q6_k_lanes_kernel<MT_, L_, float><<<grid3, block3, lds3, s>>>(w, (const float*)am, om, (int)n, (int)k, ring, ldo); \
         else                                                                                                          \
-            gemv_q6_k_lanes_kernel<L_, uint16_t><<<grid3, block3, lds3, s>>>(w, (const uint16_t*)a, out, (int)n, (int)k, ring); \
+            gemv_q6_k_lanes_kernel<MT_, L_, uint16_t><<<grid3, block3, lds3, s>>>(w, (const uint16_t*)am, om, (int)n, (int)k, ring, ldo); \
     } while (0)
-        if (k == 4096) QMM_Q6K_LANES(4);
-        else QMM_Q6K_LANES(2);
+            if (rows == 1) {
+                if (k == 4096) QMM_Q6K_LANES(1, 4);
+                else QMM_Q6K_LANES(1, 2);
+            } else {
+                if (k == 4096) QMM_Q6K_LANES(2, 4);
+                else QMM_Q6K_LANES(2, 2);
+            }
 #undef QMM_Q6K_LANES
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+        }
         *handled = true;
-        return hipGetLastError();
+        return hipSuccess;
     }
+    if (m > 4) return hipSuccess;
     if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !env_flag_qmm_q6k_rows()) {
         const size_t lds2 = 4 * (size_t)kRunBytes + 4 * (size_t)kParkRows * 4;
         // enough wavefronts that none has more rows than its LDS parking slots

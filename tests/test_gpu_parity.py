@@ -533,19 +533,22 @@ def test_q6_k_decode_many_rows(lhs_bf16):
     assert_close(got, want, f"Q6_K 1x{n}x{k} bf16={lhs_bf16}")
 
 
-@pytest.mark.parametrize("n,k,lhs_bf16", [(12418, 4096, False), (12301, 4096, True), (13000, 2048, False)])
-def test_q6_k_decode_vocabulary_shapes(n, k, lhs_bf16):
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(1, 12418, 4096, False), (1, 12301, 4096, True), (1, 13000, 2048, False),
+                                            (2, 12418, 4096, False), (3, 12301, 4096, True), (5, 13000, 2048, False),
+                                            (16, 12290, 4096, False)])
+def test_q6_k_decode_vocabulary_shapes(m, n, k, lhs_bf16):
     """K = 4096 / 2048 with many rows: the kernel with compile-time field alignment and rows delivered straight
-    into LDS (16 and 8 super-blocks per row; a row count that is not a multiple of the wavefront count)."""
-    w, a = synth(42, n, k, 1)
+    into LDS (16 and 8 super-blocks per row; a row count that is not a multiple of the wavefront count); several
+    lhs rows go through it in passes of two (an odd count ends with a pass of one)."""
+    w, a = synth(42, n, k, m)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
     wq = O.quantize(O.Q6_K, w)
     want = O.matmul_f32(O.Q6_K, a, wq)
     truth = O.matmul_f64(O.Q6_K, a, wq)
     got = qmatmul(QE.Q6_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
-    assert_close(got, want, f"Q6_K 1x{n}x{k} bf16={lhs_bf16} vs fp32 oracle")
-    assert_close(got, truth, f"Q6_K 1x{n}x{k} bf16={lhs_bf16} vs fp64 truth")
+    assert_close(got, want, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp32 oracle")
+    assert_close(got, truth, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp64 truth")
 
 
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(200, 300, 1024, False), (64, 130, 4096, True), (17, 16, 96, False),
