@@ -15,9 +15,9 @@
 // 32 sc asum16, one 16-column group per lane.  Activations come through the vector cache (a
 // 16 KB row stays resident), which keeps the LDS pipe for the weights.
 //
-// The vocabulary projection (one lhs row, K = 2048 or 4096, a 16-byte aligned tensor, many rows) takes
-// gemv_q6_k_lanes_kernel instead: a row of 8 or 16 super-blocks is a multiple of 16 bytes, so whole rows go
-// global -> LDS directly into a private ring, two rows ahead; the super-blocks of a row are dealt four to a
+// The vocabulary projection and other matrices with many rows (K a multiple of 2048, a 16-byte aligned tensor) take
+// gemv_q6_k_lanes_kernel instead: a row of 8 n super-blocks is a multiple of 16 bytes, so rows (or, beyond 16
+// super-blocks, their 2 or 4 parts, one wavefront each) go global -> LDS directly into a private ring, two ahead; the super-blocks of a row are dealt four to a
 // 16-lane group (block = 4 group + round), which makes the 2-byte misalignment of every field a compile-time
 // constant per round; a lane keeps the 64 activations of its four blocks in registers for the whole kernel.
 #include <stdlib.h>
@@ -193,6 +193,7 @@ __global__ __launch_bounds__(256) void gemv_q6_k_rows_kernel(const uint8_t* __re
 // the weights of all its rows stream through.  Per-row partial sums wait in LDS until the last
 // run (one slot per row of the wavefront, kParkRows at most).
 constexpr int kParkRows = 128;
+constexpr int kLanesSlot = (12 + 16 * Q6_K_BPB + 15) / 16 * 16 + 16;  // 3392: LDS slot of the vocabulary kernel
 
 template <int MT, typename AT>
 __global__ __launch_bounds__(256) void gemv_q6_k_slab_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
@@ -357,28 +358,40 @@ static size_t q6k_rows_lds(int mt, int64_t k) {
 template <int MT, int L, typename AT>
 __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
                                                               float* __restrict__ out, int n, int k, int ring_slots,
-                                                              int64_t ldo) {
+                                                              int64_t ldo, int wpr, int bpw) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nblk = k >> 8;                       // 8 or 16
+    const int nblk = k >> 8;                       // a multiple of 8: rows are whole 16-byte pieces
     const int64_t row_bytes = (int64_t)nblk * Q6_K_BPB;
-    const int pieces = (int)(row_bytes / 16);      // 105 or 210
-    const int kSlot = pieces * 16 + 16;            // one dword of read-ahead past the last block
+    // Rows longer than 16 super-blocks are cut into wpr (2 or 4) parts of bpw (even) super-blocks, one wavefront
+    // each; a part starts 4, 8 or 12 bytes after a 16-byte boundary at most (bpw * 210 is a multiple of 4), so the
+    // pieces are taken from the boundary below it and every field keeps its dword parity.
+    const int part = wave % wpr, blk0 = part * bpw;
+    const int nbp = max(0, min(bpw, nblk - blk0));                    // super-blocks of this part
+    const int lead = (blk0 * Q6_K_BPB) & 15;                          // bytes before the part in its first piece
+    const int pieces = (12 + bpw * Q6_K_BPB + 15) / 16;               // per slot: the longest lead-in and a full part
+    const int last_piece = (lead + max(nbp, 1) * Q6_K_BPB + 15) / 16 - 1;  // of this part (nothing past it is read)
+    const int kSlot = kLanesSlot;                  // room for 16 super-blocks whatever bpw is: lanes of a last,
+                                                   // partial group of four read (and discard) what lies behind the part
     uint8_t* ring = smem + wave * (ring_slots * kSlot);
     const uint32_t ring_lds = lds_address(ring);
     float* park = (float*)(smem + 4 * ring_slots * kSlot) + wave * MT * kParkRows;  // [row][MT]
-    const int total_waves = (int)gridDim.x * 4, gw = (int)blockIdx.x * 4 + wave;
+    const int spw = 4 / wpr;                                          // row streams per workgroup
+    const int total_waves = (int)gridDim.x * spw, gw = (int)blockIdx.x * spw + wave / wpr;
     const int my_rows = gw < n ? (n - gw + total_waves - 1) / total_waves : 0;
     const int bq = lane >> 4, t = lane & 15, h = t >> 3, j = t & 7;
     const int sc_shift = 8 * (j >> 2);
 
     // the first rows are requested before the activations, so that their latencies overlap
+    // (the mask follows the slot size, the same for every part, so each of the L instructions has a live lane in
+    // every wavefront and the wait counts stay exact; a shorter part repeats its last piece)
     auto issue = [&](int ri, int slot) {
-        const uint8_t* base = w + (int64_t)(gw + (int64_t)ri * total_waves) * row_bytes;
+        const uint8_t* base = w + (int64_t)(gw + (int64_t)ri * total_waves) * row_bytes + (int64_t)blk0 * Q6_K_BPB - lead;
 #pragma unroll
         for (int i = 0; i < L; i++)
-            if (lane + 64 * i < pieces) load16_to_lds(base + 16 * (lane + 64 * i), ring_lds + slot * kSlot + i * 1024);
+            if (lane + 64 * i < pieces)
+                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
     };
     int issued = 0, islot = 0, cslot = 0;
     for (; issued < min(ring_slots - 1, my_rows); issued++) {
@@ -388,13 +401,14 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
     // this lane's activations: per super-block slot `it`, four quartets at columns 128 h + 4 j + {0, 32, 64, 96};
     // and -32 times the sum of one 16-column group per lane (group t of the super-block)
     float4 x[MT][4][4];
-    float os[MT][4], lv[4];
+    float os[MT][4];
+    bool lv[4];  // the lane's super-block `it` exists in this part
     float keep = 0.0f;
 #pragma unroll
     for (int it = 0; it < 4; it++) {
-        const int bl = 4 * bq + it;
-        lv[it] = bl < nblk ? 1.0f : 0.0f;
-        const int blc = min(bl, nblk - 1);
+        const int bl = 4 * bq + it;                 // super-block of the part
+        lv[it] = bl < nbp;
+        const int blc = min(blk0 + bl, nblk - 1);   // of the row
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
             const AT* ar = a + (int64_t)mi * k + blc * 256;
@@ -423,8 +437,8 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             issued++;
         }
         wait_items<L, 0>(issued - 1 - ri, false);
-        // super-block 4 bq: byte 840 bq (groups past the row read the last group's blocks again; their lv is 0)
-        const uint32_t* l32 = (const uint32_t*)(ring + cslot * kSlot) + 210 * min(bq, nblk / 4 - 1);
+        // super-block 4 bq of the part: byte lead + 840 bq (groups past the part read its last group again; discarded)
+        const uint32_t* l32 = (const uint32_t*)(ring + cslot * kSlot) + (lead >> 2) + 210 * min(bq, (max(nbp, 1) - 1) / 4);
         cslot = cslot + 1 == ring_slots ? 0 : cslot + 1;
         float v[MT];
 #pragma unroll
@@ -439,7 +453,7 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             const uint32_t A = rd(o_ql), B = rd(o_ql + 8), H = rd(o_qh);
             const uint32_t s0 = rd(o_sc), s1 = rd(o_sc + 1);
             const uint32_t dv = odd ? l32[q0 + 52] >> 16 : l32[q0 + 52] & 0xffffu;
-            const float d = h2f((uint16_t)dv) * lv[it];
+            const float d = h2f((uint16_t)dv);
             const uint32_t q1 = (A & 0x0F0F0F0Fu) | ((H << 4) & 0x30303030u);
             const uint32_t q2 = (B & 0x0F0F0F0Fu) | ((H << 2) & 0x30303030u);
             const uint32_t q3 = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
@@ -454,7 +468,7 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
                 u = fmaf(c3, dot4u(x[mi][it][2], q3), u);
                 u = fmaf(c4, dot4u(x[mi][it][3], q4), u);
                 u = fmaf(cg, os[mi][it], u);
-                v[mi] = fmaf(d, u, v[mi]);
+                v[mi] = lv[it] ? fmaf(d, u, v[mi]) : v[mi];  // (a select: what a missing super-block's lanes read is arbitrary)
             }
         }
 #pragma unroll
@@ -463,10 +477,15 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             if (lane == 63) park[ri * MT + mi] = sum;
         }
     }
-    __builtin_amdgcn_wave_barrier();
-    for (int i = lane; i < my_rows * MT; i += 64) {
-        const int r = i / MT, mi = i - r * MT;
-        out[(int64_t)mi * ldo + gw + (int64_t)r * total_waves] = park[i];
+    if (wpr > 1) __syncthreads();  // (every wavefront gets here: no early exit above)
+    else __builtin_amdgcn_wave_barrier();
+    if (part == 0) {
+        for (int i = lane; i < my_rows * MT; i += 64) {
+            const int r = i / MT, mi = i - r * MT;
+            float v = park[i];
+            for (int q = 1; q < wpr; q++) v += park[q * MT * kParkRows + i];  // the other parts of the row
+            out[(int64_t)mi * ldo + gw + (int64_t)r * total_waves] = v;
+        }
     }
 }
 
@@ -485,34 +504,44 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     static const int pc_env = getenv("QMM_Q6K_WG_PER_CU") ? atoi(getenv("QMM_Q6K_WG_PER_CU")) : 0;
     const int pc = pc_env > 0 ? pc_env : 3;
     static const bool lanes_off = getenv("QMM_Q6K_LANES_OFF") != nullptr;  // read once: fallback switch
-    // The vocabulary shape: the kernel with whole rows global -> LDS and the activations in registers, one or two
-    // lhs rows per pass over the weights (up to 16 rows: passes of two).
-    if ((k == 2048 || k == 4096) && !((uintptr_t)w & 15) && n >= (int64_t)cus * pc * 4 * 4 && !lanes_off && !env_flag_qmm_q6k_rows()) {
+    // Rows of whole 16-byte pieces (K a multiple of 2048, up to 16384) and enough of them: the kernel with the rows
+    // global -> LDS and the activations in registers, one or two lhs rows per pass over the weights (up to 16 rows:
+    // passes of two).  Rows longer than 16 super-blocks are cut into 2 or 4 parts, one wavefront each.
+    const int nblk = (int)(k / 256);
+    const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
+    static const int64_t min_parts = getenv("QMM_Q6K_LANES_MIN") ? atoll(getenv("QMM_Q6K_LANES_MIN")) : 0;  // read once: tuning
+    const int64_t need_parts = min_parts > 0 ? min_parts : (int64_t)cus * 4 * 8;  // below 8 row parts per wavefront of a one-workgroup-per-CU grid the row-at-a-time kernel is faster
+    if (k % 2048 == 0 && nblk <= 64 && !((uintptr_t)w & 15) && n * wpr >= need_parts && !lanes_off && !env_flag_qmm_q6k_rows()) {
         const int ring = 3;
-        const size_t slot = (size_t)(k / 256) * Q6_K_BPB + 16;
+        const int bpw = nblk / wpr;                                  // 8 .. 16, even
+        const int pieces = (12 + bpw * Q6_K_BPB + 15) / 16;
+        const int l = (pieces + 63) / 64;                            // 2 .. 4 load instructions per row part
+        const int spw = 4 / wpr;
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
         for (int m0 = 0; m0 < m; m0 += 2) {
             const int rows = min(2, m - m0);
             const int pcl = rows == 1 ? pc : min(pc, 2);  // two lhs rows: twice the registers, two wavefronts per SIMD
-            const size_t lds3 = 4 * ring * slot + 4 * (size_t)rows * kParkRows * 4;
-            const int64_t wgs = max((int64_t)cus * pcl, (n + 4 * kParkRows - 1) / (4 * kParkRows));
-            dim3 grid3((unsigned)min(wgs, (n + 3) / 4)), block3(256);
+            const size_t lds3 = 4 * ring * (size_t)kLanesSlot + 4 * (size_t)rows * kParkRows * 4;
+            const int64_t wgs = max((int64_t)cus * pcl, (n + (int64_t)spw * kParkRows - 1) / ((int64_t)spw * kParkRows));
+            dim3 grid3((unsigned)min(wgs, (n + spw - 1) / spw)), block3(256);
             const void* am = (const char*)a + (int64_t)m0 * k * esz;
             float* om = out + (int64_t)m0 * ldo;
 #define QMM_Q6K_LANES(MT_, L_)                                                                                        \
     do {                                                                                                              \
         if (a_dtype == QMM_F32)                                                                                       \
-            gemv_q6_k_lanes_kernel<MT_, L_, float><<<grid3, block3, lds3, s>>>(w, (const float*)am, om, (int)n, (int)k, ring, ldo); \
+            gemv_q6_k_lanes_kernel<MT_, L_, float><<<grid3, block3, lds3, s>>>(w, (const float*)am, om, (int)n, (int)k, ring, ldo, wpr, bpw); \
         else                                                                                                          \
-            gemv_q6_k_lanes_kernel<MT_, L_, uint16_t><<<grid3, block3, lds3, s>>>(w, (const uint16_t*)am, om, (int)n, (int)k, ring, ldo); \
+            gemv_q6_k_lanes_kernel<MT_, L_, uint16_t><<<grid3, block3, lds3, s>>>(w, (const uint16_t*)am, om, (int)n, (int)k, ring, ldo, wpr, bpw); \
     } while (0)
-            if (rows == 1) {
-                if (k == 4096) QMM_Q6K_LANES(1, 4);
-                else QMM_Q6K_LANES(1, 2);
-            } else {
-                if (k == 4096) QMM_Q6K_LANES(2, 4);
-                else QMM_Q6K_LANES(2, 2);
-            }
+#define QMM_Q6K_LANES_L(MT_)               \
+    do {                                   \
+        if (l == 2) QMM_Q6K_LANES(MT_, 2); \
+        else if (l == 3) QMM_Q6K_LANES(MT_, 3); \
+        else QMM_Q6K_LANES(MT_, 4);        \
+    } while (0)
+            if (rows == 1) QMM_Q6K_LANES_L(1);
+            else QMM_Q6K_LANES_L(2);
+#undef QMM_Q6K_LANES_L
 #undef QMM_Q6K_LANES
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) return e;

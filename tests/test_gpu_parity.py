@@ -535,11 +535,14 @@ def test_q6_k_decode_many_rows(lhs_bf16):
 
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(1, 12418, 4096, False), (1, 12301, 4096, True), (1, 13000, 2048, False),
                                             (2, 12418, 4096, False), (3, 12301, 4096, True), (5, 13000, 2048, False),
-                                            (16, 12290, 4096, False)])
+                                            (16, 12290, 4096, False), (1, 4096, 14336, False), (2, 2100, 14336, True),
+                                            (1, 4100, 6144, False), (3, 2050, 10240, False), (1, 2049, 16384, True),
+                                            (1, 8200, 2048, False)])
 def test_q6_k_decode_vocabulary_shapes(m, n, k, lhs_bf16):
     """K = 4096 / 2048 with many rows: the kernel with compile-time field alignment and rows delivered straight
     into LDS (16 and 8 super-blocks per row; a row count that is not a multiple of the wavefront count); several
-    lhs rows go through it in passes of two (an odd count ends with a pass of one)."""
+    lhs rows go through it in passes of two (an odd count ends with a pass of one); rows longer than 16 super-blocks
+    are cut into 2 or 4 parts of 10, 12, 14 or 16 super-blocks (a last group of four with two blocks missing)."""
     w, a = synth(42, n, k, m)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
