@@ -250,7 +250,7 @@ def test_q5_k_decode_shapes(m, n, k, bf16):
     assert_close(got, truth, f"Q5_K {m}x{n}x{k} bf16={bf16}")
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256)])
+@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256), (1, 14336, 4096), (3, 200, 14336)])
 def test_gptq_matmul(m, n, k):
     w, a = synth(5, n, k, m)
     qw, sc, qz, gi = O.quantize_gptq(w)
@@ -280,6 +280,24 @@ def test_non_finite_lhs_values_stay_in_their_row(enc, m):
         assert O.isclose(got[0][fin], want[0][fin], RTOL, ATOL).all()
         if m > 1:
             assert_close(got[1:], want[1:], f"{enc.name} m={m}: rows next to a non-finite one")
+
+
+@pytest.mark.parametrize("m,n,k,group,bf16", [(1, 264, 1024, 32, False), (2, 72, 2048, 64, True), (4, 136, 4096, 256, False),
+                                               (1, 64, 28672, 128, False), (3, 8, 512, 128, False), (1, 128, 480, 96, False)])
+def test_gptq_decode_group_sizes(m, n, k, group, bf16):
+    """Group sizes 32, 64, 96, 128 and 256 through the decode kernel (4 or 16 packed rows per inner step), a long K,
+    N of eight columns, arbitrary zero points."""
+    w, a = synth(71, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    rng = np.random.Generator(np.random.PCG64(72))
+    qz = rng.integers(0, 2**32, size=qz.shape, dtype=np.uint64).astype(np.uint32).view(np.int32)  # any zero point
+    truth = O.matmul_gptq(a, qw, sc, qz, group, f64=True)
+    cfg = QuantizationConfig(group_size=group, sym=False)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.GPTQ, cfg, lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, truth, f"GPTQ decode {m}x{n}x{k} group={group}")
 
 
 def test_leading_dims_broadcast():
