@@ -5,9 +5,11 @@
 // 256 contiguous bytes.  The eight wavefronts of a workgroup share 64 columns and split the groups
 // of K between them; every wavefront issues all the loads of a group (group/8 dwords per lane)
 // before it touches the first one, so the memory latency is paid once per group, not once per row.
-// The activations a wavefront needs for a k8 row are the same for all its lanes; they are read with
-// wave-uniform addresses.  Per-group activation sums (for the zero point) are computed once per
-// workgroup into LDS:  sum_k a_k s (q_k - z) = s (sum a_k q_k - z asum_g).
+// The activations a wavefront needs for a k8 row are the same for all its lanes: the wavefront loads
+// a group's activations once (coalesced), parks them in LDS lines of its own and reads them back as
+// broadcasts; their sum, for the zero point, falls out on the way:
+// sum_k a_k s (q_k - z) = s (sum a_k q_k - z asum_g).  Nothing is shared between wavefronts before
+// the final sum over the K shares.
 #include <stdlib.h>
 
 #include "qmm_internal.h"
@@ -41,21 +43,8 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols_kernel(const uint3
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ngroups = k / group, rows_per_group = group >> 3;
-    float* asum = gsm;                       // [MT][ngroups]
-    float* red = gsm + MT * ngroups;         // [kWaves][MT][64]
-
-    // per-group activation sums: one wavefront per (lhs row, group) item, lanes stride the group
-    for (int gi = wave; gi < MT * ngroups; gi += kWaves) {
-        const int mi = gi / ngroups, g = gi - mi * ngroups;
-        float s = 0.0f;
-        if (mi < m) {
-            const AT* ar = a + (int64_t)mi * k + (int64_t)g * group;
-            for (int i = lane; i < group; i += 64) s += act(ar, i);
-        }
-        s = wave_sum(s);
-        if (lane == 0) asum[gi] = s;
-    }
-    __syncthreads();
+    float* red = gsm;                                  // [kWaves][MT][64]
+    float* mine = gsm + kWaves * MT * 64 + wave * MT * group;  // this wavefront's copy of a group's activations: [MT][group]
 
     const int col = (int)blockIdx.x * 64 + lane;
     const int ccol = min(col, n - 1);
@@ -67,9 +56,22 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols_kernel(const uint3
     for (int g = wave; g < ngroups; g += kWaves) {
         const float sc = h2f(scales[(int64_t)g * n + ccol]);
         const float z = (float)(((qzeros[(int64_t)g * (n >> 3) + (ccol >> 3)] >> zshift) & 0xFu) + 1u);
-        float part[MT];
+        // The group's activations: loaded once by the wavefront (coalesced), parked in its own LDS lines and read
+        // back as broadcasts (every lane needs the same value at the same time); their sum for the zero point on
+        // the way.  LDS operations of one wavefront are performed in order, so no barrier is needed.
+        float gsum[MT], part[MT];
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++) part[mi] = 0.0f;
+        for (int mi = 0; mi < MT; mi++) {
+            const AT* ar = a + (int64_t)min(mi, m - 1) * k + (int64_t)g * group;
+            float s = 0.0f;
+            for (int i = lane; i < group; i += 64) {
+                const float v = act(ar, i);
+                mine[mi * group + i] = v;
+                s += v;
+            }
+            gsum[mi] = wave_sum(s);
+            part[mi] = 0.0f;
+        }
         for (int r0 = 0; r0 < rows_per_group; r0 += ROWS) {
             const int64_t k8 = (int64_t)g * rows_per_group + r0;
             uint32_t x[ROWS];
@@ -82,21 +84,22 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols_kernel(const uint3
                 const float w1 = gub0(qo), w3 = gub1(qo), w5 = gub2(qo), w7 = gub3(qo);
 #pragma unroll
                 for (int mi = 0; mi < MT; mi++) {
-                    const AT* ar = a + (int64_t)(mi < m ? mi : 0) * k + (k8 + j) * 8;  // wave-uniform address
+                    const float4* ap = (const float4*)(mine + mi * group + (r0 + j) * 8);  // the same address in every lane
+                    const float4 a0 = ap[0], a1 = ap[1];
                     float t = part[mi];
-                    t = fmaf(w0, act(ar, 0), t);
-                    t = fmaf(w1, act(ar, 1), t);
-                    t = fmaf(w2, act(ar, 2), t);
-                    t = fmaf(w3, act(ar, 3), t);
-                    t = fmaf(w4, act(ar, 4), t);
-                    t = fmaf(w5, act(ar, 5), t);
-                    t = fmaf(w6, act(ar, 6), t);
-                    part[mi] = fmaf(w7, act(ar, 7), t);
+                    t = fmaf(w0, a0.x, t);
+                    t = fmaf(w1, a0.y, t);
+                    t = fmaf(w2, a0.z, t);
+                    t = fmaf(w3, a0.w, t);
+                    t = fmaf(w4, a1.x, t);
+                    t = fmaf(w5, a1.y, t);
+                    t = fmaf(w6, a1.z, t);
+                    part[mi] = fmaf(w7, a1.w, t);
                 }
             }
         }
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++) acc[mi] = fmaf(sc, fmaf(-z, asum[mi * ngroups + g], part[mi]), acc[mi]);
+        for (int mi = 0; mi < MT; mi++) acc[mi] = fmaf(sc, fmaf(-z, gsum[mi], part[mi]), acc[mi]);
     }
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) red[(wave * MT + mi) * 64 + lane] = acc[mi];
@@ -120,7 +123,7 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
     *handled = false;
     if (m > 4 || group % 32) return hipSuccess;
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
-    const size_t lds = ((size_t)mt * (k / group) + (size_t)kWaves * mt * 64) * 4;
+    const size_t lds = ((size_t)kWaves * mt * group + (size_t)kWaves * mt * 64) * 4;
     if (lds > 64 * 1024) return hipSuccess;
     dim3 grid((unsigned)((n + 63) / 64)), block(64 * kWaves);
 #define QMM_GPTQ_GO(MT_, ROWS_)                                                                                       \
