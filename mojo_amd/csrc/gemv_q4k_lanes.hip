@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
                 load16_to_lds(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
     };
 
-    // --- the lane's chunk: super-block blk0 + lane / 4 (clamped: lanes past the part get zero activations),
+    // --- the lane's chunk: super-block blk0 + lane / 4 (clamped: lanes past the part repeat its last super-block; their sum is dropped),
     //     chunk c = lane % 4.  The lhs rows are staged once per workgroup: coalesced 16-byte pieces straight
     //     into LDS, laid out as one record per 64-column chunk (its pieces plus one piece of padding, so that
     //     the lanes' 16-byte reads of their own records spread over the banks), issued before the first weight
@@ -140,8 +140,8 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
         float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
         for (int i = 0; i < 32; i++) {
-            alo[mi][i] = live ? v[i] : 0.0f;
-            ahi[mi][i] = live ? v[32 + i] : 0.0f;
+            alo[mi][i] = v[i];
+            ahi[mi][i] = v[32 + i];
         }
 #pragma unroll
         for (int i = 0; i < 32; i += 4) {
@@ -204,6 +204,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             t = fmaf(-m1, slo_a[mi], t);
             t = fmaf(d2, shi[mi], t);
             t = fmaf(-m2, shi_a[mi], t);
+            t = live ? t : 0.0f;  // lanes past the part decoded its last super-block again (valid data): dropped here
             const float v = wave_sum_dpp_lane63(t);
             if (lane == 63) res[ri * MT + mi] = v;
         }
