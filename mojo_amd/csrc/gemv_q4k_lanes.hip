@@ -48,8 +48,16 @@ __device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ub
 // (matrix j owns rows [end[j - 1], end[j])), so one launch serves q|k|v or gate|up.
 template <int MT, int WPR, int L, typename AT>
 __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const LanesMats mats, const AT* __restrict__ a,
-                                                                        int m, int k, int64_t ldo, int ring_slots) {
-    const int n = mats.end[mats.count - 1];
+                                                                        int m, int k, int64_t ldo, int ring_slots,
+                                                                        int streams, int rows_each, int rows_extra) {
+    // One matrix (the plain call) needs nothing from the argument block per row.  With several, the row's matrix is
+    // looked up in the block: a dependent scalar load per row, a round trip to memory while the scalar cache is
+    // cold, which a short launch cannot hide; the grouped launches are long enough.
+    const bool single = mats.count == 1;
+    const uint8_t* const w0 = mats.w[0];
+    float* const o0 = mats.out[0];
+    const int e0 = mats.end[0];
+    const int n = mats.end[kLanesMaxMats - 1];  // (entries past count repeat the last one)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -65,27 +73,34 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     uint8_t* ring = smem + wave * (kRing * kSlot);
     const uint32_t ring_lds = lds_address(ring);
     float* res = (float*)(smem + kWaves * kRing * kSlot) + wave * kMaxRows * MT;
-    const int gs = (int)blockIdx.x * (kWaves / WPR) + wave / WPR, GS = (int)gridDim.x * (kWaves / WPR);
+    const int gs = (int)blockIdx.x * (kWaves / WPR) + wave / WPR, GS = streams;  // streams = workgroups * kWaves / WPR
     // Rows of this row stream.  Plain: gs, gs + GS, ...  Gated pair (mats.swiglu): the stream owns the row PAIRS
     // gs, gs + GS, ... and walks gate row, up row, gate row, ...: both results of a pair end up in its own slots.
     const bool paired = mats.swiglu != 0;
-    const int np = paired ? mats.end[0] : n;
-    const int my_rows = gs < np ? ((np - gs + GS - 1) / GS) * (paired ? 2 : 1) : 0;
-    auto row_of = [&](int ri) { return paired ? (ri & 1) * np + gs + (ri >> 1) * GS : gs + ri * GS; };
+    const int np = paired ? e0 : n;
+    // rows (or pairs) of this stream: np / GS, one more for the first np % GS streams (the host did the division)
+    const int my_rows = (rows_each + (gs < rows_extra ? 1 : 0)) * (paired ? 2 : 1);
+    auto row_of = [&](int ri) __attribute__((always_inline)) { return paired ? (ri & 1) * np + gs + (ri >> 1) * GS : gs + ri * GS; };
 
     // a row part into a slot.  Every one of the L instructions has a live lane in every wavefront (the mask
     // follows the full part length, a shorter last part repeats its last piece), so the wait counts stay exact.
     const int last_piece = max(nb, 1) * 9 - 1;
-    auto issue = [&](int ri, int slot) {
+    auto issue = [&](int ri, int slot) __attribute__((always_inline)) {
         const int row = row_of(ri);
-        int j = 0;
-        while (j + 1 < mats.count && row >= mats.end[j]) j++;  // (uniform: a few scalar compares)
-        const int local = row - (j ? mats.end[j - 1] : 0);
-        const uint8_t* base = mats.w[j] + (int64_t)local * row_bytes + (int64_t)blk0 * Q4_K_BPB;
+        const uint8_t* wp = w0;
+        int local = row;
+        if (!single) {
+            int j = 0;
+            while (j + 1 < mats.count && row >= mats.end[j]) j++;  // (uniform: a few scalar compares)
+            local = row - (j ? mats.end[j - 1] : 0);
+            wp = mats.w[j];
+        }
+        const uint8_t* base = wp + (int64_t)local * row_bytes + (int64_t)blk0 * Q4_K_BPB;
 #pragma unroll
         for (int i = 0; i < L; i++)
             if (lane + 64 * i < pieces)
-                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
+                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece),
+                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(ring_lds + slot * kSlot + i * 1024)));  // (uniform; says so)
     };
 
     // --- the lane's chunk: super-block blk0 + lane / 4 (clamped: lanes past the part repeat its last super-block; their sum is dropped),
@@ -209,15 +224,20 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             if (lane == 63) res[ri * MT + mi] = v;
         }
     }
-    auto store_row = [&](int mi, int row, float v) {
-        int j = 0;
-        while (j + 1 < mats.count && row >= mats.end[j]) j++;
-        const int local = row - (j ? mats.end[j - 1] : 0);
-        const int nj = mats.end[j] - (j ? mats.end[j - 1] : 0);
-        mats.out[j][(int64_t)mi * (ldo ? ldo : nj) + local] = v;
+    auto store_row = [&](int mi, int row, float v) __attribute__((always_inline)) {
+        float* op = o0;
+        int local = row, nj = e0;
+        if (!single) {
+            int j = 0;
+            while (j + 1 < mats.count && row >= mats.end[j]) j++;
+            local = row - (j ? mats.end[j - 1] : 0);
+            nj = mats.end[j] - (j ? mats.end[j - 1] : 0);
+            op = mats.out[j];
+        }
+        op[(int64_t)mi * (ldo ? ldo : nj) + local] = v;
     };
     // result slot idx of this stream, the K parts added
-    auto result = [&](int idx) {
+    auto result = [&](int idx) __attribute__((always_inline)) {
         float v = res[idx];
 #pragma unroll
         for (int q = 1; q < WPR; q++) v += res[q * kMaxRows * MT + idx];
@@ -229,7 +249,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             // (one lhs row) out[pair] = silu(gate) * up, silu(x) = x / (1 + exp(-x))
             for (int idx = lane; idx < my_rows / 2; idx += 64) {
                 const float g = result(2 * idx), u = result(2 * idx + 1);
-                mats.out[0][gs + idx * GS] = g / (1.0f + expf(-g)) * u;
+                o0[gs + idx * GS] = g / (1.0f + expf(-g)) * u;
             }
         } else {
             for (int idx = lane; idx < my_rows * MT; idx += 64) {
@@ -293,11 +313,14 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     const int64_t min_wgs = (n + (int64_t)streams * kMaxRows - 1) / ((int64_t)streams * kMaxRows);
     if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots
     dim3 grid((unsigned)wgs), block(64 * kWaves);
+    const int total_streams = (int)wgs * streams;
 #define QMM_GO3(MT_, WPR_, L_, AT_)                                                                                   \
     do {                                                                                                              \
         hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_>>();                                \
         if (e_ != hipSuccess) return e_;                                                                              \
-        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring); \
+        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring,   \
+                                                                            total_streams, (int)(units / total_streams), \
+                                                                            (int)(units % total_streams));           \
     } while (0)
 #define QMM_GO2(MT_, WPR_, L_)                            \
     do {                                                  \

@@ -81,7 +81,13 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
     uint8_t* ring = smem + wave * (kSlots * kSlotBytes);
     const uint32_t ring_lds = lds_address(ring);
     float* accs = (float*)(smem + kRingBytes);  // [kWaves][kMaxTiles][4][64]
-    const int ntiles = mats.tile_end[mats.count - 1];  // 16-row tiles, numbered through the matrices
+    const int ntiles = mats.tile_end[kLanesMaxMats - 1];  // 16-row tiles, numbered through the matrices (entries past count repeat the last)
+    // One matrix (the plain call) needs nothing from the argument block per item; with several, the tile's matrix is
+    // looked up there (dependent scalar loads per item).
+    const bool single = mats.count == 1;
+    const uint8_t* const w_first = mats.w[0];
+    float* const out_first = mats.out[0];
+    const int n_first = mats.n[0];
     const int my_tiles = min(kMaxTiles, (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
     // group g is super-blocks [16 g, 16 g + 16): two per wavefront, or, when 8 or fewer are left, one
     const int ngrp = (nblk + kRunBlk * kWaves - 1) / (kRunBlk * kWaves);
@@ -105,13 +111,19 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
     // item (group g, tile index t) -> ring slot `slot`
     auto issue = [&](int g, int t, int slot) {
         const int tile = (int)blockIdx.x + t * (int)gridDim.x;
-        int j = 0;
-        while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;  // (uniform: a few scalar compares)
-        const int n0 = (tile - (j ? mats.tile_end[j - 1] : 0)) * 16, n = mats.n[j];
+        int n0 = tile * 16, n = n_first;
+        const uint8_t* wj = w_first;
+        if (!single) {
+            int j = 0;
+            while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;  // (uniform: a few scalar compares)
+            n0 = (tile - (j ? mats.tile_end[j - 1] : 0)) * 16;
+            n = mats.n[j];
+            wj = mats.w[j];
+        }
         int bc, cnt;
         group_share(g, bc, cnt);
         const int last_piece = max(cnt, 1) * 9 - 1;
-        const uint8_t* base = mats.w[j] + (int64_t)bc * Q4_K_BPB;
+        const uint8_t* base = wj + (int64_t)bc * Q4_K_BPB;
 #pragma unroll
         for (int i = 0; i < kLoads; i++) {
             const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * min(pidx[i], last_piece);
@@ -372,11 +384,16 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
     for (int pr = wave; pr < my_tiles * 4; pr += kWaves) {
         const int t = pr >> 2, r = pr & 3;
         const int tile = (int)blockIdx.x + t * (int)gridDim.x;
-        int j = 0;
-        while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;
-        const int n = mats.n[j];
-        float* out = mats.out[j];
-        const int col = (tile - (j ? mats.tile_end[j - 1] : 0)) * 16 + nn, row = 4 * kg + r;
+        int n = n_first, tile0 = 0;
+        float* out = out_first;
+        if (!single) {
+            int j = 0;
+            while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;
+            n = mats.n[j];
+            out = mats.out[j];
+            tile0 = j ? mats.tile_end[j - 1] : 0;
+        }
+        const int col = (tile - tile0) * 16 + nn, row = 4 * kg + r;
         float v = 0.0f;
 #pragma unroll
         for (int ww = 0; ww < kWaves; ww++) {
