@@ -586,3 +586,60 @@ def test_q4_0_matmul_int8_matrix_cores(m, n, k, lhs_bf16):
     want = O.matmul_q4_0(a, wq)
     got = qmatmul(QE.Q4_0, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
     assert_close(got, want, f"Q4_0 {m}x{n}x{k} bf16={lhs_bf16}")
+
+
+def test_graph_capture_and_replay_match_eager():
+    """The library only enqueues kernels on the caller's stream (no allocation, no synchronisation, no memset), so
+    calls can be captured into a HIP graph: replays with new lhs values in the same buffers must give what eager
+    calls give, for a decode call, a small-batch call, a Q4_0 call with its workspace, a gated pair and a prefill GEMM
+    with its lhs pass."""
+    from mojo_amd import _lib
+    import ctypes as C
+
+    lib = _lib.load()
+    n, k = 512, 1024
+    w, _ = synth(81, 2 * n, k, 1)
+    wk = gpu(O.quantize(O.Q4_K, w))
+    w0 = gpu(O.quantize(O.Q4_0, w[:n]))
+    cases = [(QE.Q4_K, wk[:n], 1), (QE.Q4_K, wk[:n], 4), (QE.Q4_0, w0, 3), (QE.Q4_K, wk[:n], 40)]
+    bufs = []
+    for enc, wt, m in cases:
+        a = torch.zeros((m, k), dtype=torch.float32, device=DEV)
+        out = torch.empty((m, n), dtype=torch.float32, device=DEV)
+        need = lib.qmm_matmul_workspace_bytes(enc.code, _lib.QMM_F32, m, n, k)
+        ws = torch.empty((max(need, 1),), dtype=torch.uint8, device=DEV)
+        bufs.append((enc, wt, m, a, out, ws, need))
+    ag = torch.zeros((1, k), dtype=torch.float32, device=DEV)
+    og = torch.empty((1, n), dtype=torch.float32, device=DEV)
+
+    def enqueue(stream):
+        for enc, wt, m, a, out, ws, need in bufs:
+            ptrs = (C.c_void_p * 1)(wt.data_ptr())
+            rc = lib.qmm_matmul(enc.code, None, C.c_void_p(a.data_ptr()), _lib.QMM_F32, m, k, ptrs, 1, n,
+                                C.c_void_p(out.data_ptr()), C.c_void_p(ws.data_ptr()), need, 0, C.c_void_p(stream))
+            assert rc == 0, lib.qmm_last_error()
+        rc = lib.qmm_matmul_swiglu(QE.Q4_K.code, C.c_void_p(ag.data_ptr()), _lib.QMM_F32, 1, k, C.c_void_p(wk[:n].data_ptr()),
+                                   C.c_void_p(wk[n:].data_ptr()), n, C.c_void_p(og.data_ptr()), None, 0, C.c_void_p(stream))
+        assert rc == 0, lib.qmm_last_error()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        enqueue(side.cuda_stream)  # warm every kernel outside the capture
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            enqueue(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    rng = np.random.Generator(np.random.PCG64(82))
+    for rep in range(3):
+        for _, _, m, a, _, _, _ in bufs:
+            a.copy_(gpu(rng.standard_normal((m, k), dtype=np.float32)))
+        ag.copy_(gpu(rng.standard_normal((1, k), dtype=np.float32)))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for enc, wt, m, a, out, _, _ in bufs:
+            want = qmatmul(enc, None, a, wt)
+            assert torch.equal(out, want), f"replay {rep}: {enc.name} m={m} differs from the eager call"
+        assert torch.equal(og, qmatmul_swiglu(QE.Q4_K, ag, wk[:n], wk[n:])), f"replay {rep}: gated pair differs"
