@@ -643,3 +643,38 @@ def test_graph_capture_and_replay_match_eager():
             want = qmatmul(enc, None, a, wt)
             assert torch.equal(out, want), f"replay {rep}: {enc.name} m={m} differs from the eager call"
         assert torch.equal(og, qmatmul_swiglu(QE.Q4_K, ag, wk[:n], wk[n:])), f"replay {rep}: gated pair differs"
+
+
+def test_concurrent_calls_on_two_streams():
+    """Entry points are re-entrant: two host threads, each with its own stream, issue different encodings at the same
+    time (ctypes drops the GIL inside the calls); every result equals the single-threaded one."""
+    import threading
+
+    n, k = 1024, 2048
+    w, a = synth(91, n, k, 4)
+    jobs = [(QE.Q4_K, gpu(O.quantize(O.Q4_K, w)), gpu(a[:1])), (QE.Q6_K, gpu(O.quantize(O.Q6_K, w)), gpu(a[:1])),
+            (QE.Q4_0, gpu(O.quantize(O.Q4_0, w)), gpu(a)), (QE.Q4_K, gpu(O.quantize(O.Q4_K, w)), gpu(a))]
+    want = [qmatmul(enc, None, lhs, wq).clone() for enc, wq, lhs in jobs]
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(offset):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                for it in range(40):
+                    j = (it + offset) % len(jobs)
+                    enc, wq, lhs = jobs[j]
+                    got = qmatmul(enc, None, lhs, wq)
+                    s.synchronize()
+                    if not torch.equal(got, want[j]):
+                        errors.append(f"thread {offset} iteration {it}: {enc.name} differs")
+        except Exception as e:  # noqa: BLE001
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(o,)) for o in (0, 2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]
