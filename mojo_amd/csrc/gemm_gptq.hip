@@ -5,7 +5,13 @@
 // the order (0,4,1,5,2,6,3,7) inside each 8-group and its odd columns pre-multiplied
 // by 1/16, the four fp16 pairs  x & 0x000F000F,  x & 0x00F000F0,  (x>>8) & 0x000F000F,
 // (x>>8) & 0x00F000F0  are the matrix-core B operand directly: fp16 subnormals q*2^-24
-// (or 16q*2^-24), no multiply needed because the scale is per group, not per 32.
+// (or 16q*2^-24), no multiply needed because the scale is per group, not per 32.  For an
+// fp32 lhs the nibbles are moved two bits up inside the subnormal's mantissa (x << 2 and
+// x >> 6, masks shifted likewise: q*2^-22): the matrix core does not normalise subnormal
+// inputs before it aligns the products of a step, and the low bits of long products (the
+// residual plane's most of all) then fall off the end of the adder, always towards minus
+// infinity: with non-negative codes a bias that grows with K (unit-size activations,
+// K = 14336: 2e-4 with the nibbles low, 4.5e-5 with them here; bf16 lhs: 1e-6).
 // Per group g the matrix cores produce  P[m][n] = sum_k a[m][k]*q[k][n]  exactly (fp32
 // sums), and the lanes apply  acc += scale[g][n] * P.  The zero-point term
 // -scale*zero * sum_k a[m][k]  is a second small matrix product over the 32-wide
@@ -28,7 +34,7 @@ namespace {
 
 constexpr int BM = 128, BN = 256;
 constexpr int A_STRIDE = 72;
-constexpr float kTwo24 = 16777216.0f;
+constexpr float kTwo24 = 16777216.0f, kTwo22 = 4194304.0f;
 
 }  // namespace
 
@@ -186,7 +192,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
 #pragma unroll
                 for (int i = 0; i < GB; i++) {
                     const uint32_t sb = sc_n[ni][i] & 0xffffu;
-                    gscale[ni][i] = h2f((uint16_t)sb) * kTwo24;
+                    gscale[ni][i] = h2f((uint16_t)sb) * (NPART == 2 ? kTwo22 : kTwo24);
                     const float z = (float)(((zw_n[ni][i] >> (ni == 0 ? zshift0 : zshift1)) & 0xFu) + 1u);
                     const uint32_t nsc = (sb ^ 0x8000u) * 0x00010001u;  // (-scale, -scale)
                     const uint32_t zp = pack_half2(z, z);
@@ -213,12 +219,16 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
         }
 
         // ---- one 64-wide chunk: four 16-wide operand slices, one packed dword per column each
-        const uint32_t M1 = 0x000F000Fu, M2 = 0x00F000F0u;
+        // nibble positions inside the fp16 halves: bits 2..5 / 6..9 for an fp32 lhs (two planes), 0..3 / 4..7 for a
+        // bf16 lhs (one shift less; its products are four bits shorter and lose next to nothing)
+        constexpr int UP = NPART == 2 ? 2 : 0;
+        const uint32_t M1 = 0x000F000Fu << UP, M2 = 0x00F000F0u << UP;
 #pragma unroll
         for (int f = 0; f < 4; f++) {
             half8 bfrag[2];
-            bfrag[0] = pack4(qa[f] & M1, qa[f] & M2, (qa[f] >> 8) & M1, (qa[f] >> 8) & M2);
-            bfrag[1] = pack4(qb[f] & M1, qb[f] & M2, (qb[f] >> 8) & M1, (qb[f] >> 8) & M2);
+            const uint32_t qa_lo = UP ? qa[f] << UP : qa[f], qb_lo = UP ? qb[f] << UP : qb[f];
+            bfrag[0] = pack4(qa_lo & M1, qa_lo & M2, (qa[f] >> (8 - UP)) & M1, (qa[f] >> (8 - UP)) & M2);
+            bfrag[1] = pack4(qb_lo & M1, qb_lo & M2, (qb[f] >> (8 - UP)) & M1, (qb[f] >> (8 - UP)) & M2);
 #pragma unroll
             for (int p = 0; p < NPART; p++) {
 #pragma unroll

@@ -224,7 +224,11 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
             }
             return QMM_OK;
         }
-        if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size))
+        // up to 48 rows the small-batch kernel, 16 rows a pass, is faster than the 128-row tiles of the GEMM
+        // (14336 x 4096: 24 us a pass against 105 us)
+        static const int gemm_min = getenv("QMM_GPTQ_GEMM_MIN") ? atoi(getenv("QMM_GPTQ_GEMM_MIN")) : 49;
+        if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size) &&
+            (m >= gemm_min || !qmm::gemv_gptq_mm_supported(rhs[0], n, k, cfg->group_size)))
             return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
                                                     (const uint32_t*)rhs[2], m, n, k, cfg->group_size, out, workspace, s),
                               "qmm_matmul(GPTQ GEMM)");

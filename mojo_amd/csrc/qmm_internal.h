@@ -85,6 +85,10 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
 hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                  const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                                  int64_t ldo, hipStream_t s, bool* handled);
+bool gemv_gptq_mm_supported(const void* qweight, int64_t n, int64_t k, int group);
+hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
+                               const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out, int64_t ldo,
+                               hipStream_t s, bool* handled);
 hipError_t launch_gemv_gptq_act_order(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                       const uint32_t* qzeros, const int32_t* g_idx, int m, int64_t n, int64_t k, int group,
                                       float* out, int64_t ldo, hipStream_t s);

@@ -282,6 +282,50 @@ def test_non_finite_lhs_values_stay_in_their_row(enc, m):
             assert_close(got[1:], want[1:], f"{enc.name} m={m}: rows next to a non-finite one")
 
 
+@pytest.mark.parametrize("m,n,k,group,bf16", [
+    (2, 72, 256, 128, False), (5, 1000, 1024, 128, False), (8, 8, 4096, 64, False), (13, 136, 4096, 256, True),
+    (16, 520, 8192, 128, False), (16, 200, 14336, 128, True), (7, 264, 4352, 64, False), (3, 2048, 2048, 256, True),
+    (33, 96, 4096, 128, False)])
+def test_gptq_small_batch(m, n, k, group, bf16):
+    """2 to 16 lhs rows (and 33 as passes) through the matrix-core small-batch kernel: one to sixteen wavefronts of
+    256 k each, K beyond 4096 as launches that add to the output (8192 = 2 x 16, 14336 = 3 x 16 + 8, 4352 = 16 + 1
+    wavefronts), ragged N, N of eight columns, arbitrary zero points, lhs rows of very different magnitude."""
+    w, a = synth(81, n, k, m)
+    a[0] *= 1e-6
+    a[m - 1] *= 3e4
+    if m > 2:
+        a[1, : k // 2] = 0.0
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    rng = np.random.Generator(np.random.PCG64(82))
+    qz = rng.integers(0, 2**32, size=qz.shape, dtype=np.uint64).astype(np.uint32).view(np.int32)
+    truth = O.matmul_gptq(a, qw, sc, qz, group, f64=True)
+    cfg = QuantizationConfig(group_size=group, sym=False)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.GPTQ, cfg, lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    assert_close(got, truth, f"GPTQ small batch {m}x{n}x{k} group={group} bf16={bf16}")
+
+
+@pytest.mark.parametrize("m,bf16,bound", [(5, False, 5e-6), (5, True, 5e-6), (64, True, 3e-5), (64, False, 7e-5)])
+def test_gptq_long_k_mean_error(m, bf16, bound):
+    """K = 14336 with unit-size activations: the mean of (result - fp64 truth) over all outputs stays small.  The matrix
+    cores cut the low bits of products of fp16 subnormals towards minus infinity; with the non-negative GPTQ codes held
+    as q * 2^-24 that was a bias of 6e-5 (small-batch kernel) to 2e-4 (GEMM, fp32 lhs) at this K, more than the absolute
+    tolerance.  The kernels now hold the codes higher in the subnormal's mantissa: no measurable bias in the small-batch
+    kernel, 1.5e-5 (bf16 lhs) and 4.5e-5 (fp32 lhs, whose residual plane shares the accumulators) in the GEMM."""
+    n, k = 64, 14336
+    w, a = synth(91, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    qw, sc, qz, gi = O.quantize_gptq(w)
+    truth = O.matmul_gptq(a, qw, sc, qz, f64=True)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.GPTQ, QuantizationConfig(), lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi)).cpu().numpy()
+    assert_close(got, truth, f"GPTQ {m}x{n}x{k} bf16={bf16}")
+    assert abs(float((got - truth).mean())) < bound
+
+
 @pytest.mark.parametrize("m,n,k,group,bf16", [(1, 264, 1024, 32, False), (2, 72, 2048, 64, True), (4, 136, 4096, 256, False),
                                                (1, 64, 28672, 128, False), (3, 8, 512, 128, False), (1, 128, 480, 96, False)])
 def test_gptq_decode_group_sizes(m, n, k, group, bf16):
