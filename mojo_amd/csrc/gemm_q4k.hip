@@ -1,8 +1,8 @@
 // Q4_K prefill kernel (m > 16 lhs rows): matrix-core GEMM over exact integer codes.
 //
 // Arithmetic.  As in the decode kernel, a masked nibble is the fp16 subnormal
-// q*2^-24 and one packed fp16 multiply folds the 6-bit sub-block scale in
-// (q*sc <= 945, exact).  lhs values are scaled per row by a power of two and
+// q*2^-24 and one packed fp16 multiply folds the 6-bit sub-block scale in,
+// times 64 (sc*q*2^-18 with q*sc <= 945: exact, and normal from 16 on).  lhs values are scaled per row by a power of two and
 // narrowed to fp16 (exact for bf16 inputs of ordinary range), so every product
 // inside v_mfma_f32_32x32x16_f16 is exact and the sums are fp32.  Per 256-wide
 // super-block b the matrix cores produce P_b[m][n] = sum_k a[m][k]*(sc*q)[n][k];
@@ -43,7 +43,7 @@ namespace {
 
 constexpr int BN = 256;
 constexpr int A_STRIDE = 72;  // halfs per LDS row of a 64-wide chunk (144 bytes: conflict-free b128 reads)
-constexpr float kTwo24 = 16777216.0f;
+constexpr float kTwo18 = 262144.0f;
 
 // Tile order inside an XCD's range: `gm` lhs tile rows stay fixed while the order walks N.
 __device__ __forceinline__ void tile_coords(int o, int tiles_m, int tiles_n, int gm, int& tile_m, int& tile_n) {
@@ -175,14 +175,18 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
 #pragma unroll
             for (int ni = 0; ni < 2; ni++) {
                 const uint4 hdr = ni == 0 ? hdr_n0 : hdr_n1;
-                dscale[ni] = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo24;
+                dscale[ni] = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo18;
                 const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
                 const uint32_t sc_lo = s0 & 0x3F3F3F3Fu, sc_hi = (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u);
                 const uint32_t mn_lo = s1 & 0x3F3F3F3Fu, mn_hi = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
-                const float e0 = (float)(sc_lo & 0xffu), e1 = 0.0625f * (float)((sc_lo >> 8) & 0xffu);
-                const float e2 = (float)((sc_lo >> 16) & 0xffu), e3 = 0.0625f * (float)(sc_lo >> 24);
-                const float e4 = (float)(sc_hi & 0xffu), e5 = 0.0625f * (float)((sc_hi >> 8) & 0xffu);
-                const float e6 = (float)((sc_hi >> 16) & 0xffu), e7 = 0.0625f * (float)(sc_hi >> 24);
+                // 64 * sc for the low nibbles (q * 2^-24), 4 * sc for the high ones (16 q * 2^-24): the operand is
+                // sc * q * 2^-18, a normal fp16 number from sc * q = 16 on.  (With sc * q * 2^-24, always a subnormal,
+                // the matrix core drops low bits of the products of small sc * q towards minus infinity: a bias
+                // growing with K, 5e-5 at K = 14336 for sub-block scales of 1.)
+                const float e0 = 64.0f * (float)(sc_lo & 0xffu), e1 = 4.0f * (float)((sc_lo >> 8) & 0xffu);
+                const float e2 = 64.0f * (float)((sc_lo >> 16) & 0xffu), e3 = 4.0f * (float)(sc_lo >> 24);
+                const float e4 = 64.0f * (float)(sc_hi & 0xffu), e5 = 4.0f * (float)((sc_hi >> 8) & 0xffu);
+                const float e6 = 64.0f * (float)((sc_hi >> 16) & 0xffu), e7 = 4.0f * (float)(sc_hi >> 24);
                 sp[ni][0] = pack_half2(e0, e0); sp[ni][1] = pack_half2(e1, e1);
                 sp[ni][2] = pack_half2(e2, e2); sp[ni][3] = pack_half2(e3, e3);
                 sp[ni][4] = pack_half2(e4, e4); sp[ni][5] = pack_half2(e5, e5);

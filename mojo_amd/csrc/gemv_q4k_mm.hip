@@ -2,7 +2,7 @@
 // matrix-core products over exact integer codes.
 //
 // Arithmetic is that of the prefill kernel (gemm_q4k.hip): a masked nibble is the fp16 subnormal
-// q*2^-24, one packed fp16 multiply folds the 6-bit sub-block scale in, the lhs is narrowed to fp16
+// q*2^-24, one packed fp16 multiply folds the 6-bit sub-block scale in (times 64), the lhs is narrowed to fp16
 // (hi, plus a residual plane) after an exact power-of-two scaling, the fp32 super-block scale is
 // applied in the lanes and the min term is one extra matrix product per super-block.
 //
@@ -46,7 +46,7 @@ constexpr int kPieces = 16 * kRowBytes / 16;    // 288 pieces per item, piece p 
 constexpr int kLoads = (kPieces + 63) / 64;     // 5 load instructions per item, the last one by 32 lanes
 constexpr int kSlotBytes = kPieces * 16;        // 4608
 constexpr int kSlots = 3;                       // ring: one item being decoded, two in flight
-constexpr float kTwo24f = 16777216.0f;
+constexpr float kTwo18f = 262144.0f;
 constexpr int kWaves = 8;                       // wavefronts per workgroup
 constexpr int kMaxTiles = 4;                    // tiles per workgroup (private LDS accumulators per wavefront)
 constexpr int kPlaneStride = 528;               // staged lhs plane of one super-block: 512 bytes + 16 (bank spread)
@@ -335,7 +335,10 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
             const uint32_t p0 = (hdr.y >> sh) & 0xffffu, p1 = (hdr.z >> sh) & 0xffffu, p2 = (hdr.w >> sh) & 0xffffu;
             const uint32_t sc_pair = upper ? ((p2 & 0x0F0Fu) | ((p0 >> 2) & 0x3030u)) : (p0 & 0x3F3Fu);
             const uint32_t mn_pair = upper ? (((p2 >> 4) & 0x0F0Fu) | ((p1 >> 2) & 0x3030u)) : (p1 & 0x3F3Fu);
-            const float e0 = (float)(sc_pair & 0xffu), e1 = 0.0625f * (float)(sc_pair >> 8);
+            // 64 * sc for the low nibbles (q * 2^-24), 4 * sc for the high ones (16 q * 2^-24): the operand is
+            // sc * q * 2^-18, a normal fp16 number from sc * q = 16 on (as sc * q * 2^-24, always a subnormal, the
+            // matrix core drops low bits of the products of small sc * q towards minus infinity: a bias growing with K)
+            const float e0 = 64.0f * (float)(sc_pair & 0xffu), e1 = 4.0f * (float)(sc_pair >> 8);
             const uint32_t sp_lo = pack_half2(e0, e0), sp_hi = pack_half2(e1, e1);
             // min term: weight slots (bh0, bh0, bl0, bh1, bh1, bl1, 0, 0) of -(dmin * mn_j), hi and residual parts
             float4v Bk = {0.f, 0.f, 0.f, 0.f};
@@ -364,7 +367,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
                     Q = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[bb][p][1][1], bhi, Q, 0, 0, 0);
                 }
             }
-            const float dsc = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo24f;
+            const float dsc = h2f((uint16_t)(hdr.x & 0xffffu)) * kTwo18f;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const float v = fmaf(dsc, P[r] + Q[r], Bk[r]);

@@ -307,6 +307,27 @@ def test_gptq_small_batch(m, n, k, group, bf16):
     assert_close(got, truth, f"GPTQ small batch {m}x{n}x{k} group={group} bf16={bf16}")
 
 
+@pytest.mark.parametrize("m", [4, 16, 64])
+def test_q4_k_unit_sub_block_scales_long_k(m):
+    """Q4_K rows whose 6-bit scales and mins are all 1, K = 14336, fp32 lhs, through the matrix-core kernels: the
+    operand sc * q is then at most 15, and held as the fp16 subnormal sc * q * 2^-24 the matrix cores dropped low
+    product bits towards minus infinity (mean error -2e-5 to -5e-5 here).  Held as sc * q * 2^-18 there is none."""
+    n, k = 64, 14336
+    rng = np.random.Generator(np.random.PCG64(93))
+    blocks = rng.integers(0, 256, size=(n, k // 256, 144), dtype=np.uint8)
+    blocks[:, :, 4:12] = 1      # scales and mins of sub-blocks 0..3 (and zero top bits for 4..7)
+    blocks[:, :, 12:16] = 0x11  # low nibbles of the scales and mins of sub-blocks 4..7
+    d = np.full((n, k // 256, 1), 0.02 / 7.5, dtype=np.float16)
+    blocks[:, :, 0:2] = d.view(np.uint8)
+    blocks[:, :, 2:4] = d.view(np.uint8)
+    wq = blocks.reshape(n, -1)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a), gpu(wq)).cpu().numpy()
+    assert_close(got, truth, f"Q4_K unit scales {m}x{n}x{k}")
+    assert abs(float((got - truth).mean())) < 3e-6
+
+
 @pytest.mark.parametrize("m,bf16,bound", [(5, False, 5e-6), (5, True, 5e-6), (64, True, 3e-5), (64, False, 7e-5)])
 def test_gptq_long_k_mean_error(m, bf16, bound):
     """K = 14336 with unit-size activations: the mean of (result - fp64 truth) over all outputs stays small.  The matrix
