@@ -5,13 +5,15 @@
 // the order (0,4,1,5,2,6,3,7) inside each 8-group and its odd columns pre-multiplied
 // by 1/16, the four fp16 pairs  x & 0x000F000F,  x & 0x00F000F0,  (x>>8) & 0x000F000F,
 // (x>>8) & 0x00F000F0  are the matrix-core B operand directly: fp16 subnormals q*2^-24
-// (or 16q*2^-24), no multiply needed because the scale is per group, not per 32.  For an
-// fp32 lhs the nibbles are moved two bits up inside the subnormal's mantissa (x << 2 and
-// x >> 6, masks shifted likewise: q*2^-22): the matrix core does not normalise subnormal
-// inputs before it aligns the products of a step, and the low bits of long products (the
-// residual plane's most of all) then fall off the end of the adder, always towards minus
-// infinity: with non-negative codes a bias that grows with K (unit-size activations,
-// K = 14336: 2e-4 with the nibbles low, 4.5e-5 with them here; bf16 lhs: 1e-6).
+// (or 16q*2^-24), no multiply needed because the scale is per group, not per 32.
+// The matrix core does not normalise subnormal inputs before it aligns the products of a
+// step, and the low bits of long products then fall off the end of the adder, always towards
+// minus infinity: with non-negative codes a bias that grows with K.  With unit-size
+// activations at K = 14336 it is 1.5e-5 for a bf16 lhs (short products).  For an fp32 lhs it
+// was 2e-4 with the main and the residual plane in one launch; now each plane is a launch of
+// its own (the residual plane's small products no longer sit next to the main plane's large
+// sums) and the nibbles are moved two bits up inside the subnormal's mantissa (x << 2 and
+// x >> 6, masks shifted likewise: q*2^-22), which leaves 6e-6.
 // Per group g the matrix cores produce  P[m][n] = sum_k a[m][k]*q[k][n]  exactly (fp32
 // sums), and the lanes apply  acc += scale[g][n] * P.  The zero-point term
 // -scale*zero * sum_k a[m][k]  is a second small matrix product over the 32-wide
@@ -39,16 +41,20 @@ constexpr float kTwo24 = 16777216.0f, kTwo22 = 4194304.0f;
 }  // namespace
 
 // GB = groups per 256-column chunk (group size 256 / GB: 256, 128 or 64).
-template <int NPART, int GB>
+// One launch multiplies one fp16 plane of the lhs (`a16`) with the weights.  `with_zero` adds the zero-point term (it
+// uses the full-precision sub-block sums, so it belongs to exactly one launch); `accumulate` adds the result to
+// what `out` already holds (second launch of an fp32 lhs: its residual plane, with accumulators of its own: next to
+// the large sums of the main plane the small residual products would lose their low bits inside the matrix core).
+// UP: how many bits the nibbles are moved up inside the fp16 halves (2 for an fp32 lhs, 0 for a bf16 lhs).
+template <int UP, int GB, bool with_zero, bool accumulate>
 __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restrict__ qweight,
                                                         const uint16_t* __restrict__ scales,
                                                         const uint32_t* __restrict__ qzeros,
                                                         const _Float16* __restrict__ a16,
-                                                        const _Float16* __restrict__ a16_lo,
                                                         const _Float16* __restrict__ asum, const float* __restrict__ inv,
                                                         float* __restrict__ out, int m, int n, int k, int tiles_m,
                                                         int tiles_n) {
-    __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][NPART][BM * A_STRIDE];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) _Float16 lds_s[BM * 16];
     __shared__ __attribute__((aligned(16))) float lds_inv[BM];
     constexpr int SPG = 4 / GB;  // 64-wide steps per group
@@ -77,29 +83,19 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
     const int a_row = tid >> 2, a_seg = tid & 3;
     const int64_t a_off = (int64_t)min(m0 + a_row, m - 1) * k + a_seg * 8;
     const uint4* a_base0 = (const uint4*)(a16 + a_off);
-    const uint4* a_base1 = NPART == 2 ? (const uint4*)(a16_lo + a_off) : nullptr;
-    uint4 ax0_p0s0, ax0_p0s1, ax0_p1s0, ax0_p1s1, ax1_p0s0, ax1_p0s1, ax1_p1s0, ax1_p1s1;
-    ax0_p1s0 = ax0_p1s1 = ax1_p1s0 = ax1_p1s1 = make_uint4(0, 0, 0, 0);
-    _Float16* a_dst = &lds_a[0][0][a_row * A_STRIDE + a_seg * 8];
+    uint4 ax0_p0s0, ax0_p0s1, ax1_p0s0, ax1_p0s1;
+    _Float16* a_dst = &lds_a[0][a_row * A_STRIDE + a_seg * 8];
 #define QMM_A_LOAD(SET, STEP)                                         \
     do {                                                              \
         const int chunk_ = min((STEP), nsteps - 1);                   \
         SET##_p0s0 = a_base0[chunk_ * 8];                             \
         SET##_p0s1 = a_base0[chunk_ * 8 + 4];                         \
-        if constexpr (NPART == 2) {                                   \
-            SET##_p1s0 = a_base1[chunk_ * 8];                         \
-            SET##_p1s1 = a_base1[chunk_ * 8 + 4];                     \
-        }                                                             \
     } while (0)
 #define QMM_A_STORE(SET, BUF)                                                     \
     do {                                                                          \
-        _Float16* d_ = a_dst + (size_t)(BUF) * NPART * BM * A_STRIDE;             \
+        _Float16* d_ = a_dst + (size_t)(BUF) * BM * A_STRIDE;                     \
         *(uint4*)d_ = SET##_p0s0;                                                 \
         *(uint4*)(d_ + 32) = SET##_p0s1;                                          \
-        if constexpr (NPART == 2) {                                               \
-            *(uint4*)(d_ + BM * A_STRIDE) = SET##_p1s0;                           \
-            *(uint4*)(d_ + BM * A_STRIDE + 32) = SET##_p1s1;                      \
-        }                                                                         \
     } while (0)
 
     // this lane's two weight columns; the lane half g takes the odd k8 rows
@@ -192,7 +188,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
 #pragma unroll
                 for (int i = 0; i < GB; i++) {
                     const uint32_t sb = sc_n[ni][i] & 0xffffu;
-                    gscale[ni][i] = h2f((uint16_t)sb) * (NPART == 2 ? kTwo22 : kTwo24);
+                    gscale[ni][i] = h2f((uint16_t)sb) * (UP == 2 ? kTwo22 : kTwo24);
                     const float z = (float)(((zw_n[ni][i] >> (ni == 0 ? zshift0 : zshift1)) & 0xFu) + 1u);
                     const uint32_t nsc = (sb ^ 0x8000u) * 0x00010001u;  // (-scale, -scale)
                     const uint32_t zp = pack_half2(z, z);
@@ -201,6 +197,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
                 }
             }
             hdr_prefetch(blk + 1);
+            if constexpr (with_zero)
 #pragma unroll
             for (int mi = 0; mi < 2; mi++) {
                 // A operand: lanes g=0 carry the hi parts of the 8 sub-block sums, g=1 the lo parts
@@ -219,9 +216,8 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
         }
 
         // ---- one 64-wide chunk: four 16-wide operand slices, one packed dword per column each
-        // nibble positions inside the fp16 halves: bits 2..5 / 6..9 for an fp32 lhs (two planes), 0..3 / 4..7 for a
-        // bf16 lhs (one shift less; its products are four bits shorter and lose next to nothing)
-        constexpr int UP = NPART == 2 ? 2 : 0;
+        // nibble positions inside the fp16 halves: bits 2..5 / 6..9 for an fp32 lhs, 0..3 / 4..7 for a bf16 lhs
+        // (one shift less; its products are three bits shorter and lose next to nothing)
         const uint32_t M1 = 0x000F000Fu << UP, M2 = 0x00F000F0u << UP;
 #pragma unroll
         for (int f = 0; f < 4; f++) {
@@ -230,14 +226,11 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
             bfrag[0] = pack4(qa_lo & M1, qa_lo & M2, (qa[f] >> (8 - UP)) & M1, (qa[f] >> (8 - UP)) & M2);
             bfrag[1] = pack4(qb_lo & M1, qb_lo & M2, (qb[f] >> (8 - UP)) & M1, (qb[f] >> (8 - UP)) & M2);
 #pragma unroll
-            for (int p = 0; p < NPART; p++) {
+            for (int mi = 0; mi < 2; mi++) {
+                const half8 afrag = *(const half8*)(&lds_a[buf][(wm * 64 + mi * 32 + nl) * A_STRIDE + f * 16 + g * 8]);
 #pragma unroll
-                for (int mi = 0; mi < 2; mi++) {
-                    const half8 afrag = *(const half8*)(&lds_a[buf][p][(wm * 64 + mi * 32 + nl) * A_STRIDE + f * 16 + g * 8]);
-#pragma unroll
-                    for (int ni = 0; ni < 2; ni++)
-                        P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[ni], P[mi][ni], 0, 0, 0);
-                }
+                for (int ni = 0; ni < 2; ni++)
+                    P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[ni], P[mi][ni], 0, 0, 0);
             }
         }
         if constexpr ((c + 1) % SPG == 0) {  // group end: apply its scale
@@ -296,8 +289,8 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
             const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
             if (row < m) {
                 float* o = out + (int64_t)row * n;
-                if (c0_ok) o[ocol0] = acc[mi][0][r] * is;
-                if (c1_ok) o[ocol1] = acc[mi][1][r] * is;
+                if (c0_ok) o[ocol0] = accumulate ? fmaf(acc[mi][0][r], is, o[ocol0]) : acc[mi][0][r] * is;
+                if (c1_ok) o[ocol1] = accumulate ? fmaf(acc[mi][1][r], is, o[ocol1]) : acc[mi][1][r] * is;
             }
         }
     }
@@ -321,12 +314,18 @@ hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qwei
     dim3 grid((unsigned)(per_xcd * 8)), block(512);
 #define QMM_GPTQ_LAUNCH(GB_)                                                                                          \
     do {                                                                                                              \
-        if (lhs_dtype == QMM_F32)                                                                                     \
-            gemm_gptq_kernel<2, GB_><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.a16_lo, p.asum, p.inv,  \
-                                                            out, (int)m, (int)n, (int)k, tiles_m, tiles_n);          \
-        else                                                                                                          \
-            gemm_gptq_kernel<1, GB_><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, nullptr, p.asum, p.inv,   \
-                                                            out, (int)m, (int)n, (int)k, tiles_m, tiles_n);          \
+        if (lhs_dtype == QMM_F32) { /* main plane, then the residual plane added on top */                            \
+            gemm_gptq_kernel<2, GB_, true, false><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.asum,    \
+                                                                         p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
+                                                                         tiles_n);                                   \
+            gemm_gptq_kernel<2, GB_, false, true><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16_lo, p.asum, \
+                                                                         p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
+                                                                         tiles_n);                                   \
+        } else {                                                                                                      \
+            gemm_gptq_kernel<0, GB_, true, false><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.asum,    \
+                                                                         p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
+                                                                         tiles_n);                                   \
+        }                                                                                                             \
     } while (0)
     if (group == 256) QMM_GPTQ_LAUNCH(1);
     else if (group == 128) QMM_GPTQ_LAUNCH(2);
