@@ -475,6 +475,12 @@ def extra_timings(layers, acts, gen):
     dev_s, _ = time_graphs([g], 20, 3)
     us = dev_s * 1e6 / (20 * 8)
     out["gptq_g128_act_order_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round((14336 * 4096 * 0.5176 + 4096 * 8 + 14336 * 4) / us / 1e3, 1)}
+    # sixteen lhs rows: the small-batch matrix-core kernel
+    am16 = torch.randn((16, 4096), dtype=torch.float32, device="cuda:0", generator=gen)
+    g = capture([GptqMatmul(c.t, am16) for c in cs])
+    dev_s, _ = time_graphs([g], 20, 3)
+    us = dev_s * 1e6 / (20 * 8)
+    out["gptq_g128_m16_14336x4096"] = {"us": round(us, 3), "GB/s": round((14336 * 4096 * 0.5176 + 16 * 4096 * 4 + 16 * 14336 * 4) / us / 1e3, 1)}
     del cs
     # Q5_K decode on the gate shape
     cs = [Gemv(QE.Q5_K, make_weight(QE.Q5_K, 14336, 4096, gen), am1) for _ in range(8)]
