@@ -36,6 +36,8 @@ constexpr int kPartK = 256;         // k values of a wavefront
 constexpr int kKB = kPartK / 32;    // matrix-core steps of a wavefront per strip
 constexpr int kStrip = 32;          // columns of a strip
 constexpr int kMaxWaves = 16;
+constexpr int kLoReg = 2;            // residual-plane operands of a wavefront kept in registers; the other kKB - kLoReg in LDS
+constexpr int kLoLds = kKB - kLoReg;
 
 __device__ __forceinline__ half8 nibble_operand(uint32_t w) {
     constexpr uint32_t kTop = 0x03C003C0u;  // mantissa bits 6..9 of both halves
@@ -86,7 +88,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
     }
 
     // --- this wavefront's lhs part: lane (row c, k quarter kq) holds a[c][256 wave + 32 kb + 8 kq + 0..7] ---
-    half8 ahi[kKB], alo[PLANES == 2 ? kKB : 1];
+    // (fp32 lhs: main and residual operands, 64 registers, do not fit next to the loads in flight in the 128
+    // registers of a 16-wavefront workgroup: with all of them in registers the compiler spilled a dozen to scratch
+    // memory and 14336 x 4096 with 16 rows took 24.7 us; with six of the eight residual operands in LDS, each lane
+    // reading back what it wrote, 21.3 us.  One plane alone: 18.5 us.)
+    half8 ahi[kKB], alo[PLANES == 2 ? kLoReg : 1];
+    half8* lo_w = (half8*)(mm_lds + nw * 512 + nw * (NG + 1) * 16) + wave * kLoLds * 64 + lane;  // [kLoLds][64] per wavefront
     {
         float x[kKB][8];
         const AT* ar = a + (int64_t)min(c, m - 1) * lda + wave * kPartK + kq * 8;
@@ -139,7 +146,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
                 gs[kb / GK] += s0 + s1;
             }
             ahi[kb] = pack4(hi[0], hi[1], hi[2], hi[3]);
-            if constexpr (PLANES == 2) alo[kb] = pack4(lo[0], lo[1], lo[2], lo[3]);
+            if constexpr (PLANES == 2) {
+                if (kb < kLoReg) alo[kb] = pack4(lo[0], lo[1], lo[2], lo[3]);
+                else lo_w[(kb - kLoReg) * 64] = pack4(lo[0], lo[1], lo[2], lo[3]);
+            }
         }
         // group sums over the four k quarters, then row c -> the lanes that hold row 4 * kq + r of the results
 #pragma unroll
@@ -180,7 +190,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
                     const int kb = g * GK + kk;
                     const half8 b = nibble_operand(j == 0 ? wq[kb].x : wq[kb].y);
                     P = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi[kb], b, P, 0, 0, 0);
-                    if constexpr (PLANES == 2) R = __builtin_amdgcn_mfma_f32_16x16x32_f16(alo[kb], b, R, 0, 0, 0);
+                    if constexpr (PLANES == 2)
+                        R = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb < kLoReg ? alo[kb] : lo_w[(kb - kLoReg) * 64], b, R, 0, 0, 0);
                 }
                 if constexpr (PLANES == 2) P += R;
                 const float sc = j == 0 ? sz0 : sz1, zp = j == 0 ? zp0 : zp1;
@@ -246,7 +257,8 @@ hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweig
     const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
     for (int64_t k0 = 0; k0 < k; k0 += (int64_t)kMaxWaves * kPartK) {
         const int nw = (int)std::min<int64_t>(kMaxWaves, (k - k0) / kPartK);
-        const size_t lds = ((size_t)nw * 512 + (size_t)nw * (ng + 1) * 16) * sizeof(float);  // at most 34 KB
+        const size_t lds = ((size_t)nw * 512 + (size_t)nw * (ng + 1) * 16) * sizeof(float) +  // at most 34 KB
+                           (a_dtype == QMM_F32 ? (size_t)nw * kLoLds * 64 * 16 : 0);            // + 96 KB
         const int per_cu = std::max(1, kMaxWaves / nw);
         dim3 grid((unsigned)std::min<int64_t>(nstrips, (int64_t)cus * per_cu)), block(64 * nw);
         const uint32_t* qw = qweight + (k0 / 8) * n;
@@ -256,6 +268,11 @@ hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweig
         const int accumulate = k0 > 0;
 #define QMM_GPTQ_MM(PL_, GK_, AT_)                                                                                   \
     do {                                                                                                             \
+        if (lds > 64 * 1024) {                                                                                       \
+            hipError_t e_ = hipFuncSetAttribute((const void*)gemv_gptq_mm_kernel<PL_, GK_, AT_>,                     \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);               \
+            if (e_ != hipSuccess) return e_;                                                                         \
+        }                                                                                                            \
         gemv_gptq_mm_kernel<PL_, GK_, AT_><<<grid, block, lds, s>>>(qw, sc, qz, (const AT_*)ap, out, m, (int)n, k, ldo, \
                                                                     nstrips, accumulate);                            \
     } while (0)
