@@ -17,8 +17,9 @@
 //
 // Shape.  Wavefront w of a workgroup owns the 256 k values [256 w, 256 w + 256) for the whole kernel and keeps
 // its lhs operands (16 rows x 256 k: 32 registers a plane), the group sums and the inverse row scales in
-// registers; a workgroup of K / 256 wavefronts (K up to 4096 per launch, longer K as further launches that add
-// to the output) walks over strips of 32 columns.  The eight loads of a strip are replaced, as they are
+// registers; a workgroup of up to 16 wavefronts walks over strips of 32 columns.  K beyond 4096 is cut into equal
+// chunks of at most 16 wavefront parts, one per value of blockIdx.y: the chunks write their partial results to a
+// workspace, [chunk][row][N], and a second kernel adds them in chunk order.  The eight loads of a strip are replaced, as they are
 // consumed, by those of the workgroup's next strip.  The wavefronts' partial sums of a strip meet in LDS and are
 // added in wavefront order: results do not depend on timing.
 #include <stdlib.h>
@@ -49,20 +50,26 @@ template <int PLANES, int GK, typename AT>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
     const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qzeros,
     const AT* __restrict__ a, float* __restrict__ out, int m, int n, int64_t lda, int64_t ldo, int nstrips,
-    int accumulate) {
+    int parts_total, int64_t chunk_stride) {
     constexpr int NG = kKB / GK;  // groups of a wavefront's part
     extern __shared__ __attribute__((aligned(16))) float mm_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nw = (int)(blockDim.x >> 6);
     const int c = lane & 15, kq = lane >> 4;
+    // this wavefront's 256 k: part `part` of the row; the wavefronts of the last chunk beyond the end of the row redo
+    // the last part (every address stays valid, the barriers stay uniform) and contribute zeros
+    const int part_raw = (int)blockIdx.y * nw + wave;
+    const bool part_live = part_raw < parts_total;
+    const int part = __builtin_amdgcn_readfirstlane(min(part_raw, parts_total - 1));
+    out += (int64_t)blockIdx.y * chunk_stride;
     float* park = mm_lds;                                // [nw][512]
     float* tr = mm_lds + nw * 512 + wave * (NG + 1) * 16;  // this wavefront's [NG + 1][16]
 
     // --- the first strip's loads go out before anything else ---
-    // word row of (wave, step kb, lane row kq): 32 * wave + 4 * kb + kq; columns n0 + 2c, n0 + 2c + 1.  Lanes
+    // word row of (part, step kb, lane row kq): 32 * part + 4 * kb + kq; columns n0 + 2c, n0 + 2c + 1.  Lanes
     // beyond N read the last column pair instead (their outputs are not stored).
-    const uint32_t* wrow = qweight + (int64_t)(32 * wave + kq) * n;
+    const uint32_t* wrow = qweight + (int64_t)(32 * part + kq) * n;
     const int n_half = n >> 3;
     auto col_of = [&](int strip) { return min(strip * kStrip + 2 * c, n - 2); };
     uint2 wq[kKB];
@@ -76,7 +83,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
         const int col = col_of(strip);
 #pragma unroll
         for (int g = 0; g < NG; g++) {
-            const int64_t gi = (int64_t)wave * NG + g;
+            const int64_t gi = (int64_t)part * NG + g;
             sc2[g] = *(const uint32_t*)(scales + gi * n + col);
             zw[g] = qzeros[gi * n_half + (col >> 3)];
         }
@@ -87,7 +94,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
         load_params(strip);
     }
 
-    // --- this wavefront's lhs part: lane (row c, k quarter kq) holds a[c][256 wave + 32 kb + 8 kq + 0..7] ---
+    // --- this wavefront's lhs part: lane (row c, k quarter kq) holds a[c][256 part + 32 kb + 8 kq + 0..7] ---
     // (fp32 lhs: main and residual operands, 64 registers, do not fit next to the loads in flight in the 128
     // registers of a 16-wavefront workgroup: with all of them in registers the compiler spilled a dozen to scratch
     // memory and 14336 x 4096 with 16 rows took 24.7 us; with six of the eight residual operands in LDS, each lane
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
     half8* lo_w = (half8*)(mm_lds + nw * 512 + nw * (NG + 1) * 16) + wave * kLoLds * 64 + lane;  // [kLoLds][64] per wavefront
     {
         float x[kKB][8];
-        const AT* ar = a + (int64_t)min(c, m - 1) * lda + wave * kPartK + kq * 8;
+        const AT* ar = a + (int64_t)min(c, m - 1) * lda + part * kPartK + kq * 8;
 #pragma unroll
         for (int kb = 0; kb < kKB; kb++) {
             if constexpr (sizeof(AT) == 4) {
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) mine[(j * 4 + r) * 64 + lane] = acc[j][r] * inv[r];
+            for (int r = 0; r < 4; r++) mine[(j * 4 + r) * 64 + lane] = part_live ? acc[j][r] * inv[r] : 0.0f;
         __syncthreads();
         for (int t = tid; t < 512; t += (int)blockDim.x) {
             float v = 0.0f;
@@ -220,8 +227,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
             const int j = t >> 8, r = (t >> 6) & 3, l = t & 63;
             const int row = 4 * (l >> 4) + r, col = strip * kStrip + 2 * (l & 15) + j;
             if (row < m && col < n) {
-                float* o = out + (int64_t)row * ldo + col;
-                *o = accumulate ? *o + v : v;
+                out[(int64_t)row * ldo + col] = v;
             }
         }
         if (more) __syncthreads();  // the next strip's partial sums go to the same place
@@ -236,12 +242,41 @@ bool gemv_gptq_mm_supported(const void* qweight, int64_t n, int64_t k, int group
            (group == 64 || group == 128 || group == 256);
 }
 
-// 2..16 lhs rows, K a multiple of 256, group 64 / 128 / 256, qweight 8-byte aligned: otherwise *handled stays
-// false and nothing is launched.  K beyond 4096 goes as several launches over K ranges, in order on the stream,
-// each adding to what the one before wrote.
+namespace {
+
+// K = chunks * (wavefronts per workgroup) * 256 at most, chunks as few as 16 wavefronts allow, of equal size
+struct MmChunks {
+    int chunks, nw;
+};
+MmChunks mm_chunks(int64_t k) {
+    const int parts = (int)(k / kPartK);
+    const int chunks = (parts + kMaxWaves - 1) / kMaxWaves;
+    return {chunks, (parts + chunks - 1) / chunks};
+}
+
+// out[r][c] = sum over the chunks of part[chunk][r][c], in chunk order
+__global__ __launch_bounds__(256) void gemv_gptq_mm_sum_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                               int m, int n, int64_t ldo, int chunks) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, count = (int64_t)m * n;
+    if (i >= count) return;
+    float v = 0.0f;
+    for (int ch = 0; ch < chunks; ch++) v += part[ch * count + i];
+    out[(i / n) * ldo + i % n] = v;
+}
+
+}  // namespace
+
+// Workspace of one call with up to 16 lhs rows: the chunks' partial results when K is beyond 4096.
+int64_t gemv_gptq_mm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    if (k % kPartK || k <= (int64_t)kMaxWaves * kPartK) return 0;
+    return (int64_t)mm_chunks(k).chunks * std::min<int64_t>(m, 16) * n * 4;
+}
+
+// 1..16 lhs rows, K a multiple of 256, group 64 / 128 / 256, qweight 8-byte aligned: otherwise *handled stays
+// false and nothing is launched.  `workspace` holds gemv_gptq_mm_workspace_bytes(m, n, k) bytes.
 hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out, int64_t ldo,
-                               hipStream_t s, bool* handled) {
+                               void* workspace, hipStream_t s, bool* handled) {
     *handled = false;
     if (m < 1 || m > 16 || !gemv_gptq_mm_supported(qweight, n, k, group)) return hipSuccess;
     if (a_dtype != QMM_F32 && a_dtype != QMM_BF16) return hipSuccess;
@@ -254,18 +289,16 @@ hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweig
     }
     const int gk = group / 32, ng = kKB / gk;
     const int nstrips = (int)((n + kStrip - 1) / kStrip);
-    const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
-    for (int64_t k0 = 0; k0 < k; k0 += (int64_t)kMaxWaves * kPartK) {
-        const int nw = (int)std::min<int64_t>(kMaxWaves, (k - k0) / kPartK);
-        const size_t lds = ((size_t)nw * 512 + (size_t)nw * (ng + 1) * 16) * sizeof(float) +  // at most 34 KB
-                           (a_dtype == QMM_F32 ? (size_t)nw * kLoLds * 64 * 16 : 0);            // + 96 KB
-        const int per_cu = std::max(1, kMaxWaves / nw);
-        dim3 grid((unsigned)std::min<int64_t>(nstrips, (int64_t)cus * per_cu)), block(64 * nw);
-        const uint32_t* qw = qweight + (k0 / 8) * n;
-        const uint16_t* sc = scales + (k0 / group) * n;
-        const uint32_t* qz = qzeros + (k0 / group) * (n / 8);
-        const char* ap = (const char*)a + k0 * esz;
-        const int accumulate = k0 > 0;
+    const MmChunks cc = mm_chunks(k);
+    if (cc.chunks > 1 && !workspace) return hipErrorInvalidValue;
+    const int nw = cc.nw, parts_total = (int)(k / kPartK);
+    const size_t lds = ((size_t)nw * 512 + (size_t)nw * (ng + 1) * 16) * sizeof(float) +  // at most 34 KB
+                       (a_dtype == QMM_F32 ? (size_t)nw * kLoLds * 64 * 16 : 0);            // + 96 KB
+    const int per_cu = std::max(1, kMaxWaves / nw);
+    const int64_t wgs_x = std::max<int64_t>(1, std::min<int64_t>(nstrips, (int64_t)cus * per_cu / cc.chunks));
+    dim3 grid((unsigned)wgs_x, (unsigned)cc.chunks), block(64 * nw);
+    float* dst = cc.chunks > 1 ? (float*)workspace : out;
+    const int64_t dst_ld = cc.chunks > 1 ? n : ldo, chunk_stride = cc.chunks > 1 ? (int64_t)m * n : 0;
 #define QMM_GPTQ_MM(PL_, GK_, AT_)                                                                                   \
     do {                                                                                                             \
         if (lds > 64 * 1024) {                                                                                       \
@@ -273,20 +306,27 @@ hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweig
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);               \
             if (e_ != hipSuccess) return e_;                                                                         \
         }                                                                                                            \
-        gemv_gptq_mm_kernel<PL_, GK_, AT_><<<grid, block, lds, s>>>(qw, sc, qz, (const AT_*)ap, out, m, (int)n, k, ldo, \
-                                                                    nstrips, accumulate);                            \
+        gemv_gptq_mm_kernel<PL_, GK_, AT_><<<grid, block, lds, s>>>(qweight, scales, qzeros, (const AT_*)a, dst, m,  \
+                                                                    (int)n, k, dst_ld, nstrips, parts_total,         \
+                                                                    chunk_stride);                                   \
     } while (0)
 #define QMM_GPTQ_MM_GK(GK_)                                  \
     do {                                                     \
         if (a_dtype == QMM_F32) QMM_GPTQ_MM(2, GK_, float);  \
         else QMM_GPTQ_MM(1, GK_, uint16_t);                  \
     } while (0)
-        if (gk == 2) QMM_GPTQ_MM_GK(2);
-        else if (gk == 4) QMM_GPTQ_MM_GK(4);
-        else QMM_GPTQ_MM_GK(8);
+    if (gk == 2) QMM_GPTQ_MM_GK(2);
+    else if (gk == 4) QMM_GPTQ_MM_GK(4);
+    else QMM_GPTQ_MM_GK(8);
 #undef QMM_GPTQ_MM_GK
 #undef QMM_GPTQ_MM
-        hipError_t e = hipGetLastError();
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (cc.chunks > 1) {
+        const int64_t count = (int64_t)m * n;
+        gemv_gptq_mm_sum_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s>>>((const float*)workspace, out, m,
+                                                                                            (int)n, ldo, cc.chunks);
+        e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     *handled = true;

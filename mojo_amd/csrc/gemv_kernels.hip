@@ -375,17 +375,9 @@ hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight,
                             const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                             int64_t ldo, hipStream_t s) {
     if (!env_flag_qmm_gptq_v1()) {
-        static const int mm_min = getenv("QMM_GPTQ_MM_MIN") ? atoi(getenv("QMM_GPTQ_MM_MIN")) : 3;
-        bool handled = false;
-        if (m >= mm_min) {
-            // three or more lhs rows: one pass of the matrix-core kernel for up to 16 of them (two rows: 19 us
-            // against 16 us of the column kernel on 14336 x 4096)
-            hipError_t e = launch_gemv_gptq_mm(a, a_dtype, qweight, scales, qzeros, m, n, k, group, out, ldo, s, &handled);
-            if (e != hipSuccess || handled) return e;
-        }
         // up to four lhs rows per pass of the column kernel; more rows take more passes over the weights
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
-        handled = true;
+        bool handled = true;
         for (int m0 = 0; m0 < m && handled; m0 += 4) {
             hipError_t e = launch_gemv_gptq_cols((const char*)a + (int64_t)m0 * k * esz, a_dtype, qweight, scales, qzeros,
                                                  min(4, m - m0), n, k, group, out + (int64_t)m0 * ldo, ldo, s, &handled);

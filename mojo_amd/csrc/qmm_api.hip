@@ -181,7 +181,10 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     }
     if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) return qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);  // 0 up to 8 rows
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
-    if (encoding == QMM_GPTQ && m > 16 && k % 256 == 0) return qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k);
+    if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
+        const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k) : 0;
+        return a > b ? a : b;
+    }
     return 0;
 }
 
@@ -232,8 +235,20 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
             return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
                                                     (const uint32_t*)rhs[2], m, n, k, cfg->group_size, out, workspace, s),
                               "qmm_matmul(GPTQ GEMM)");
+        // one pass of the matrix-core small-batch kernel per 16 lhs rows; one row, and two fp32 rows, go to the column
+        // kernel (two rows on 14336 x 4096: 12.3 us with a bf16 lhs, 16 us with an fp32 lhs, column kernel 16.5 us)
+        static const int mm_min_env = getenv("QMM_GPTQ_MM_MIN") ? atoi(getenv("QMM_GPTQ_MM_MIN")) : 0;
+        const int mm_min = mm_min_env > 0 ? mm_min_env : (lhs_dtype == QMM_F32 ? 3 : 2);
         for (int64_t m0 = 0; m0 < m; m0 += 16) {
             int mt = (int)(m - m0 < 16 ? m - m0 : 16);
+            bool handled = false;
+            if (m >= mm_min) {
+                hipError_t e = qmm::launch_gemv_gptq_mm((const char*)lhs + m0 * k * esz, lhs_dtype, (const uint32_t*)rhs[0],
+                                                        (const uint16_t*)rhs[1], (const uint32_t*)rhs[2], mt, n, k,
+                                                        cfg->group_size, out + m0 * n, n, workspace, s, &handled);
+                if (e != hipSuccess) return hip_status(e, "qmm_matmul(GPTQ small batch)");
+            }
+            if (handled) continue;
             hipError_t e = qmm::launch_gemv_gptq((const char*)lhs + m0 * k * esz, lhs_dtype, (const uint32_t*)rhs[0],
                                                  (const uint16_t*)rhs[1], (const uint32_t*)rhs[2], mt, n, k,
                                                  cfg->group_size, out + m0 * n, n, s);

@@ -86,9 +86,10 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
                                  const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                                  int64_t ldo, hipStream_t s, bool* handled);
 bool gemv_gptq_mm_supported(const void* qweight, int64_t n, int64_t k, int group);
+int64_t gemv_gptq_mm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out, int64_t ldo,
-                               hipStream_t s, bool* handled);
+                               void* workspace, hipStream_t s, bool* handled);
 hipError_t launch_gemv_gptq_act_order(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                       const uint32_t* qzeros, const int32_t* g_idx, int m, int64_t n, int64_t k, int group,
                                       float* out, int64_t ldo, hipStream_t s);
