@@ -120,6 +120,30 @@ def test_prefill_configuration_full_size(kind):
     check_all(got, a.double(), w32, f"{kind} prefill {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("m,n,k,bf16", [(16, 14336, 4096, False), (16, 14336, 4096, True), (4, 4096, 14336, False),
+                                        (48, 4096, 14336, True), (2, 1024, 4096, True)])
+def test_gptq_small_batch_full_size(m, n, k, bf16):
+    """The GPTQ small-batch kernel on the projection shapes: 448 column strips on 256 workgroups (14336 x 4096), four K
+    chunks with partial sums in the workspace (4096 x 14336), three passes of 16 rows (m = 48).  Sampled columns against
+    the oracle's fp64 sums, every output against the fp64 product on the GPU."""
+    w, gen = weights(300 + m, n, k)
+    a = torch.randn((m, k), dtype=torch.float32, device=DEV, generator=gen)
+    if bf16:
+        a = a.to(torch.bfloat16)
+    cfg = QuantizationConfig()
+    qw, sc, qz, gi = quantize_gptq(w)
+    got = qmatmul(QE.GPTQ, cfg, a, qw, sc, qz, gi)
+    assert got.shape == (m, n)
+    words = np.sort(np.random.default_rng(m + n).choice(n // 8, 6, replace=False))
+    cols = (words[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+    tcols = torch.from_numpy(cols).to(DEV)
+    truth = O.matmul_gptq(a.float().cpu().numpy(), qw[:, tcols].cpu().numpy(), sc[:, tcols].cpu().numpy().view(np.uint16),
+                          np.ascontiguousarray(qz.cpu().numpy()[:, words]), f64=True)
+    ok = O.isclose(got[:, tcols].cpu().numpy(), truth, RTOL, ATOL)
+    assert ok.all(), f"GPTQ {m}x{n}x{k}: {(~ok).sum()}/{ok.size} sampled outputs differ from the oracle"
+    check_all(got, a.double(), dequantize(QE.GPTQ, qw, sc, qz, gi, config=cfg), f"GPTQ small batch {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("enc,m,k,period,reps", [
     (QE.Q4_K, 1, 4096, 9600, 100),    # 960 000 rows x 2304 B = 2.2 GB: the decode kernel's row offsets pass 2^31
     (QE.Q4_K, 4, 4096, 9600, 100),    # the small-batch kernel
