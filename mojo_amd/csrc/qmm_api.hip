@@ -41,6 +41,19 @@ int hip_status(hipError_t e, const char* what) {
 
 bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
+// GPTQ with more than 16 lhs rows: do passes of the small-batch kernel (16 rows each, bound by the bytes of the weights)
+// beat the GEMM (128 x 256 output tiles, one workgroup each, bound by K per round of 256 tiles)?  Times in
+// microseconds as measured on 14336 x 4096, 4096 x 14336 and 4096 x 4096 with 64 to 128 rows: a GEMM round costs
+// 64 us per 4096 of K (bf16 lhs; 2.1 x that for an fp32 lhs, which runs two launches) whatever N is, so few column tiles
+// (N = 4096: 16 of 256 compute units) and long K favour the passes: 4096 x 14336 with 128 bf16 rows 126 against 209 us.
+bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    const bool f32 = lhs_dtype == QMM_F32;
+    const double tiles = (double)((m + 127) / 128) * (double)((n + 255) / 256);
+    const double gemm_us = (double)(int64_t)((tiles + 255.0) / 256.0) * ((double)k / 4096.0) * 64.0 * (f32 ? 2.1 : 1.0);
+    const double pass_us = (f32 ? 10.0 : 8.0) + (double)n * (double)k * 0.52 / (f32 ? 1.9e6 : 3.9e6) + (k > 4096 ? 2.0 : 0.0);
+    return (double)((m + 15) / 16) * pass_us < gemm_us;
+}
+
 bool block_params(int enc, int64_t& epb, int64_t& bpb) {
     switch (enc) {
         case QMM_Q4_0: epb = 32; bpb = 18; return true;
@@ -227,11 +240,12 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
             }
             return QMM_OK;
         }
-        // up to 48 rows the small-batch kernel, 16 rows a pass, is faster than the 128-row tiles of the GEMM
-        // (14336 x 4096: 24 us a pass against 105 us)
-        static const int gemm_min = getenv("QMM_GPTQ_GEMM_MIN") ? atoi(getenv("QMM_GPTQ_GEMM_MIN")) : 49;
+        // GEMM (128 x 256 tiles) or passes of the small-batch kernel (16 rows each)?  QMM_GPTQ_GEMM_MIN=<rows> overrides
+        // the estimate of gptq_small_batch_wins.
+        static const int gemm_min = getenv("QMM_GPTQ_GEMM_MIN") ? atoi(getenv("QMM_GPTQ_GEMM_MIN")) : 0;
+        const bool gemm_wins = gemm_min > 0 ? m >= gemm_min : !gptq_small_batch_wins(lhs_dtype, m, n, k);
         if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size) &&
-            (m >= gemm_min || !qmm::gemv_gptq_mm_supported(rhs[0], n, k, cfg->group_size)))
+            (gemm_wins || !qmm::gemv_gptq_mm_supported(rhs[0], n, k, cfg->group_size)))
             return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
                                                     (const uint32_t*)rhs[2], m, n, k, cfg->group_size, out, workspace, s),
                               "qmm_matmul(GPTQ GEMM)");
