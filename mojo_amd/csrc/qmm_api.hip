@@ -46,6 +46,16 @@ bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0;
 // microseconds as measured on 14336 x 4096, 4096 x 14336 and 4096 x 4096 with 64 to 128 rows: a GEMM round costs
 // 64 us per 4096 of K (bf16 lhs; 2.1 x that for an fp32 lhs, which runs two launches) whatever N is, so few column tiles
 // (N = 4096: 16 of 256 compute units) and long K favour the passes: 4096 x 14336 with 128 bf16 rows 126 against 209 us.
+// Q4_K with 2..16 lhs rows: the kernel that cuts K across workgroups, or the one that gives a workgroup whole rows?
+// QMM_Q4K_KC=1 / 0 forces the answer.
+bool q4k_kc_wins(int64_t m, int64_t n, int64_t k) {
+    static const int force = getenv("QMM_Q4K_KC") ? atoi(getenv("QMM_Q4K_KC")) : -1;
+    if (force >= 0) return force != 0;
+    // measured, 4096 x 14336: 16 rows 29.5 against 49.9 us (fp32 lhs), 22.2 against 35.0 us (bf16); 8 rows about even;
+    // 4 rows 26.8 against 19.1 us.  On 14336 x 4096 and on K = 4096 the row kernel wins at every row count.
+    return m >= 9 && n <= 4096 && k > 4096;
+}
+
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     const bool f32 = lhs_dtype == QMM_F32;
     const double tiles = (double)((m + 127) / 128) * (double)((n + 255) / 256);
@@ -192,7 +202,10 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         return a > b ? a : b;
     }
-    if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) return qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);  // 0 up to 8 rows
+    if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) {  // lhs planes from 9 rows on; partial sums of K chunks
+        const int64_t a = qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k), b = m >= 2 ? qmm::gemv_q4_k_kc_workspace_bytes(m, n, k) : 0;
+        return a > b ? a : b;
+    }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
         const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k) : 0;
@@ -330,6 +343,13 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         return QMM_OK;
     }
 
+    // 2..16 lhs rows on few weight rows and long K: the small-batch kernel that cuts K across workgroups
+    if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && q4k_kc_wins(m, n, k) && qmm::gemv_q4_k_kc_supported(w, k)) {
+        bool handled = false;
+        hipError_t e = qmm::launch_gemv_q4_k_kc(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s, &handled);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K small batch, K chunks)");
+        if (handled) return QMM_OK;
+    }
     // 3..16 lhs rows: the small-batch matrix-core kernel; more: the prefill kernel
     if (encoding == QMM_Q4_K && m >= env_q4k_mm_min_m() && m <= 16 && !env_flag_qmm_q4k_small_gemv())
         return hip_status(qmm::launch_gemv_q4_k_mm(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K small batch)");

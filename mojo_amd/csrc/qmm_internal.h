@@ -93,6 +93,10 @@ hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweig
 hipError_t launch_gemv_gptq_act_order(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                       const uint32_t* qzeros, const int32_t* g_idx, int m, int64_t n, int64_t k, int group,
                                       float* out, int64_t ldo, hipStream_t s);
+bool gemv_q4_k_kc_supported(const void* w, int64_t k);
+int64_t gemv_q4_k_kc_workspace_bytes(int64_t m, int64_t n, int64_t k);
+hipError_t launch_gemv_q4_k_kc(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                               int64_t ldo, void* workspace, hipStream_t s, bool* handled);
 int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
 hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                float* out, void* workspace, hipStream_t s);

@@ -63,6 +63,7 @@ def q8_0_round_trip(a: np.ndarray) -> np.ndarray:
     (QE.Q4_K, 1, 1024, 4096), (QE.Q4_K, 4, 1024, 4096),        # k / v
     (QE.Q4_K, 1, 14336, 4096), (QE.Q4_K, 4, 14336, 4096),      # gate / up
     (QE.Q4_K, 1, 4096, 14336), (QE.Q4_K, 4, 4096, 14336),      # down
+    (QE.Q4_K, 16, 4096, 14336),    # down with 16 rows: the small-batch kernel that cuts K across workgroups
     (QE.Q6_K, 1, 128256, 4096),    # lm_head
 ])
 def test_decode_configurations_full_size(enc, m, n, k):

@@ -307,6 +307,29 @@ def test_gptq_small_batch(m, n, k, group, bf16):
     assert_close(got, truth, f"GPTQ small batch {m}x{n}x{k} group={group} bf16={bf16}")
 
 
+@pytest.mark.parametrize("m,n,k,bf16", [(13, 64, 14336, False), (16, 520, 8192, True), (9, 33, 4352, False), (12, 1, 4608, True),
+                                        (16, 100, 28672, False)])
+def test_q4_k_small_batch_k_chunks(m, n, k, bf16):
+    """9 to 16 lhs rows, at most 4096 weight rows and K beyond 4096: the small-batch kernel that cuts K across
+    workgroups (2 x 16, 4 x 14, 2 x 9 with an idle wavefront, 2 x 9 and 7 x 16 super-blocks), partial sums through the
+    workspace; a third of the rows carry arbitrary bit patterns, lhs rows of very different magnitude."""
+    w, a = synth(95, n, k, m)
+    a[0] *= 1e-5
+    a[m - 1] *= 1e4
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    blocks = O.quantize(O.Q4_K, w).reshape(n, k // 256, 144)
+    rng = np.random.Generator(np.random.PCG64(96))
+    blocks[::3] = rng.integers(0, 256, size=blocks[::3].shape, dtype=np.uint8)
+    blocks[::3, :, 0:2] = np.frombuffer(np.float16(0.001).tobytes(), dtype=np.uint8)
+    blocks[::3, :, 2:4] = np.frombuffer(np.float16(0.0007).tobytes(), dtype=np.uint8)
+    wq = np.ascontiguousarray(blocks.reshape(n, -1))
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.Q4_K, None, lhs, gpu(wq))
+    assert_close(got, truth, f"Q4_K small batch, K chunks {m}x{n}x{k} bf16={bf16}")
+
+
 @pytest.mark.parametrize("m", [4, 16, 64])
 def test_q4_k_unit_sub_block_scales_long_k(m):
     """Q4_K rows whose 6-bit scales and mins are all 1, K = 14336, fp32 lhs, through the matrix-core kernels: the
