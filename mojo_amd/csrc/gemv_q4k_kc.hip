@@ -9,9 +9,9 @@
 // its own) in registers, and the workgroup walks over strips of 32 weight rows (two matrix-core tiles of 16).  A lane
 // (row c = l % 16, quarter kq = l / 16) loads the 16-byte header of its row's super-block and, for each of the four
 // 64-weight pairs, the 8 quant bytes 32 p + 8 kq .. + 7: their low nibbles are its share of sub-block 2p, the high
-// nibbles of sub-block 2p + 1.  A masked nibble is the fp16 subnormal q * 2^-24; one packed multiply by 64 * sc
-// makes it sc * q * 2^-18 (exact; a normal number from 16 on, which the matrix cores need to keep the low product
-// bits).  acc += d * 2^18 * P  -  dmin * sum_s mn_s * (sum of the scaled lhs row over sub-block s).
+// nibbles of sub-block 2p + 1.  One shift and one mask put two nibbles at the top of the fp16 subnormal mantissa,
+// q * 2^-18; one packed multiply by sc makes it sc * q * 2^-18 (exact; a normal number from 16 on, which the matrix
+// cores need to keep the low product bits).  acc += d * 2^18 * P  -  dmin * sum_s mn_s * (sum of the scaled lhs row over sub-block s).
 // The wavefronts' partial sums meet in LDS and are added in wavefront order; the chunks' partial results go to the
 // workspace, [chunk][row][N], and a second kernel adds them in chunk order.
 #include <stdlib.h>
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_q4_k_kc_kernel(const uint
         __syncthreads();
     }
 
-    const uint32_t M1 = 0x000F000Fu;
+    const uint32_t M1 = 0x03C003C0u;  // mantissa bits 6..9 of both fp16 halves
     for (; strip < nstrips; strip += (int)gridDim.x) {
         const int next = strip + (int)gridDim.x;
         const bool more = next < nstrips;  // uniform
@@ -167,12 +167,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_q4_k_kc_kernel(const uint
             for (int s = 0; s < 8; s++) {
                 uint32_t sc, mn;
                 q4k_scale_min(s, s3, sc, mn);
-                const float e = 64.0f * (float)sc;
-                const uint32_t sp = pack_half2(e, e);
+                const uint32_t sp = (uint32_t)f2h((float)sc) * 0x00010001u;  // (sc, sc)
                 const uint2 q = qs[j][s >> 1];
-                const int sh = (s & 1) ? 4 : 0;
-                const half8 b = pack4(pk_mul((q.x >> sh) & M1, sp), pk_mul((q.x >> (sh + 8)) & M1, sp),
-                                      pk_mul((q.y >> sh) & M1, sp), pk_mul((q.y >> (sh + 8)) & M1, sp));
+                // nibbles of bytes 0 and 2, then 1 and 3, moved to bits 6..9 of the fp16 halves: q * 2^-18
+                const half8 b = (s & 1) ? pack4(pk_mul((q.x << 2) & M1, sp), pk_mul((q.x >> 6) & M1, sp),
+                                                pk_mul((q.y << 2) & M1, sp), pk_mul((q.y >> 6) & M1, sp))
+                                        : pack4(pk_mul((q.x << 6) & M1, sp), pk_mul((q.x >> 2) & M1, sp),
+                                                pk_mul((q.y << 6) & M1, sp), pk_mul((q.y >> 2) & M1, sp));
                 P = __builtin_amdgcn_mfma_f32_16x16x32_f16(ahi[s], b, P, 0, 0, 0);
                 if constexpr (PLANES == 2)
                     R = __builtin_amdgcn_mfma_f32_16x16x32_f16(s < kLoReg ? alo[s] : lo_w[(s - kLoReg) * 64], b, R, 0, 0, 0);

@@ -48,12 +48,13 @@ bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0;
 // (N = 4096: 16 of 256 compute units) and long K favour the passes: 4096 x 14336 with 128 bf16 rows 126 against 209 us.
 // Q4_K with 2..16 lhs rows: the kernel that cuts K across workgroups, or the one that gives a workgroup whole rows?
 // QMM_Q4K_KC=1 / 0 forces the answer.
-bool q4k_kc_wins(int64_t m, int64_t n, int64_t k) {
+bool q4k_kc_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     static const int force = getenv("QMM_Q4K_KC") ? atoi(getenv("QMM_Q4K_KC")) : -1;
     if (force >= 0) return force != 0;
-    // measured, 4096 x 14336: 16 rows 29.5 against 49.9 us (fp32 lhs), 22.2 against 35.0 us (bf16); 8 rows about even;
-    // 4 rows 26.8 against 19.1 us.  On 14336 x 4096 and on K = 4096 the row kernel wins at every row count.
-    return m >= 9 && n <= 4096 && k > 4096;
+    // measured, 4096 x 14336, this kernel against the row kernel: 16 rows 29.5 / 49.9 us (fp32 lhs), 22.2 / 35.0 us (bf16);
+    // 8 rows 27.1 / 26.9 us (fp32), 21.1 / 26.4 us (bf16); 4 rows 26.6 / 18.8 us, 20.9 / 18.7 us.  On 14336 x 4096 and on
+    // K = 4096 the row kernel wins at every row count.
+    return m >= (lhs_dtype == QMM_F32 ? 9 : 5) && n <= 4096 && k > 4096;
 }
 
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
@@ -344,7 +345,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     }
 
     // 2..16 lhs rows on few weight rows and long K: the small-batch kernel that cuts K across workgroups
-    if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && q4k_kc_wins(m, n, k) && qmm::gemv_q4_k_kc_supported(w, k)) {
+    if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && q4k_kc_wins(lhs_dtype, m, n, k) && qmm::gemv_q4_k_kc_supported(w, k)) {
         bool handled = false;
         hipError_t e = qmm::launch_gemv_q4_k_kc(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s, &handled);
         if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K small batch, K chunks)");

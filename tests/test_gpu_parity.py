@@ -308,9 +308,9 @@ def test_gptq_small_batch(m, n, k, group, bf16):
 
 
 @pytest.mark.parametrize("m,n,k,bf16", [(13, 64, 14336, False), (16, 520, 8192, True), (9, 33, 4352, False), (12, 1, 4608, True),
-                                        (16, 100, 28672, False)])
+                                        (16, 100, 28672, False), (5, 72, 8192, True)])
 def test_q4_k_small_batch_k_chunks(m, n, k, bf16):
-    """9 to 16 lhs rows, at most 4096 weight rows and K beyond 4096: the small-batch kernel that cuts K across
+    """9 to 16 lhs rows (from 5 with a bf16 lhs), at most 4096 weight rows and K beyond 4096: the small-batch kernel that cuts K across
     workgroups (2 x 16, 4 x 14, 2 x 9 with an idle wavefront, 2 x 9 and 7 x 16 super-blocks), partial sums through the
     workspace; a third of the rows carry arbitrary bit patterns, lhs rows of very different magnitude."""
     w, a = synth(95, n, k, m)
