@@ -427,6 +427,13 @@ def extra_timings(layers, acts, gen):
         dev_s, _ = time_graphs(graphs, 100, 10)
         b = sum(alg_bytes(QE.Q4_K, 4, n, k) for _, n, k in PROJ)
         out["q4_k_m4_GB/s"] = round(b * 100 / dev_s / 1e9, 1)
+        # sixteen lhs rows, one step = the same seven projections (small-batch kernels)
+        acts16 = {k: torch.randn((16, k), dtype=torch.float32, device="cuda:0", generator=gen) for k in (4096, 14336)}
+        graphs = [capture([Gemv(QE.Q4_K, w, acts16[k]) for w, (_, n, k) in zip(lw, PROJ)]) for lw in layers]
+        dev_s, _ = time_graphs(graphs, 100, 10)
+        b = sum(alg_bytes(QE.Q4_K, 16, n, k) for _, n, k in PROJ)
+        out["q4_k_m16"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(b * 100 / dev_s / 1e9, 1)}
+        del graphs
     # cfg4: Q6_K lm_head, M=1 (431 MB: larger than the cache by itself)
     w6 = make_weight(QE.Q6_K, 128256, 4096, gen)
     a1 = torch.randn((1, 4096), dtype=torch.float32, device="cuda:0", generator=gen)
