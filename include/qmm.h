@@ -119,8 +119,9 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
  *     pass over the weights; the matrix-core kernel takes plain groups only.
  *   lhs_dtype QMM_F32 or QMM_BF16.  Q4_0 quantises lhs rows to Q8_0 and takes
  *   integer block dots (the reference CPU path); the others keep lhs as given.
- *   flags: bit 0 (QMM_FLAG_W_BF16) rounds dequantised weights to bf16 before
- *   the product in the M > 16 kernels.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K only: the
+ *   flags: bit 0 (QMM_FLAG_W_BF16) is reserved for a mode that rounds the dequantised
+ *   weights to bf16 before the product; no kernel implements it and a call that sets
+ *   it returns QMM_ERR_UNSUPPORTED.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K only: the
  *   lhs is quantised to Q8_K blocks (256 wide, fp32 scale) and the product is the
  *   integer sub-block dot of the ggml-lineage CPU kernels instead of the default
  *   floating-point one; K <= 16384, any m (passes of four rows).

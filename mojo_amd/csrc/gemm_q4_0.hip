@@ -85,9 +85,9 @@ __global__ __launch_bounds__(256) void quantize_q8_0_operand_kernel(const InT* _
     float amax = fabsf(v);
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
-    const float d = amax / 127.0f;
-    const float id = d != 0.0f ? 1.0f / d : 0.0f;
-    const int q = (int)roundf(v * id);
+    uint16_t dh;
+    const float id = q8_0_block_rule(amax, dh);
+    const int q = q8_0_code(v, id);
     int sum = q;
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 32);
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256) void quantize_q8_0_operand_kernel(const InT* _
     const int64_t tb = tile * nkb + kb;
     codes[(tb * 64 + g * 16 + mm) * 8 + (l & 7)] = (int8_t)q;
     if (l == 0) {
-        dscale[tb * 16 + mm] = h2f(f2h(d));
+        dscale[tb * 16 + mm] = h2f(dh);
         csum[tb * 16 + mm] = sum;
     }
 }

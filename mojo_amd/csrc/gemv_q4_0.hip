@@ -119,11 +119,11 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
                                fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
             amax = fmaxf(amax, dpp_move<0xB1>(amax));
             amax = fmaxf(amax, dpp_move<0x4E>(amax));  // the four threads of a block hold its amax
-            const float d = amax / 127.0f;
-            const float id = d != 0.0f ? 1.0f / d : 0.0f;
+            uint16_t dh;
+            const float id = q8_0_block_rule(amax, dh);
             int q[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) q[i] = (int)roundf(v[i] * id);
+            for (int i = 0; i < 8; i++) q[i] = q8_0_code(v[i], id);
             int sum = ((q[0] + q[1]) + (q[2] + q[3])) + ((q[4] + q[5]) + (q[6] + q[7]));
             sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
             sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xf, 0xf, true);
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
                                     ((uint32_t)q[7] << 24);
                 *(uint2*)(lds_codes + ((size_t)mi * nblk + blk) * 8 + 2 * (t & 3)) = make_uint2(c0, c1);
                 if ((t & 3) == 0) {
-                    lds_scale[mi * nblk + blk] = h2f(f2h(d));
+                    lds_scale[mi * nblk + blk] = h2f(dh);
                     lds_sum[mi * nblk + blk] = sum;
                 }
             }

@@ -221,6 +221,8 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
     hipStream_t s = (hipStream_t)stream;
     if (!lhs || !rhs || !out) return fail(QMM_ERR_INVALID, "qmm_matmul: null pointer");
     if (flags & ~(QMM_FLAG_W_BF16 | QMM_FLAG_ACT_Q8K)) return fail(QMM_ERR_INVALID, "qmm_matmul: unknown flag bits 0x%x", flags);
+    if (flags & QMM_FLAG_W_BF16)
+        return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: QMM_FLAG_W_BF16 (weights rounded to bf16 before the product) has no kernel in this build");
     if (m <= 0 || n <= 0 || k <= 0)
         return fail(QMM_ERR_INVALID, "qmm_matmul: M=%lld N=%lld K=%lld must all be positive", (long long)m,
                     (long long)n, (long long)k);

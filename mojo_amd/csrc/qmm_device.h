@@ -41,6 +41,17 @@ __device__ __forceinline__ float load_f32(const InT* p, int64_t i) {
     else return bf2f(p[i]);
 }
 
+// The per-block rule of the Q8_0 activation quantiser (GGUF quantize_row_q8_0), shared by the stand-alone
+// quantiser and by every Q4_0 matmul kernel that quantises its lhs itself: d = amax / 127 in fp32, the stored
+// scale is d narrowed to fp16 (returned as its bit pattern), and a code is round-half-away(x * (1 / d)) with the
+// fp32 d (all codes 0 for an all-zero block).
+__device__ __forceinline__ float q8_0_block_rule(float amax, uint16_t& d_half) {
+    const float d = amax / 127.0f;
+    d_half = f2h(d);
+    return d != 0.0f ? 1.0f / d : 0.0f;
+}
+__device__ __forceinline__ int q8_0_code(float v, float inv_d) { return (int)roundf(v * inv_d); }
+
 __device__ __forceinline__ uint32_t byte_of(uint32_t w, int i) { return (w >> (8 * i)) & 0xffu; }
 
 // Q4_K: 6-bit scale and min of sub-block j (0..7) from the 12 packed bytes,

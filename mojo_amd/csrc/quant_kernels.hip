@@ -182,10 +182,9 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const InT* __restric
     float amax = fabsf(v);
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 32));
-    float d = amax / 127.0f;
-    float id = d != 0.0f ? 1.0f / d : 0.0f;
-    int q = (int)roundf(v * id);
-    uint16_t dh = f2h(d);
+    uint16_t dh;
+    const float id = q8_0_block_rule(amax, dh);
+    int q = q8_0_code(v, id);
     int sum = q;
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 32);

@@ -51,6 +51,8 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
     ``lhs`` is float32 or bfloat16.  Q4_0 quantises ``lhs`` to Q8_0 blocks and
     takes integer block dots; the other encodings use ``lhs`` as given.  ``act_q8k=True`` (Q4_K only)
     quantises ``lhs`` to Q8_K blocks and takes the integer sub-block dots of the ggml-lineage CPU kernels instead.
+    ``w_bf16=True`` asks for the reserved mode that rounds the dequantised weights to bfloat16 first; the library
+    has no kernel for it and raises ``NotImplementedError``.
     """
     if not isinstance(encoding, QuantizationEncoding):
         raise TypeError("encoding must be a QuantizationEncoding")

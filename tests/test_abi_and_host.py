@@ -50,6 +50,9 @@ def test_argument_validation_happens_before_any_launch():
         return lib.qmm_matmul(enc, cfg, lhs, dt, m, k, rhs_arr, n_rhs, n, fake, ws, ws_bytes, 0, None)
 
     assert matmul(1, 1, 4100, 8) == -1 and b"multiple of the block size" in lib.qmm_last_error()
+    # the reserved bf16-weights mode has no kernel: refused, never silently ignored
+    assert lib.qmm_matmul(1, None, fake, 0, 1, 4096, rhs, 1, 8, fake, None, 0, _lib.QMM_FLAG_W_BF16, None) == -2
+    assert b"W_BF16" in lib.qmm_last_error()
     assert matmul(1, 0, 4096, 8) == -1 and b"positive" in lib.qmm_last_error()
     assert matmul(1, 1, 4096, 8, lhs=None) == -1
     assert matmul(7, 1, 4096, 8) == -1 and b"unknown encoding" in lib.qmm_last_error()

@@ -167,6 +167,54 @@ def test_block_dots_extremes():
     assert got.tolist() == [[32 * 8 * 127, -32 * 7 * 127], [-32 * 8 * 127, 32 * 7 * 127]]
 
 
+def _integer_dot_case(m, n, k, one_hot, bf16, seed):
+    """Inputs on which the fp32 output of the Q4_0 path IS the integer block dot: weight blocks with scale 1.0 (fp16
+    0x3C00; with one_hot only block (7 row + 3) % nblocks of a row has it, the others 0.0), random nibbles; lhs
+    values integers or .5 ties of magnitude <= 127 with one +-127 per 32-block, so that the Q8_0 scale is exactly 1
+    and a code is round-half-away of its value.  Every partial sum is an integer below 2^24, so fp32 adds them
+    exactly in any order: out[i, j] == sum_b scale[j, b] * isum[i, j, b] bit for bit."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    nb = k // 32
+    blocks = rng.integers(0, 256, (n, nb, 18), dtype=np.uint8)
+    hot = np.ones((n, nb), bool)
+    if one_hot:
+        hot[:] = False
+        hot[np.arange(n), (7 * np.arange(n) + 3) % nb] = True
+    blocks[:, :, 0] = 0
+    blocks[:, :, 1] = np.where(hot, 0x3C, 0)
+    wq = np.ascontiguousarray(blocks.reshape(n, nb * 18))
+    a = rng.integers(-127, 128, (m, nb, 32)).astype(np.float32)
+    ties = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, -126.5], np.float32)  # (all exact in bf16)
+    a[:, ::3, 8:16] = ties  # x / d lands on a .5 tie in every third block
+    a[:, 1::5, 16:24] = 0.0
+    peak = rng.integers(0, 8, (m, nb))
+    sign = rng.choice(np.array([-127.0, 127.0], np.float32), (m, nb))
+    np.put_along_axis(a, peak[:, :, None], sign[:, :, None], axis=2)
+    a = np.ascontiguousarray(a.reshape(m, k))
+    aq = O.quantize_q8_0(a)
+    assert (aq.reshape(m, nb, 34)[:, :, :2] == np.array([0x00, 0x3C], np.uint8)).all()  # every activation scale is 1.0
+    isum = O.block_dots_q4_0_q8_0(aq, wq, k).astype(np.int64)
+    want = (isum * hot[None, :, :]).sum(axis=2)
+    assert np.abs(want).max() < 2**24
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    return lhs, gpu(wq), want.astype(np.float32)
+
+
+# (m, n, k) -> kernel: 1, 4: the decode kernel that quantises the lhs itself; K = 8224: the first-version decode kernel
+# behind the stand-alone quantiser; 5, 16: small-batch int8 matrix-core kernel; 9 with K % 256 != 0, 33, 64: the
+# 16-row-tile kernel (1, 4 tiles per group); 65, 256: the wide prefill kernel
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("one_hot", [True, False])
+@pytest.mark.parametrize("m,n,k", [(1, 200, 4096), (4, 200, 4096), (2, 70, 8224), (5, 200, 4096), (16, 200, 4096),
+                                   (9, 72, 1056), (33, 200, 1024), (64, 72, 4096), (65, 200, 1024), (256, 136, 4096)])
+def test_q4_0_production_kernels_give_the_integer_block_dots(m, n, k, one_hot, bf16):
+    """The int8 block dots of every Q4_0 matmul kernel, read off its fp32 output, equal the oracle's bit for bit
+    (Q8_0 codes with .5 ties included)."""
+    lhs, wq, want = _integer_dot_case(m, n, k, one_hot, bf16, seed=31 + m)
+    got = qmatmul(QE.Q4_0, None, lhs, wq).cpu().numpy()
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} outputs differ from the integer dots"
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (16, 1024, 4096), (5, 130, 64), (3, 7, 32), (33, 64, 256)])
 def test_q4_0_matmul(m, n, k):
     w, a = synth(0, n, k, m)
