@@ -134,6 +134,22 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
                void* workspace, int64_t workspace_bytes, int flags, void* stream);
 
 /*
+ * qmm_matmul for callers that cannot allocate or pass device memory of their own for scratch: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments and results as qmm_matmul without the workspace pair: the kernels' scratch
+ * (the planes and partial sums qmm_matmul_workspace_bytes sizes) lives in a buffer of
+ * QMM_STATIC_SCRATCH_BYTES that is part of the loaded library, one copy per GPU, held until the process
+ * ends.  The call allocates and frees nothing.  A problem that needs more scratch than that returns
+ * QMM_ERR_WORKSPACE (use qmm_matmul with a workspace).  All calls on one GPU share the buffer: calls that
+ * can overlap there (different streams, different host threads) race and must be ordered by the caller.
+ * Nothing in the buffer is expected to be zero or to survive from one call to the next.
+ */
+#define QMM_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
+int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m,
+                      int64_t k, const void* const* rhs, int n_rhs, int64_t n, float* out, int flags,
+                      void* stream);
+
+/*
  * Several GGUF weight matrices applied to one lhs, as the callers of ops.qmatmul in a transformer
  * block do (q | k | v, and gate | up, take the same activations):
  *   out[j] fp32[m, n[j]] = lhs[m, k] . dequant(rhs[j])^T,  j < count, all rhs of `encoding` and of row length k.

@@ -6,6 +6,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <atomic>
 
 #include "qmm_internal.h"
 
@@ -112,9 +113,41 @@ Q8Planes q8_planes(void* ws, int64_t m, int64_t k) {
 
 }  // namespace
 
+// Scratch memory of qmm_matmul_static: device memory that belongs to the loaded library, one copy per GPU, held
+// until the process ends.  In host code the array's name is only a handle for the runtime, not a device
+// address; the address on each GPU comes from hipGetSymbolAddress with that GPU current, once, and only that
+// pointer is ever handed to a kernel.  (No kernel names the array, so it is the host use in static_scratch() that
+// makes the compiler emit it, with a symbol the runtime can look up; marking it `used` instead keeps that
+// symbol local to the code object and the lookup then fails.)
+static __device__ __align__(256) unsigned char scratch[QMM_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_scratch(void** ws) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul_static: device ordinal %d out of range", dev);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        // (two threads that get here together read the same address for this device)
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_status(e, "hipGetSymbolAddress(scratch)");
+        if (!p || !aligned(p, 256)) return fail(QMM_ERR_HIP, "qmm_matmul_static: the static scratch buffer has no usable device address");
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *ws = p;
+    return QMM_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
-int qmm_version(void) { return 100; }
+int qmm_version(void) { return 101; }
 
 const char* qmm_last_error(void) { return g_err; }
 
@@ -367,6 +400,19 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         if (e != hipSuccess) return hip_status(e, "qmm_matmul");
     }
     return QMM_OK;
+}
+
+int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
+                      const void* const* rhs, int n_rhs, int64_t n, float* out, int flags, void* stream) {
+    const int64_t need = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    if (need > (int64_t)QMM_STATIC_SCRATCH_BYTES)
+        return fail(QMM_ERR_WORKSPACE,
+                    "qmm_matmul_static: this problem needs %lld bytes of scratch and the static buffer holds %lld; "
+                    "use qmm_matmul with a workspace of the caller's",
+                    (long long)need, (long long)QMM_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return qmm_matmul(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, out, ws, (int64_t)QMM_STATIC_SCRATCH_BYTES, flags, stream);
 }
 
 int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, int count,

@@ -42,7 +42,8 @@ def _gptq_cfg(config: Optional[QuantizationConfig]) -> _lib.GptqConfig:
 
 
 def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], lhs: torch.Tensor,
-            *rhs: torch.Tensor, w_bf16: bool = False, act_q8k: bool = False) -> torch.Tensor:
+            *rhs: torch.Tensor, w_bf16: bool = False, act_q8k: bool = False, out: Optional[torch.Tensor] = None,
+            static_scratch: bool = False) -> torch.Tensor:
     """``out[..., N] = lhs[..., K] @ dequantize(rhs)^T`` in fp32.
 
     GGUF encodings take one ``uint8[N, K/epb*bpb]`` tensor of packed blocks (the
@@ -53,6 +54,11 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
     quantises ``lhs`` to Q8_K blocks and takes the integer sub-block dots of the ggml-lineage CPU kernels instead.
     ``w_bf16=True`` asks for the reserved mode that rounds the dequantised weights to bfloat16 first; the library
     has no kernel for it and raises ``NotImplementedError``.
+
+    ``out`` (contiguous float32 ``[M, N]`` on the device of ``lhs``) receives the result instead of a new tensor.
+    ``static_scratch=True`` goes through ``qmm_matmul_static``: the kernels' scratch is the buffer that is part of
+    the library (64 MiB per GPU) instead of a tensor allocated here, so with ``out`` given the call allocates no
+    device memory; calls that may overlap on one GPU must then be ordered by the caller.
     """
     if not isinstance(encoding, QuantizationEncoding):
         raise TypeError("encoding must be a QuantizationEncoding")
@@ -106,14 +112,25 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
         raise ValueError(f"{encoding.name} is not a weight encoding of qmatmul")
     if m == 0 or n == 0:
         raise ValueError("qmatmul of an empty tensor")
-    out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+    else:
+        _require_gpu(out, "out")
+        if out.dtype != torch.float32 or out.numel() != m * n or out.device != lhs.device:
+            raise TypeError(f"out must be a contiguous float32 tensor of {m} x {n} elements on the device of lhs")
     lhs_dt = _DTYPES[lhs.dtype]
-    need = lib.qmm_matmul_workspace_bytes(encoding.code, lhs_dt, m, n, k)
-    ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
+    flags = (_lib.QMM_FLAG_W_BF16 if w_bf16 else 0) | (_lib.QMM_FLAG_ACT_Q8K if act_q8k else 0)
     ptrs = (C.c_void_p * len(rhs))(*[t.data_ptr() for t in rhs])
-    rc = lib.qmm_matmul(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), _ptr(ws),
-                        need, (_lib.QMM_FLAG_W_BF16 if w_bf16 else 0) | (_lib.QMM_FLAG_ACT_Q8K if act_q8k else 0),
-                        _stream(lhs))
+    if static_scratch:
+        rc = lib.qmm_matmul_static(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), flags,
+                                   _stream(lhs))
+    else:
+        need = lib.qmm_matmul_workspace_bytes(encoding.code, lhs_dt, m, n, k)
+        ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
+        rc = lib.qmm_matmul(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), _ptr(ws),
+                            need, flags, _stream(lhs))
+    if rc == -4:
+        raise ValueError("qmatmul: " + lib.qmm_last_error().decode("utf-8", "replace"))
     _lib.check(rc, "qmatmul")
     return out.reshape(*lead, n)
 
