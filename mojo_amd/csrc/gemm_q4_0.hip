@@ -278,7 +278,7 @@ __global__ __launch_bounds__(64 * kSWaves) void gemm_q4_0_small_kernel(const uin
         for (int i = 0; i < kSLoads; i++) {
             const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * pidx[i];
             if (i < kSLoads - 1 || lane < kSPieces - 64 * (kSLoads - 1))
-                load16_to_lds(src, ring_lds + slot * kSSlot + i * 1024);
+                load16_to_lds_once(src, ring_lds + slot * kSSlot + i * 1024);
         }
     };
     int last_issued = -1, ig = 0, it_t = 0, islot = 0;

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
         const uint8_t* base = (const uint8_t*)(ad - (uintptr_t)dl);
 #pragma unroll
         for (int i = 0; i < L; i++)
-            load16_to_lds(base + 16 * (int64_t)min(lane + 64 * i, last), ring_lds + slot * kSlot + i * 1024);
+            load16_to_lds_once(base + 16 * (int64_t)min(lane + 64 * i, last), ring_lds + slot * kSlot + i * 1024);
     };
 
     // --- the lhs, quantised to Q8_0 once per workgroup: thread t takes values 8 t .. 8 t + 7 of every 4096

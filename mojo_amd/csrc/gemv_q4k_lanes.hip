@@ -99,7 +99,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
 #pragma unroll
         for (int i = 0; i < L; i++)
             if (lane + 64 * i < pieces)
-                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece),
+                load16_to_lds_once(base + 16 * min(lane + 64 * i, last_piece),
                               (uint32_t)__builtin_amdgcn_readfirstlane((int)(ring_lds + slot * kSlot + i * 1024)));  // (uniform; says so)
     };
 
@@ -299,16 +299,18 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     static const int ring_env = [] { const char* e = getenv("QMM_Q4K_LANES_RING"); return e ? atoi(e) : 0; }();   // read once: tuning
     static const int percu_env = [] { const char* e = getenv("QMM_Q4K_LANES_WGS"); return e ? atoi(e) : 0; }();  // read once: tuning
     const size_t fixed = (size_t)kWaves * kMaxRows * mt * 4 + act_bytes, slot = (size_t)bpw * Q4_K_BPB;
-    // three slots (two row parts in flight per wavefront), one workgroup per compute unit: measured best over
-    // (2..4 slots) x (1..3 workgroups per compute unit) on the Llama-3-8B shapes
-    int ring = ring_env >= 2 && ring_env <= 4 ? ring_env : 3;
-    const int per_cu = percu_env > 0 ? percu_env : 1;
-    if (!ring_env && (size_t)kWaves * ring * slot + fixed > 160 * 1024) ring = 2;
+    // Two slots (one row part in flight per wavefront while it decodes the other) and one workgroup per compute
+    // unit; two workgroups per compute unit where a row stream is long (16 rows or more) and both fit the LDS.
+    // Measured over (2..4 slots) x (1, 2 workgroups per compute unit), weight loads non-temporal: more slots
+    // never help (14336 x 4096: 7.9 / 8.1 / 8.4 us with 2 / 3 / 4; 196608 x 4096: 85 / 91 / 93 us), the second
+    // workgroup takes the 453 MB tensor from 85 to 75 us (6.05 TB/s) and costs the short launches up to 20 %.
+    int ring = ring_env >= 2 && ring_env <= 4 ? ring_env : 2;
     const size_t lds = (size_t)kWaves * ring * slot + fixed;
     if (lds > (size_t)kLdsPerCu) return hipSuccess;
     const int streams = kWaves / wpr;  // rows in progress per workgroup
-    int64_t wgs = (int64_t)cus * per_cu;
     const int64_t units = swiglu ? n / 2 : n;  // rows, or gate / up row pairs, to deal to the streams
+    const int per_cu = percu_env > 0 ? percu_env : (units >= (int64_t)16 * cus * streams && 2 * lds + 2048 <= (size_t)kLdsPerCu ? 2 : 1);
+    int64_t wgs = (int64_t)cus * per_cu;
     if (wgs * streams > units) wgs = (units + streams - 1) / streams;
     const int64_t min_wgs = (n + (int64_t)streams * kMaxRows - 1) / ((int64_t)streams * kMaxRows);
     if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots

@@ -128,7 +128,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
         for (int i = 0; i < kLoads; i++) {
             const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * min(pidx[i], last_piece);
             if (i < kLoads - 1 || lane < kPieces - 64 * (kLoads - 1))  // the last instruction: 32 lanes
-                load16_to_lds(src, ring_lds + slot * kSlotBytes + i * 1024);
+                load16_to_lds_once(src, ring_lds + slot * kSlotBytes + i * 1024);
         }
     };
 

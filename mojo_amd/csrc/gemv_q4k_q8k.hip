@@ -138,7 +138,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_k_q8k_kernel(const uin
 #pragma unroll
         for (int i = 0; i < L; i++)
             if (lane + 64 * i < pieces)
-                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
+                load16_to_lds_once(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
     };
     // the first weight rows are issued before the lhs is touched: the compiler's waits for the lhs loads below also
     // wait for these rows, which the first decode needs anyway

@@ -391,7 +391,7 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
 #pragma unroll
         for (int i = 0; i < L; i++)
             if (lane + 64 * i < pieces)
-                load16_to_lds(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
+                load16_to_lds_once(base + 16 * min(lane + 64 * i, last_piece), ring_lds + slot * kSlot + i * 1024);
     };
     int issued = 0, islot = 0, cslot = 0;
     for (; issued < min(ring_slots - 1, my_rows); issued++) {

@@ -30,6 +30,15 @@ __device__ __forceinline__ void load16_to_lds(const void* g, uint32_t lds_base) 
                  : "v"(g), "s"(lds_base)
                  : "memory");
 }
+// The same for data that is read exactly once (weight streams): marked non-temporal, so that the caches do not
+// keep it (a plain read of a 453 MB buffer runs at 7.0 TB/s with the mark against 6.3 TB/s without).
+__device__ __forceinline__ void load16_to_lds_once(const void* g, uint32_t lds_base) {
+    uint32_t keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(g), "s"(lds_base)
+                 : "memory");
+}
 
 // Plain global loads into registers, hidden the same way.  The destination may only be used after
 // wait_vmcnt and tie() on it.

@@ -266,6 +266,30 @@ def swiglu(gate, up) -> np.ndarray:
         return g / (1.0 + np.exp(-g)) * np.asarray(up, np.float64)
 
 
+class _Native:
+    """The same source built with -march=native (``make -C oracle native``): only the timed CPU baseline of
+    ``bench.py`` uses it, never a test."""
+
+    def __init__(self, path: str):
+        self._lib = C.CDLL(path)
+
+    def set_num_threads(self, n: int) -> None:
+        self._lib.qo_set_num_threads(C.c_int(n))
+
+    def matmul_f32(self, enc: int, a, w) -> np.ndarray:
+        a, m, k = _rows_k(a)
+        w = _c(w, np.uint8)
+        n = w.shape[0]
+        out = np.empty((m, n), np.float32)
+        rc = self._lib.qo_matmul_f32(C.c_int(enc), _p(a), _p(w), _i64(m), _i64(n), _i64(k), C.c_int(0), _p(out))
+        assert rc == 0
+        return out
+
+
+def native() -> _Native:
+    return _Native(os.path.join(_HERE, "_native", "libqmm_oracle_native.so"))
+
+
 def num_threads() -> int:
     return int(lib().qo_num_threads())
 
