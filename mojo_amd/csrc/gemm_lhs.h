@@ -47,7 +47,11 @@ __device__ __forceinline__ uint32_t pk_fma(uint32_t x, uint32_t s, uint32_t c) {
 // registers.  Left to the compiler, the three-operand form puts the result where P was; the 16-register
 // tuples of the matrix-core accumulators then swap roles and fragment the register file, and the
 // multiply-adds get sunk past the next group's matrix-core instructions.
+// The compiler does not see which registers an asm statement reads, so it cannot place the wait states the
+// hardware wants between a matrix-core instruction that writes P and a vector instruction that reads it (they
+// are not interlocked): twelve idle states in front cover the eight passes of v_mfma_f32_32x32x16_f16.
 __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float16v& P) {
+    asm volatile("s_nop 7\n\ts_nop 3");
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         float t = acc[r];
@@ -62,7 +66,9 @@ __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float1
 //                  (their codes are used in place in the high nibble position, 16*q)
 //   kLhsOrderQ4K16: 8*(pos/8) + (0,2,1,3,4,6,5,7)[slot]   (natural order, the two middle pairs of every 8 swapped:
 //                  the operand order of the 16x16x32 small-batch kernel)
-constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1, kLhsOrderQ4K16 = 2;
+//   kLhsOrderTile: 32*g + 8*f + (0,2,1,3,4,6,5,7)[slot]   (slice f pairs 8 columns of the low-nibble sub-block
+//                  with the same 8 of the high-nibble one: what one lane of the tile kernels unpacks from 8 code bytes)
+constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1, kLhsOrderQ4K16 = 2, kLhsOrderTile = 3;
 
 template <typename AT, int ORDER>
 __global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
@@ -93,6 +99,11 @@ __global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a,
             const int hin = kl >> 5, gg = (kl >> 4) & 1, odd = (kl >> 3) & 1;
             const int pos = (2 * hin + odd) * 16 + gg * 8 + (kl & 4);
             const int64_t o = (int64_t)row * k + (i & ~63) + pos;
+            *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
+            if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
+        } else if constexpr (ORDER == kLhsOrderTile) {
+            const int gg = kl >> 5, f = (kl >> 3) & 3;
+            const int64_t o = (int64_t)row * k + (i & ~63) + f * 16 + gg * 8 + (kl & 4);
             *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
             if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
         } else if constexpr (ORDER == kLhsOrderQ4K16) {
@@ -133,8 +144,11 @@ struct LhsPlanes {
     int64_t bytes;
 };
 
-inline LhsPlanes lhs_planes(void* workspace, int lhs_dtype, int64_t m, int64_t k) {
+// row_pad: the planes are sized for m rounded up to a multiple of it (kernels that read whole row tiles past the
+// last row; the pass leaves those rows unwritten, and nothing computed from them is ever stored).
+inline LhsPlanes lhs_planes(void* workspace, int lhs_dtype, int64_t m, int64_t k, int64_t row_pad = 1) {
     auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
+    m = (m + row_pad - 1) / row_pad * row_pad;
     LhsPlanes p;
     char* ws = (char*)workspace;
     int64_t off = 0;

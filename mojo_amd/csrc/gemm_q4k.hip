@@ -384,12 +384,14 @@ int k_shares(int64_t m, int64_t n, int64_t k, int bm) {
 }  // namespace
 
 int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    if (gemm_q4_k_tile_wanted(m, n, k)) return gemm_q4_k_tile_workspace_bytes(lhs_dtype, m, k);
     const int ks = k_shares(m, n, k, 64);
     return lhs_planes(nullptr, lhs_dtype, m, k).bytes + (ks > 1 ? (int64_t)ks * m * n * 4 : 0);
 }
 
 hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                float* out, void* workspace, hipStream_t s) {
+    if (gemm_q4_k_tile_wanted(m, n, k)) return launch_gemm_q4_k_tile(lhs, lhs_dtype, w, m, n, k, out, workspace, s);
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
     hipError_t e = launch_prep_lhs<kLhsOrderQ4K>(lhs, lhs_dtype, m, k, p, s);
     if (e != hipSuccess) return e;

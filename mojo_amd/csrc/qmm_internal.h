@@ -112,6 +112,12 @@ hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight,
 int64_t gemm_q4_k_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                             float* out, void* workspace, hipStream_t s);
+// The kernel that unpacks each weight tile once per workgroup into LDS (256 x 128 output tiles): taken by
+// launch_gemm_q4_k where gemm_q4_k_tile_wanted says so.
+bool gemm_q4_k_tile_wanted(int64_t m, int64_t n, int64_t k);
+int64_t gemm_q4_k_tile_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
+hipError_t launch_gemm_q4_k_tile(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                                 float* out, void* workspace, hipStream_t s);
 
 hipError_t launch_block_dots_q4_0(const uint8_t* a_q8, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                   int32_t* out, hipStream_t s);

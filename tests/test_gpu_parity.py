@@ -609,6 +609,26 @@ def test_q4_k_gemm_f32_lhs(m, n, k):
     assert_close(got, want, f"Q4_K GEMM fp32 lhs {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("m,n,k,bf16", [(1024, 8192, 512, True), (1000, 9300, 768, True), (300, 32768, 256, True),
+                                        (520, 8200, 512, False)])
+def test_q4_k_gemm_tile_kernel(m, n, k, bf16):
+    """Shapes with at least 256 output tiles of 256 x 128 go to the kernel that unpacks each weight tile once per
+    workgroup into LDS: whole rounds of tiles (256), a last round cut in two K halves that meet through atomic adds
+    (292 tiles: 37 per XCD, 5 in the last round; K = 768 gives halves of 1 and 2 super-blocks), a single super-block
+    (no halves possible), ragged edges, and an fp32 lhs (two planes; the second one adds to the first)."""
+    w, a = synth(14, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_K, w)
+    want = O.matmul_f32(O.Q4_K, a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    wq_d = gpu(wq)
+    got = qmatmul(QE.Q4_K, None, lhs, wq_d)
+    assert_close(got, want, f"Q4_K tile GEMM {m}x{n}x{k}")
+    again = qmatmul(QE.Q4_K, None, lhs, wq_d)  # the two halves of a tile may arrive in either order: same sum
+    assert torch.equal(got, again)
+
+
 def test_q4_k_gemm_wide_range_lhs():
     """Rows of very different magnitude: the per-row power-of-two scaling keeps fp16 operands exact."""
     w, a = synth(13, 96, 512, 40)
