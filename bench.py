@@ -36,7 +36,7 @@ from mojo_amd import _lib, qmatmul, quantize, quantize_gptq  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
 BF16_PEAK_TFLOPS = 2500.0
-PREFILL_KERNEL = "gemm_q4_k_kernel"
+PREFILL_KERNEL = "gemm_q4_k_tile_kernel"
 
 # (name, N, K) of the Llama-3-8B projections
 PROJ = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
@@ -505,7 +505,7 @@ def prefill_main(args, gen) -> int:
     steps, warmup = min(args.steps, 50), min(args.warmup, 5)
     ab = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
     if args.workload == "prefill":
-        call, name, kern = Gemv(QE.Q4_K, make_weight(QE.Q4_K, n, k, gen), ab), "Q4_K", "gemm_q4_k_kernel"
+        call, name, kern = Gemv(QE.Q4_K, make_weight(QE.Q4_K, n, k, gen), ab), "Q4_K", PREFILL_KERNEL
     else:
         wg = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
         call, name, kern = GptqMatmul(wg, ab), "GPTQ g128", "gemm_gptq_kernel"
@@ -601,18 +601,21 @@ def extra_timings(layers, acts, gen):
         b = sum(alg_bytes(QE.Q4_K, 16, n, k) for _, n, k in PROJ)
         out["q4_k_m16"] = {"us_per_step": round(dev_s * 1e6 / 100, 2), "GB/s": round(b * 100 / dev_s / 1e9, 1)}
         del graphs
-    # the decode kernel's asymptote: one Q4_K tensor of 196608 x 4096 (453 MB, beyond every cache), M = 1
+    # the decode kernel's asymptote: single Q4_K tensors of 196608 x 4096 (453 MB) and 393216 x 4096 (906 MB), beyond
+    # every cache, M = 1; and the plain read of the same bytes
     if m == 1:
-        wbig = make_weight(QE.Q4_K, 196608, 4096, gen)
-        g = capture([Gemv(QE.Q4_K, wbig, acts[4096])])
-        dev_s, _ = time_graphs([g], 10, 3)
-        b = alg_bytes(QE.Q4_K, 1, 196608, 4096)
-        out["q4_k_m1_196608x4096_453MB"] = {"us": round(dev_s * 1e6 / 10, 2), "GB/s": round(b * 10 / dev_s / 1e9, 1),
-                                            "frac_of_8000": round(b * 10 / dev_s / 1e9 / HBM_PEAK_GBS, 4)}
-        g = capture([ReadProbe(wbig)])
-        dev_s, _ = time_graphs([g], 10, 3)
-        out["plain_read_453MB"] = {"us": round(dev_s * 1e6 / 10, 2), "GB/s": round(wbig.numel() * 10 / dev_s / 1e9, 1)}
-        del wbig, g
+        for rows in (196608, 393216):
+            wbig = make_weight(QE.Q4_K, rows, 4096, gen)
+            mb = wbig.numel() // 1000000
+            g = capture([Gemv(QE.Q4_K, wbig, acts[4096])])
+            dev_s, _ = time_graphs([g], 10, 3)
+            b = alg_bytes(QE.Q4_K, 1, rows, 4096)
+            out[f"q4_k_m1_{rows}x4096_{mb}MB"] = {"us": round(dev_s * 1e6 / 10, 2), "GB/s": round(b * 10 / dev_s / 1e9, 1),
+                                                  "frac_of_8000": round(b * 10 / dev_s / 1e9 / HBM_PEAK_GBS, 4)}
+            g = capture([ReadProbe(wbig)])
+            dev_s, _ = time_graphs([g], 10, 3)
+            out[f"plain_read_{mb}MB"] = {"us": round(dev_s * 1e6 / 10, 2), "GB/s": round(wbig.numel() * 10 / dev_s / 1e9, 1)}
+            del wbig, g
     # cfg4: Q6_K lm_head, M=1 (431 MB: larger than the cache by itself)
     w6 = make_weight(QE.Q6_K, 128256, 4096, gen)
     a1 = torch.randn((1, 4096), dtype=torch.float32, device="cuda:0", generator=gen)

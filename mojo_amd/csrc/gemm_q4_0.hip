@@ -524,8 +524,7 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
     if (e != hipSuccess) return e;
     // Few lhs rows: the weights are read once and the kernel lives on HBM latency, so K is cut eight
     // ways for more wavefronts in flight; otherwise four.
-    static const bool small_off = getenv("QMM_Q4_0_SMALL_V1") != nullptr;  // read once: fallback switch
-    if (tiles == 1 && k % 256 == 0 && !small_off) {
+    if (tiles == 1 && k % 256 == 0 && !kernel_disabled("q4_0_small")) {
         static int cus = 0;
         if (!cus) {
             int dev = 0;
@@ -546,8 +545,7 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
                                                                                    (int)k);
         return hipGetLastError();
     }
-    static const bool wide_off = getenv("QMM_Q4_0_WIDE_OFF") != nullptr;  // read once: fallback switch
-    if (tiles > 4 && !wide_off) {
+    if (tiles > 4 && !kernel_disabled("q4_0_wide")) {
         const size_t wlds = (size_t)kWWaves * kWNT * kWaveLds;
         static bool wide_set = false;
         if (!wide_set) {

@@ -395,9 +395,9 @@ hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, in
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k);
     hipError_t e = launch_prep_lhs<kLhsOrderQ4K>(lhs, lhs_dtype, m, k, p, s);
     if (e != hipSuccess) return e;
-    // QMM_GEMM_WM=2 selects 8-wavefront workgroups on 128-row tiles (one per compute unit); the default
-    // is 4-wavefront workgroups on 64-row tiles, two per compute unit, which run out of phase.
-    static const int wm_env = getenv("QMM_GEMM_WM") && atoi(getenv("QMM_GEMM_WM")) == 2 ? 2 : 1;
+    // 4-wavefront workgroups on 64-row tiles, two per compute unit, which run out of phase; with that shape
+    // disabled ("q4k_gemm64"), 8-wavefront workgroups on 128-row tiles, one per compute unit.
+    const int wm_env = kernel_disabled("q4k_gemm64") ? 2 : 1;
     const int ksplit = k_shares(m, n, k, 64);
     const int wm_rows = ksplit > 1 ? 1 : wm_env;
     const int bm = 64 * wm_rows;

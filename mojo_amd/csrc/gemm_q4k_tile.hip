@@ -507,9 +507,10 @@ __global__ __launch_bounds__(256) void zero_split_tiles_kernel(float* __restrict
 }
 
 bool gemm_q4_k_tile_wanted(int64_t m, int64_t n, int64_t k) {
-    static const int force = getenv("QMM_Q4K_TILE") ? atoi(getenv("QMM_Q4K_TILE")) : -1;  // read once: 0 / 1 forces the choice
-    if (k % 256 || k < 256) return false;
-    if (force >= 0) return force != 0 && m > 16;
+    // QMM_Q4K_TILE=1 (read once) sends every prefill shape here, for tests of the kernel on small problems
+    static const bool force = getenv("QMM_Q4K_TILE") != nullptr && atoi(getenv("QMM_Q4K_TILE")) == 1;
+    if (k % 256 || k < 256 || kernel_disabled("q4k_tile")) return false;
+    if (force) return m > 16;
     const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
     return m > 128 && tiles >= 256;
 }

@@ -237,8 +237,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_gptq_mm_kernel(
 }  // namespace
 
 bool gemv_gptq_mm_supported(const void* qweight, int64_t n, int64_t k, int group) {
-    static const bool off = getenv("QMM_GPTQ_MM_OFF") != nullptr;  // read once: fallback switch
-    return !off && k % kPartK == 0 && n >= 8 && n % 8 == 0 && ((uintptr_t)qweight & 7) == 0 &&
+    return !kernel_disabled("gptq_mm") && k % kPartK == 0 && n >= 8 && n % 8 == 0 && ((uintptr_t)qweight & 7) == 0 &&
            (group == 64 || group == 128 || group == 256);
 }
 

@@ -9,18 +9,6 @@
 
 namespace qmm {
 
-static bool env_flag_qmm_q4k_v1() {
-    static const bool v = getenv("QMM_Q4K_V1") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
-static bool env_flag_qmm_q6k_v1() {
-    static const bool v = getenv("QMM_Q6K_V1") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
-static bool env_flag_qmm_gptq_v1() {
-    static const bool v = getenv("QMM_GPTQ_V1") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
 
 template <typename AT>
 __device__ __forceinline__ float4 load_a4(const AT* __restrict__ a, int64_t i) {
@@ -320,13 +308,13 @@ __global__ __launch_bounds__(256) void gemv_gptq_kernel(const uint32_t* __restri
 // small-batch matrix-core kernel instead; this is what is left when that is switched off.)
 hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
-    if (m <= 2 && !env_flag_qmm_q4k_v1()) {
+    const bool rows_ok = !kernel_disabled("q4k_rows_v2");  // (the streaming / row kernels of gemv_q4k_valu.hip)
+    if (m <= 2) {
         bool handled = false;
-        hipError_t e = launch_gemv_q4_k_lanes(a, a_dtype, w, m, n, k, out, ldo, s, &handled);
+        hipError_t e = launch_gemv_q4_k_lanes(a, a_dtype, w, m, n, k, out, ldo, s, &handled);  // (declines when disabled)
         if (e != hipSuccess || handled) return e;
-        return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
-    }
-    if (m <= 4 && !env_flag_qmm_q4k_v1()) {
+        if (rows_ok) return launch_gemv_q4_k_rows(a, a_dtype, w, m, n, k, out, ldo, s);
+    } else if (m <= 4 && rows_ok) {
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
         hipError_t e = launch_gemv_q4_k_rows(a, a_dtype, w, 2, n, k, out, ldo, s);
         if (e != hipSuccess) return e;
@@ -345,7 +333,7 @@ hipError_t launch_gemv_q4_k(const void* a, int a_dtype, const uint8_t* w, int m,
 
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                             float* out, int64_t ldo, hipStream_t s) {
-    if (!env_flag_qmm_q6k_v1()) {
+    if (!kernel_disabled("q6k_staged")) {
         bool handled = false;
         hipError_t e = launch_gemv_q6_k_rows(a, a_dtype, w, m, n, k, out, ldo, s, &handled);
         if (e != hipSuccess || handled) return e;
@@ -374,7 +362,7 @@ hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const i
 hipError_t launch_gemv_gptq(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                             const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                             int64_t ldo, hipStream_t s) {
-    if (!env_flag_qmm_gptq_v1()) {
+    if (!kernel_disabled("gptq_cols")) {
         // up to four lhs rows per pass of the column kernel; more rows take more passes over the weights
         const int64_t esz = a_dtype == QMM_F32 ? 4 : 2;
         bool handled = true;

@@ -212,8 +212,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
 hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
                                    int64_t ldo, hipStream_t s, bool* handled) {
     *handled = false;
-    static const bool off = getenv("QMM_Q4_0_V1") != nullptr;  // read once: fallback switch
-    if (off || m > 4 || k < 8) return hipSuccess;
+    if (kernel_disabled("q4_0_stream") || m > 4 || k < 8) return hipSuccess;
     const int nblk = (int)(k / 32);
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const int bpl = nblk <= 128 ? 2 : nblk <= 256 ? 4 : 0;

@@ -211,8 +211,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_q4_k_kc_kernel(const uint
 }  // namespace
 
 bool gemv_q4_k_kc_supported(const void* w, int64_t k) {
-    static const bool off = getenv("QMM_Q4K_KC_OFF") != nullptr;  // read once: fallback switch
-    return !off && k % 256 == 0 && ((uintptr_t)w & 15) == 0;
+    return !kernel_disabled("q4k_kc") && k % 256 == 0 && ((uintptr_t)w & 15) == 0;
 }
 
 // Partial results of the K chunks (none up to K = 4096).

@@ -267,7 +267,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
                                           bool swiglu) {
     *handled = false;
     if (swiglu && (count != 2 || ns[0] != ns[1] || m != 1)) return hipSuccess;
-    static const bool off = getenv("QMM_Q4K_LANES_OFF") != nullptr;  // read once: fallback switch
+    const bool off = kernel_disabled("q4k_lanes");
     const int nblk = (int)(k / 256);
     if (off || m > 1 || nblk > 64 || count < 1 || count > kLanesMaxMats) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
     LanesMats mats;
@@ -296,20 +296,18 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
     // staged lhs rows: one padded record per chunk, each row rounded up to whole load instructions (1 KB)
     const size_t act_bytes = (size_t)mt * (((size_t)(k / 64) * (64 * esz + 16) + 1023) / 1024 * 1024);
-    static const int ring_env = [] { const char* e = getenv("QMM_Q4K_LANES_RING"); return e ? atoi(e) : 0; }();   // read once: tuning
-    static const int percu_env = [] { const char* e = getenv("QMM_Q4K_LANES_WGS"); return e ? atoi(e) : 0; }();  // read once: tuning
     const size_t fixed = (size_t)kWaves * kMaxRows * mt * 4 + act_bytes, slot = (size_t)bpw * Q4_K_BPB;
     // Two slots (one row part in flight per wavefront while it decodes the other) and one workgroup per compute
     // unit; two workgroups per compute unit where a row stream is long (16 rows or more) and both fit the LDS.
     // Measured over (2..4 slots) x (1, 2 workgroups per compute unit), weight loads non-temporal: more slots
     // never help (14336 x 4096: 7.9 / 8.1 / 8.4 us with 2 / 3 / 4; 196608 x 4096: 85 / 91 / 93 us), the second
     // workgroup takes the 453 MB tensor from 85 to 75 us (6.05 TB/s) and costs the short launches up to 20 %.
-    int ring = ring_env >= 2 && ring_env <= 4 ? ring_env : 2;
+    const int ring = 2;
     const size_t lds = (size_t)kWaves * ring * slot + fixed;
     if (lds > (size_t)kLdsPerCu) return hipSuccess;
     const int streams = kWaves / wpr;  // rows in progress per workgroup
     const int64_t units = swiglu ? n / 2 : n;  // rows, or gate / up row pairs, to deal to the streams
-    const int per_cu = percu_env > 0 ? percu_env : (units >= (int64_t)16 * cus * streams && 2 * lds + 2048 <= (size_t)kLdsPerCu ? 2 : 1);
+    const int per_cu = (units >= (int64_t)16 * cus * streams && 2 * lds + 2048 <= (size_t)kLdsPerCu ? 2 : 1);
     int64_t wgs = (int64_t)cus * per_cu;
     if (wgs * streams > units) wgs = (units + streams - 1) / streams;
     const int64_t min_wgs = (n + (int64_t)streams * kMaxRows - 1) / ((int64_t)streams * kMaxRows);

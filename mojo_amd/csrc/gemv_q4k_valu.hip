@@ -15,14 +15,6 @@
 
 namespace qmm {
 
-static bool env_flag_qmm_gemv_nolds() {
-    static const bool v = getenv("QMM_GEMV_NOLDS") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
-static bool env_flag_qmm_gemv_rows() {
-    static const bool v = getenv("QMM_GEMV_ROWS") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
 
 namespace {
 
@@ -437,9 +429,7 @@ __global__ __launch_bounds__(512, MT == 1 ? 4 : 2) void gemv_q4_k_stream_kernel(
 
 hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s) {
-    static const int r_env = [] { const char* e = getenv("QMM_GEMV_R"); return e ? atoi(e) : 0; }();
-    static const int g_env = [] { const char* e = getenv("QMM_GEMV_G"); return e ? atoi(e) : 0; }();
-    static const int w_env = [] { const char* e = getenv("QMM_GEMV_WAVES"); return e ? atoi(e) : 0; }();
+    const int r_env = 0, g_env = 0, w_env = 0;  // (launch-shape overrides of earlier tuning runs: none)
     const int mt = m <= 1 ? 1 : 2;
     // rows per wavefront: as many as keep at least ~2000 wavefronts in the grid
     const int r = r_env > 0 ? r_env : (n >= 8192 ? 4 : (n >= 4096 ? 2 : 1));
@@ -447,10 +437,10 @@ hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     // staged lhs rows, padded to 8 super-blocks, plus 512 bytes of lane sums per step, plus result slots
     const int wv_stream = (w_env == 4 || w_env == 8) ? w_env : 8;  // wavefronts per workgroup of the streaming kernel
     const size_t lds = (size_t)mt * ((nblk + 7) / 8) * (8192 + 512) + (size_t)wv_stream * kStreamMaxRows * mt * 4;
-    const bool ldsa = lds <= 64 * 1024 && !env_flag_qmm_gemv_nolds();
+    const bool ldsa = lds <= 64 * 1024;
     const int waves = w_env > 0 ? w_env : (lds > 32 * 1024 ? 8 : 4);
     const int g = g_env > 0 ? g_env : 1;  // row groups per wavefront
-    if (ldsa && !env_flag_qmm_gemv_rows()) {
+    if (ldsa && !kernel_disabled("q4k_stream")) {
         // streaming kernel: persistent workgroups, as many as fill the machine at 4 wavefronts per SIMD
         static const int num_cu = [] {
             int dev = 0, cu = 256;

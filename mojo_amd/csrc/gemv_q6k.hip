@@ -27,10 +27,6 @@
 
 namespace qmm {
 
-static bool env_flag_qmm_q6k_rows() {
-    static const bool v = getenv("QMM_Q6K_ROWS") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
 
 namespace {
 
@@ -501,17 +497,15 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipGetLastError();
         cus = prop.multiProcessorCount;
     }
-    static const int pc_env = getenv("QMM_Q6K_WG_PER_CU") ? atoi(getenv("QMM_Q6K_WG_PER_CU")) : 0;
-    const int pc = pc_env > 0 ? pc_env : 3;
-    static const bool lanes_off = getenv("QMM_Q6K_LANES_OFF") != nullptr;  // read once: fallback switch
+    const int pc_env = 0, pc = 3;
+    const bool lanes_off = kernel_disabled("q6k_lanes");
     // Rows of whole 16-byte pieces (K a multiple of 2048, up to 16384) and enough of them: the kernel with the rows
     // global -> LDS and the activations in registers, one or two lhs rows per pass over the weights (up to 16 rows:
     // passes of two).  Rows longer than 16 super-blocks are cut into 2 or 4 parts, one wavefront each.
     const int nblk = (int)(k / 256);
     const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
-    static const int64_t min_parts = getenv("QMM_Q6K_LANES_MIN") ? atoll(getenv("QMM_Q6K_LANES_MIN")) : 0;  // read once: tuning
-    const int64_t need_parts = min_parts > 0 ? min_parts : (int64_t)cus * 4 * 8;  // below 8 row parts per wavefront of a one-workgroup-per-CU grid the row-at-a-time kernel is faster
-    if (k % 2048 == 0 && nblk <= 64 && !((uintptr_t)w & 15) && n * wpr >= need_parts && !lanes_off && !env_flag_qmm_q6k_rows()) {
+    const int64_t need_parts = (int64_t)cus * 4 * 8;  // below 8 row parts per wavefront of a one-workgroup-per-CU grid the row-at-a-time kernel is faster
+    if (k % 2048 == 0 && nblk <= 64 && !((uintptr_t)w & 15) && n * wpr >= need_parts && !lanes_off) {
         const int ring = 3;
         const int bpw = nblk / wpr;                                  // 8 .. 16, even
         const int pieces = (12 + bpw * Q6_K_BPB + 15) / 16;
@@ -550,7 +544,7 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
         return hipSuccess;
     }
     if (m > 4) return hipSuccess;
-    if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !env_flag_qmm_q6k_rows()) {
+    if (mt == 1 && n >= (int64_t)cus * pc * 4 * 4 && !kernel_disabled("q6k_slab")) {
         const size_t lds2 = 4 * (size_t)kRunBytes + 4 * (size_t)kParkRows * 4;
         // enough wavefronts that none has more rows than its LDS parking slots
         const int64_t wgs = max((int64_t)cus * pc, (n + 4 * kParkRows - 1) / (4 * kParkRows));

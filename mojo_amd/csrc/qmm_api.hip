@@ -7,21 +7,22 @@
 
 #include <algorithm>
 #include <atomic>
+#include <string>
 
 #include "qmm_internal.h"
 
-static bool env_flag_qmm_q4k_small_gemv() {
-    static const bool v = getenv("QMM_Q4K_SMALL_GEMV") != nullptr;  // read once: 5..16 lhs rows through the decode kernels
-    return v;
+namespace qmm {
+
+bool kernel_disabled(const char* family) {
+    // (parsed on first use; a C++11 static initialiser runs once, also when two host threads get here together)
+    static const std::string list = [] {
+        const char* e = getenv("QMM_DISABLE");
+        return std::string(",") + (e ? e : "") + ",";
+    }();
+    return list.size() > 2 && list.find(std::string(",") + family + ",") != std::string::npos;
 }
-static int env_q4k_mm_min_m() {
-    static const int v = [] { const char* e = getenv("QMM_Q4K_MM_MIN_M"); return e ? atoi(e) : 2; }();  // read once: tuning switch
-    return v;
-}
-static bool env_flag_qmm_q4_0_gemv() {
-    static const bool v = getenv("QMM_Q4_0_GEMV") != nullptr;  // read once: tuning and fallback switch
-    return v;
-}
+
+}  // namespace qmm
 
 namespace {
 
@@ -48,10 +49,7 @@ bool aligned(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0;
 // 64 us per 4096 of K (bf16 lhs; 2.1 x that for an fp32 lhs, which runs two launches) whatever N is, so few column tiles
 // (N = 4096: 16 of 256 compute units) and long K favour the passes: 4096 x 14336 with 128 bf16 rows 126 against 209 us.
 // Q4_K with 2..16 lhs rows: the kernel that cuts K across workgroups, or the one that gives a workgroup whole rows?
-// QMM_Q4K_KC=1 / 0 forces the answer.
 bool q4k_kc_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    static const int force = getenv("QMM_Q4K_KC") ? atoi(getenv("QMM_Q4K_KC")) : -1;
-    if (force >= 0) return force != 0;
     // measured, 4096 x 14336, this kernel against the row kernel: 16 rows 29.5 / 49.9 us (fp32 lhs), 22.2 / 35.0 us (bf16);
     // 8 rows 27.1 / 26.9 us (fp32), 21.1 / 26.4 us (bf16); 4 rows 26.6 / 18.8 us, 20.9 / 18.7 us.  On 14336 x 4096 and on
     // K = 4096 the row kernel wins at every row count.
@@ -289,10 +287,8 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
             }
             return QMM_OK;
         }
-        // GEMM (128 x 256 tiles) or passes of the small-batch kernel (16 rows each)?  QMM_GPTQ_GEMM_MIN=<rows> overrides
-        // the estimate of gptq_small_batch_wins.
-        static const int gemm_min = getenv("QMM_GPTQ_GEMM_MIN") ? atoi(getenv("QMM_GPTQ_GEMM_MIN")) : 0;
-        const bool gemm_wins = gemm_min > 0 ? m >= gemm_min : !gptq_small_batch_wins(lhs_dtype, m, n, k);
+        // GEMM (128 x 256 tiles) or passes of the small-batch kernel (16 rows each)?
+        const bool gemm_wins = !gptq_small_batch_wins(lhs_dtype, m, n, k);
         if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size) &&
             (gemm_wins || !qmm::gemv_gptq_mm_supported(rhs[0], n, k, cfg->group_size)))
             return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
@@ -300,8 +296,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
                               "qmm_matmul(GPTQ GEMM)");
         // one pass of the matrix-core small-batch kernel per 16 lhs rows; one row, and two fp32 rows, go to the column
         // kernel (two rows on 14336 x 4096: 12.3 us with a bf16 lhs, 16 us with an fp32 lhs, column kernel 16.5 us)
-        static const int mm_min_env = getenv("QMM_GPTQ_MM_MIN") ? atoi(getenv("QMM_GPTQ_MM_MIN")) : 0;
-        const int mm_min = mm_min_env > 0 ? mm_min_env : (lhs_dtype == QMM_F32 ? 3 : 2);
+        const int mm_min = lhs_dtype == QMM_F32 ? 3 : 2;
         for (int64_t m0 = 0; m0 < m; m0 += 16) {
             int mt = (int)(m - m0 < 16 ? m - m0 : 16);
             bool handled = false;
@@ -357,7 +352,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         }
         return QMM_OK;
     }
-    if (encoding == QMM_Q4_0 && m >= 5 && !env_flag_qmm_q4_0_gemv())
+    if (encoding == QMM_Q4_0 && m >= 5 && !qmm::kernel_disabled("q4_0_mfma"))
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0 && m <= 4) {
         // decode: the kernel that quantises the lhs itself (takes K <= 8192)
@@ -387,7 +382,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         if (handled) return QMM_OK;
     }
     // 3..16 lhs rows: the small-batch matrix-core kernel; more: the prefill kernel
-    if (encoding == QMM_Q4_K && m >= env_q4k_mm_min_m() && m <= 16 && !env_flag_qmm_q4k_small_gemv())
+    if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && !qmm::kernel_disabled("q4k_mm"))
         return hip_status(qmm::launch_gemv_q4_k_mm(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K small batch)");
     if (encoding == QMM_Q4_K && m > 16)
         return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");
@@ -441,7 +436,7 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
             if (e != hipSuccess) return hip_status(e, "qmm_matmul_grouped(Q4_K decode)");
             if (handled) return QMM_OK;
         }
-        if (ok && total <= INT32_MAX && m >= env_q4k_mm_min_m() && !env_flag_qmm_q4k_small_gemv()) {
+        if (ok && total <= INT32_MAX && m >= 2 && !qmm::kernel_disabled("q4k_mm")) {
             // the lhs is narrowed once (in the kernel up to 8 rows, by the separate pass beyond) for all the matrices
             const int64_t need = qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);
             if (need > 0 && (!workspace || workspace_bytes < need))

@@ -9,6 +9,12 @@
 
 namespace qmm {
 
+// Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
+// per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
+// in the dispatch order serves it.  Names: q4k_lanes, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_rows_v2,
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q6k_lanes, q6k_slab, q6k_staged, gptq_mm, gptq_cols.  Nothing is disabled by default.
+bool kernel_disabled(const char* family);
+
 hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
 hipError_t launch_dequant(int enc, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
                           hipStream_t s);
