@@ -300,9 +300,8 @@ hipError_t launch_gemv_gptq_mm(const void* a, int a_dtype, const uint32_t* qweig
     const int64_t dst_ld = cc.chunks > 1 ? n : ldo, chunk_stride = cc.chunks > 1 ? (int64_t)m * n : 0;
 #define QMM_GPTQ_MM(PL_, GK_, AT_)                                                                                   \
     do {                                                                                                             \
-        if (lds > 64 * 1024) {                                                                                       \
-            hipError_t e_ = hipFuncSetAttribute((const void*)gemv_gptq_mm_kernel<PL_, GK_, AT_>,                     \
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);               \
+        if (lds > 64 * 1024) { /* (raised once, to the whole LDS) */                                                 \
+            hipError_t e_ = allow_full_lds<gemv_gptq_mm_kernel<PL_, GK_, AT_>>();                                    \
             if (e_ != hipSuccess) return e_;                                                                         \
         }                                                                                                            \
         gemv_gptq_mm_kernel<PL_, GK_, AT_><<<grid, block, lds, s>>>(qweight, scales, qzeros, (const AT_*)a, dst, m,  \

@@ -246,9 +246,8 @@ hipError_t launch_gemv_q4_k_kc(const void* a, int a_dtype, const uint8_t* w, int
     const int64_t dst_ld = cc.chunks > 1 ? n : ldo, chunk_stride = cc.chunks > 1 ? (int64_t)m * n : 0;
 #define QMM_Q4K_KC(PL_, AT_)                                                                                          \
     do {                                                                                                              \
-        if (lds > 64 * 1024) {                                                                                        \
-            hipError_t e_ = hipFuncSetAttribute((const void*)gemv_q4_k_kc_kernel<PL_, AT_>,                           \
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                \
+        if (lds > 64 * 1024) { /* (the limit is raised once, to the whole LDS: two host threads cannot interleave it) */ \
+            hipError_t e_ = allow_full_lds<gemv_q4_k_kc_kernel<PL_, AT_>>();                                          \
             if (e_ != hipSuccess) return e_;                                                                          \
         }                                                                                                             \
         gemv_q4_k_kc_kernel<PL_, AT_><<<grid, block, lds, s>>>(w, (const AT_*)a, dst, m, (int)n, k, dst_ld, nstrips,  \

@@ -231,7 +231,14 @@ def dequantize(encoding: QuantizationEncoding, *quantized: torch.Tensor, k: Opti
         qweight, scales, qzeros = quantized[:3]
         g_idx = quantized[3] if len(quantized) == 4 else None
         cfg = _gptq_cfg(config)
+        for t, name, dt in ((qweight, "qweight", torch.int32), (scales, "scales", torch.float16), (qzeros, "qzeros", torch.int32)):
+            if t.dtype != dt or t.dim() != 2:
+                raise TypeError(f"{name} must be a rank-2 {dt} tensor")
         kk, n = qweight.shape[0] * 8, qweight.shape[1]
+        g = cfg.group_size
+        # (a group size smaller than the checkpoint's would make the kernel read scales and qzeros past their end)
+        if g <= 0 or kk % g or n % 8 or tuple(scales.shape) != (kk // g, n) or tuple(qzeros.shape) != (kk // g, n // 8):
+            raise ValueError("scales/qzeros shapes do not match (K/group, N) and (K/group, N/8) of this config")
         if g_idx is not None and (g_idx.dtype != torch.int32 or tuple(g_idx.shape) != (kk,)):
             raise TypeError("g_idx must be int32[K]")
         if g_idx is None and cfg.desc_act:

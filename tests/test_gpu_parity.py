@@ -101,6 +101,17 @@ def test_dequantize_gptq_bit_exact():
     assert np.array_equal(bits(got), want.view(np.uint8).reshape(128, -1))
 
 
+def test_dequantize_gptq_rejects_tensors_that_do_not_fit_the_config():
+    """A group size smaller than the checkpoint's would index scales / qzeros past their end: refused on the host."""
+    w, _ = synth(8, 64, 512, 1)
+    qw, sc, qz, gi = O.quantize_gptq(w, 128)
+    t = [gpu(qw), gpu(sc.view(np.float16)), gpu(qz)]
+    with pytest.raises(ValueError, match="scales/qzeros"):
+        dequantize(QE.GPTQ, *t, config=QuantizationConfig(group_size=64))
+    with pytest.raises(TypeError, match="scales"):
+        dequantize(QE.GPTQ, t[0], gpu(sc.view(np.int16)), t[2], config=QuantizationConfig())
+
+
 @pytest.mark.parametrize("m", [1, 4, 64])
 def test_gptq_asymmetric_checkpoint(m):
     """sym=False: zero points other than 8 in qzeros (stored value + 1), through dequantize and every matmul kernel."""
