@@ -70,12 +70,12 @@ __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float1
 //                  with the same 8 of the high-nibble one: what one lane of the tile kernels unpacks from 8 code bytes)
 constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1, kLhsOrderQ4K16 = 2, kLhsOrderTile = 3;
 
+// One lhs row by one workgroup of 256 threads.
 template <typename AT, int ORDER>
-__global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
-                                                       _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum,
-                                                       float* __restrict__ inv) {
+__device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
+                                             _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum, float* __restrict__ inv) {
     __shared__ uint32_t wmax[4];
-    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const AT* ar = a + (int64_t)row * k;
     float mx = 0.0f;
     for (int i = tid * 4; i < k; i += 1024) {
@@ -134,6 +134,13 @@ __global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a,
             as[8 + j] = (_Float16)(sum - sh);
         }
     }
+}
+
+template <typename AT, int ORDER>
+__global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
+                                                       _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum,
+                                                       float* __restrict__ inv) {
+    prep_lhs_row<AT, ORDER>((int)blockIdx.x, a, k, a16, a16_lo, asum, inv);
 }
 
 struct LhsPlanes {

@@ -1,0 +1,510 @@
+// Prefill (m > 16 lhs rows) for Q5_K and Q6_K on the matrix cores, in two steps: a conversion pass turns the
+// packed weights into planes of exact small integers in fp16, already in the LDS image of the matrix-core operand
+// tiles, and a GEMM that is the Q4_K tile kernel without the unpack streams lhs and plane tiles global -> LDS
+// directly and applies the fp32 super-block scales in the lanes.
+//
+// Arithmetic (exact products, fp32 sums, as in gemm_q4k_tile.hip):
+//   Q5_K  w = d * (sc * q) - dmin * mn,  q = nibble | fifth bit << 4 <= 31, sc <= 63: one plane, sc * q <= 1953 (an
+//         fp16 integer); the min term as two extra matrix-core products per super-block over the lhs sub-block sums.
+//   Q6_K  w = d * (sc * q),  q in [-32, 31], sc an int8 per 16 weights: sc * q reaches 4096 and odd values above
+//         2048 are no fp16 numbers, so sc = 16 hi + lo (hi = sc >> 4 in [-8, 7], lo = sc & 15) gives two planes,
+//         (16 hi) * q (a multiple of 16 with at most 9 significant bits) and lo * q (<= 480), both exact.  The GEMM
+//         walks K once per plane; a super-block's partial product of either plane is scaled by the same d.
+// The planes cost workspace (2 bytes per weight and plane) and one pass over the weights (tens of microseconds at
+// the sizes this path is chosen for); they buy a GEMM whose only vector-ALU work is the rescale.
+//
+// Plane layout: [n_tile][plane * steps + step][128 columns][64 halfs] with the 16-byte pieces of a column's row at
+// piece index p ^ ((column / 2) % 8) (the swizzle of the tile kernel's LDS buffers), piece p = 2 f + g holding the
+// weights k = 64 step + 32 g + 8 f + (0,2,1,3,4,6,5,7)[slot] (the lhs order kLhsOrderTile): one (tile, step) is 16 KB
+// of contiguous memory that goes to LDS as it is.  Tables per (n_tile, super-block): d as fp32 [128], and for Q5_K
+// the min operands -(dmin * mn) split exactly into fp16 hi + lo, [128 columns][8 hi, 8 lo].
+#include <stdlib.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "gemm_lhs.h"
+#include "gemm_tile.h"
+#include "lds_stream.h"
+#include "qmm_internal.h"
+
+namespace qmm {
+
+namespace {
+
+constexpr int TM = 256, TN = 128;
+constexpr int kABuf = TM * 128, kBBuf = TN * 128, kSBuf = TM * 32, kMBuf = TN * 32, kDBuf = TN * 4;
+constexpr int kOffA = 0, kOffB = kOffA + 3 * kABuf, kOffS = kOffB + 3 * kBBuf, kOffM = kOffS + kSBuf, kOffD = kOffM + kMBuf;
+constexpr int kOffInv = kOffD + kDBuf, kPlanesLds = kOffInv + TM * 4;
+static_assert(kPlanesLds <= kLdsPerCu, "planes kernel LDS");
+constexpr int kPerm[8] = {0, 2, 1, 3, 4, 6, 5, 7};
+
+struct PlaneSpace {
+    uint8_t* planes;  // [tiles_n][nplanes * steps][16 KB]
+    float* dtab;      // [tiles_n][nblk][128]
+    uint8_t* mtab;    // [tiles_n][nblk][128][32 bytes]   (Q5_K)
+    int64_t bytes;
+};
+PlaneSpace plane_space(void* base, int64_t n, int64_t k, int nplanes, bool with_min) {
+    auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
+    const int64_t tiles_n = (n + TN - 1) / TN, nblk = k / 256;
+    PlaneSpace p;
+    int64_t off = 0;
+    p.planes = (uint8_t*)base + off;
+    off += up(tiles_n * nplanes * nblk * 4 * kBBuf);
+    p.dtab = (float*)((uint8_t*)base + off);
+    off += up(tiles_n * nblk * kDBuf);
+    p.mtab = (uint8_t*)base + off;
+    off += with_min ? up(tiles_n * nblk * kMBuf) : 0;
+    p.bytes = off;
+    return p;
+}
+
+__device__ __forceinline__ uint32_t pack_ints(int a, int b) { return pack_half2((float)a, (float)b); }
+
+}  // namespace
+
+// The conversion.  One workgroup of 256 threads per (n_tile, super-block, quarter of the tile's columns).  The 32 blocks of its
+// columns are first copied into LDS with coalesced two-byte loads (rows of Q6_K blocks start on even addresses only) at a
+// stride that is a multiple of four bytes, so that the code bytes can be read eight at a time; thread t then takes piece
+// t % 8 of column t / 8 of each of the four steps, so that eight neighbouring threads write one 128-byte row of the tile.
+template <int ENC>
+__device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quarter, const uint8_t* __restrict__ w, int n, int nblk,
+                                                   uint8_t* __restrict__ planes, float* __restrict__ dtab, uint8_t* __restrict__ mtab) {
+    constexpr int BPB = ENC == QMM_Q6_K ? Q6_K_BPB : ENC == QMM_Q5_K ? Q5_K_BPB : Q4_K_BPB;
+    constexpr int STRIDE = (BPB + 3) / 4 * 4;  // 212 for Q6_K
+    constexpr int NPL = ENC == QMM_Q6_K ? 2 : 1;
+    constexpr int COLS = TN / 4;
+    __shared__ __attribute__((aligned(16))) uint16_t stage[COLS * STRIDE / 2];
+    const int tid = (int)threadIdx.x, col0 = quarter * COLS;
+    for (int i = tid; i < COLS * (BPB / 2); i += 256) {
+        const int c = i / (BPB / 2), e = i - c * (BPB / 2);
+        const int64_t src_col = min(tile_n * TN + col0 + c, n - 1);
+        stage[c * (STRIDE / 2) + e] = ((const uint16_t*)(w + (src_col * nblk + rb) * BPB))[e];
+    }
+    __syncthreads();
+    const int piece = tid & 7, g = piece & 1, f = piece >> 1;
+    const int64_t steps_row = (int64_t)nblk * 4;
+    {
+        const int col = col0 + (tid >> 3), ncol = tile_n * TN + col;
+        const bool live = ncol < n;
+        const uint8_t* blk = (const uint8_t*)stage + (tid >> 3) * STRIDE;
+        const uint32_t dst_in_tile = (uint32_t)(col * 128 + ((piece ^ ((col >> 1) & 7)) << 4));
+        // Q4_K / Q5_K header fields of this column's block
+        uint32_t sc5[8], mn5[8];
+        uint2 fifth = make_uint2(0, 0);
+        if constexpr (ENC != QMM_Q6_K) {
+            const uint32_t s3[3] = {*(const uint32_t*)(blk + 4), *(const uint32_t*)(blk + 8), *(const uint32_t*)(blk + 12)};
+#pragma unroll
+            for (int q = 0; q < 8; q++) q4k_scale_min(q, s3, sc5[q], mn5[q]);
+            if constexpr (ENC == QMM_Q5_K) fifth = *(const uint2*)(blk + 16 + 8 * f);  // fifth bits of elements 8 f .. 8 f + 7 of every sub-block
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            // the eight weights 64 c + 32 g + 8 f + (0..7) of the super-block: their code bytes are eight neighbours
+            int v0[8], v1[8];
+            if constexpr (ENC == QMM_Q6_K) {
+                const int h = c >> 1, quad = (2 * c + g) & 3;
+                // (columns are 212 bytes apart in the stage: four-byte reads)
+                const uint32_t* qlp = (const uint32_t*)(blk + 64 * h + (quad & 1) * 32 + 8 * f);
+                const uint32_t* qhp = (const uint32_t*)(blk + 128 + 32 * h + 8 * f);
+                const uint2 ql = make_uint2(qlp[0], qlp[1]), qh = make_uint2(qhp[0], qhp[1]);
+                const int sc = (int)(int8_t)blk[192 + 8 * h + 2 * quad + (f >> 1)];
+                const int hi16 = (sc >> 4) * 16, lo = sc & 15;  // sc = 16 hi + lo
+                const int nsh = (quad & 2) ? 4 : 0, hsh = 2 * quad;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int e = kPerm[i];
+                    const uint32_t lw = e < 4 ? ql.x : ql.y, hw = e < 4 ? qh.x : qh.y;
+                    const int q = (int)(((lw >> (8 * (e & 3) + nsh)) & 15u) | (((hw >> (8 * (e & 3) + hsh)) & 3u) << 4)) - 32;
+                    v0[i] = live ? hi16 * q : 0;
+                    v1[i] = live ? lo * q : 0;
+                }
+            } else {
+                const int sb = 2 * c + g;
+                const uint2 qs = *(const uint2*)(blk + (ENC == QMM_Q5_K ? 48 : 16) + 32 * c + 8 * f);
+                const int scale = live ? (int)sc5[sb] : 0;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int e = kPerm[i];
+                    const uint32_t lw = e < 4 ? qs.x : qs.y;
+                    int q = (int)((lw >> (8 * (e & 3) + 4 * g)) & 15u);
+                    if constexpr (ENC == QMM_Q5_K) q |= (int)((((e < 4 ? fifth.x : fifth.y) >> (8 * (e & 3) + sb)) & 1u) << 4);
+                    v0[i] = scale * q;
+                    v1[i] = 0;
+                }
+            }
+            const int64_t step = (int64_t)rb * 4 + c;
+#pragma unroll
+            for (int pl = 0; pl < NPL; pl++) {
+                const int* v = pl == 0 ? v0 : v1;
+                uint8_t* tile = planes + (((int64_t)tile_n * NPL + pl) * steps_row + step) * kBBuf;
+                *(uint4*)(tile + dst_in_tile) = make_uint4(pack_ints(v[0], v[1]), pack_ints(v[2], v[3]), pack_ints(v[4], v[5]), pack_ints(v[6], v[7]));
+            }
+        }
+        // tables: one thread per column
+        if (piece == 0) {
+            const int64_t tb = (int64_t)tile_n * nblk + rb;
+            const uint16_t dbits = *(const uint16_t*)(blk + (ENC == QMM_Q6_K ? 208 : 0));
+            dtab[tb * TN + col] = live ? h2f(dbits) : 0.0f;
+            if constexpr (ENC != QMM_Q6_K) {
+                const uint32_t ndm = ((uint32_t)(*(const uint16_t*)(blk + 2)) ^ 0x8000u) * 0x00010001u;  // (-dmin, -dmin)
+                uint32_t hi[4], lo[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t mp = live ? pack_half2((float)mn5[2 * q], (float)mn5[2 * q + 1]) : 0u;
+                    hi[q] = pk_mul(ndm, mp);
+                    lo[q] = pk_fma(ndm, mp, hi[q] ^ 0x80008000u);
+                }
+                uint8_t* mt = mtab + (tb * TN + col) * 32;
+                *(uint4*)mt = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                *(uint4*)(mt + 16) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            }
+        }
+    }
+}
+
+// Everything the GEMM needs done first, in one launch of 256-thread workgroups: [0, conv) convert weights (the long part,
+// so it starts first), the next m narrow one lhs row each, the rest zero the output tiles that the GEMM fills with atomic adds.
+template <int ENC, typename AT>
+__global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __restrict__ w, int nblk, uint8_t* __restrict__ planes,
+                                                              float* __restrict__ dtab, uint8_t* __restrict__ mtab, int conv,
+                                                              const AT* __restrict__ a, int k, LhsPlanes p, SplitTiles z) {
+    const int b = (int)blockIdx.x;
+    if (b < conv) {
+        const int t = b >> 2, rb = t / z.tiles_n;
+        planes_from_kquant<ENC>(t - rb * z.tiles_n, rb, b & 3, w, z.n, nblk, planes, dtab, mtab);
+    } else if (b < conv + z.m) {
+        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv);
+    } else {
+        const int e = b - conv - z.m;
+        zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
+    }
+}
+
+// The GEMM over the planes.  Structure, buffers and schedule are those of gemm_q4_k_tile_kernel (see there); what differs:
+// the weight operands of a step arrive ready-made (16 KB per tile and step, global -> LDS directly, two steps ahead in a
+// ring of three buffers like the lhs), K is walked once per plane (virtual super-blocks vb = plane * nblk + rb), and the
+// tables of a super-block come from memory.  WITH_MIN: the encoding has a min term (Q5_K).
+template <bool WITH_MIN>
+__global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __restrict__ planes, const float* __restrict__ dtab,
+                                                            const uint8_t* __restrict__ mtab, const _Float16* __restrict__ a16,
+                                                            const _Float16* __restrict__ asum, const float* __restrict__ inv,
+                                                            float* __restrict__ out, int m, int n, int k, int nplanes, int tiles_m,
+                                                            int tiles_n, int with_min, int accumulate, int allow_split) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t lds0 = lds_address(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int nl = lane & 31, g = lane >> 5;
+    const int nblk_row = k >> 8, nblk_virtual = nblk_row * nplanes;
+    const uint32_t fb0 = (uint32_t)(kOffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
+    const int a_minus_b = (kOffA + wm * 64 * 128) - (kOffB + wn * 64 * 128);
+    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
+    const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
+    int full;
+    const int units = xcd_units(n_x, wgs_per_xcd, nblk_virtual, allow_split, full);
+    for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
+        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_virtual);
+        // (uniform values that come out of integer divisions live in vector registers unless told otherwise; everything
+        // below that is derived from them, the base pointers above all, would follow them there)
+        const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * 4;  // this unit's share of the virtual K
+        const int kb0 = __builtin_amdgcn_readfirstlane(unit.kb0), unit_half = __builtin_amdgcn_readfirstlane(unit.half);
+        int tile_m, tile_n;
+        tile_order(unit.tile, tiles_m, tiles_n, kTileGm, tile_m, tile_n);
+        tile_m = __builtin_amdgcn_readfirstlane(tile_m);
+        tile_n = __builtin_amdgcn_readfirstlane(tile_n);
+        const int m0 = tile_m * TM, n0 = tile_n * TN;
+        const uint32_t lane16 = (uint32_t)(lane * 16);
+
+        uint32_t a_off[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            a_off[i] = (uint32_t)((lane >> 3) * (k * 2) + (((lane & 7) ^ ((4 * i + (lane >> 4)) & 7)) << 4));
+        const uint8_t* a_base = (const uint8_t*)a16 + (int64_t)(m0 + wave * 32) * k * 2;
+        const uint32_t s_off = (uint32_t)((wave * 32 + (lane >> 1)) * (nblk_row * 32) + (lane & 1) * 16);
+        const uint8_t* s_base = (const uint8_t*)asum + (int64_t)m0 * nblk_row * 32;
+        const uint8_t* b_base = planes + ((int64_t)tile_n * nblk_virtual + kb0) * 4 * kBBuf;  // (virtual steps of a tile are contiguous)
+        const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * nblk_row * kDBuf;
+        const uint8_t* m_base = mtab + (int64_t)tile_n * nblk_row * kMBuf;
+        auto real_blk = [&](int blk) __attribute__((always_inline)) {  // virtual super-block of this unit -> super-block of the row
+            const int vb = kb0 + min(blk, nblk - 1);
+            return vb >= nblk_row ? vb - nblk_row : vb;  // (at most two planes)
+        };
+
+        auto issue_A1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
+            const int sv = kb0 * 4 + min(step, ns - 1), steps_row = nblk_row * 4;
+            const int sr = sv >= steps_row ? sv - steps_row : sv;
+            const uint32_t dst = lds0 + kOffA + buf * kABuf + wave * 4096;
+            load16_to_lds(a_off[i & 1], a_base + (int64_t)sr * 128 + (int64_t)i * 16 * k,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
+        };
+        // the i-th (0, 1) of this wavefront's two 1 KB pieces of the weight tile of step `step`
+        auto issue_B1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
+            const int piece = (wave * 2 + i) * 1024;
+            load16_to_lds(lane16, b_base + (int64_t)min(step, ns - 1) * kBBuf + piece,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffB + buf * kBBuf + piece)));
+        };
+        // tables and lhs sums of super-block `blk` (of this unit): every wavefront brings an eighth of each
+        auto issue_tables = [&](int blk) __attribute__((always_inline)) {
+            const int rb = real_blk(blk);
+            if (lane < 4)
+                load16_to_lds(lane16, d_base + (int64_t)rb * kDBuf + wave * 64,
+                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffD + wave * 64)));
+            if constexpr (WITH_MIN) {
+                if (lane < 32)
+                    load16_to_lds(lane16, m_base + (int64_t)rb * kMBuf + wave * 512,
+                                  (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffM + wave * 512)));
+                load16_to_lds(s_off, s_base + (int64_t)rb * 32, (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffS + wave * 1024)));
+            }
+        };
+
+        float16v acc[2][2], P[2][2];
+#pragma unroll
+        for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    acc[mi][ni][r] = 0.0f;
+                    P[mi][ni][r] = 0.0f;
+                }
+        half8 afr[2][2], bfr[2][2];
+        float dcur[2] = {0.f, 0.f};
+
+        // ---- tile prologue
+        __syncthreads();  // every wavefront is done with the previous tile's LDS contents
+        issue_tables(0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_A1(0, 0, i);
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_A1(1, 1, i);
+        issue_B1(0, 0, 0);
+        issue_B1(0, 0, 1);
+        issue_B1(1, 1, 0);
+        issue_B1(1, 1, 1);
+        if (tid < TM) *(float*)(smem + kOffInv + tid * 4) = inv[min(m0 + tid, m - 1)];
+        wait_vmcnt<0>();
+        int abuf = 0;  // buffer of the current step (step % 3), lhs and weights alike
+        __syncthreads();
+
+        // Operand addresses of the current step: recomputed every phase from the buffer index behind an empty asm statement.
+        // (Left to itself the compiler keeps the addresses of all three buffers in registers and rotates them, some twenty
+        // registers that push accumulators out to scratch memory.)
+        uint32_t fa = 0, fbb = 0;
+        auto step_bases = [&](int ab) __attribute__((always_inline)) {
+            int ao = a_minus_b + ab * kABuf, bo = ab * kBBuf;
+            asm volatile("" : "+s"(ao), "+s"(bo));
+            fa = fb0 + (uint32_t)ao;
+            fbb = fb0 + (uint32_t)bo;
+        };
+        auto read_frags = [&](int f, int slot) __attribute__((always_inline)) {
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + (uint32_t)((fa ^ (uint32_t)(f << 5)) + mi * 4096));
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++) bfr[slot][ni] = *(const half8*)(smem + (uint32_t)((fbb ^ (uint32_t)(f << 5)) + ni * 4096));
+        };
+        auto mfma_slice = [&](int slot, bool fresh, auto&& between) __attribute__((always_inline)) {
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    if (fresh) P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][ni], zero16, 0, 0, 0);
+                    else P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][ni], P[mi][ni], 0, 0, 0);
+                    between(mi * 2 + ni);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        };
+        auto rescale_tile = [&](int t) __attribute__((always_inline)) {
+            const int mi = t >> 1, ni = t & 1;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mi][ni][r] = fmaf(dcur[ni], P[mi][ni][r], acc[mi][ni][r]);
+        };
+
+        // One phase = from the barrier inside step s - 1 to the barrier inside step s (see gemm_q4_k_tile_kernel).
+        auto phase = [&](int blk, auto CC) __attribute__((always_inline)) {
+            constexpr int c = decltype(CC)::value;
+            const int s = blk * 4 + c;
+            step_bases(abuf);
+            read_frags(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            const int ab2 = abuf == 0 ? 2 : abuf - 1;  // (step + 2) % 3
+            if (s > 0) mfma_slice(1, false, [&](int i) __attribute__((always_inline)) { if (i == 3) issue_A1(s + 2, ab2, 0); });
+            else issue_A1(s + 2, ab2, 0);
+            issue_B1(s + 2, ab2, 0);
+            // tables of super-block blk + 1: the current ones were last read in phase 1 (d in phase 0)
+            if constexpr (c == 2) issue_tables(blk + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            half8 sfr[2], mh, ml;
+            const bool min_now = WITH_MIN && c == 1 && with_min && kb0 + blk < nblk_row;  // (once per super-block of the row: with its first plane)
+            if (min_now) {
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++) sfr[mi] = *(const half8*)(smem + kOffS + (wm * 64 + mi * 32 + nl) * 32 + g * 16);
+                mh = *(const half8*)(smem + kOffM + (wn * 64 + nl) * 32);
+                ml = *(const half8*)(smem + kOffM + (wn * 64 + nl) * 32 + 16);
+            }
+            read_frags(1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (c == 0 && s > 0) {
+                // the finished super-block's rescale, sub-tile by sub-tile, in front of the instruction that restarts its P
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    rescale_tile(t);
+                    __builtin_amdgcn_sched_barrier(0);
+                    P[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][t & 1], zero16, 0, 0, 0);
+                    if (t == 3) issue_A1(s + 2, ab2, 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                mfma_slice(0, c == 0, [&](int i) __attribute__((always_inline)) { if (i == 3) issue_A1(s + 2, ab2, 1); });
+            }
+            if (c == 0) {
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) dcur[ni] = *(const float*)(smem + kOffD + (wn * 64 + ni * 32 + nl) * 4);
+            }
+            if (min_now) {
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+#pragma unroll
+                    for (int mi = 0; mi < 2; mi++) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sfr[mi], mh, acc[mi][ni], 0, 0, 0);
+#pragma unroll
+                    for (int mi = 0; mi < 2; mi++) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sfr[mi], ml, acc[mi][ni], 0, 0, 0);
+                    if (ni == 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        mh = *(const half8*)(smem + kOffM + (wn * 64 + 32 + nl) * 32);
+                        ml = *(const half8*)(smem + kOffM + (wn * 64 + 32 + nl) * 32 + 16);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            read_frags(2, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_slice(1, false, [&](int i) __attribute__((always_inline)) {
+                if (i == 1) issue_B1(s + 2, ab2, 1);
+                if (i == 3) issue_A1(s + 2, ab2, 2);
+            });
+            read_frags(3, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_slice(0, false, [&](int i) __attribute__((always_inline)) { if (i == 3) issue_A1(s + 2, ab2, 3); });
+            // everything issued before this phase has landed: lhs and weights of step s + 1 (and, after phase 3, the tables)
+            if constexpr (c == 2) wait_vmcnt<WITH_MIN ? 9 : 7>();
+            else wait_vmcnt<6>();
+            __syncthreads();
+            abuf = abuf == 2 ? 0 : abuf + 1;
+        };
+        for (int blk = 0; blk < nblk; blk++) {
+            phase(blk, std::integral_constant<int, 0>{});
+            phase(blk, std::integral_constant<int, 1>{});
+            phase(blk, std::integral_constant<int, 2>{});
+            phase(blk, std::integral_constant<int, 3>{});
+        }
+        mfma_slice(1, false, [](int) __attribute__((always_inline)) {});  // last slice of the last step
+#pragma unroll
+        for (int t = 0; t < 4; t++) rescale_tile(t);
+
+        // ---- tile epilogue: undo the row scale, store
+        {
+            const int col0 = n0 + wn * 64 + nl, col1 = col0 + 32;
+            const bool c0_ok = col0 < n, c1_ok = col1 < n;
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+                float4 iv[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) iv[j] = *(const float4*)(smem + kOffInv + (wm * 64 + mi * 32 + 8 * j + 4 * g) * 4);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    const float4 q = iv[r >> 2];
+                    const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
+                    if (row < m) {
+                        float* o_ = out + (int64_t)row * n;
+                        const float v0 = acc[mi][0][r] * is, v1 = acc[mi][1][r] * is;
+                        if (unit_half) {  // one of the two K halves of this tile: out holds zero or the other half
+                            if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
+                            if (c1_ok) unsafeAtomicAdd(o_ + col1, v1);
+                        } else if (accumulate) {
+                            if (c0_ok) o_[col0] += v0;
+                            if (c1_ok) o_[col1] += v1;
+                        } else {
+                            if (c0_ok) __builtin_nontemporal_store(v0, o_ + col0);
+                            if (c1_ok) __builtin_nontemporal_store(v1, o_ + col1);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
+    if (kernel_disabled("kquant_planes") || k % 256 || k < 256) return false;
+    if (encoding == QMM_Q4_K) {  // QMM_Q4K_PLANES=1 (read once) sends every Q4_K prefill shape here, for tests and comparisons
+        static const bool force = getenv("QMM_Q4K_PLANES") != nullptr && atoi(getenv("QMM_Q4K_PLANES")) == 1;
+        return force && m > 16;
+    }
+    if (encoding != QMM_Q5_K && encoding != QMM_Q6_K) return false;
+    // Below these row counts the passes of the decode kernels (16 lhs rows a pass for Q6_K, 1 to 4 for Q5_K) cost less than
+    // the conversion pass plus a GEMM whose 256-row tiles are mostly empty.
+    return encoding == QMM_Q6_K ? m > 64 : m > 32;
+}
+
+int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    const bool q6 = encoding == QMM_Q6_K;
+    const int64_t lhs = (lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes + 255) / 256 * 256;
+    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6).bytes;
+}
+
+hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                              float* out, void* workspace, hipStream_t s) {
+    const bool q6 = encoding == QMM_Q6_K;
+    const int nplanes = q6 ? 2 : 1;
+    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
+    const PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, nplanes, !q6);
+    hipError_t e = q6 ? allow_full_lds<gemm_planes_kernel<false>>() : allow_full_lds<gemm_planes_kernel<true>>();
+    if (e != hipSuccess) return e;
+    const int tiles_m = (int)((m + TM - 1) / TM), tiles_n = (int)((n + TN - 1) / TN), nblk = (int)(k / 256);
+    const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
+    const int nblk_virtual = nblk * nplanes;
+    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, nblk_virtual, wg);
+    const int max_split = z.max_split;
+    const int64_t conv = (int64_t)tiles_n * nblk * 4, blocks = conv + m + (int64_t)max_split * 64;
+    if (blocks > INT32_MAX) return hipErrorInvalidValue;
+    const dim3 pgrid((unsigned)blocks);
+    auto prologue = [&](auto enc_c) {
+        constexpr int ENC = decltype(enc_c)::value;
+        if (lhs_dtype == QMM_F32)
+            planes_prologue_kernel<ENC, float><<<pgrid, dim3(256), 0, s>>>(w, nblk, ps.planes, ps.dtab, ps.mtab, (int)conv, (const float*)lhs, (int)k, p, z);
+        else
+            planes_prologue_kernel<ENC, uint16_t><<<pgrid, dim3(256), 0, s>>>(w, nblk, ps.planes, ps.dtab, ps.mtab, (int)conv, (const uint16_t*)lhs, (int)k, p, z);
+    };
+    if (q6) prologue(std::integral_constant<int, QMM_Q6_K>{});
+    else if (encoding == QMM_Q4_K) prologue(std::integral_constant<int, QMM_Q4_K>{});
+    else prologue(std::integral_constant<int, QMM_Q5_K>{});
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    for (int pass = 0; pass < (p.a16_lo ? 2 : 1); pass++) {
+        // fp32 lhs: the residual plane of the lhs in a second launch, added on top (whole tiles only, no min term)
+        const _Float16* a = pass == 0 ? p.a16 : p.a16_lo;
+        const int split = pass == 0 && max_split > 0 ? 1 : 0;
+        if (q6)
+            gemm_planes_kernel<false><<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m,
+                                                                                    (int)n, (int)k, nplanes, tiles_m, tiles_n, 0, pass, split);
+        else
+            gemm_planes_kernel<true><<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m,
+                                                                                   (int)n, (int)k, nplanes, tiles_m, tiles_n, pass == 0, pass, split);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace qmm

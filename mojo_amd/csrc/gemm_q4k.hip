@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
     // second kernel adds up in a fixed order.  (For large m, cutting only the leftover tiles of the last
     // round along K was tried and lost: a workgroup that has its compute unit to itself runs its last tile
     // about 1.6x faster, and the partial sums cost traffic.)
-    for (int it = 0, tq = (int)(blockIdx.x >> 3); tq < per_xcd; it++, tq += (int)(gridDim.x >> 3)) {
+    for (int tq = (int)(blockIdx.x >> 3); tq < per_xcd; tq += (int)(gridDim.x >> 3)) {
         const int o = (int)(blockIdx.x & 7) * per_xcd + tq;
         if (o >= total) break;
         const int tile = o / ksplit, ks = o - tile * ksplit;

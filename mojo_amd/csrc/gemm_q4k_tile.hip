@@ -51,6 +51,7 @@
 #include <type_traits>
 
 #include "gemm_lhs.h"
+#include "gemm_tile.h"
 #include "lds_stream.h"
 #include "qmm_internal.h"
 
@@ -71,47 +72,6 @@ constexpr int kOffD = kOffM + kMBuf, kOffInv = kOffD + kDBuf, kOffQ = kOffInv + 
 constexpr int kTileLds = kOffH + 2 * kHBuf;
 static_assert(kTileLds <= kLdsPerCu, "tile kernel LDS");
 constexpr float kTwo18f = 262144.0f;
-constexpr int kTileGm = 8;  // lhs tile rows that stay fixed while the tile order of an XCD walks N
-
-__device__ __forceinline__ void tile_order(int o, int tiles_m, int tiles_n, int gm, int& tile_m, int& tile_n) {
-    const int span = gm * tiles_n;
-    const int grp = o / span, rem = o - grp * span;
-    const int rows_here = min(gm, tiles_m - grp * gm);
-    tile_n = rem / rows_here;
-    tile_m = grp * gm + rem - tile_n * rows_here;
-}
-
-// Work units of one XCD.  The tiles are dealt to the 8 XCDs in contiguous ranges (workgroup ids congruent mod 8 share an
-// XCD and its L2); inside a range the W persistent workgroups of the XCD take units u = slot, slot + W, ...  When the
-// range is not a multiple of W, the last round would keep only `rem` of the W compute units busy for a whole tile; if
-// rem <= W / 2, each of those last tiles is cut into two halves of K that go to different workgroups and are added in
-// `out` with atomic adds (onto zeros written beforehand: exactly two terms per element, so the sum does not depend on
-// their order).  That round then takes half a tile's time.
-struct TileUnit {
-    int tile;   // global tile index
-    int kb0;    // first super-block
-    int nb;     // super-blocks
-    int half;   // 0: whole K, plain stores; 1: one of two halves, atomic adds
-};
-__device__ __host__ inline int xcd_units(int n_x, int wgs_per_xcd, int nblk, int allow_split, int& full) {
-    const int rem = n_x % wgs_per_xcd;
-    const bool split = allow_split && rem > 0 && 2 * rem <= wgs_per_xcd && nblk >= 2;
-    full = split ? n_x - rem : n_x;
-    return full + 2 * (n_x - full);
-}
-__device__ __host__ inline TileUnit xcd_unit(int u, int base, int full, int nblk) {
-    TileUnit t;
-    if (u < full) {
-        t.tile = base + u; t.kb0 = 0; t.nb = nblk; t.half = 0;
-    } else {
-        const int j = u - full;
-        t.tile = base + full + (j >> 1);
-        t.kb0 = (j & 1) ? nblk / 2 : 0;
-        t.nb = (j & 1) ? nblk - nblk / 2 : nblk / 2;
-        t.half = 1;
-    }
-    return t;
-}
 
 // the value of lane (lane & ~3) + Q of every quad, in all four of its lanes
 template <int Q>
@@ -485,24 +445,16 @@ __global__ __launch_bounds__(512, 1) void gemm_q4_k_tile_kernel(const uint8_t* _
     }
 }
 
-// Zeros the output tiles that the kernel above will fill with atomic adds of two K halves (same unit arithmetic).
-__global__ __launch_bounds__(256) void zero_split_tiles_kernel(float* __restrict__ out, int m, int n, int tiles_m, int tiles_n,
-                                                               int nblk_row, int wgs_per_xcd, int gm) {
-    const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-    const int x = (int)blockIdx.y, xcd_base = x * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
-    int full;
-    xcd_units(n_x, wgs_per_xcd, nblk_row, 1, full);
-    const int j = (int)blockIdx.x;  // j-th split tile of this XCD
-    if (full + j >= n_x) return;
-    int tile_m, tile_n;
-    tile_order(xcd_base + full + j, tiles_m, tiles_n, gm, tile_m, tile_n);
-    const int m0 = tile_m * TM, n0 = tile_n * TN;
-    for (int e = (int)threadIdx.x; e < TM * (TN / 4); e += 256) {
-        const int row = m0 + e / (TN / 4), col = n0 + (e % (TN / 4)) * 4;
-        if (row >= m) break;
-        float* o = out + (int64_t)row * n + col;
-        for (int q = 0; q < 4; q++)
-            if (col + q < n) o[q] = 0.0f;
+// Everything the GEMM needs done first, in one launch: workgroups [0, m) narrow one lhs row each; the rest zero the
+// output tiles that the GEMM will fill with atomic adds of two K halves.
+template <typename AT>
+__global__ __launch_bounds__(256) void tile_prologue_kernel(const AT* __restrict__ a, int k, LhsPlanes p, SplitTiles z) {
+    const int b = (int)blockIdx.x;
+    if (b < z.m) {
+        prep_lhs_row<AT, kLhsOrderTile>(b, a, k, p.a16, p.a16_lo, p.asum, p.inv);
+    } else {
+        const int e = b - z.m;
+        zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
     }
 }
 
@@ -520,9 +472,7 @@ int64_t gemm_q4_k_tile_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { re
 hipError_t launch_gemm_q4_k_tile(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out,
                                  void* workspace, hipStream_t s) {
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
-    hipError_t e = launch_prep_lhs<kLhsOrderTile>(lhs, lhs_dtype, m, k, p, s);
-    if (e != hipSuccess) return e;
-    e = allow_full_lds<gemm_q4_k_tile_kernel>();
+    hipError_t e = allow_full_lds<gemm_q4_k_tile_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n = (int)((n + TN - 1) / TN);
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
@@ -534,16 +484,13 @@ hipError_t launch_gemm_q4_k_tile(const void* lhs, int lhs_dtype, const uint8_t* 
     }
     const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));  // persistent: one workgroup per compute unit
     // the tiles of a last, at most half-full round are cut in two along K (see TileUnit): their outputs start from zero
-    const int wgs_per_xcd = wg / 8, nblk_row = (int)(k / 256);
-    int full, max_split = 0;
-    for (int x = 0; x < 8; x++) {
-        const int n_x = std::max(0, std::min(per_xcd, total - x * per_xcd));
-        xcd_units(n_x, wgs_per_xcd, nblk_row, 1, full);
-        max_split = std::max(max_split, n_x - full);
-    }
-    if (max_split > 0)
-        zero_split_tiles_kernel<<<dim3((unsigned)max_split, 8), dim3(256), 0, s>>>(out, (int)m, (int)n, tiles_m, tiles_n, nblk_row,
-                                                                                 wgs_per_xcd, kTileGm);
+    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, (int)(k / 256), wg);
+    const int max_split = z.max_split;
+    const dim3 pgrid((unsigned)(m + (int64_t)max_split * 64));
+    if (lhs_dtype == QMM_F32) tile_prologue_kernel<float><<<pgrid, dim3(256), 0, s>>>((const float*)lhs, (int)k, p, z);
+    else tile_prologue_kernel<uint16_t><<<pgrid, dim3(256), 0, s>>>((const uint16_t*)lhs, (int)k, p, z);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
     gemm_q4_k_tile_kernel<<<dim3((unsigned)wg), dim3(512), kTileLds, s>>>(w, p.a16, p.asum, p.inv, out, (int)m, (int)n, (int)k, tiles_m,
                                                                           tiles_n, 1, 0, max_split > 0 ? 1 : 0);
     if (p.a16_lo)  // fp32 lhs: the residual plane, added on top (whole tiles only: every element gets one more term, in a fixed order)

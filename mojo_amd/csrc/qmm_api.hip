@@ -230,6 +230,7 @@ int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int
 
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || k <= 0) return 0;
+    if (qmm::gemm_planes_wanted(encoding, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (encoding == QMM_Q4_0) {
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         return a > b ? a : b;
@@ -338,8 +339,11 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         }
         return QMM_OK;
     }
+    // Q5_K and Q6_K with many lhs rows: weights to fp16 integer planes in the workspace, then the matrix cores
+    if (qmm::gemm_planes_wanted(encoding, m, n, k))
+        return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
     if (encoding == QMM_Q5_K) {
-        // one decode-shaped kernel for every m; a pass takes as many lhs rows as fit its LDS copy of the lhs
+        // a decode-shaped kernel; a pass takes as many lhs rows as fit its LDS copy of the lhs
         const int64_t ngroups = (k / 256 + 15) / 16;
         const int64_t pass = ngroups <= 2 ? 4 : ngroups <= 4 ? 2 : 1;
         if (ngroups > 8) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q5_K takes K <= 32768 (K = %lld)", (long long)k);

@@ -12,7 +12,7 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q6k_lanes, q6k_slab, q6k_staged, gptq_mm, gptq_cols.  Nothing is disabled by default.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, gptq_mm, gptq_cols.  Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 
 hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
@@ -124,6 +124,12 @@ bool gemm_q4_k_tile_wanted(int64_t m, int64_t n, int64_t k);
 int64_t gemm_q4_k_tile_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
 hipError_t launch_gemm_q4_k_tile(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                  float* out, void* workspace, hipStream_t s);
+// Q5_K and Q6_K (Q4_K on request) on the matrix cores: a pass that turns the weights into fp16 integer planes in the
+// workspace, then a tile GEMM over them.
+bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k);
+int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
+hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                              float* out, void* workspace, hipStream_t s);
 
 hipError_t launch_block_dots_q4_0(const uint8_t* a_q8, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                   int32_t* out, hipStream_t s);

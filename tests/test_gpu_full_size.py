@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 
 RTOL, ATOL = 1e-3, 1e-4
 DEV = "cuda:0"
-ENC = {QE.Q4_0: O.Q4_0, QE.Q4_K: O.Q4_K, QE.Q6_K: O.Q6_K}
+ENC = {QE.Q4_0: O.Q4_0, QE.Q4_K: O.Q4_K, QE.Q6_K: O.Q6_K, QE.Q5_K: O.Q5_K}
 
 
 def close_on_gpu(got: torch.Tensor, want64: torch.Tensor) -> torch.Tensor:
@@ -88,7 +88,7 @@ def test_decode_configurations_full_size(enc, m, n, k):
     check_all(got, torch.from_numpy(a_eff).to(DEV).double(), dequantize(enc, packed), f"{enc.name} {m}x{n}x{k}")
 
 
-@pytest.mark.parametrize("kind", ["Q4_K", "GPTQ"])
+@pytest.mark.parametrize("kind", ["Q4_K", "Q6_K", "Q5_K", "GPTQ"])
 def test_prefill_configuration_full_size(kind):
     m, n, k = 2048, 14336, 4096
     w, gen = weights(7, n, k)
@@ -96,11 +96,12 @@ def test_prefill_configuration_full_size(kind):
     idx = np.sort(np.random.default_rng(5).choice(n, 32, replace=False))
     tidx = torch.from_numpy(idx).to(DEV)
     a_np = a.float().cpu().numpy()
-    if kind == "Q4_K":
-        packed = quantize(QE.Q4_K, w)
-        got = qmatmul(QE.Q4_K, None, a, packed)
-        truth = O.matmul_f64(O.Q4_K, a_np, packed[tidx].cpu().numpy())
-        w32 = dequantize(QE.Q4_K, packed)
+    if kind != "GPTQ":
+        enc = QE[kind]
+        packed = quantize(enc, w)
+        got = qmatmul(enc, None, a, packed)
+        truth = O.matmul_f64(ENC[enc], a_np, packed[tidx].cpu().numpy())
+        w32 = dequantize(enc, packed)
     else:
         cfg = QuantizationConfig()
         qw, sc, qz, gi = quantize_gptq(w)

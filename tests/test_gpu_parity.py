@@ -640,6 +640,53 @@ def test_q4_k_gemm_tile_kernel(m, n, k, bf16):
     assert torch.equal(got, again)
 
 
+@pytest.mark.parametrize("enc,m,n,k,bf16", [
+    (QE.Q6_K, 65, 130, 512, True), (QE.Q6_K, 300, 257, 1024, False), (QE.Q6_K, 1000, 9300, 768, True), (QE.Q6_K, 256, 128, 256, True),
+    (QE.Q5_K, 33, 130, 512, True), (QE.Q5_K, 300, 257, 1024, False), (QE.Q5_K, 1000, 9300, 768, True), (QE.Q5_K, 520, 8200, 256, False),
+    (QE.Q5_K, 40, 24, 36864, True)])
+def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
+    """Q5_K above 32 and Q6_K above 64 lhs rows: the weights become fp16 integer planes (Q5_K sc * q; Q6_K two planes,
+    (16 hi) * q and lo * q with sc = 16 hi + lo) and a tile GEMM multiplies them.  Ragged edges in m and n, one super-block,
+    a last round of tiles cut in two K halves (292 tiles; for Q6_K the cut falls between or inside the planes), fp32 lhs
+    (second pass on the residual), a K beyond what the Q5_K decode kernel takes; a third of the blocks carry random bytes
+    (every scale byte value including negative Q6_K scales and the extremes -128 and 127, every code combination)."""
+    e = ENC[enc]
+    bpb = 210 if enc == QE.Q6_K else 176
+    w, a = synth(61, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(e, w)
+    rng = np.random.default_rng(62)
+    blocks = wq.reshape(-1, bpb)
+    rnd = rng.integers(0, 256, blocks.shape, dtype=np.uint8)
+    keep = slice(208, 210) if enc == QE.Q6_K else slice(0, 4)  # the fp16 super-block scales stay finite
+    rnd[:, keep] = blocks[:, keep]
+    blocks[::3] = rnd[::3]
+    if enc == QE.Q6_K:
+        blocks[1, 192:208] = np.array([-128, 127, -1, 0, 15, 16, -16, -17, 1, -127, 126, 64, -64, 100, -100, 8], dtype=np.int8).view(np.uint8)
+    truth = O.matmul_f64(e, a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    wq_d = gpu(wq)
+    got = qmatmul(enc, None, lhs, wq_d)
+    assert_close(got, truth, f"{enc.name} planes GEMM {m}x{n}x{k} bf16={bf16}")
+    if bf16 and n * k <= 1 << 22:
+        assert_close(got, O.matmul_f32(e, a, wq), f"{enc.name} planes GEMM {m}x{n}x{k} vs fp32 oracle")
+    again = qmatmul(enc, None, lhs, wq_d)
+    assert torch.equal(got, again)
+
+
+def test_q6_k_prefill_equals_the_decode_kernel_passes():
+    """The same product through the planes GEMM (72 rows at once) and through the decode kernel (the rows in three calls
+    of at most 64): two summation orders of the same exact products."""
+    w, a = synth(63, 700, 2048, 72)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq_d = gpu(O.quantize(O.Q6_K, w))
+    lhs = gpu(a).to(torch.bfloat16)
+    whole = qmatmul(QE.Q6_K, None, lhs, wq_d)
+    parts = torch.cat([qmatmul(QE.Q6_K, None, lhs[i:i + 24], wq_d) for i in range(0, 72, 24)])
+    assert_close(whole, parts.cpu().numpy(), "Q6_K planes GEMM against decode passes")
+
+
 def test_q4_k_gemm_wide_range_lhs():
     """Rows of very different magnitude: the per-row power-of-two scaling keeps fp16 operands exact."""
     w, a = synth(13, 96, 512, 40)
