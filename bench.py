@@ -363,9 +363,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "calib"), default="decode",
-                    help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill: the M=2048 GEMM of the "
-                         "same model's gate projection (second target, matrix-core roofline); calib: a plain "
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "calib"), default="decode",
+                    help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill / q6k_prefill / q5k_prefill: the M=2048 "
+                         "GEMM of the same model's gate projection (second target, matrix-core roofline); calib: a plain "
                          "read and a plain copy of 256 MiB, the yardsticks for the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip per-shape and secondary-config timings")
@@ -506,6 +506,10 @@ def prefill_main(args, gen) -> int:
     ab = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
     if args.workload == "prefill":
         call, name, kern = Gemv(QE.Q4_K, make_weight(QE.Q4_K, n, k, gen), ab), "Q4_K", PREFILL_KERNEL
+    elif args.workload == "q6k_prefill":
+        call, name, kern = Gemv(QE.Q6_K, make_weight(QE.Q6_K, n, k, gen), ab), "Q6_K", "planes_prologue_kernel + gemm_planes_kernel"
+    elif args.workload == "q5k_prefill":
+        call, name, kern = Gemv(QE.Q5_K, make_weight(QE.Q5_K, n, k, gen), ab), "Q5_K", "planes_prologue_kernel + gemm_planes_kernel"
     else:
         wg = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
         call, name, kern = GptqMatmul(wg, ab), "GPTQ g128", "gemm_gptq_kernel"
@@ -519,11 +523,11 @@ def prefill_main(args, gen) -> int:
         "steps": steps, "warmup": warmup, "ms_per_step": round(us / 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 products, f32 sums", "data": "synthetic",
         "config": {"workload": f"{name} prefill GEMM, bf16 lhs [{mm}, {k}] x weights [{n}, {k}], fp32 out; one step = "
-                               f"lhs preparation + one GEMM launch", "m": mm, "n": n, "k": k},
+                               f"lhs preparation (for Q5_K / Q6_K also the weight conversion) + one GEMM launch", "m": mm, "n": n, "k": k},
         "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": kern,
                      "flops_per_launch": flops, "launch_us": round(us, 2),
-                     "note": "launch_us includes the lhs preparation kernel (a few microseconds)"},
+                     "note": "launch_us includes the preparation kernel (lhs narrowing; for Q5_K / Q6_K also the weight planes)"},
         "cpu_baseline": None,
     }))
     return 0
@@ -633,6 +637,15 @@ def extra_timings(layers, acts, gen):
     tf = 2 * 2048 * 14336 * 4096 / us / 1e6
     out["q4_k_prefill_m2048"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
     del wp
+    # the same shape with Q6_K and Q5_K weights (weights to fp16 integer planes, then a tile GEMM: the times include both)
+    for enc, tag in ((QE.Q6_K, "q6_k_prefill_m2048"), (QE.Q5_K, "q5_k_prefill_m2048")):
+        wk = make_weight(enc, 14336, 4096, gen)
+        g = capture([Gemv(enc, wk, ab)])
+        dev_s, _ = time_graphs([g], 10, 2)
+        us = dev_s * 1e6 / 10
+        tf = 2 * 2048 * 14336 * 4096 / us / 1e6
+        out[tag] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
+        del wk, g
     # cfg5, second weight set: GPTQ (group 128) prefill on the same shape
     wg = quantize_gptq(torch.randn((14336, 4096), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
     g = capture([GptqMatmul(wg, ab)])
