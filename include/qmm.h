@@ -107,8 +107,10 @@ int qmm_quantize(int encoding, const float* x, int64_t rows, int64_t k, void* ou
 int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int64_t k,
                       void* qweight, void* scales, void* qzeros, void* g_idx, void* stream);
 
-/* Bytes of device scratch qmm_matmul needs for this problem (may be 0). */
+/* Bytes of device scratch qmm_matmul needs for this problem (may be 0); the second form for a call with `flags`
+ * (QMM_FLAG_OUT_BF16 adds room for an fp32 result wherever the kernel does not store bf16 itself). */
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
+int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags);
 
 /*
  * ops.qmatmul: out fp32[m, n] = lhs[m, k] . dequant(rhs)^T.
@@ -124,11 +126,17 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
  *   it returns QMM_ERR_UNSUPPORTED.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K only: the
  *   lhs is quantised to Q8_K blocks (256 wide, fp32 scale) and the product is the
  *   integer sub-block dot of the ggml-lineage CPU kernels instead of the default
- *   floating-point one; K <= 16384, any m (passes of four rows).
+ *   floating-point one; K <= 16384, any m (passes of four rows).  Bit 2 (QMM_FLAG_OUT_BF16): `out`
+ *   points to bf16[m, n] instead of fp32 (the caller's next op takes bf16 activations): the fp32 result is
+ *   rounded to nearest even with NaN mapped to the canonical quiet NaN, the reference's narrowing rule
+ *   (stdlib/src/builtin/simd.mojo:3279-3300).  The Q4_K decode kernel (m = 1, K <= 16384) stores bf16 itself;
+ *   every other problem computes fp32 into the workspace and narrows in a second launch, which takes
+ *   qmm_matmul_workspace_bytes_flags bytes of workspace.
  * rhs is a host array of device pointers.
  */
 #define QMM_FLAG_W_BF16 1
 #define QMM_FLAG_ACT_Q8K 2
+#define QMM_FLAG_OUT_BF16 4
 int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m,
                int64_t k, const void* const* rhs, int n_rhs, int64_t n, float* out,
                void* workspace, int64_t workspace_bytes, int flags, void* stream);

@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(HERE, "libqmm.so")
 QMM_F32, QMM_BF16, QMM_F16 = 0, 1, 2
 QMM_FLAG_W_BF16 = 1
 QMM_FLAG_ACT_Q8K = 2
+QMM_FLAG_OUT_BF16 = 4
 QMM_STATIC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 
@@ -31,6 +32,7 @@ SIGNATURES = {
     "qmm_quantize": (_int, [_int, _vp, _i64, _i64, _vp, _vp]),
     "qmm_quantize_gptq": (_int, [C.POINTER(GptqConfig), _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "qmm_matmul_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64]),
+    "qmm_matmul_workspace_bytes_flags": (_i64, [_int, _int, _i64, _i64, _i64, _int]),
     "qmm_matmul": (_int, [_int, C.POINTER(GptqConfig), _vp, _int, _i64, _i64, C.POINTER(_vp), _int, _i64, _vp, _vp,
                           _i64, _int, _vp]),
     "qmm_matmul_static": (_int, [_int, C.POINTER(GptqConfig), _vp, _int, _i64, _i64, C.POINTER(_vp), _int, _i64, _vp, _int,

@@ -234,7 +234,9 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             nj = mats.end[j] - (j ? mats.end[j - 1] : 0);
             op = mats.out[j];
         }
-        op[(int64_t)mi * (ldo ? ldo : nj) + local] = v;
+        const int64_t at = (int64_t)mi * (ldo ? ldo : nj) + local;
+        if (mats.out_bf16) ((uint16_t*)op)[at] = f2bf(v);
+        else op[at] = v;
     };
     // result slot idx of this stream, the K parts added
     auto result = [&](int idx) __attribute__((always_inline)) {
@@ -249,7 +251,9 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
             // (one lhs row) out[pair] = silu(gate) * up, silu(x) = x / (1 + exp(-x))
             for (int idx = lane; idx < my_rows / 2; idx += 64) {
                 const float g = result(2 * idx), u = result(2 * idx + 1);
-                o0[gs + idx * GS] = g / (1.0f + expf(-g)) * u;
+                const float v = g / (1.0f + expf(-g)) * u;
+                if (mats.out_bf16) ((uint16_t*)o0)[gs + idx * GS] = f2bf(v);
+                else o0[gs + idx * GS] = v;
             }
         } else {
             for (int idx = lane; idx < my_rows * MT; idx += 64) {
@@ -264,7 +268,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
 // lhs; out[j] is fp32 [m, n[j]] (ldo = 0: dense; a single matrix may give its own leading dimension).
 hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
                                           float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled,
-                                          bool swiglu) {
+                                          bool swiglu, bool out_bf16) {
     *handled = false;
     if (swiglu && (count != 2 || ns[0] != ns[1] || m != 1)) return hipSuccess;
     const bool off = kernel_disabled("q4k_lanes");
@@ -281,6 +285,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     }
     mats.count = count;
     mats.swiglu = swiglu ? 1 : 0;
+    mats.out_bf16 = out_bf16 ? 1 : 0;
     if (n > 0x7fffffff) return hipSuccess;
     const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
     const int bpw = (nblk + wpr - 1) / wpr;
@@ -362,8 +367,8 @@ hipError_t launch_swiglu(const float* gate, const float* up, float* out, int64_t
 }
 
 hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
-                                  int64_t ldo, hipStream_t s, bool* handled) {
-    return launch_gemv_q4_k_lanes_grouped(a, a_dtype, 1, &w, &n, &out, m, k, ldo, s, handled, false);
+                                  int64_t ldo, hipStream_t s, bool* handled, bool out_bf16) {
+    return launch_gemv_q4_k_lanes_grouped(a, a_dtype, 1, &w, &n, &out, m, k, ldo, s, handled, false, out_bf16);
 }
 
 }  // namespace qmm

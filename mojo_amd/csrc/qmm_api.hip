@@ -247,9 +247,55 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     return 0;
 }
 
+static int64_t up256(int64_t v) { return (v + 255) / 256 * 256; }
+
+// Does the kernel that serves this problem store bf16 itself?  (The Q4_K decode kernel does; everything else goes
+// through an fp32 result in the workspace and a narrowing pass.)
+static bool stores_bf16_itself(int encoding, int64_t m, int64_t k, int flags) {
+    return encoding == QMM_Q4_K && m == 1 && k % 256 == 0 && k <= 16384 && !(flags & QMM_FLAG_ACT_Q8K) && !qmm::kernel_disabled("q4k_lanes");
+}
+
+int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags) {
+    const int64_t base = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    if (!(flags & QMM_FLAG_OUT_BF16) || m <= 0 || n <= 0 || stores_bf16_itself(encoding, m, k, flags)) return base;
+    return up256(base) + up256(m * n * 4);
+}
+
+static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
+                      const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
+                      int flags, void* stream);
+
 int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
                int flags, void* stream) {
+    if (!(flags & QMM_FLAG_OUT_BF16) || (flags & ~(QMM_FLAG_W_BF16 | QMM_FLAG_ACT_Q8K | QMM_FLAG_OUT_BF16)))
+        return matmul_f32(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, out, workspace, workspace_bytes, flags, stream);
+    // bf16 output
+    const int inner = flags & ~QMM_FLAG_OUT_BF16;
+    if (!lhs || !rhs || !out) return fail(QMM_ERR_INVALID, "qmm_matmul: null pointer");
+    if (!aligned(out, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: bf16 out must be 2-byte aligned");
+    if (m > 0 && n > 0 && k > 0 && m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX && n_rhs == 1 && rhs[0] &&
+        (lhs_dtype == QMM_F32 || lhs_dtype == QMM_BF16) && aligned(lhs, 16) && aligned(rhs[0], 16) && !(inner & QMM_FLAG_W_BF16) &&
+        stores_bf16_itself(encoding, m, k, inner)) {
+        bool handled = false;
+        hipError_t e = qmm::launch_gemv_q4_k_lanes(lhs, lhs_dtype, (const uint8_t*)rhs[0], (int)m, n, k, out, n, (hipStream_t)stream, &handled, true);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K decode, bf16 out)");
+        if (handled) return QMM_OK;
+    }
+    if (m <= 0 || n <= 0) return fail(QMM_ERR_INVALID, "qmm_matmul: M=%lld N=%lld must be positive", (long long)m, (long long)n);
+    const int64_t base = up256(qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k)), need = base + up256(m * n * 4);
+    if (!workspace || workspace_bytes < need)
+        return fail(QMM_ERR_WORKSPACE, "qmm_matmul: bf16 output of this problem goes through an fp32 result in the workspace: %lld bytes required "
+                                       "(qmm_matmul_workspace_bytes_flags), %lld given", (long long)need, (long long)workspace_bytes);
+    if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul: workspace must be 256-byte aligned");
+    float* tmp = (float*)((char*)workspace + base);
+    if (int rc = matmul_f32(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, tmp, workspace, base, inner, stream)) return rc;
+    return hip_status(qmm::launch_f32_to_bf16(tmp, (uint16_t*)out, m * n, (hipStream_t)stream), "qmm_matmul(narrow to bf16)");
+}
+
+static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
+                      const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
+                      int flags, void* stream) {
     hipStream_t s = (hipStream_t)stream;
     if (!lhs || !rhs || !out) return fail(QMM_ERR_INVALID, "qmm_matmul: null pointer");
     if (flags & ~(QMM_FLAG_W_BF16 | QMM_FLAG_ACT_Q8K)) return fail(QMM_ERR_INVALID, "qmm_matmul: unknown flag bits 0x%x", flags);
@@ -403,7 +449,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
 
 int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                       const void* const* rhs, int n_rhs, int64_t n, float* out, int flags, void* stream) {
-    const int64_t need = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    const int64_t need = qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags);
     if (need > (int64_t)QMM_STATIC_SCRATCH_BYTES)
         return fail(QMM_ERR_WORKSPACE,
                     "qmm_matmul_static: this problem needs %lld bytes of scratch and the static buffer holds %lld; "

@@ -61,6 +61,7 @@ struct LanesMats {
     int end[kLanesMaxMats];  // running row count: matrix j owns rows [end[j - 1], end[j])
     int count;
     int swiglu;              // 1: two matrices (gate, up) of equal size; out[0][r] = silu(gate row r) * (up row r)
+    int out_bf16;            // 1: the out pointers are bf16 arrays (round to nearest even, canonical NaN)
 };
 // The same for the small-batch matrix-core kernel: 16-row tiles are numbered through the matrices.
 struct MmMats {
@@ -74,11 +75,13 @@ hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count
                                        float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s);
 hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
                                           float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled,
-                                          bool swiglu = false);
+                                          bool swiglu = false, bool out_bf16 = false);
 // out[i] = silu(gate[i]) * up[i], i < count (fp32)
 hipError_t launch_swiglu(const float* gate, const float* up, float* out, int64_t count, hipStream_t s);
 hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
-                                  int64_t ldo, hipStream_t s, bool* handled);
+                                  int64_t ldo, hipStream_t s, bool* handled, bool out_bf16 = false);
+// out[i] = bf16(x[i]), i < count: round to nearest even, NaN to the canonical quiet NaN
+hipError_t launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count, hipStream_t s);
 hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,

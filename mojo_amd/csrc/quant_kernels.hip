@@ -140,6 +140,17 @@ hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s) {
     return hipGetLastError();
 }
 
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, int64_t count) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256) out[i] = f2bf(x[i]);
+}
+
+hipError_t launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count, hipStream_t s) {
+    int64_t g = (count + 255) / 256;
+    if (g > 256 * 32) g = 256 * 32;
+    f32_to_bf16_kernel<<<dim3((unsigned)(g > 0 ? g : 1)), dim3(256), 0, s>>>(x, out, count);
+    return hipGetLastError();
+}
+
 static int grid_for(int64_t total, int threads) {
     int64_t g = (total + threads - 1) / threads;
     const int64_t cap = 256 * 64;

@@ -43,8 +43,12 @@ def _gptq_cfg(config: Optional[QuantizationConfig]) -> _lib.GptqConfig:
 
 def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], lhs: torch.Tensor,
             *rhs: torch.Tensor, w_bf16: bool = False, act_q8k: bool = False, out: Optional[torch.Tensor] = None,
-            static_scratch: bool = False) -> torch.Tensor:
+            static_scratch: bool = False, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """``out[..., N] = lhs[..., K] @ dequantize(rhs)^T`` in fp32.
+
+    ``out_dtype=torch.bfloat16`` returns the fp32 result rounded to bfloat16 (nearest even, canonical NaN:
+    the narrowing rule of stdlib/src/builtin/simd.mojo:3279-3300) for a consumer that takes bf16 activations; the
+    Q4_K decode kernel stores it directly, other shapes narrow an fp32 result held in the workspace.
 
     GGUF encodings take one ``uint8[N, K/epb*bpb]`` tensor of packed blocks (the
     transposed, quantised weight).  GPTQ takes the AutoGPTQ tensors
@@ -112,20 +116,23 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
         raise ValueError(f"{encoding.name} is not a weight encoding of qmatmul")
     if m == 0 or n == 0:
         raise ValueError("qmatmul of an empty tensor")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError("out_dtype must be float32 or bfloat16")
     if out is None:
-        out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+        out = torch.empty((m, n), dtype=out_dtype, device=lhs.device)
     else:
         _require_gpu(out, "out")
-        if out.dtype != torch.float32 or out.numel() != m * n or out.device != lhs.device:
-            raise TypeError(f"out must be a contiguous float32 tensor of {m} x {n} elements on the device of lhs")
+        if out.dtype != out_dtype or out.numel() != m * n or out.device != lhs.device:
+            raise TypeError(f"out must be a contiguous {out_dtype} tensor of {m} x {n} elements on the device of lhs")
     lhs_dt = _DTYPES[lhs.dtype]
-    flags = (_lib.QMM_FLAG_W_BF16 if w_bf16 else 0) | (_lib.QMM_FLAG_ACT_Q8K if act_q8k else 0)
+    flags = ((_lib.QMM_FLAG_W_BF16 if w_bf16 else 0) | (_lib.QMM_FLAG_ACT_Q8K if act_q8k else 0) |
+             (_lib.QMM_FLAG_OUT_BF16 if out_dtype == torch.bfloat16 else 0))
     ptrs = (C.c_void_p * len(rhs))(*[t.data_ptr() for t in rhs])
     if static_scratch:
         rc = lib.qmm_matmul_static(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), flags,
                                    _stream(lhs))
     else:
-        need = lib.qmm_matmul_workspace_bytes(encoding.code, lhs_dt, m, n, k)
+        need = lib.qmm_matmul_workspace_bytes_flags(encoding.code, lhs_dt, m, n, k, flags)
         ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
         rc = lib.qmm_matmul(encoding.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(rhs), n, _ptr(out), _ptr(ws),
                             need, flags, _stream(lhs))

@@ -687,6 +687,36 @@ def test_q6_k_prefill_equals_the_decode_kernel_passes():
     assert_close(whole, parts.cpu().numpy(), "Q6_K planes GEMM against decode passes")
 
 
+@pytest.mark.parametrize("enc,m,n,k,lhs_bf16", [
+    (QE.Q4_K, 1, 1030, 4096, False), (QE.Q4_K, 1, 4096, 14336, True), (QE.Q4_K, 1, 66, 20480, False), (QE.Q4_K, 4, 512, 4096, False),
+    (QE.Q4_K, 200, 300, 1024, True), (QE.Q6_K, 1, 777, 2048, False), (QE.Q6_K, 70, 130, 512, True), (QE.Q4_0, 3, 130, 4096, False),
+    (QE.Q4_0, 40, 64, 1024, True), (QE.Q5_K, 40, 256, 512, True), (QE.GPTQ, 1, 256, 1024, False), (QE.GPTQ, 24, 128, 512, True)])
+def test_bf16_output_is_the_fp32_result_narrowed(enc, m, n, k, lhs_bf16):
+    """out_dtype=bfloat16: the bits are those of the fp32 result under the reference's narrowing rule (round to nearest
+    even, NaN to the canonical quiet NaN; stdlib/src/builtin/simd.mojo:3279-3300, the oracle's f32_to_bf16), both where
+    the kernel stores bf16 itself (Q4_K decode) and where an fp32 result in the workspace is narrowed afterwards.  A NaN
+    in the first lhs row makes that whole output row NaN."""
+    w, a = synth(71, n, k, m)
+    a[0, 5] = np.nan
+    lhs = gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a)
+    if enc == QE.GPTQ:
+        qw, sc, qz, gi = O.quantize_gptq(w, 128)
+        args = (QuantizationConfig(group_size=128), lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    else:
+        args = (None, lhs, gpu(O.quantize(ENC[enc], w)))
+    f32 = qmatmul(enc, *args)
+    b16 = qmatmul(enc, *args, out_dtype=torch.bfloat16)
+    assert b16.dtype == torch.bfloat16 and b16.shape == f32.shape
+    want = O.f32_to_bf16(f32.cpu().numpy())
+    got = b16.cpu().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    if enc != QE.Q4_0:  # (Q4_0 quantises the lhs first: a NaN does not survive as one)
+        assert np.all((got[0] & 0x7fff) == 0x7fc0)
+    into = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    qmatmul(enc, *args, out=into, out_dtype=torch.bfloat16)
+    assert torch.equal(into.view(torch.int16), b16.view(torch.int16))
+
+
 def test_q4_k_gemm_wide_range_lhs():
     """Rows of very different magnitude: the per-row power-of-two scaling keeps fp16 operands exact."""
     w, a = synth(13, 96, 512, 40)
