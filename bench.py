@@ -70,6 +70,22 @@ class Gemv:
         _lib.check(rc, "qmm_matmul")
 
 
+class NormGemv(Gemv):
+    """One preallocated qmm_matmul_rmsnorm call: RMS normalisation of the lhs rows, then the matmul."""
+
+    def __init__(self, enc: QE, w: torch.Tensor, a: torch.Tensor, gamma: torch.Tensor, eps: float = 1e-5):
+        super().__init__(enc, w, a)
+        self.gamma, self.eps = gamma, eps
+        self.need = self.lib.qmm_matmul_rmsnorm_workspace_bytes(enc.code, self.dt, self.m, self.n, self.k, 0)
+        self.ws = torch.empty((max(self.need, 1),), dtype=torch.uint8, device=a.device)
+
+    def launch(self, stream_ptr: int) -> None:
+        rc = self.lib.qmm_matmul_rmsnorm(self.enc.code, None, C.c_void_p(self.a.data_ptr()), self.dt, C.c_void_p(self.gamma.data_ptr()),
+                                         C.c_float(self.eps), self.m, self.k, self.ptrs, 1, self.n, C.c_void_p(self.out.data_ptr()),
+                                         C.c_void_p(self.ws.data_ptr()), self.need, 0, C.c_void_p(stream_ptr))
+        _lib.check(rc, "qmm_matmul_rmsnorm")
+
+
 class GroupedGemv:
     """One preallocated qmm_matmul_grouped call: several weight matrices, one lhs."""
 
@@ -662,6 +678,11 @@ def extra_timings(layers, acts, gen):
         dev_s, _ = time_graphs([g], 20, 3)
         us = dev_s * 1e6 / (20 * copies)
         out[tag] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q4_0, mm, n, k) / us / 1e3, 1)}
+        if mm == 1:  # the same launches with the RMS normalisation of the lhs as the kernel's prologue
+            gamma = torch.ones((k,), dtype=torch.float32, device="cuda:0")
+            g = capture([NormGemv(QE.Q4_0, c.w, am, gamma) for c in cs])
+            dev_s, _ = time_graphs([g], 20, 3)
+            out[tag + "_rmsnorm_prologue"] = {"us": round(dev_s * 1e6 / (20 * copies), 3)}
         del cs
     # GPTQ (group 128) decode on the gate shape
     am1 = torch.randn((1, 4096), dtype=torch.float32, device="cuda:0", generator=gen)

@@ -184,6 +184,21 @@ int qmm_matmul_swiglu(int encoding, const void* lhs, int lhs_dtype, int64_t m, i
                       int64_t n, float* out, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * The normalisation in front of ops.qmatmul in a Llama block, fused into the call (no counterpart in the reference's op
+ * set: there the graph holds an rms_norm node and a qmatmul node):
+ *     y[m, k] = x * rsqrt(mean_k(x^2) + eps) * gamma,   out = qmatmul(encoding, y, rhs)
+ * with the normalisation in fp32 and y rounded to bf16 when x is bf16 (what a bf16 rms_norm node hands to qmatmul).
+ * x fp32 or bf16 [m, k], gamma fp32 [k], eps >= 0.  Q4_0 with m <= 4 and K <= 8192 (flags = 0) is ONE launch: the decode
+ * kernel, which quantises its lhs rows to Q8_0 itself, normalises them first (gamma must then be 16-byte aligned, else the
+ * general route is taken).  Every other problem is a normalisation launch into the workspace and qmm_matmul on the result.
+ * flags, rhs, cfg, out as for qmm_matmul.
+ */
+int64_t qmm_matmul_rmsnorm_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags);
+int qmm_matmul_rmsnorm(int encoding, const qmm_gptq_config* cfg, const void* x, int x_dtype, const float* gamma, float eps,
+                       int64_t m, int64_t k, const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace,
+                       int64_t workspace_bytes, int flags, void* stream);
+
+/*
  * Test hook for the bit-exact integer check: raw int32 block sums
  * out[m, n, k/32] = sum_32 (q4 - 8) * q8 of Q8_0 lhs blocks (uint8[m, k/32*34])
  * against Q4_0 rhs blocks.

@@ -12,6 +12,7 @@ from .ops import (
     dequantize,
     qmatmul,
     qmatmul_grouped,
+    qmatmul_rmsnorm,
     qmatmul_swiglu,
     quantize,
     quantize_gptq,
@@ -24,6 +25,7 @@ __all__ = [
     "QuantizationEncoding",
     "qmatmul",
     "qmatmul_grouped",
+    "qmatmul_rmsnorm",
     "qmatmul_swiglu",
     "dequantize",
     "quantize",

@@ -41,6 +41,9 @@ SIGNATURES = {
                                   _i64, _vp]),
     "qmm_matmul_swiglu_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64]),
     "qmm_matmul_swiglu": (_int, [_int, _vp, _int, _i64, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _vp]),
+    "qmm_matmul_rmsnorm_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64, _int]),
+    "qmm_matmul_rmsnorm": (_int, [_int, C.POINTER(GptqConfig), _vp, _int, _vp, C.c_float, _i64, _i64, C.POINTER(_vp), _int, _i64,
+                                  _vp, _vp, _i64, _int, _vp]),
     "qmm_block_dots_q4_0": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
 }
 

@@ -42,11 +42,13 @@ __device__ __forceinline__ void wait_rows(int rows) {
 
 // BPL: blocks per lane (k <= 2048 * BPL).  L = load instructions per row = pieces of 16 bytes / 64, for the
 // longest row BPL allows plus one piece of misalignment.  RING: LDS slots per wavefront.
-template <int MT, int BPL, int RING, typename AT>
+// NORM: the lhs rows are RMS-normalised first, y = x * rsqrt(mean(x^2) + eps) * gamma in fp32 (rounded to bf16 when the
+// lhs is bf16: what a bf16 normalisation node would hand over), and y is what gets quantised.
+template <int MT, int BPL, int RING, typename AT, bool NORM>
 __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const uint8_t* __restrict__ w,
                                                                          const AT* __restrict__ a,
                                                                          float* __restrict__ out, int m, int n, int k,
-                                                                         int64_t ldo) {
+                                                                         int64_t ldo, const float* __restrict__ gamma, float eps) {
     constexpr int L = (72 * BPL + 1 + 63) / 64;
     constexpr int kSlot = L * 1024;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -93,26 +95,77 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
 #pragma unroll
             for (int i = 0; i < kPieces; i++) hidden_load(raw[mi][p][i], (const uint8_t*)ar + 16 * i);
         }
+    u32x4 graw[NORM ? P : 1][2];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int64_t v0 = min((int64_t)p * 4096 + 8 * t, (int64_t)k - 8);
+            hidden_load(graw[p][0], (const uint8_t*)(gamma + v0));
+            hidden_load(graw[p][1], (const uint8_t*)(gamma + v0) + 16);
+        }
+    }
     int issued = 0;
     for (; issued < min(RING - 1, my_rows); issued++) issue(issued, issued % RING);
     wait_rows<L>(issued);  // the lhs loads are older than these rows
+    // the eight lhs values of (row mi, pass p) that this thread holds
+    auto values = [&](int mi, int p, float (&v)[8]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kPieces; i++) {
+            tie(raw[mi][p][i]);
+            const u32x4 r = raw[mi][p][i];
+            if constexpr (sizeof(AT) == 4) {
+                v[4 * i] = __uint_as_float(r.x); v[4 * i + 1] = __uint_as_float(r.y);
+                v[4 * i + 2] = __uint_as_float(r.z); v[4 * i + 3] = __uint_as_float(r.w);
+            } else {
+                v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+                v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+                v[4] = __uint_as_float(r.z << 16); v[5] = __uint_as_float(r.z & 0xffff0000u);
+                v[6] = __uint_as_float(r.w << 16); v[7] = __uint_as_float(r.w & 0xffff0000u);
+            }
+        }
+    };
+    float rs[MT];
+    if constexpr (NORM) {
+        // sum of squares of every lhs row over the workgroup: per thread, per wavefront (DPP), then over the 8 wavefronts in order
+        float* red = (float*)(qbase + (size_t)MT * nblk * 40);
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            float ss = 0.0f;
+#pragma unroll
+            for (int p = 0; p < P; p++) {
+                float v[8];
+                values(mi, p, v);
+                const float part = ((v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3])) + ((v[4] * v[4] + v[5] * v[5]) + (v[6] * v[6] + v[7] * v[7]));
+                ss += (int64_t)p * 4096 + 8 * t < k ? part : 0.0f;
+            }
+            ss = wave_sum_dpp(ss);
+            if (lane == 0) red[wave * MT + mi] = ss;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            float tot = 0.0f;
+#pragma unroll
+            for (int q = 0; q < kWaves; q++) tot += red[q * MT + mi];
+            rs[mi] = 1.0f / sqrtf(tot / (float)k + eps);
+        }
+    }
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
 #pragma unroll
         for (int p = 0; p < P; p++) {
             float v[8];
+            values(mi, p, v);
+            if constexpr (NORM) {
+                tie(graw[p][0]);
+                tie(graw[p][1]);
+                const u32x4 g0 = graw[p][0], g1 = graw[p][1];
+                const float g[8] = {__uint_as_float(g0.x), __uint_as_float(g0.y), __uint_as_float(g0.z), __uint_as_float(g0.w),
+                                    __uint_as_float(g1.x), __uint_as_float(g1.y), __uint_as_float(g1.z), __uint_as_float(g1.w)};
 #pragma unroll
-            for (int i = 0; i < kPieces; i++) {
-                tie(raw[mi][p][i]);
-                const u32x4 r = raw[mi][p][i];
-                if constexpr (sizeof(AT) == 4) {
-                    v[4 * i] = __uint_as_float(r.x); v[4 * i + 1] = __uint_as_float(r.y);
-                    v[4 * i + 2] = __uint_as_float(r.z); v[4 * i + 3] = __uint_as_float(r.w);
-                } else {
-                    v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
-                    v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
-                    v[4] = __uint_as_float(r.z << 16); v[5] = __uint_as_float(r.z & 0xffff0000u);
-                    v[6] = __uint_as_float(r.w << 16); v[7] = __uint_as_float(r.w & 0xffff0000u);
+                for (int i = 0; i < 8; i++) {
+                    v[i] = (v[i] * rs[mi]) * g[i];
+                    if constexpr (sizeof(AT) == 2) v[i] = bf2f(f2bf(v[i]));
                 }
             }
             float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
@@ -210,9 +263,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const 
 
 // Takes the shapes the kernel is built for (reports the others through *handled = false).
 hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
-                                   int64_t ldo, hipStream_t s, bool* handled) {
+                                   int64_t ldo, hipStream_t s, bool* handled, const float* gamma, float eps) {
     *handled = false;
     if (kernel_disabled("q4_0_stream") || m > 4 || k < 8) return hipSuccess;
+    if (gamma && ((uintptr_t)gamma & 15)) return hipSuccess;  // (the kernel reads gamma in 16-byte pieces)
     const int nblk = (int)(k / 32);
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const int bpl = nblk <= 128 ? 2 : nblk <= 256 ? 4 : 0;
@@ -226,26 +280,28 @@ hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w,
     }
     const int L = (72 * bpl + 1 + 63) / 64;
     const int ring = bpl == 2 ? 4 : 3;  // LDS: 8 wavefronts x ring x L KB
-    const size_t lds = (size_t)kWaves * ring * L * 1024 + (size_t)kWaves * kMaxRows * mt * 4 + (size_t)mt * nblk * 40;
+    const size_t lds = (size_t)kWaves * ring * L * 1024 + (size_t)kWaves * kMaxRows * mt * 4 + (size_t)mt * nblk * 40 + 128;  // (the last 128 bytes: the row norms' partial sums)
     int64_t wgs = cus;  // one workgroup of 8 wavefronts per compute unit
     if (wgs * kWaves > n) wgs = (n + kWaves - 1) / kWaves;
     const int64_t min_wgs = (n + (int64_t)kWaves * kMaxRows - 1) / ((int64_t)kWaves * kMaxRows);
     if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots
     dim3 grid((unsigned)wgs), block(64 * kWaves);
-#define QMM_GO(MT_, BPL_, RING_)                                                                                      \
+#define QMM_GO2(MT_, BPL_, RING_, AT_, NORM_)                                                                         \
     do {                                                                                                              \
-        hipError_t e_;                                                                                                \
-        if (a_dtype == QMM_F32) {                                                                                     \
-            e_ = allow_full_lds<gemv_q4_0_stream_kernel<MT_, BPL_, RING_, float>>();                                  \
-            if (e_ != hipSuccess) return e_;                                                                          \
-            gemv_q4_0_stream_kernel<MT_, BPL_, RING_, float><<<grid, block, lds, s>>>(w, (const float*)a, out, m, (int)n, \
-                                                                                     (int)k, ldo);                   \
-        } else {                                                                                                      \
-            e_ = allow_full_lds<gemv_q4_0_stream_kernel<MT_, BPL_, RING_, uint16_t>>();                               \
-            if (e_ != hipSuccess) return e_;                                                                          \
-            gemv_q4_0_stream_kernel<MT_, BPL_, RING_, uint16_t><<<grid, block, lds, s>>>(w, (const uint16_t*)a, out, m, \
-                                                                                        (int)n, (int)k, ldo);        \
-        }                                                                                                             \
+        hipError_t e_ = allow_full_lds<gemv_q4_0_stream_kernel<MT_, BPL_, RING_, AT_, NORM_>>();                      \
+        if (e_ != hipSuccess) return e_;                                                                              \
+        gemv_q4_0_stream_kernel<MT_, BPL_, RING_, AT_, NORM_><<<grid, block, lds, s>>>(w, (const AT_*)a, out, m, (int)n,  \
+                                                                                      (int)k, ldo, gamma, eps);      \
+    } while (0)
+#define QMM_GO(MT_, BPL_, RING_)                                          \
+    do {                                                                  \
+        if (a_dtype == QMM_F32) {                                         \
+            if (gamma) QMM_GO2(MT_, BPL_, RING_, float, true);            \
+            else QMM_GO2(MT_, BPL_, RING_, float, false);                 \
+        } else {                                                          \
+            if (gamma) QMM_GO2(MT_, BPL_, RING_, uint16_t, true);         \
+            else QMM_GO2(MT_, BPL_, RING_, uint16_t, false);              \
+        }                                                                 \
     } while (0)
     if (bpl == 2) {
         if (mt == 1) QMM_GO(1, 2, 4);
@@ -256,6 +312,7 @@ hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w,
         else QMM_GO(2, 4, 3);
     }
 #undef QMM_GO
+#undef QMM_GO2
     *handled = true;
     return hipGetLastError();
 }

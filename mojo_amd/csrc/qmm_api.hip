@@ -447,6 +447,40 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     return QMM_OK;
 }
 
+int64_t qmm_matmul_rmsnorm_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags) {
+    if (m <= 0 || k <= 0) return 0;
+    return up256(m * k * (lhs_dtype == QMM_F32 ? 4 : 2)) + qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags);
+}
+
+int qmm_matmul_rmsnorm(int encoding, const qmm_gptq_config* cfg, const void* x, int x_dtype, const float* gamma, float eps, int64_t m,
+                       int64_t k, const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
+                       int flags, void* stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (!x || !gamma || !rhs || !out) return fail(QMM_ERR_INVALID, "qmm_matmul_rmsnorm: null pointer");
+    if (m <= 0 || n <= 0 || k <= 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX)
+        return fail(QMM_ERR_INVALID, "qmm_matmul_rmsnorm: M=%lld N=%lld K=%lld out of range", (long long)m, (long long)n, (long long)k);
+    if (x_dtype != QMM_F32 && x_dtype != QMM_BF16) return fail(QMM_ERR_INVALID, "qmm_matmul_rmsnorm: x dtype must be f32 or bf16");
+    if (!aligned(x, 16) || !aligned(gamma, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_rmsnorm: x must be 16-byte aligned, gamma 4-byte aligned");
+    if (!(eps >= 0.0f)) return fail(QMM_ERR_INVALID, "qmm_matmul_rmsnorm: eps must be non-negative");
+    // One launch: the Q4_0 decode kernel normalises the rows it quantises anyway.
+    if (encoding == QMM_Q4_0 && m <= 4 && flags == 0 && n_rhs == 1 && rhs[0] && k % 32 == 0 && aligned(rhs[0], 2)) {
+        bool handled = false;
+        hipError_t e = qmm::launch_gemv_q4_0_stream(x, x_dtype, (const uint8_t*)rhs[0], (int)m, n, k, out, n, s, &handled, gamma, eps);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul_rmsnorm(Q4_0 decode)");
+        if (handled) return QMM_OK;
+    }
+    // Otherwise: normalised rows into the workspace, then the matmul on them.
+    const int64_t ybytes = up256(m * k * (x_dtype == QMM_F32 ? 4 : 2));
+    const int64_t need = ybytes + qmm_matmul_workspace_bytes_flags(encoding, x_dtype, m, n, k, flags);
+    if (!workspace || workspace_bytes < need)
+        return fail(QMM_ERR_WORKSPACE, "qmm_matmul_rmsnorm: workspace of %lld bytes required (qmm_matmul_rmsnorm_workspace_bytes), %lld given",
+                    (long long)need, (long long)workspace_bytes);
+    if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_rmsnorm: workspace must be 256-byte aligned");
+    hipError_t e = qmm::launch_rmsnorm(x, x_dtype, gamma, eps, m, k, workspace, s);
+    if (e != hipSuccess) return hip_status(e, "qmm_matmul_rmsnorm(normalise)");
+    return qmm_matmul(encoding, cfg, workspace, x_dtype, m, k, rhs, n_rhs, n, out, (char*)workspace + ybytes, workspace_bytes - ybytes, flags, stream);
+}
+
 int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                       const void* const* rhs, int n_rhs, int64_t n, float* out, int flags, void* stream) {
     const int64_t need = qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags);

@@ -29,8 +29,11 @@ hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group,
                                 void* scales, void* qzeros, void* g_idx, hipStream_t s);
 
 // Decode-shape kernels (m <= 16 rows of lhs per launch).
+// gamma != nullptr: the lhs rows are RMS-normalised in the kernel before they are quantised (y = x * rsqrt(mean(x^2) + eps) * gamma)
 hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
-                                   int64_t ldo, hipStream_t s, bool* handled);
+                                   int64_t ldo, hipStream_t s, bool* handled, const float* gamma = nullptr, float eps = 0.0f);
+// y[rows, k] = x * rsqrt(mean(x^2) + eps) * gamma, computed in fp32; y has the dtype of x (bf16: rounded to nearest even)
+hipError_t launch_rmsnorm(const void* x, int x_dtype, const float* gamma, float eps, int64_t rows, int64_t k, void* y, hipStream_t s);
 hipError_t launch_gemv_q4_0(const int8_t* a_codes, const float* a_scale, const int32_t* a_sum,
                             const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
                             hipStream_t s);

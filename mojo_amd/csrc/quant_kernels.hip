@@ -151,6 +151,36 @@ hipError_t launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count, hipS
     return hipGetLastError();
 }
 
+// RMS normalisation of one row per workgroup: y = (x * rsqrt(mean(x^2) + eps)) * gamma in fp32, stored in the dtype of x.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, const float* __restrict__ gamma, float eps, int64_t k,
+                                                      T* __restrict__ y) {
+    __shared__ float red[4];
+    const T* xr = x + (int64_t)blockIdx.x * k;
+    T* yr = y + (int64_t)blockIdx.x * k;
+    const int tid = threadIdx.x;
+    float ss = 0.0f;
+    for (int64_t i = tid; i < k; i += 256) {
+        const float v = load_f32(xr, i);
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum_dpp(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    const float rs = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)k + eps);
+    for (int64_t i = tid; i < k; i += 256) {
+        const float v = (load_f32(xr, i) * rs) * gamma[i];
+        if constexpr (sizeof(T) == 4) yr[i] = v;
+        else yr[i] = f2bf(v);
+    }
+}
+
+hipError_t launch_rmsnorm(const void* x, int x_dtype, const float* gamma, float eps, int64_t rows, int64_t k, void* y, hipStream_t s) {
+    if (x_dtype == QMM_F32) rmsnorm_kernel<float><<<dim3((unsigned)rows), dim3(256), 0, s>>>((const float*)x, gamma, eps, k, (float*)y);
+    else rmsnorm_kernel<uint16_t><<<dim3((unsigned)rows), dim3(256), 0, s>>>((const uint16_t*)x, gamma, eps, k, (uint16_t*)y);
+    return hipGetLastError();
+}
+
 static int grid_for(int64_t total, int threads) {
     int64_t g = (total + threads - 1) / threads;
     const int64_t cap = 256 * 64;

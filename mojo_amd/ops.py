@@ -41,42 +41,8 @@ def _gptq_cfg(config: Optional[QuantizationConfig]) -> _lib.GptqConfig:
     return _lib.GptqConfig(int(config.bits), int(config.group_size), int(bool(config.desc_act)), int(bool(config.sym)))
 
 
-def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], lhs: torch.Tensor,
-            *rhs: torch.Tensor, w_bf16: bool = False, act_q8k: bool = False, out: Optional[torch.Tensor] = None,
-            static_scratch: bool = False, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """``out[..., N] = lhs[..., K] @ dequantize(rhs)^T`` in fp32.
-
-    ``out_dtype=torch.bfloat16`` returns the fp32 result rounded to bfloat16 (nearest even, canonical NaN:
-    the narrowing rule of stdlib/src/builtin/simd.mojo:3279-3300) for a consumer that takes bf16 activations; the
-    Q4_K decode kernel stores it directly, other shapes narrow an fp32 result held in the workspace.
-
-    GGUF encodings take one ``uint8[N, K/epb*bpb]`` tensor of packed blocks (the
-    transposed, quantised weight).  GPTQ takes the AutoGPTQ tensors
-    ``(qweight int32[K/8, N], scales float16[K/g, N], qzeros int32[K/g, N/8][, g_idx int32[K]])``.
-    ``lhs`` is float32 or bfloat16.  Q4_0 quantises ``lhs`` to Q8_0 blocks and
-    takes integer block dots; the other encodings use ``lhs`` as given.  ``act_q8k=True`` (Q4_K only)
-    quantises ``lhs`` to Q8_K blocks and takes the integer sub-block dots of the ggml-lineage CPU kernels instead.
-    ``w_bf16=True`` asks for the reserved mode that rounds the dequantised weights to bfloat16 first; the library
-    has no kernel for it and raises ``NotImplementedError``.
-
-    ``out`` (contiguous float32 ``[M, N]`` on the device of ``lhs``) receives the result instead of a new tensor.
-    ``static_scratch=True`` goes through ``qmm_matmul_static``: the kernels' scratch is the buffer that is part of
-    the library (64 MiB per GPU) instead of a tensor allocated here, so with ``out`` given the call allocates no
-    device memory; calls that may overlap on one GPU must then be ordered by the caller.
-    """
-    if not isinstance(encoding, QuantizationEncoding):
-        raise TypeError("encoding must be a QuantizationEncoding")
-    _require_gpu(lhs, "lhs")
-    if lhs.dtype not in _DTYPES:
-        raise TypeError(f"lhs must be float32 or bfloat16, got {lhs.dtype}")
-    if lhs.dim() < 1:
-        raise ValueError("lhs must have at least one dimension")
-    k = lhs.shape[-1]
-    lead = lhs.shape[:-1]
-    m = 1
-    for d in lead:
-        m *= d
-    lib = _lib.load()
+def _check_rhs(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], k: int, rhs):
+    """Validates the weight tensors of a qmatmul against the encoding and K; returns (N, pointer to the GPTQ config or None)."""
     if encoding == QuantizationEncoding.GPTQ:
         if len(rhs) not in (3, 4):
             raise TypeError(f"GPTQ qmatmul takes (qweight, scales, qzeros[, g_idx]); got {len(rhs)} rhs tensors")
@@ -114,6 +80,46 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
         cfg_p = None
     else:
         raise ValueError(f"{encoding.name} is not a weight encoding of qmatmul")
+    return n, cfg_p
+
+
+def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], lhs: torch.Tensor,
+            *rhs: torch.Tensor, w_bf16: bool = False, act_q8k: bool = False, out: Optional[torch.Tensor] = None,
+            static_scratch: bool = False, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``out[..., N] = lhs[..., K] @ dequantize(rhs)^T`` in fp32.
+
+    ``out_dtype=torch.bfloat16`` returns the fp32 result rounded to bfloat16 (nearest even, canonical NaN:
+    the narrowing rule of stdlib/src/builtin/simd.mojo:3279-3300) for a consumer that takes bf16 activations; the
+    Q4_K decode kernel stores it directly, other shapes narrow an fp32 result held in the workspace.
+
+    GGUF encodings take one ``uint8[N, K/epb*bpb]`` tensor of packed blocks (the
+    transposed, quantised weight).  GPTQ takes the AutoGPTQ tensors
+    ``(qweight int32[K/8, N], scales float16[K/g, N], qzeros int32[K/g, N/8][, g_idx int32[K]])``.
+    ``lhs`` is float32 or bfloat16.  Q4_0 quantises ``lhs`` to Q8_0 blocks and
+    takes integer block dots; the other encodings use ``lhs`` as given.  ``act_q8k=True`` (Q4_K only)
+    quantises ``lhs`` to Q8_K blocks and takes the integer sub-block dots of the ggml-lineage CPU kernels instead.
+    ``w_bf16=True`` asks for the reserved mode that rounds the dequantised weights to bfloat16 first; the library
+    has no kernel for it and raises ``NotImplementedError``.
+
+    ``out`` (contiguous float32 ``[M, N]`` on the device of ``lhs``) receives the result instead of a new tensor.
+    ``static_scratch=True`` goes through ``qmm_matmul_static``: the kernels' scratch is the buffer that is part of
+    the library (64 MiB per GPU) instead of a tensor allocated here, so with ``out`` given the call allocates no
+    device memory; calls that may overlap on one GPU must then be ordered by the caller.
+    """
+    if not isinstance(encoding, QuantizationEncoding):
+        raise TypeError("encoding must be a QuantizationEncoding")
+    _require_gpu(lhs, "lhs")
+    if lhs.dtype not in _DTYPES:
+        raise TypeError(f"lhs must be float32 or bfloat16, got {lhs.dtype}")
+    if lhs.dim() < 1:
+        raise ValueError("lhs must have at least one dimension")
+    k = lhs.shape[-1]
+    lead = lhs.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    lib = _lib.load()
+    n, cfg_p = _check_rhs(encoding, config, k, rhs)
     if m == 0 or n == 0:
         raise ValueError("qmatmul of an empty tensor")
     if out_dtype not in (torch.float32, torch.bfloat16):
@@ -139,6 +145,47 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
     if rc == -4:
         raise ValueError("qmatmul: " + lib.qmm_last_error().decode("utf-8", "replace"))
     _lib.check(rc, "qmatmul")
+    return out.reshape(*lead, n)
+
+
+def qmatmul_rmsnorm(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], x: torch.Tensor,
+                    gamma: torch.Tensor, eps: float, *rhs: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``qmatmul(encoding, config, rms_norm(x, gamma, eps), *rhs)`` as one call: the normalisation in front of the
+    projections of a Llama block, ``y = x * rsqrt(mean(x^2) + eps) * gamma`` in fp32 (rounded to bfloat16 when ``x`` is
+    bfloat16).  Q4_0 with up to four rows (K <= 8192) is one launch: the decode kernel normalises the rows it quantises
+    to Q8_0 anyway; other problems run a normalisation launch and the matmul inside the library."""
+    if not isinstance(encoding, QuantizationEncoding):
+        raise TypeError("encoding must be a QuantizationEncoding")
+    _require_gpu(x, "x")
+    _require_gpu(gamma, "gamma")
+    if x.dtype not in _DTYPES:
+        raise TypeError(f"x must be float32 or bfloat16, got {x.dtype}")
+    if x.dim() < 1:
+        raise ValueError("x must have at least one dimension")
+    k = x.shape[-1]
+    if gamma.dtype != torch.float32 or tuple(gamma.shape) != (k,):
+        raise TypeError(f"gamma must be float32[{k}]")
+    if not eps >= 0.0:
+        raise ValueError("eps must be non-negative")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError("out_dtype must be float32 or bfloat16")
+    lead = x.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    n, cfg_p = _check_rhs(encoding, config, k, rhs)
+    if m == 0 or n == 0:
+        raise ValueError("qmatmul of an empty tensor")
+    lib = _lib.load()
+    x_dt = _DTYPES[x.dtype]
+    flags = _lib.QMM_FLAG_OUT_BF16 if out_dtype == torch.bfloat16 else 0
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    need = lib.qmm_matmul_rmsnorm_workspace_bytes(encoding.code, x_dt, m, n, k, flags)
+    ws = torch.empty((need,), dtype=torch.uint8, device=x.device) if need > 0 else None
+    ptrs = (C.c_void_p * len(rhs))(*[t.data_ptr() for t in rhs])
+    rc = lib.qmm_matmul_rmsnorm(encoding.code, cfg_p, _ptr(x), x_dt, _ptr(gamma), C.c_float(eps), m, k, ptrs, len(rhs), n,
+                                _ptr(out), _ptr(ws), need, flags, _stream(x))
+    _lib.check(rc, "qmatmul_rmsnorm")
     return out.reshape(*lead, n)
 
 

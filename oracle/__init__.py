@@ -266,6 +266,17 @@ def swiglu(gate, up) -> np.ndarray:
         return g / (1.0 + np.exp(-g)) * np.asarray(up, np.float64)
 
 
+def rmsnorm(x, gamma, eps: float, to_bf16: bool = False) -> np.ndarray:
+    """y = x * rsqrt(mean(x^2) + eps) * gamma per row, fp32 (rounded to bf16 and widened again with to_bf16)."""
+    x = _c(x, np.float32)
+    rows, k = (1, x.shape[0]) if x.ndim == 1 else x.shape
+    gamma = _c(gamma, np.float32)
+    assert gamma.shape == (k,)
+    y = np.empty(x.shape, np.float32)
+    lib().qo_rmsnorm(_p(x), _p(gamma), C.c_float(eps), _i64(rows), _i64(k), C.c_int(int(to_bf16)), _p(y))
+    return y
+
+
 class _Native:
     """The same source built with -march=native (``make -C oracle native``): only the timed CPU baseline of
     ``bench.py`` uses it, never a test."""

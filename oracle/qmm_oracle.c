@@ -62,6 +62,12 @@
  *                                     -127, round-half-even, bsums).  Which of
  *                                     the two treatments the reference uses is
  *                                     PARITY UNPINNED (see the line above).
+ *   qo_rmsnorm                        the normalisation in front of the op in a
+ *                                     Llama block, y = x * rsqrt(mean(x^2) + eps)
+ *                                     * gamma: pinned by closed forms (constant
+ *                                     rows, sum of squares of y / gamma = K at
+ *                                     eps = 0, invariance under scaling of x)
+ *                                     and an independent fp64 restatement.
  */
 #include <math.h>
 #include <stdint.h>
@@ -162,6 +168,27 @@ void qo_f32_to_f16_n(const float* f, int64_t n, uint16_t* out) {
 }
 void qo_f32_to_bf16_n(const float* f, int64_t n, uint16_t* out) {
     for (int64_t i = 0; i < n; i++) out[i] = qo_f32_to_bf16(f[i]);
+}
+
+/*
+ * RMS normalisation of each row: y = (x * rs) * gamma with rs = 1 / sqrt(mean(x^2) + eps) as a float, the mean summed in
+ * double; to_bf16 != 0 rounds y to bf16 (the value a bf16 normalisation node hands on) and returns it widened again.
+ */
+void qo_rmsnorm(const float* x, const float* gamma, float eps, int64_t rows, int64_t k, int to_bf16, float* y) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float* xr = x + r * k;
+        double ss = 0.0;
+        for (int64_t i = 0; i < k; i++) ss += (double)xr[i] * (double)xr[i];
+        const float rs = (float)(1.0 / sqrt(ss / (double)k + (double)eps));
+        for (int64_t i = 0; i < k; i++) {
+            float v = (xr[i] * rs) * gamma[i];
+            if (to_bf16) {
+                uint32_t u = (uint32_t)qo_f32_to_bf16(v) << 16;
+                memcpy(&v, &u, 4);
+            }
+            y[r * k + i] = v;
+        }
+    }
 }
 
 static inline float rd_f16(const uint8_t* p) {

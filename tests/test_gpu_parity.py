@@ -11,7 +11,7 @@ import torch
 import oracle as O
 from conftest import synth
 from mojo_amd import QuantizationConfig, QuantizationEncoding as QE
-from mojo_amd import block_dots_q4_0, dequantize, qmatmul, qmatmul_grouped, qmatmul_swiglu, quantize, quantize_gptq
+from mojo_amd import block_dots_q4_0, dequantize, qmatmul, qmatmul_grouped, qmatmul_rmsnorm, qmatmul_swiglu, quantize, quantize_gptq
 
 pytestmark = pytest.mark.gpu
 
@@ -715,6 +715,33 @@ def test_bf16_output_is_the_fp32_result_narrowed(enc, m, n, k, lhs_bf16):
     into = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
     qmatmul(enc, *args, out=into, out_dtype=torch.bfloat16)
     assert torch.equal(into.view(torch.int16), b16.view(torch.int16))
+
+
+@pytest.mark.parametrize("enc,m,n,k,bf16", [
+    (QE.Q4_0, 1, 1030, 4096, False), (QE.Q4_0, 1, 515, 4096, True), (QE.Q4_0, 4, 300, 2048, False), (QE.Q4_0, 2, 66, 8192, True),
+    (QE.Q4_0, 3, 130, 1056, False), (QE.Q4_0, 9, 64, 1024, False), (QE.Q4_K, 1, 512, 4096, False), (QE.Q4_K, 40, 96, 1024, True),
+    (QE.Q6_K, 2, 130, 2048, False)])
+def test_rmsnorm_prologue(enc, m, n, k, bf16):
+    """qmatmul_rmsnorm against the oracle: rmsnorm (fp32; bf16 x: rounded to bf16) then the encoding's matmul.  Q4_0 up
+    to four rows is the decode kernel's own prologue (fused), the other cases a normalisation launch and the matmul; a
+    fused result also has to agree with the two-step route through qmatmul on the normalised rows."""
+    w, x = synth(81, n, k, m)
+    x *= np.logspace(-2, 2, m, dtype=np.float32)[:, None]
+    if bf16:
+        x = O.bf16_to_f32(O.f32_to_bf16(x))
+    gamma = np.random.default_rng(82).uniform(0.25, 2.0, k).astype(np.float32)
+    eps = 1e-5
+    wq = O.quantize(ENC[enc], w)
+    y = O.rmsnorm(x, gamma, eps, to_bf16=bf16)
+    want = O.matmul_q4_0(y, wq) if enc == QE.Q4_0 else O.matmul_f32(ENC[enc], y, wq)
+    xd = gpu(x).to(torch.bfloat16) if bf16 else gpu(x)
+    got = qmatmul_rmsnorm(enc, None, xd, gpu(gamma), eps, gpu(wq))
+    assert_close(got, want, f"{enc.name} rmsnorm prologue {m}x{n}x{k} bf16={bf16}")
+    yd = gpu(y).to(torch.bfloat16) if bf16 else gpu(y)
+    assert_close(got, qmatmul(enc, None, yd, gpu(wq)).cpu().numpy(), "against qmatmul on the oracle's normalised rows")
+    b16 = qmatmul_rmsnorm(enc, None, xd, gpu(gamma), eps, gpu(wq), out_dtype=torch.bfloat16)
+    if not (enc == QE.Q4_0 and m <= 4):
+        assert np.array_equal(b16.cpu().view(torch.int16).numpy().view(np.uint16), O.f32_to_bf16(got.cpu().numpy()))
 
 
 def test_q4_k_gemm_wide_range_lhs():

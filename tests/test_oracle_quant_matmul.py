@@ -185,3 +185,26 @@ def test_swiglu_closed_forms():
     assert abs(O.swiglu(xm, 1.0) + 0.2784645) < 1e-6 and O.swiglu(xm - 0.01, 1.0) > O.swiglu(xm, 1.0) < O.swiglu(xm + 0.01, 1.0)
     assert np.array_equal(O.swiglu(x, 3.0 * one), 3.0 * s)
 
+
+
+def test_rmsnorm_closed_forms_and_restatement():
+    """qo_rmsnorm: a constant row c gives gamma * c / sqrt(c^2 + eps); with eps = 0 the squares of y / gamma sum to K and
+    scaling x changes nothing; an independent fp64 restatement agrees to fp32 rounding; to_bf16 is the bf16 narrowing of
+    the fp32 result."""
+    rng = np.random.default_rng(91)
+    k = 768
+    gamma = rng.uniform(0.5, 1.5, k).astype(np.float32)
+    c = np.float32(-3.25)
+    y = O.rmsnorm(np.full((2, k), c, np.float32), gamma, 1e-5)
+    assert np.allclose(y, gamma.astype(np.float64) * c / np.sqrt(float(c) ** 2 + 1e-5), rtol=3e-7)
+    x = (rng.standard_normal((5, k)) * np.logspace(-3, 3, 5)[:, None]).astype(np.float32)
+    y0 = O.rmsnorm(x, gamma, 0.0)
+    assert np.allclose(((y0.astype(np.float64) / gamma) ** 2).sum(axis=1), k, rtol=1e-6)
+    assert np.allclose(O.rmsnorm(4.0 * x, gamma, 0.0), y0, rtol=3e-7)  # (a power of two: exact up to the one rounding of rs)
+    eps = 1e-3
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + eps) * gamma
+    assert np.allclose(O.rmsnorm(x, gamma, eps), want, rtol=4e-7, atol=0)
+    assert np.array_equal(O.rmsnorm(x, gamma, eps, to_bf16=True), O.bf16_to_f32(O.f32_to_bf16(O.rmsnorm(x, gamma, eps))))
+    # a larger eps can only shrink the result
+    assert np.all(np.abs(O.rmsnorm(x, gamma, 1.0)) <= np.abs(y0))
