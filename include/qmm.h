@@ -123,10 +123,13 @@ int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m,
  *   integer block dots (the reference CPU path); the others keep lhs as given.
  *   flags: bit 0 (QMM_FLAG_W_BF16) is reserved for a mode that rounds the dequantised
  *   weights to bf16 before the product; no kernel implements it and a call that sets
- *   it returns QMM_ERR_UNSUPPORTED.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K only: the
- *   lhs is quantised to Q8_K blocks (256 wide, fp32 scale) and the product is the
- *   integer sub-block dot of the ggml-lineage CPU kernels instead of the default
- *   floating-point one; K <= 16384, any m (passes of four rows).  Bit 2 (QMM_FLAG_OUT_BF16): `out`
+ *   it returns QMM_ERR_UNSUPPORTED.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K / Q5_K / Q6_K: the
+ *   lhs is quantised to Q8_K blocks (256 wide, fp32 scale) and the products are those of the
+ *   integer sub-block dots of the ggml-lineage CPU kernels instead of the default
+ *   floating-point ones.  Q4_K with m <= 4 and K <= 16384 takes the integer dots in the kernel;
+ *   every other problem writes d8 * code as fp32 rows into the workspace and runs the
+ *   floating-point kernels on them (same products, fp32 sums; workspace from
+ *   qmm_matmul_workspace_bytes_flags).  Bit 2 (QMM_FLAG_OUT_BF16): `out`
  *   points to bf16[m, n] instead of fp32 (the caller's next op takes bf16 activations): the fp32 result is
  *   rounded to nearest even with NaN mapped to the canonical quiet NaN, the reference's narrowing rule
  *   (stdlib/src/builtin/simd.mojo:3279-3300).  The Q4_K decode kernel (m = 1, K <= 16384) stores bf16 itself;

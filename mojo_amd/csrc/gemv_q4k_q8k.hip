@@ -106,6 +106,37 @@ __global__ __launch_bounds__(256) void quantize_q8_k_kernel(const AT* __restrict
     if ((l & 1) == 0) *(int16_t*)(ob + 260 + 2 * (l >> 1)) = (int16_t)s16;
 }
 
+// x [rows, k] -> d8 * code of its Q8_K quantisation as fp32 [rows, k]: the activations that the integer treatment multiplies,
+// for the kernels that take a floating-point lhs.  Same quantiser, same 32 threads per block.
+template <typename AT>
+__global__ __launch_bounds__(256) void q8k_round_trip_kernel(const AT* __restrict__ x, int64_t nblocks, float* __restrict__ y) {
+    const int64_t blk = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    const int l = threadIdx.x & 31;
+    const int64_t bc = min(blk, nblocks - 1);
+    uint32_t c0, c1;
+    float d8;
+    int s8;
+    q8k_quantise8(x + bc * 256 + 8 * l, 8 * l, c0, c1, d8, s8);
+    if (blk >= nblocks) return;
+    float* yo = y + blk * 256 + 8 * l;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        v[i] = d8 * (float)(int)(int8_t)((c0 >> (8 * i)) & 0xffu);
+        v[4 + i] = d8 * (float)(int)(int8_t)((c1 >> (8 * i)) & 0xffu);
+    }
+    *(float4*)yo = make_float4(v[0], v[1], v[2], v[3]);
+    *(float4*)(yo + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+hipError_t launch_q8k_round_trip(const void* x, int x_dtype, int64_t rows, int64_t k, float* y, hipStream_t s) {
+    const int64_t nblocks = rows * (k / 256), threads = nblocks * 32;
+    const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+    if (x_dtype == QMM_F32) q8k_round_trip_kernel<float><<<grid, block, 0, s>>>((const float*)x, nblocks, y);
+    else q8k_round_trip_kernel<uint16_t><<<grid, block, 0, s>>>((const uint16_t*)x, nblocks, y);
+    return hipGetLastError();
+}
+
 template <int MT, int WPR, int L, typename AT>
 __global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_k_q8k_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
                                                                       float* __restrict__ out, int m, int n, int k, int64_t ldo,

@@ -255,8 +255,14 @@ static bool stores_bf16_itself(int encoding, int64_t m, int64_t k, int flags) {
     return encoding == QMM_Q4_K && m == 1 && k % 256 == 0 && k <= 16384 && !(flags & QMM_FLAG_ACT_Q8K) && !qmm::kernel_disabled("q4k_lanes");
 }
 
+// Q8_K activations: Q4_K with up to four lhs rows has a kernel that takes the integer sub-block dots itself; every other
+// problem quantises the lhs, writes d8 * code as fp32 rows into the workspace and runs the floating-point path on those.
+static bool q8k_integer_kernel(int encoding, int64_t m, int64_t k) { return encoding == QMM_Q4_K && m <= 4 && k <= 16384; }
+
 int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags) {
-    const int64_t base = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    int64_t base = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    if ((flags & QMM_FLAG_ACT_Q8K) && m > 0 && k > 0 && !q8k_integer_kernel(encoding, m, k))
+        base = up256(m * k * 4) + qmm_matmul_workspace_bytes(encoding, QMM_F32, m, n, k);
     if (!(flags & QMM_FLAG_OUT_BF16) || m <= 0 || n <= 0 || stores_bf16_itself(encoding, m, k, flags)) return base;
     return up256(base) + up256(m * n * 4);
 }
@@ -309,7 +315,7 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         return fail(QMM_ERR_INVALID, "qmm_matmul: lhs dtype must be f32 or bf16");
     if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul: lhs must be 16-byte aligned");
     int64_t esz = lhs_dtype == QMM_F32 ? 4 : 2;
-    int64_t need = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    int64_t need = qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags & QMM_FLAG_ACT_Q8K);
     if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(QMM_ERR_WORKSPACE, "qmm_matmul: workspace of %lld bytes required, %lld given", (long long)need,
                     (long long)workspace_bytes);
@@ -375,15 +381,22 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     if (!aligned(w, 2)) return fail(QMM_ERR_INVALID, "qmm_matmul: rhs must be 2-byte aligned");
 
     if (flags & QMM_FLAG_ACT_Q8K) {
-        if (encoding != QMM_Q4_K) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations are implemented for Q4_K weights only");
-        for (int64_t m0 = 0; m0 < m; m0 += 4) {
+        if (encoding != QMM_Q4_K && encoding != QMM_Q5_K && encoding != QMM_Q6_K)
+            return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations go with Q4_K, Q5_K and Q6_K weights");
+        if (q8k_integer_kernel(encoding, m, k)) {
             bool handled = false;
-            hipError_t e = qmm::launch_gemv_q4_k_q8k((const char*)lhs + m0 * k * esz, lhs_dtype, w, (int)std::min<int64_t>(4, m - m0), n, k,
-                                                     out + m0 * n, n, s, &handled);
+            hipError_t e = qmm::launch_gemv_q4_k_q8k(lhs, lhs_dtype, w, (int)m, n, k, out, n, s, &handled);
             if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K x Q8_K)");
-            if (!handled) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations need K <= 16384 (K = %lld)", (long long)k);
+            if (handled) return QMM_OK;
+            return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q4_K x Q8_K shape not taken (M=%lld K=%lld)", (long long)m, (long long)k);
         }
-        return QMM_OK;
+        // the quantised activations as fp32 rows (d8 * code), then the floating-point path on them: the products are those of
+        // the integer treatment, summed in fp32
+        const int64_t ybytes = up256(m * k * 4);
+        float* y = (float*)workspace;
+        hipError_t e = qmm::launch_q8k_round_trip(lhs, lhs_dtype, m, k, y, s);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q8_K round trip)");
+        return matmul_f32(encoding, cfg, y, QMM_F32, m, k, rhs, n_rhs, n, out, (char*)workspace + ybytes, workspace_bytes - ybytes, 0, stream);
     }
     // Q5_K and Q6_K with many lhs rows: weights to fp16 integer planes in the workspace, then the matrix cores
     if (qmm::gemm_planes_wanted(encoding, m, n, k))

@@ -25,6 +25,8 @@ hipError_t launch_quantize(int enc, const float* x, int64_t rows, int64_t k, voi
 hipError_t launch_quantize_q8_0(const void* x, int x_dtype, int64_t rows, int64_t k, void* blocks,
                                 void* codes, void* dscale, void* csum, hipStream_t s);
 hipError_t launch_quantize_q8_k(const void* x, int x_dtype, int64_t rows, int64_t k, void* out, hipStream_t s);
+// y fp32[rows, k] = d8 * code of the Q8_K quantisation of x (k a multiple of 256)
+hipError_t launch_q8k_round_trip(const void* x, int x_dtype, int64_t rows, int64_t k, float* y, hipStream_t s);
 hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group, void* qweight,
                                 void* scales, void* qzeros, void* g_idx, hipStream_t s);
 

@@ -215,6 +215,27 @@ def matmul_q4_k_q8_k(a_q8k, w, k: int) -> np.ndarray:
     return out
 
 
+def block_sums_kquant_q8_k(enc: int, a_q8k, w, k: int):
+    """(isum, msum) int32 [M, N, K/256] of Q4_K / Q5_K / Q6_K blocks against Q8_K blocks (msum = 0 for Q6_K)."""
+    a_q8k, w = _c(a_q8k, np.uint8), _c(w, np.uint8)
+    m, n = a_q8k.shape[0], w.shape[0]
+    isum, msum = np.empty((m, n, k // 256), np.int32), np.empty((m, n, k // 256), np.int32)
+    rc = lib().qo_block_sums_kquant_q8_k(C.c_int(enc), _p(a_q8k), _p(w), _i64(m), _i64(n), _i64(k), _p(isum), _p(msum))
+    assert rc == 0
+    return isum, msum
+
+
+def matmul_kquant_act_q8_k(enc: int, a, w) -> np.ndarray:
+    """The integer-activation path for Q4_K / Q5_K / Q6_K weights: fp32 activations -> Q8_K, integer sub-block dots."""
+    a, m, k = _rows_k(a)
+    w = _c(w, np.uint8)
+    n = w.shape[0]
+    out = np.empty((m, n), np.float32)
+    rc = lib().qo_matmul_kquant_act_q8_k(C.c_int(enc), _p(a), _p(w), _i64(m), _i64(n), _i64(k), _p(out))
+    assert rc == 0
+    return out
+
+
 def matmul_q4_k_act_q8_k(a, w) -> np.ndarray:
     """The integer-activation Q4_K path: fp32 activations -> Q8_K, integer sub-block dots."""
     a, m, k = _rows_k(a)

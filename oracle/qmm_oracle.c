@@ -62,6 +62,15 @@
  *                                     -127, round-half-even, bsums).  Which of
  *                                     the two treatments the reference uses is
  *                                     PARITY UNPINNED (see the line above).
+ *   qo_block_sums_kquant_q8_k, qo_matmul_kquant_act_q8_k
+ *                                     the same treatment for Q5_K and Q6_K
+ *                                     weights: integer sums pinned by brute
+ *                                     force vs int64 over an independent
+ *                                     unpack of the blocks, the matmul by the
+ *                                     identity with the fp64 product on
+ *                                     activations that Q8_K represents exactly,
+ *                                     and by equality with the Q4_K functions
+ *                                     above for enc = Q4_K.
  *   qo_rmsnorm                        the normalisation in front of the op in a
  *                                     Llama block, y = x * rsqrt(mean(x^2) + eps)
  *                                     * gamma: pinned by closed forms (constant
@@ -763,6 +772,107 @@ void qo_matmul_q4_k_q8_k(const uint8_t* a_q8k, const uint8_t* w, int64_t m, int6
             out[i * n + j] = acc;
         }
     }
+}
+
+/* The same for Q5_K (codes 0..31 with the fifth bit from qh) and for Q6_K (codes -32..31, an int8 scale per 16 weights, no
+ * min term): integer sums of one weight block against one Q8_K block. */
+static void block_sums_q5_k_q8_k(const uint8_t* wb, const uint8_t* ab, int32_t* isum, int32_t* msum) {
+    uint8_t sc[8], mn[8];
+    qo_unpack_scales_q4_k(wb + 4, sc, mn);
+    const int8_t* q8 = (const int8_t*)(ab + 4);
+    const uint8_t* qh = wb + 16;
+    const uint8_t* qs = wb + 48;
+    int32_t is = 0, ms = 0;
+    for (int c = 0; c < 4; c++) {
+        int32_t lo = 0, hi = 0;
+        for (int t = 0; t < 32; t++) {
+            lo += (int)((qs[32 * c + t] & 0xF) + (((qh[t] >> (2 * c)) & 1) << 4)) * (int)q8[64 * c + t];
+            hi += (int)((qs[32 * c + t] >> 4) + (((qh[t] >> (2 * c + 1)) & 1) << 4)) * (int)q8[64 * c + 32 + t];
+        }
+        is += (int32_t)sc[2 * c] * lo + (int32_t)sc[2 * c + 1] * hi;
+    }
+    for (int sub = 0; sub < 8; sub++) {
+        int16_t b0, b1;
+        memcpy(&b0, ab + 260 + 4 * sub, 2);
+        memcpy(&b1, ab + 262 + 4 * sub, 2);
+        ms += (int32_t)mn[sub] * ((int32_t)b0 + (int32_t)b1);
+    }
+    *isum = is;
+    *msum = ms;
+}
+static int32_t block_sum_q6_k_q8_k(const uint8_t* wb, const uint8_t* ab) {
+    const int8_t* q8 = (const int8_t*)(ab + 4);
+    int32_t is = 0;
+    for (int h = 0; h < 2; h++) {
+        const uint8_t* ql = wb + 64 * h;
+        const uint8_t* qh = wb + 128 + 32 * h;
+        const int8_t* sc = (const int8_t*)(wb + 192 + 8 * h);
+        const int8_t* a = q8 + 128 * h;
+        int32_t part[8] = {0, 0, 0, 0, 0, 0, 0, 0};  /* the eight 16-weight groups of this half, in scale order */
+        for (int l = 0; l < 32; l++) {
+            int g = l / 16;
+            part[g + 0] += ((int)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32) * (int)a[l];
+            part[g + 2] += ((int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32) * (int)a[l + 32];
+            part[g + 4] += ((int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32) * (int)a[l + 64];
+            part[g + 6] += ((int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32) * (int)a[l + 96];
+        }
+        for (int g = 0; g < 8; g++) is += (int32_t)sc[g] * part[g];
+    }
+    return is;
+}
+
+/* out int32[M, N, K/256]: isum (and msum, zero for Q6_K) of every block pair, enc = Q4_K, Q5_K or Q6_K */
+int qo_block_sums_kquant_q8_k(int enc, const uint8_t* a_q8k, const uint8_t* w, int64_t m, int64_t n, int64_t k, int32_t* isum, int32_t* msum) {
+    int64_t epb, bpb;
+    if ((enc != QO_Q4_K && enc != QO_Q5_K && enc != QO_Q6_K) || qo_block_params(enc, &epb, &bpb) || k % 256) return -1;
+    int64_t nb = k / 256;
+#pragma omp parallel for schedule(static)
+    for (int64_t j = 0; j < n; j++)
+        for (int64_t i = 0; i < m; i++)
+            for (int64_t b = 0; b < nb; b++) {
+                const uint8_t* wb = w + (j * nb + b) * bpb;
+                const uint8_t* ab = a_q8k + (i * nb + b) * 292;
+                int32_t* is = isum + (i * n + j) * nb + b;
+                int32_t* ms = msum + (i * n + j) * nb + b;
+                if (enc == QO_Q4_K) block_sums_q4_k_q8_k(wb, ab, is, ms);
+                else if (enc == QO_Q5_K) block_sums_q5_k_q8_k(wb, ab, is, ms);
+                else { *is = block_sum_q6_k_q8_k(wb, ab); *ms = 0; }
+            }
+    return 0;
+}
+
+/* fp32 activations in, quantised to Q8_K on the way: out[m, n] = sum_b (d8 * f32(d)) * isum - (d8 * f32(dmin)) * msum, blocks
+ * in ascending order (Q6_K: d at byte 208, no min term) */
+int qo_matmul_kquant_act_q8_k(int enc, const float* a, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out) {
+    int64_t epb, bpb;
+    if ((enc != QO_Q4_K && enc != QO_Q5_K && enc != QO_Q6_K) || qo_block_params(enc, &epb, &bpb) || k % 256) return -1;
+    int64_t nb = k / 256;
+    uint8_t* aq = (uint8_t*)malloc((size_t)(m * nb * 292));
+    qo_quantize_q8_k(a, m, k, aq);
+#pragma omp parallel for schedule(static)
+    for (int64_t j = 0; j < n; j++) {
+        for (int64_t i = 0; i < m; i++) {
+            float acc = 0.0f;
+            for (int64_t b = 0; b < nb; b++) {
+                const uint8_t* wb = w + (j * nb + b) * bpb;
+                const uint8_t* ab = aq + (i * nb + b) * 292;
+                float d8;
+                memcpy(&d8, ab, 4);
+                if (enc == QO_Q6_K) {
+                    acc += (d8 * rd_f16(wb + 208)) * (float)block_sum_q6_k_q8_k(wb, ab);
+                } else {
+                    int32_t is, ms;
+                    if (enc == QO_Q4_K) block_sums_q4_k_q8_k(wb, ab, &is, &ms);
+                    else block_sums_q5_k_q8_k(wb, ab, &is, &ms);
+                    acc += (d8 * rd_f16(wb)) * (float)is;
+                    acc -= (d8 * rd_f16(wb + 2)) * (float)ms;
+                }
+            }
+            out[i * n + j] = acc;
+        }
+    }
+    free(aq);
+    return 0;
 }
 
 /* fp32 activations in, quantised to Q8_K on the way */

@@ -538,10 +538,30 @@ def test_q4_k_matmul_with_q8_k_activations(m, n, k, lhs_bf16):
         assert not O.isclose(got, O.matmul_f32(O.Q4_K, a, wq), 1e-4, 1e-5).all()
 
 
-def test_q8_k_activations_only_for_q4_k():
+@pytest.mark.parametrize("enc,m,n,k,lhs_bf16", [
+    (QE.Q6_K, 1, 1000, 4096, False), (QE.Q6_K, 4, 130, 2048, True), (QE.Q6_K, 16, 64, 14336, False), (QE.Q6_K, 100, 257, 1024, False),
+    (QE.Q5_K, 1, 515, 4096, False), (QE.Q5_K, 3, 70, 8192, True), (QE.Q5_K, 48, 130, 768, False),
+    (QE.Q4_K, 5, 300, 4096, False), (QE.Q4_K, 16, 96, 14336, True), (QE.Q4_K, 300, 520, 1024, False), (QE.Q4_K, 2, 40, 20480, False)])
+def test_kquant_matmul_with_q8_k_activations(enc, m, n, k, lhs_bf16):
+    """Q8_K activations for every K-quant and row count: where no kernel takes the integer sub-block dots itself, the
+    quantised activations go through the floating-point kernels as d8 * code, which differs from the integer treatment
+    (the oracle's) only by fp32 summation; and the result is not the unquantised-activation one."""
+    w, a = synth(73, n, k, m)
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(ENC[enc], w)
+    want = O.matmul_kquant_act_q8_k(ENC[enc], a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a)
+    got = qmatmul(enc, None, lhs, gpu(wq), act_q8k=True).cpu().numpy()
+    assert O.isclose(got, want, 1e-4, 1e-5).all(), f"max abs err {np.abs(got - want).max()}"
+    if n * m >= 64 and k >= 1024:
+        assert not O.isclose(got, O.matmul_f32(ENC[enc], a, wq), 1e-4, 1e-5).all()
+
+
+def test_q8_k_activations_only_for_k_quants():
     w, a = synth(72, 8, 256, 1)
     with pytest.raises(NotImplementedError):
-        qmatmul(QE.Q6_K, None, gpu(a), gpu(O.quantize(O.Q6_K, w)), act_q8k=True)
+        qmatmul(QE.Q4_0, None, gpu(a), gpu(O.quantize(O.Q4_0, w)), act_q8k=True)
 
 
 # ------------------------------------------------------------------ matrices that share their lhs

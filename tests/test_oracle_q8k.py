@@ -1,9 +1,10 @@
-"""Pins of the oracle's integer-activation Q4_K path (activations -> Q8_K blocks, integer sub-block dots)."""
+"""Pins of the oracle's integer-activation K-quant paths (activations -> Q8_K blocks, integer sub-block dots)."""
 import numpy as np
+import pytest
 
 import oracle as O
 from conftest import synth
-from np_formats import f16, unpack_scales_q4_k
+from np_formats import dequant_q5_k, dequant_q6_k, f16, unpack_scales_q4_k
 
 
 def _fields(q8k: np.ndarray, k: int):
@@ -99,4 +100,64 @@ def test_integer_path_is_a_quantisation_of_the_fp_path():
     ip, fp = O.matmul_q4_k_act_q8_k(a, wq), O.matmul_f32(O.Q4_K, a, wq)
     rel = np.abs(ip - fp) / np.abs(fp).max()
     assert 1e-4 < rel.max() < 3e-2
+    assert not O.isclose(ip, fp, 1e-3, 1e-4).all()
+
+
+@pytest.mark.parametrize("enc,bpb,d_at,dmin_at", [(O.Q5_K, 176, 0, 2), (O.Q6_K, 210, 208, None)])
+def test_q5_k_q6_k_block_sums_against_int64_brute_force(enc, bpb, d_at, dmin_at):
+    """Blocks of random bytes (every code, fifth-bit / high-bit and scale pattern) with d = 1 and dmin = 0 dequantise, in
+    the independent NumPy restatement, to the integers sc * q: their int64 dot with the Q8_K codes is isum.  With d = 0
+    and dmin = 1 the same restatement gives -mn per weight, and the dot is -msum."""
+    n, k, m = 6, 768, 3
+    rng = np.random.default_rng(51)
+    one = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    aq = O.quantize_q8_k(a)
+    _, q8, _ = _fields(aq, k)
+    blocks = rng.integers(0, 256, (n, k // 256, bpb), dtype=np.uint8)
+    deq = dequant_q5_k if enc == O.Q5_K else dequant_q6_k
+    blocks[:, :, d_at:d_at + 2] = one
+    if dmin_at is not None:
+        blocks[:, :, dmin_at:dmin_at + 2] = 0
+    wq = blocks.reshape(n, -1)
+    isum, msum = O.block_sums_kquant_q8_k(enc, aq, wq, k)
+    ints = deq(wq, k).astype(np.float64)
+    assert np.array_equal(ints, np.rint(ints))
+    want = np.einsum("nbk,mbk->mnb", ints.reshape(n, -1, 256).astype(np.int64), q8.astype(np.int64))
+    assert np.array_equal(isum.astype(np.int64), want)
+    if dmin_at is None:
+        assert not msum.any()
+        return
+    blocks[:, :, d_at:d_at + 2] = 0
+    blocks[:, :, dmin_at:dmin_at + 2] = one
+    wq = blocks.reshape(n, -1)
+    _, msum = O.block_sums_kquant_q8_k(enc, aq, wq, k)
+    mins = deq(wq, k).astype(np.float64)
+    want = -np.einsum("nbk,mbk->mnb", mins.reshape(n, -1, 256).astype(np.int64), q8.astype(np.int64))
+    assert np.array_equal(msum.astype(np.int64), want)
+
+
+def test_generic_q8_k_functions_equal_the_q4_k_ones():
+    n, k, m = 9, 1024, 3
+    w, a = synth(52, n, k, m)
+    wq, aq = O.quantize(O.Q4_K, w), O.quantize_q8_k(a)
+    for x, y in zip(O.block_sums_kquant_q8_k(O.Q4_K, aq, wq, k), O.block_sums_q4_k_q8_k(aq, wq, k)):
+        assert np.array_equal(x, y)
+    assert np.array_equal(O.matmul_kquant_act_q8_k(O.Q4_K, a, wq), O.matmul_q4_k_act_q8_k(a, wq))
+
+
+@pytest.mark.parametrize("enc", [O.Q5_K, O.Q6_K])
+def test_q5_k_q6_k_integer_path_equals_fp_path_on_exactly_representable_activations(enc):
+    n, k, m = 33, 1024, 4
+    w, _ = synth(53, n, k, m)
+    rng = np.random.default_rng(5)
+    a = rng.integers(-126, 127, (m, k)).astype(np.float32)
+    a[:, ::256] = np.array([127.0, -127.0, 127.0, -127.0])[:, None]
+    wq = O.quantize(enc, w)
+    got = O.matmul_kquant_act_q8_k(enc, a, wq)
+    truth = O.matmul_f64(enc, a, wq)
+    assert np.abs(got - truth).max() <= 2e-6 * np.abs(truth).max() + 1e-6 * np.abs(a).max()
+    # and on ordinary activations it is a different (quantised) treatment
+    _, a2 = synth(54, n, k, m)
+    ip, fp = O.matmul_kquant_act_q8_k(enc, a2, wq), O.matmul_f32(enc, a2, wq)
     assert not O.isclose(ip, fp, 1e-3, 1e-4).all()
