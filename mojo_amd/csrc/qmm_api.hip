@@ -233,7 +233,8 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     if (qmm::gemm_planes_wanted(encoding, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (encoding == QMM_Q4_0) {
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
-        return a > b ? a : b;
+        const int64_t c = qmm::gemm_q4_0_planes_wanted(m, n, k) ? qmm::gemm_q4_0_planes_workspace_bytes(m, n, k) : 0;
+        return std::max(std::max(a, b), c);
     }
     if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) {  // lhs planes from 9 rows on; partial sums of K chunks
         const int64_t a = qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k), b = m >= 2 ? qmm::gemv_q4_k_kc_workspace_bytes(m, n, k) : 0;
@@ -415,6 +416,8 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         }
         return QMM_OK;
     }
+    if (encoding == QMM_Q4_0 && qmm::gemm_q4_0_planes_wanted(m, n, k))
+        return hip_status(qmm::launch_gemm_q4_0_planes(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 plane GEMM)");
     if (encoding == QMM_Q4_0 && m >= 5 && !qmm::kernel_disabled("q4_0_mfma"))
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0 && m <= 4) {

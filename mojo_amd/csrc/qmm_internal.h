@@ -12,7 +12,7 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, gptq_mm, gptq_cols.  Nothing is disabled by default.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, gptq_mm, gptq_cols.  Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 
 hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
@@ -94,6 +94,12 @@ hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m,
 hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s, bool* handled);
 int64_t gemm_q4_0_workspace_bytes(int64_t m, int64_t k);
+// Q4_0 prefill on the fp16 matrix cores with exact integer operands (weights as a plane of q - 8, lhs as Q8_0 codes, the
+// per-block scale products made by the matrix cores too): taken where gemm_q4_0_planes_wanted says so.
+bool gemm_q4_0_planes_wanted(int64_t m, int64_t n, int64_t k);
+int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k);
+hipError_t launch_gemm_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out,
+                                   void* workspace, hipStream_t s);
 hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                             float* out, void* workspace, hipStream_t s);
 hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,

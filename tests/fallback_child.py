@@ -1,5 +1,5 @@
 """Child process of test_gpu_fallback_kernels.py: runs a fixed set of small matmuls through the C ABI with whatever
-QMM_DISABLE / QMM_Q4K_TILE the parent put into the environment (the library reads them once per process) and checks
+QMM_DISABLE / QMM_Q4K_TILE / QMM_*_PLANES the parent put into the environment (the library reads them once per process) and checks
 every result against the CPU oracle.  Prints one line per case; exits non-zero on the first mismatch."""
 import os
 import sys
@@ -19,7 +19,7 @@ CASES = {
     "Q4_K": [(1, 300, 4096, False), (2, 130, 2048, True), (4, 200, 4096, False), (12, 64, 8192, False), (16, 72, 512, True),
              (40, 300, 1024, True), (1, 70, 32768, False), (200, 260, 512, True)],
     "Q4_0": [(1, 200, 4096, False), (4, 200, 4096, True), (9, 72, 1056, False), (16, 200, 4096, False), (80, 136, 1024, True)],
-    "Q6_K": [(1, 8200, 2048, False), (1, 300, 4096, True), (4, 200, 4096, False), (16, 72, 512, False)],
+    "Q6_K": [(1, 8200, 2048, False), (1, 300, 4096, True), (4, 200, 4096, False), (16, 72, 512, False), (70, 136, 1024, True)],
     "GPTQ": [(1, 264, 1024, False), (4, 264, 1024, True), (16, 264, 1024, False), (40, 264, 1024, True)],
 }
 

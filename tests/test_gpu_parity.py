@@ -213,7 +213,7 @@ def _integer_dot_case(m, n, k, one_hot, bf16, seed):
 
 # (m, n, k) -> kernel: 1, 4: the decode kernel that quantises the lhs itself; K = 8224: the first-version decode kernel
 # behind the stand-alone quantiser; 5, 16: small-batch int8 matrix-core kernel; 9 with K % 256 != 0, 33, 64: the
-# 16-row-tile kernel (1, 4 tiles per group); 65, 256: the wide prefill kernel
+# 16-row-tile kernel (1, 4 tiles per group); 65, 256: the plane GEMM on the fp16 matrix cores (K = 1024, 4096)
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("one_hot", [True, False])
 @pytest.mark.parametrize("m,n,k", [(1, 200, 4096), (4, 200, 4096), (2, 70, 8224), (5, 200, 4096), (16, 200, 4096),
@@ -878,6 +878,31 @@ def test_q4_0_matmul_int8_matrix_cores(m, n, k, lhs_bf16):
     want = O.matmul_q4_0(a, wq)
     got = qmatmul(QE.Q4_0, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
     assert_close(got, want, f"Q4_0 {m}x{n}x{k} bf16={lhs_bf16}")
+
+
+@pytest.mark.parametrize("m,n,k,bf16", [(1024, 8192, 512, True), (1000, 9300, 768, False), (300, 32768, 256, True), (520, 8200, 1280, False)])
+def test_q4_0_prefill_plane_gemm(m, n, k, bf16):
+    """Q4_0 with more than 64 lhs rows: the fp16 matrix-core kernel over integer planes (lhs Q8_0 codes, weights
+    q - 8; the block scale products made by the matrix cores too).  Whole rounds of tiles, a last round cut in two K halves, a
+    single group of eight blocks, ragged edges; against the oracle's integer path."""
+    w, a = synth(24, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q4_0, w)
+    want = O.matmul_q4_0(a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    wq_d = gpu(wq)
+    got = qmatmul(QE.Q4_0, None, lhs, wq_d)
+    assert_close(got, want, f"Q4_0 plane GEMM {m}x{n}x{k}")
+    assert torch.equal(got, qmatmul(QE.Q4_0, None, lhs, wq_d))
+
+
+@pytest.mark.parametrize("one_hot", [True, False])
+def test_q4_0_prefill_plane_gemm_gives_the_integer_block_dots(one_hot):
+    """The same bit-exact check as for the other Q4_0 kernels, on a problem whose last round of tiles is cut along K."""
+    lhs, wq, want = _integer_dot_case(300, 16384, 512, one_hot, False, 7)
+    got = qmatmul(QE.Q4_0, None, lhs, wq).cpu().numpy()
+    assert np.array_equal(got, want)
 
 
 def test_graph_capture_and_replay_match_eager():
