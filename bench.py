@@ -379,8 +379,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "calib"), default="decode",
-                    help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill / q6k_prefill / q5k_prefill: the M=2048 "
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib"), default="decode",
+                    help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill / q6k_prefill / q5k_prefill / q40_prefill: the M=2048 "
                          "GEMM of the same model's gate projection (second target, matrix-core roofline); calib: a plain "
                          "read and a plain copy of 256 MiB, the yardsticks for the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -524,6 +524,8 @@ def prefill_main(args, gen) -> int:
         call, name, kern = Gemv(QE.Q4_K, make_weight(QE.Q4_K, n, k, gen), ab), "Q4_K", PREFILL_KERNEL
     elif args.workload == "q6k_prefill":
         call, name, kern = Gemv(QE.Q6_K, make_weight(QE.Q6_K, n, k, gen), ab), "Q6_K", "planes_prologue_kernel + gemm_planes_kernel"
+    elif args.workload == "q40_prefill":
+        call, name, kern = Gemv(QE.Q4_0, make_weight(QE.Q4_0, n, k, gen), ab), "Q4_0", "q4_0_planes_prologue_kernel + gemm_q4_0_planes_kernel"
     elif args.workload == "q5k_prefill":
         call, name, kern = Gemv(QE.Q5_K, make_weight(QE.Q5_K, n, k, gen), ab), "Q5_K", "planes_prologue_kernel + gemm_planes_kernel"
     else:
@@ -712,12 +714,14 @@ def extra_timings(layers, acts, gen):
     us = dev_s * 1e6 / (20 * 8)
     out["q5_k_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q5_K, 1, 14336, 4096) / us / 1e3, 1)}
     del cs
-    # Q4_0 prefill on the int8 matrix cores, same shape as cfg5
+    # Q4_0 prefill, same shape as cfg5: Q8_0 lhs codes and q - 8 as exact fp16 integers on the fp16 matrix cores (the time
+    # includes the lhs quantisation and the weight plane conversion)
     ab32 = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
     g = capture([Gemv(QE.Q4_0, make_weight(QE.Q4_0, 14336, 4096, gen), ab32)])
-    dev_s, _ = time_graphs([g], 5, 1)
-    us = dev_s * 1e6 / 5
-    out["q4_0_prefill_m2048"] = {"us": round(us, 1), "TOP/s": round(2 * 2048 * 14336 * 4096 / us / 1e6, 1)}
+    dev_s, _ = time_graphs([g], 10, 2)
+    us = dev_s * 1e6 / 10
+    tf = 2 * 2048 * 14336 * 4096 / us / 1e6
+    out["q4_0_prefill_m2048"] = {"us": round(us, 1), "TOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
     return out
 
 

@@ -267,26 +267,28 @@ __global__ __launch_bounds__(512, 1) void gemm_q4_0_planes_kernel(const uint8_t*
                 }
         };
         // the scale operands of block j (0..7) of the table in buffer tb: d_a of this lane's two row groups, d_w of its two column groups
-        uint32_t sa[2] = {0, 0}, sb[2] = {0, 0};
+        // (kept as whole operands: element 0 carries the scale, the other seven stay zero for the whole kernel)
+        HalfPack oa[2], ob[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) oa[i].u[e] = ob[i].u[e] = 0u;
         auto read_scales = [&](int tb, int j) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                sa[i] = (uint32_t)(*(const uint16_t*)(smem + da_at + tb * kDaBuf + i * 512 + j * 2)) & keep;
-                sb[i] = (uint32_t)(*(const uint16_t*)(smem + dw_at + tb * kDwBuf + i * 512 + j * 2)) & keep;
+                oa[i].u[0] = (uint32_t)(*(const uint16_t*)(smem + da_at + tb * kDaBuf + i * 512 + j * 2)) & keep;
+                ob[i].u[0] = (uint32_t)(*(const uint16_t*)(smem + dw_at + tb * kDwBuf + i * 512 + j * 2)) & keep;
             }
         };
         auto scale_tile = [&](int t) __attribute__((always_inline)) {
-            return __builtin_amdgcn_mfma_f32_32x32x16_f16(pack4(sa[t >> 1], 0u, 0u, 0u), pack4(sb[t & 1], 0u, 0u, 0u), zero16, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_32x32x16_f16(oa[t >> 1].h, ob[t & 1].h, zero16, 0, 0, 0);
         };
-        // acc += isum * (d_a d_w^T) for the finished block whose dots are in P and whose scale operands are in sa / sb, sub-tile by
+        // acc += isum * (d_a d_w^T) for the finished block whose dots are in P and whose scale operands are in oa / ob, sub-tile by
         // sub-tile in front of the instruction that restarts that sub-tile's P with the first slice of the next block (slot 0)
         auto finish_and_restart = [&](bool restart, auto&& between) __attribute__((always_inline)) {
-            float16v S0 = scale_tile(0), S1 = scale_tile(1);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
+            // one sub-tile: the multiply-adds, then the instruction that restarts its dots
+            auto finish_tile = [&](int t, const float16v& S) __attribute__((always_inline)) {
                 const int mi = t >> 1, ni = t & 1;
-                const float16v& S = (t & 1) ? S1 : S0;
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[mi][ni][r] = fmaf(P[mi][ni][r], S[r], acc[mi][ni][r]);
                 // (pins the update here: left alone, the compiler defers the multiply-adds of several blocks and keeps their
@@ -294,11 +296,24 @@ __global__ __launch_bounds__(512, 1) void gemm_q4_0_planes_kernel(const uint8_t*
                 asm volatile("" : "+v"(acc[mi][ni]));
                 __builtin_amdgcn_sched_barrier(0);
                 if (restart) P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][mi], bfr[0][ni], zero16, 0, 0, 0);
-                if (t == 0) S0 = scale_tile(2);
-                if (t == 1) S1 = scale_tile(3);
-                between(t);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            };
+            // two scale products are in flight ahead of the sub-tile that uses them
+            const float16v S0 = scale_tile(0), S1 = scale_tile(1);
+            __builtin_amdgcn_sched_barrier(0);
+            finish_tile(0, S0);
+            const float16v S2 = scale_tile(2);
+            between(0);
+            __builtin_amdgcn_sched_barrier(0);
+            finish_tile(1, S1);
+            const float16v S3 = scale_tile(3);
+            between(1);
+            __builtin_amdgcn_sched_barrier(0);
+            finish_tile(2, S2);
+            between(2);
+            __builtin_amdgcn_sched_barrier(0);
+            finish_tile(3, S3);
+            between(3);
+            __builtin_amdgcn_sched_barrier(0);
         };
         auto nothing = [](int) __attribute__((always_inline)) {};
 

@@ -589,10 +589,11 @@ int qmm_matmul_swiglu(int encoding, const void* lhs, int lhs_dtype, int64_t m, i
     if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_swiglu: workspace must be 256-byte aligned");
     float* g = (float*)((char*)workspace + mm_ws);
     float* u = (float*)((char*)workspace + mm_ws + plane);
-    const void* one[1] = {gate};
-    if (int rc = qmm_matmul(encoding, nullptr, lhs, lhs_dtype, m, k, one, 1, n, g, workspace, mm_ws, 0, stream)) return rc;
-    one[0] = up;
-    if (int rc = qmm_matmul(encoding, nullptr, lhs, lhs_dtype, m, k, one, 1, n, u, workspace, mm_ws, 0, stream)) return rc;
+    // (one launch for both products where a kernel takes matrices that share their lhs: Q4_K with 2..16 rows)
+    const void* both[2] = {gate, up};
+    const int64_t ns[2] = {n, n};
+    float* outs[2] = {g, u};
+    if (int rc = qmm_matmul_grouped(encoding, lhs, lhs_dtype, m, k, 2, both, ns, outs, workspace, mm_ws, stream)) return rc;
     return hip_status(qmm::launch_swiglu(g, u, out, m * n, (hipStream_t)stream), "qmm_matmul_swiglu(combine)");
 }
 
