@@ -68,51 +68,10 @@ __device__ __forceinline__ void tie(T& d) {
     asm volatile("" : "+v"(d));
 }
 
-// Loads into FIXED accumulation registers (a[R], a[R + 1], ...), for data that stays in flight across loop
-// back-edges.  A hidden load into an ordinary variable is only safe while the compiler never copies that
-// variable between issue and use: a copy (which it may make where two definitions meet at a loop header, or
-// when it splits a live range) moves the stale contents and frees the register the data later lands in, which
-// by then holds something else.  Accumulation registers named here are never allocated by the compiler for
-// anything that lives across these statements (they are declared clobbered), so the data is where it was sent;
-// it is moved to ordinary registers with agpr_read after the wait.  A kernel that uses these must not need
-// accumulation registers of its own in that range (check its resource report: AGPRs == the range reserved).
-template <int R> __device__ __forceinline__ void agpr_load2(const void* g);
-template <int R> __device__ __forceinline__ void agpr_load4(const void* g);
-template <int R> __device__ __forceinline__ u32x2 agpr_read2();
-template <int R> __device__ __forceinline__ u32x4 agpr_read4();
-#define QMM_AGPR2(R0, R1)                                                                                                   \
-    template <> __device__ __forceinline__ void agpr_load2<R0>(const void* g) {                                             \
-        asm volatile("global_load_dwordx2 a[" #R0 ":" #R1 "], %0, off" ::"v"(g) : "memory", "a" #R0, "a" #R1);               \
-    }                                                                                                                       \
-    template <> __device__ __forceinline__ u32x2 agpr_read2<R0>() {                                                         \
-        uint32_t x, y;                                                                                                      \
-        asm volatile("v_accvgpr_read_b32 %0, a" #R0 "\n\tv_accvgpr_read_b32 %1, a" #R1 : "=v"(x), "=v"(y)::"memory");       \
-        u32x2 v;                                                                                                            \
-        v.x = x; v.y = y;                                                                                                   \
-        return v;                                                                                                           \
-    }
-#define QMM_AGPR4(R0, R1, R2, R3)                                                                                           \
-    template <> __device__ __forceinline__ void agpr_load4<R0>(const void* g) {                                             \
-        asm volatile("global_load_dwordx4 a[" #R0 ":" #R3 "], %0, off" ::"v"(g)                                              \
-                     : "memory", "a" #R0, "a" #R1, "a" #R2, "a" #R3);                                                       \
-    }                                                                                                                       \
-    template <> __device__ __forceinline__ u32x4 agpr_read4<R0>() {                                                         \
-        uint32_t x, y, z, w;                                                                                                \
-        asm volatile("v_accvgpr_read_b32 %0, a" #R0 "\n\tv_accvgpr_read_b32 %1, a" #R1 "\n\tv_accvgpr_read_b32 %2, a" #R2   \
-                     "\n\tv_accvgpr_read_b32 %3, a" #R3                                                                     \
-                     : "=v"(x), "=v"(y), "=v"(z), "=v"(w)::"memory");                                                       \
-        u32x4 v;                                                                                                            \
-        v.x = x; v.y = y; v.z = z; v.w = w;                                                                                 \
-        return v;                                                                                                           \
-    }
-QMM_AGPR2(0, 1)
-QMM_AGPR2(2, 3)
-QMM_AGPR2(4, 5)
-QMM_AGPR2(6, 7)
-QMM_AGPR4(8, 9, 10, 11)
-QMM_AGPR4(12, 13, 14, 15)
-#undef QMM_AGPR2
-#undef QMM_AGPR4
+// A hidden load into an ordinary variable is only safe while the compiler never copies that variable between issue and
+// use: a copy (which it may make where two definitions meet at a loop header, or when it splits a live range) moves the
+// stale contents and frees the register the data later lands in, which by then holds something else.  Use hidden_load
+// in straight-line prologues only; data that stays in flight across a loop back-edge goes global -> LDS (load16_to_lds).
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

@@ -79,6 +79,33 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.qmm_matmul_workspace_bytes(1, 0, 8, 4096, 4096) == 0  # up to 8 rows the kernel narrows the lhs itself
     assert lib.qmm_matmul_workspace_bytes(1, 0, 12, 4096, 4096) >= 2 * 12 * 4096 * 2  # fp16 hi and residual planes
     assert lib.qmm_matmul_workspace_bytes(1, 1, 2048, 14336, 4096) >= 2048 * 4096 * 2
+    # flags that change the workspace: a bf16 result that the kernel does not store itself goes through an fp32 copy; Q8_K
+    # activations outside the integer kernel go through fp32 rows of d8 * code
+    f = lib.qmm_matmul_workspace_bytes_flags
+    assert f(1, 0, 1, 4096, 4096, _lib.QMM_FLAG_OUT_BF16) == 0                      # Q4_K decode stores bf16 itself
+    assert f(2, 0, 1, 4096, 4096, _lib.QMM_FLAG_OUT_BF16) == 4096 * 4               # Q6_K decode: fp32 result in the workspace
+    assert f(1, 0, 4, 4096, 4096, _lib.QMM_FLAG_ACT_Q8K) == 0                       # the integer kernel
+    assert f(2, 0, 4, 4096, 4096, _lib.QMM_FLAG_ACT_Q8K) >= 4 * 4096 * 4            # Q6_K: round-tripped rows
+    assert f(1, 0, 2048, 14336, 4096, 0) == lib.qmm_matmul_workspace_bytes(1, 0, 2048, 14336, 4096)
+    # Q5_K / Q6_K prefill: lhs planes and weight planes (2 bytes per weight and plane; Q6_K has two)
+    assert lib.qmm_matmul_workspace_bytes(2, 1, 2048, 14336, 4096) >= 2 * 14336 * 4096 * 2
+    assert lib.qmm_matmul_workspace_bytes(4, 1, 2048, 14336, 4096) >= 14336 * 4096 * 2
+    assert lib.qmm_matmul_workspace_bytes(0, 1, 2048, 14336, 4096) >= 14336 * 4096 * 2 + 2048 * 4096 * 2  # Q4_0: plane + lhs codes
+    # bf16 output without the workspace it needs, Q8_K activations for an encoding that has none
+    assert lib.qmm_matmul(2, None, fake, 0, 1, 4096, rhs, 1, 8, fake, None, 0, _lib.QMM_FLAG_OUT_BF16, None) == -4
+    assert b"bf16" in lib.qmm_last_error()
+    ws = C.c_void_p(0x100000)
+    assert lib.qmm_matmul(0, None, fake, 0, 1, 4096, rhs, 1, 8, fake, ws, 1 << 30, _lib.QMM_FLAG_ACT_Q8K, None) == -2
+    assert lib.qmm_matmul(1, None, fake, 0, 1, 4096, rhs, 1, 8, fake, None, 0, 8, None) == -1 and b"flag" in lib.qmm_last_error()
+    # the normalisation prologue
+    g = C.c_void_p(0x3000)
+    rn = lib.qmm_matmul_rmsnorm
+    assert rn(0, None, fake, 0, None, 1e-5, 1, 4096, rhs, 1, 8, fake, None, 0, 0, None) == -1               # no gamma
+    assert rn(0, None, fake, 0, g, -1.0, 1, 4096, rhs, 1, 8, fake, None, 0, 0, None) == -1 and b"eps" in lib.qmm_last_error()
+    assert rn(0, None, fake, 2, g, 1e-5, 1, 4096, rhs, 1, 8, fake, None, 0, 0, None) == -1                  # fp16 x
+    assert rn(1, None, fake, 0, g, 1e-5, 1, 4096, rhs, 1, 8, fake, None, 0, 0, None) == -4                  # Q4_K: needs room for the normalised rows
+    assert lib.qmm_matmul_rmsnorm_workspace_bytes(1, 0, 1, 8, 4096, 0) == 4096 * 4
+    assert lib.qmm_matmul_rmsnorm_workspace_bytes(1, 1, 3, 8, 4096, 0) == 3 * 4096 * 2
 
 
 def test_quantization_encoding_metadata():
