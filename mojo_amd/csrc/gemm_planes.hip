@@ -8,8 +8,9 @@
 //         fp16 integer); the min term as two extra matrix-core products per super-block over the lhs sub-block sums.
 //   Q6_K  w = d * (sc * q),  q in [-32, 31], sc an int8 per 16 weights: sc * q reaches 4096 and odd values above
 //         2048 are no fp16 numbers, so sc = 16 hi + lo (hi = sc >> 4 in [-8, 7], lo = sc & 15) gives two planes,
-//         (16 hi) * q (a multiple of 16 with at most 9 significant bits) and lo * q (<= 480), both exact.  The GEMM
-//         walks K once per plane; a super-block's partial product of either plane is scaled by the same d.
+//         (16 hi) * q (a multiple of 16 with at most 9 significant bits) and lo * q (<= 480), both exact.  Its GEMM
+//         (gemm_planes2_kernel) multiplies both planes of a K step with the same lhs operands and scales the sum of the
+//         two partial products of a super-block by d.
 // The planes cost workspace (2 bytes per weight and plane) and one pass over the weights (tens of microseconds at
 // the sizes this path is chosen for); they buy a GEMM whose only vector-ALU work is the rescale.
 //
@@ -184,13 +185,11 @@ __global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __r
 
 // The GEMM over the planes.  Structure, buffers and schedule are those of gemm_q4_k_tile_kernel (see there); what differs:
 // the weight operands of a step arrive ready-made (16 KB per tile and step, global -> LDS directly, two steps ahead in a
-// ring of three buffers like the lhs), K is walked once per plane (virtual super-blocks vb = plane * nblk + rb), and the
-// tables of a super-block come from memory.  WITH_MIN: the encoding has a min term (Q5_K).
-template <bool WITH_MIN>
+// ring of three buffers like the lhs) and the tables of a super-block come from memory.  One plane with a min term (Q5_K, Q4_K).
 __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __restrict__ planes, const float* __restrict__ dtab,
                                                             const uint8_t* __restrict__ mtab, const _Float16* __restrict__ a16,
                                                             const _Float16* __restrict__ asum, const float* __restrict__ inv,
-                                                            float* __restrict__ out, int m, int n, int k, int nplanes, int tiles_m,
+                                                            float* __restrict__ out, int m, int n, int k, int tiles_m,
                                                             int tiles_n, int with_min, int accumulate, int allow_split) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = lds_address(smem);
@@ -198,7 +197,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int nl = lane & 31, g = lane >> 5;
-    const int nblk_row = k >> 8, nblk_virtual = nblk_row * nplanes;
+    const int nblk_row = k >> 8;
     const uint32_t fb0 = (uint32_t)(kOffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const int a_minus_b = (kOffA + wm * 64 * 128) - (kOffB + wn * 64 * 128);
     const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -207,12 +206,12 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
     const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
     int full;
-    const int units = xcd_units(n_x, wgs_per_xcd, nblk_virtual, allow_split, full);
+    const int units = xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
     for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
-        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_virtual);
+        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_row);
         // (uniform values that come out of integer divisions live in vector registers unless told otherwise; everything
         // below that is derived from them, the base pointers above all, would follow them there)
-        const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * 4;  // this unit's share of the virtual K
+        const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * 4;  // this unit's share of K
         const int kb0 = __builtin_amdgcn_readfirstlane(unit.kb0), unit_half = __builtin_amdgcn_readfirstlane(unit.half);
         int tile_m, tile_n;
         tile_order(unit.tile, tiles_m, tiles_n, kTileGm, tile_m, tile_n);
@@ -228,17 +227,13 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
         const uint8_t* a_base = (const uint8_t*)a16 + (int64_t)(m0 + wave * 32) * k * 2;
         const uint32_t s_off = (uint32_t)((wave * 32 + (lane >> 1)) * (nblk_row * 32) + (lane & 1) * 16);
         const uint8_t* s_base = (const uint8_t*)asum + (int64_t)m0 * nblk_row * 32;
-        const uint8_t* b_base = planes + ((int64_t)tile_n * nblk_virtual + kb0) * 4 * kBBuf;  // (virtual steps of a tile are contiguous)
+        const uint8_t* b_base = planes + ((int64_t)tile_n * nblk_row + kb0) * 4 * kBBuf;
         const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * nblk_row * kDBuf;
         const uint8_t* m_base = mtab + (int64_t)tile_n * nblk_row * kMBuf;
-        auto real_blk = [&](int blk) __attribute__((always_inline)) {  // virtual super-block of this unit -> super-block of the row
-            const int vb = kb0 + min(blk, nblk - 1);
-            return vb >= nblk_row ? vb - nblk_row : vb;  // (at most two planes)
-        };
+        auto real_blk = [&](int blk) __attribute__((always_inline)) { return kb0 + min(blk, nblk - 1); };  // super-block of the row
 
         auto issue_A1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
-            const int sv = kb0 * 4 + min(step, ns - 1), steps_row = nblk_row * 4;
-            const int sr = sv >= steps_row ? sv - steps_row : sv;
+            const int sr = kb0 * 4 + min(step, ns - 1);
             const uint32_t dst = lds0 + kOffA + buf * kABuf + wave * 4096;
             load16_to_lds(a_off[i & 1], a_base + (int64_t)sr * 128 + (int64_t)i * 16 * k,
                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
@@ -255,12 +250,10 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
             if (lane < 4)
                 load16_to_lds(lane16, d_base + (int64_t)rb * kDBuf + wave * 64,
                               (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffD + wave * 64)));
-            if constexpr (WITH_MIN) {
-                if (lane < 32)
-                    load16_to_lds(lane16, m_base + (int64_t)rb * kMBuf + wave * 512,
-                                  (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffM + wave * 512)));
-                load16_to_lds(s_off, s_base + (int64_t)rb * 32, (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffS + wave * 1024)));
-            }
+            if (lane < 32)
+                load16_to_lds(lane16, m_base + (int64_t)rb * kMBuf + wave * 512,
+                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffM + wave * 512)));
+            load16_to_lds(s_off, s_base + (int64_t)rb * 32, (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kOffS + wave * 1024)));
         };
 
         float16v acc[2][2], P[2][2];
@@ -340,7 +333,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
             if constexpr (c == 2) issue_tables(blk + 1);
             __builtin_amdgcn_sched_barrier(0);
             half8 sfr[2], mh, ml;
-            const bool min_now = WITH_MIN && c == 1 && with_min && kb0 + blk < nblk_row;  // (once per super-block of the row: with its first plane)
+            const bool min_now = c == 1 && with_min;
             if (min_now) {
 #pragma unroll
                 for (int mi = 0; mi < 2; mi++) sfr[mi] = *(const half8*)(smem + kOffS + (wm * 64 + mi * 32 + nl) * 32 + g * 16);
@@ -391,7 +384,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
             __builtin_amdgcn_sched_barrier(0);
             mfma_slice(0, false, [&](int i) __attribute__((always_inline)) { if (i == 3) issue_A1(s + 2, ab2, 3); });
             // everything issued before this phase has landed: lhs and weights of step s + 1 (and, after phase 3, the tables)
-            if constexpr (c == 2) wait_vmcnt<WITH_MIN ? 9 : 7>();
+            if constexpr (c == 2) wait_vmcnt<9>();
             else wait_vmcnt<6>();
             __syncthreads();
             abuf = abuf == 2 ? 0 : abuf + 1;
@@ -415,6 +408,239 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
                 float4 iv[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) iv[j] = *(const float4*)(smem + kOffInv + (wm * 64 + mi * 32 + 8 * j + 4 * g) * 4);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    const float4 q = iv[r >> 2];
+                    const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
+                    if (row < m) {
+                        float* o_ = out + (int64_t)row * n;
+                        const float v0 = acc[mi][0][r] * is, v1 = acc[mi][1][r] * is;
+                        if (unit_half) {  // one of the two K halves of this tile: out holds zero or the other half
+                            if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
+                            if (c1_ok) unsafeAtomicAdd(o_ + col1, v1);
+                        } else if (accumulate) {
+                            if (c0_ok) o_[col0] += v0;
+                            if (c1_ok) o_[col1] += v1;
+                        } else {
+                            if (c0_ok) __builtin_nontemporal_store(v0, o_ + col0);
+                            if (c1_ok) __builtin_nontemporal_store(v1, o_ + col1);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// The GEMM over TWO planes of one encoding (Q6_K: (16 hi) * q and lo * q, same super-block scale d): both planes of a step are
+// multiplied with the same lhs operands, so the lhs tile travels to LDS and into registers once for both, and a step holds 32
+// matrix-core instructions per wavefront instead of 16.  That lengthens the lead of every operand read (eight instructions instead of
+// four) and lets two buffers per operand do (a step ahead is as long as two steps of the one-plane kernel): lhs 2 x 32 KB, weights
+// 2 x (2 planes x 16 KB).  No min term (Q6_K has none).
+namespace {
+constexpr int k2OffA = 0, k2OffB = 2 * kABuf, k2OffD = k2OffB + 4 * kBBuf, k2OffInv = k2OffD + kDBuf, kPlanes2Lds = k2OffInv + TM * 4;
+static_assert(kPlanes2Lds <= kLdsPerCu, "two-plane kernel LDS");
+}  // namespace
+
+__global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __restrict__ planes, const float* __restrict__ dtab,
+                                                             const _Float16* __restrict__ a16, const float* __restrict__ inv,
+                                                             float* __restrict__ out, int m, int n, int k, int tiles_m, int tiles_n,
+                                                             int accumulate, int allow_split) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t lds0 = lds_address(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int nl = lane & 31, g = lane >> 5;
+    const int nblk_row = k >> 8;
+    // operand reads: row (column) nl of the wavefront's 32-row groups, piece 2 f + g, swizzled; slice f: the address xor f << 5
+    const uint32_t fa0 = (uint32_t)(k2OffA + (wm * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
+    const uint32_t fb0 = (uint32_t)(k2OffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
+    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const uint32_t lane16 = (uint32_t)(lane * 16);
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
+    const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
+    int full;
+    const int units = xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
+    for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
+        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_row);
+        const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * 4;  // this unit's share of K
+        const int kb0 = __builtin_amdgcn_readfirstlane(unit.kb0), unit_half = __builtin_amdgcn_readfirstlane(unit.half);
+        int tile_m, tile_n;
+        tile_order(unit.tile, tiles_m, tiles_n, kTileGm, tile_m, tile_n);
+        tile_m = __builtin_amdgcn_readfirstlane(tile_m);
+        tile_n = __builtin_amdgcn_readfirstlane(tile_n);
+        const int m0 = tile_m * TM, n0 = tile_n * TN;
+
+        const uint8_t* a_base = (const uint8_t*)a16 + ((int64_t)(m0 + wave * 32) * k + (int64_t)kb0 * 256) * 2;
+        const int64_t plane_bytes = (int64_t)nblk_row * 4 * kBBuf;  // one plane of one column tile
+        const uint8_t* b_base = planes + (int64_t)tile_n * 2 * plane_bytes + (int64_t)kb0 * 4 * kBBuf;
+        const uint8_t* d_base = (const uint8_t*)dtab + ((int64_t)tile_n * nblk_row + kb0) * kDBuf;
+
+        // the i-th of the four loads that bring this wavefront's 32 rows of the lhs of step `step` into buffer `buf`
+        auto issue_A1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
+            // lhs rows wave * 32 + 8 i + lane / 8; LDS position lane % 8 of a row holds piece (lane % 8) ^ ((row / 2) % 8).  The lane
+            // offset is recomputed at every use (behind an empty asm statement): kept in a register of its own it gets spilled.
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            const uint32_t a_off = (uint32_t)((l >> 3) * (k * 2) + (((l & 7) ^ ((4 * i + (l >> 4)) & 7)) << 4));
+            const uint32_t dst = lds0 + k2OffA + buf * kABuf + wave * 4096;
+            load16_to_lds(a_off, a_base + (int64_t)min(step, ns - 1) * 128 + (int64_t)i * 16 * k,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
+        };
+        // the i-th (0..3) of this wavefront's four 1 KB pieces of the two weight tiles of step `step`: plane i / 2, piece 2 wave + i % 2
+        auto issue_B1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
+            const int pl = i >> 1, piece = (wave * 2 + (i & 1)) * 1024;
+            load16_to_lds(lane16, b_base + pl * plane_bytes + (int64_t)min(step, ns - 1) * kBBuf + piece,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + k2OffB + (buf * 2 + pl) * kBBuf + piece)));
+        };
+        auto issue_D = [&](int blk) __attribute__((always_inline)) {
+            if (lane < 4)
+                load16_to_lds(lane16, d_base + (int64_t)min(blk, nblk - 1) * kDBuf + wave * 64,
+                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + k2OffD + wave * 64)));
+        };
+
+        float16v acc[2][2], P[2][2];
+#pragma unroll
+        for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    acc[mi][ni][r] = 0.0f;
+                    P[mi][ni][r] = 0.0f;
+                }
+        half8 afr[2][2], bfr[2][2][2];  // [slot][row group], [slot][plane][column group]
+        float dcur[2] = {0.f, 0.f};
+
+        // ---- tile prologue
+        __syncthreads();  // every wavefront is done with the previous tile's LDS contents
+        issue_D(0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_A1(0, 0, i);
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_B1(0, 0, i);
+        if (tid < TM) *(float*)(smem + k2OffInv + tid * 4) = inv[min(m0 + tid, m - 1)];
+        wait_vmcnt<0>();
+        __syncthreads();
+
+        // Operand addresses of the current step: recomputed every phase from the buffer offsets behind an empty asm statement
+        // (left to itself the compiler keeps the addresses of every (phase, slice, operand) in registers of their own, spills them
+        // and reloads them inside the loop, and every reload waits for all outstanding global -> LDS loads).
+        uint32_t fa = 0, fb = 0;
+        auto step_bases = [&](int buf) __attribute__((always_inline)) {
+            int ao = buf * kABuf, bo = buf * 2 * kBBuf;
+            asm volatile("" : "+s"(ao), "+s"(bo));
+            fa = fa0 + (uint32_t)ao;
+            fb = fb0 + (uint32_t)bo;
+        };
+        auto read_frags = [&](int f, int slot) __attribute__((always_inline)) {
+            const uint32_t xa = fa ^ (uint32_t)(f << 5), xb = fb ^ (uint32_t)(f << 5);
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + xa + mi * 4096);
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + xb + pl * kBBuf + ni * 4096);
+        };
+        // the eight matrix-core instructions of one slice (both planes); `between(i)` is placed after the i-th of them
+        auto mfma_slice = [&](int slot, auto&& between) __attribute__((always_inline)) {
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++)
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++) {
+                        P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][pl][ni], P[mi][ni], 0, 0, 0);
+                        between(pl * 4 + mi * 2 + ni);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+        };
+        auto rescale_tile = [&](int t) __attribute__((always_inline)) {
+            const int mi = t >> 1, ni = t & 1;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[mi][ni][r] = fmaf(dcur[ni], P[mi][ni][r], acc[mi][ni][r]);
+        };
+
+        // One phase = from the barrier inside step s - 1 to the barrier inside step s; the buffers of step s are those of index s % 2 = c % 2.
+        // All loads of step s + 1 are issued in the first half of the phase, into the buffers that step s - 1 used.
+        auto phase = [&](int blk, auto CC) __attribute__((always_inline)) {
+            constexpr int c = decltype(CC)::value, cur = c & 1, nxt = cur ^ 1;
+            const int s = blk * 4 + c;
+            step_bases(cur);
+            read_frags(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (s > 0) {
+                mfma_slice(1, [&](int i) __attribute__((always_inline)) {  // last slice of step s - 1
+                    if (i & 1) issue_A1(s + 1, nxt, i >> 1);
+                });
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) issue_A1(s + 1, nxt, i);
+            }
+            if constexpr (c == 2) issue_D(blk + 1);  // (the current scales were read in phase 0)
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (c == 0 && s > 0) {
+                // the finished super-block's rescale, sub-tile by sub-tile, in front of the instruction that restarts its P
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    rescale_tile(t);
+                    __builtin_amdgcn_sched_barrier(0);
+                    P[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][0][t & 1], zero16, 0, 0, 0);
+                    issue_B1(s + 1, nxt, t);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    P[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][1][t & 1], P[t >> 1][t & 1], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                if (c == 0) {  // the first step of the unit: P starts from zero
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) P[t >> 1][t & 1][r] = 0.0f;
+                }
+                mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < 4) issue_B1(s + 1, nxt, i); });
+            }
+            if (c == 0) {
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) dcur[ni] = *(const float*)(smem + k2OffD + (wn * 64 + ni * 32 + nl) * 4);
+            }
+            read_frags(2, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_slice(1, [](int) __attribute__((always_inline)) {});
+            read_frags(3, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_slice(0, [](int) __attribute__((always_inline)) {});
+            wait_vmcnt<0>();  // lhs and weights of step s + 1 (and, in phase 2, the next scales) have landed
+            __syncthreads();
+        };
+        for (int blk = 0; blk < nblk; blk++) {
+            phase(blk, std::integral_constant<int, 0>{});
+            phase(blk, std::integral_constant<int, 1>{});
+            phase(blk, std::integral_constant<int, 2>{});
+            phase(blk, std::integral_constant<int, 3>{});
+        }
+        mfma_slice(1, [](int) __attribute__((always_inline)) {});  // last slice of the last step
+#pragma unroll
+        for (int t = 0; t < 4; t++) rescale_tile(t);
+
+        // ---- tile epilogue: undo the row scale, store
+        {
+            const int col0 = n0 + wn * 64 + nl, col1 = col0 + 32;
+            const bool c0_ok = col0 < n, c1_ok = col1 < n;
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+                float4 iv[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) iv[j] = *(const float4*)(smem + k2OffInv + (wm * 64 + mi * 32 + 8 * j + 4 * g) * 4);
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
@@ -464,7 +690,7 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
     const int nplanes = q6 ? 2 : 1;
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
     const PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, nplanes, !q6);
-    hipError_t e = q6 ? allow_full_lds<gemm_planes_kernel<false>>() : allow_full_lds<gemm_planes_kernel<true>>();
+    hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : allow_full_lds<gemm_planes_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n = (int)((n + TN - 1) / TN), nblk = (int)(k / 256);
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
@@ -475,8 +701,7 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
             cus = 256;
     }
     const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
-    const int nblk_virtual = nblk * nplanes;
-    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, nblk_virtual, wg);
+    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, nblk, wg);
     const int max_split = z.max_split;
     const int64_t conv = (int64_t)tiles_n * nblk * 4, blocks = conv + m + (int64_t)max_split * 64;
     if (blocks > INT32_MAX) return hipErrorInvalidValue;
@@ -498,11 +723,11 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
         const _Float16* a = pass == 0 ? p.a16 : p.a16_lo;
         const int split = pass == 0 && max_split > 0 ? 1 : 0;
         if (q6)
-            gemm_planes_kernel<false><<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m,
-                                                                                    (int)n, (int)k, nplanes, tiles_m, tiles_n, 0, pass, split);
+            gemm_planes2_kernel<<<dim3((unsigned)wg), dim3(512), kPlanes2Lds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k,
+                                                                                 tiles_m, tiles_n, pass, split);
         else
-            gemm_planes_kernel<true><<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m,
-                                                                                   (int)n, (int)k, nplanes, tiles_m, tiles_n, pass == 0, pass, split);
+            gemm_planes_kernel<<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m, (int)n,
+                                                                               (int)k, tiles_m, tiles_n, pass == 0, pass, split);
     }
     return hipGetLastError();
 }
