@@ -46,7 +46,10 @@ __device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ub
 // ring: LDS slots per wavefront (2..4): one row part being decoded, the others in flight.
 // mats: up to kLanesMaxMats weight matrices that share the lhs and K; their rows are numbered through
 // (matrix j owns rows [end[j - 1], end[j])), so one launch serves q|k|v or gate|up.
-template <int MT, int WPR, int L, typename AT>
+// HALF: a lane owns one 32-column sub-block instead of a 64-column chunk (lane l: super-block l / 8, chunk (l / 2) % 4, low nibbles
+// for even l, high nibbles for odd l), which halves the activations a lane keeps per lhs row and so makes room for four lhs
+// rows; a wavefront then covers 8 super-blocks, a row of 4096 columns takes two wavefronts (WPR up to 8, parts of up to 8).
+template <int MT, int WPR, int L, typename AT, bool HALF>
 __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const LanesMats mats, const AT* __restrict__ a,
                                                                         int m, int k, int64_t ldo, int ring_slots,
                                                                         int streams, int rows_each, int rows_extra) {
@@ -108,8 +111,10 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     //     into LDS, laid out as one record per 64-column chunk (its pieces plus one piece of padding, so that
     //     the lanes' 16-byte reads of their own records spread over the banks), issued before the first weight
     //     rows and waited for together with them.
-    const int lb = min(lane >> 2, max(nb, 1) - 1), c = lane & 3;
-    const bool live = (lane >> 2) < nb;
+    const int lsb = HALF ? lane >> 3 : lane >> 2;  // this lane's super-block of the part
+    const int lb = min(lsb, max(nb, 1) - 1), c = HALF ? (lane >> 1) & 3 : lane & 3;
+    const int hn = lane & 1;  // (HALF) 0: the low nibbles, sub-block 2 c; 1: the high nibbles, sub-block 2 c + 1
+    const bool live = lsb < nb;
     constexpr int kCp = sizeof(AT) == 4 ? 16 : 8;  // 16-byte pieces of a chunk's 64 activations
     uint8_t* act = smem + kWaves * kRing * kSlot + kWaves * kMaxRows * MT * 4;
     const int nchunk = k >> 6, npos = nchunk * (kCp + 1);  // records, and their pieces (padding included)
@@ -134,11 +139,38 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     }
     wait_items<L, 0>(issued, false);  // the activation loads are older than these rows
     __syncthreads();                  // every wavefront's share of the activations has landed
-    float alo[MT][32], ahi[MT][32], slo_a[MT], shi_a[MT];
+    constexpr int kAh = HALF ? 1 : 32;  // (HALF keeps one 32-value set per lhs row, in alo)
+    float alo[MT][32], ahi[MT][kAh], slo_a[MT], shi_a[MT];
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
         float v[64];
         const uint4* rec = (const uint4*)(act + ((size_t)mi * nposp + (size_t)((blk0 + lb) * 4 + c) * (kCp + 1)) * 16);
+        if constexpr (HALF) {
+            // this lane's half of the record: pieces [hn * kCp / 2, (hn + 1) * kCp / 2)
+            constexpr int kHp = kCp / 2;
+#pragma unroll
+            for (int i = 0; i < kHp; i++) {
+                const uint4 r = rec[hn * kHp + i];
+                if constexpr (sizeof(AT) == 4) {
+                    v[4 * i] = __uint_as_float(r.x); v[4 * i + 1] = __uint_as_float(r.y);
+                    v[4 * i + 2] = __uint_as_float(r.z); v[4 * i + 3] = __uint_as_float(r.w);
+                } else {
+                    v[8 * i] = __uint_as_float(r.x << 16); v[8 * i + 1] = __uint_as_float(r.x & 0xffff0000u);
+                    v[8 * i + 2] = __uint_as_float(r.y << 16); v[8 * i + 3] = __uint_as_float(r.y & 0xffff0000u);
+                    v[8 * i + 4] = __uint_as_float(r.z << 16); v[8 * i + 5] = __uint_as_float(r.z & 0xffff0000u);
+                    v[8 * i + 6] = __uint_as_float(r.w << 16); v[8 * i + 7] = __uint_as_float(r.w & 0xffff0000u);
+                }
+            }
+            float s0 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) alo[mi][i] = v[i];
+#pragma unroll
+            for (int i = 0; i < 32; i += 4) s0 += (alo[mi][i] + alo[mi][i + 1]) + (alo[mi][i + 2] + alo[mi][i + 3]);
+            slo_a[mi] = s0;
+            shi_a[mi] = 0.0f;
+            ahi[mi][0] = 0.0f;
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < kCp; i++) {
             const uint4 r = rec[i];
@@ -186,6 +218,24 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
         float slo[MT], shi[MT];
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) slo[mi] = shi[mi] = 0.0f;
+        if constexpr (HALF) {
+            const int nsh = 4 * hn;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                // this lane's nibbles moved to the low position: q * 2^-24 as fp16 subnormals, as below
+                const uint32_t x = qd[i] >> nsh;
+                const half2v l02 = as_half2(x & 0x000F000Fu), l13 = as_half2((x >> 8) & 0x000F000Fu);
+                const float w0 = (float)l02.x, w1 = (float)l13.x, w2 = (float)l02.y, w3 = (float)l13.y;
+#pragma unroll
+                for (int mi = 0; mi < MT; mi++) {
+                    float t = slo[mi];
+                    t = fmaf(alo[mi][4 * i], w0, t);
+                    t = fmaf(alo[mi][4 * i + 1], w1, t);
+                    t = fmaf(alo[mi][4 * i + 2], w2, t);
+                    slo[mi] = fmaf(alo[mi][4 * i + 3], w3, t);
+                }
+            }
+        } else
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             // a masked nibble in a 16-bit half is the fp16 subnormal q * 2^-24 (low nibbles) or 16 q * 2^-24 (high
@@ -211,8 +261,14 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
         const uint32_t p0 = (hdr.y >> sh) & 0xffffu, p1 = (hdr.z >> sh) & 0xffffu, p2 = (hdr.w >> sh) & 0xffffu;
         const uint32_t sc_pair = upper ? ((p2 & 0x0F0Fu) | ((p0 >> 2) & 0x3030u)) : (p0 & 0x3F3Fu);
         const uint32_t mn_pair = upper ? (((p2 >> 4) & 0x0F0Fu) | ((p1 >> 2) & 0x3030u)) : (p1 & 0x3F3Fu);
-        const float d1 = d * ubyte0(sc_pair) * 16777216.0f, d2 = d * ubyte1(sc_pair) * 1048576.0f;  // 2^24, 2^24 / 16
-        const float m1 = dmin * ubyte0(mn_pair), m2 = dmin * ubyte1(mn_pair);
+        float d1 = d * ubyte0(sc_pair) * 16777216.0f, d2 = d * ubyte1(sc_pair) * 1048576.0f;  // 2^24, 2^24 / 16
+        float m1 = dmin * ubyte0(mn_pair), m2 = dmin * ubyte1(mn_pair);
+        if constexpr (HALF) {  // one sub-block per lane: its scale and min; nibbles sit in the low position either way
+            d1 = hn ? d * ubyte1(sc_pair) * 16777216.0f : d1;
+            m1 = hn ? m2 : m1;
+            d2 = 0.0f;
+            m2 = 0.0f;
+        }
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
             float t = d1 * slo[mi];
@@ -321,9 +377,9 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     const int total_streams = (int)wgs * streams;
 #define QMM_GO3(MT_, WPR_, L_, AT_)                                                                                   \
     do {                                                                                                              \
-        hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_>>();                                \
+        hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_, false>>();                         \
         if (e_ != hipSuccess) return e_;                                                                              \
-        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring,   \
+        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_, false><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring, \
                                                                             total_streams, (int)(units / total_streams), \
                                                                             (int)(units % total_streams));           \
     } while (0)
@@ -350,6 +406,97 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     return hipGetLastError();
 }
 
+// Two to four lhs rows with the sub-block-per-lane mapping (HALF): count matrices that share the lhs, K <= 16384; out[j] is
+// fp32 [m, n[j]] (ldo = 0: dense).  Four rows need their activations staged in LDS four times over; where that does not
+// fit (K > 8192 with an fp32 lhs) the rows go in two passes of two.
+hipError_t launch_gemv_q4_k_lanes_rows_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
+                                               float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled) {
+    *handled = false;
+    const int nblk = (int)(k / 256);
+    if (kernel_disabled("q4k_lanes_rows") || m < 2 || m > 4 || k % 256 || nblk > 64 || count < 1 || count > kLanesMaxMats) return hipSuccess;
+    int64_t n = 0;
+    for (int j = 0; j < count; j++) n += ns[j];
+    if (n > 0x7fffffff) return hipSuccess;
+    const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
+    const int wpr = nblk <= 8 ? 1 : nblk <= 16 ? 2 : nblk <= 32 ? 4 : 8;
+    const int bpw = (nblk + wpr - 1) / wpr;  // <= 8
+    const int l = (bpw * 9 + 63) / 64;       // 1 or 2
+    const int ring = 2;
+    const size_t slot = (size_t)bpw * Q4_K_BPB;
+    auto lds_for = [&](int mt) {
+        const size_t act_bytes = (size_t)mt * (((size_t)(k / 64) * (64 * esz + 16) + 1023) / 1024 * 1024);
+        return (size_t)kWaves * ring * slot + (size_t)kWaves * kMaxRows * mt * 4 + act_bytes;
+    };
+    int mt = m <= 2 ? 2 : 4;
+    if (lds_for(mt) > (size_t)kLdsPerCu) mt = 2;
+    if (lds_for(mt) > (size_t)kLdsPerCu) return hipSuccess;
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    const size_t lds = lds_for(mt);
+    const int streams = kWaves / wpr;
+    int64_t wgs = cus;
+    if (wgs * streams > n) wgs = (n + streams - 1) / streams;
+    const int64_t min_wgs = (n + (int64_t)streams * kMaxRows - 1) / ((int64_t)streams * kMaxRows);
+    if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots
+    const dim3 grid((unsigned)wgs), block(64 * kWaves);
+    const int total_streams = (int)wgs * streams;
+    for (int m0 = 0; m0 < m; m0 += mt) {
+        const int rows = std::min(mt, m - m0);
+        LanesMats mats;
+        int64_t end = 0;
+        for (int j = 0; j < kLanesMaxMats; j++) {
+            const int jj = j < count ? j : count - 1;
+            if (j < count) end += ns[j];
+            mats.w[j] = ws[jj];
+            mats.out[j] = outs[jj] + (int64_t)m0 * (ldo ? ldo : ns[jj]);
+            mats.end[j] = (int)end;
+        }
+        mats.count = count;
+        mats.swiglu = 0;
+        mats.out_bf16 = 0;
+        const void* am = (const char*)a + (size_t)m0 * k * esz;
+#define QMM_H3(MT_, WPR_, L_, AT_)                                                                                                  \
+    do {                                                                                                                            \
+        hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_, true>>();                                         \
+        if (e_ != hipSuccess) return e_;                                                                                            \
+        gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_, true><<<grid, block, lds, s>>>(mats, (const AT_*)am, rows, (int)k, ldo, ring,    \
+                                                                                  total_streams, (int)(n / total_streams),         \
+                                                                                  (int)(n % total_streams));                       \
+    } while (0)
+#define QMM_H2(MT_, WPR_, L_)                               \
+    do {                                                    \
+        if (a_dtype == QMM_F32) QMM_H3(MT_, WPR_, L_, float); \
+        else QMM_H3(MT_, WPR_, L_, uint16_t);               \
+    } while (0)
+#define QMM_H1(MT_, WPR_)              \
+    do {                               \
+        if (l == 1) QMM_H2(MT_, WPR_, 1); \
+        else QMM_H2(MT_, WPR_, 2);     \
+    } while (0)
+#define QMM_H0(MT_)                    \
+    do {                               \
+        if (wpr == 1) QMM_H1(MT_, 1);  \
+        else if (wpr == 2) QMM_H1(MT_, 2); \
+        else if (wpr == 4) QMM_H1(MT_, 4); \
+        else QMM_H1(MT_, 8);           \
+    } while (0)
+        if (mt == 2) QMM_H0(2);
+        else QMM_H0(4);
+#undef QMM_H0
+#undef QMM_H1
+#undef QMM_H2
+#undef QMM_H3
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    *handled = true;
+    return hipSuccess;
+}
+
 // The gated-MLP combination as a kernel of its own, for the shapes the fused epilogue above does not take.
 __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
                                                      float* __restrict__ out, int64_t count) {
@@ -364,6 +511,11 @@ hipError_t launch_swiglu(const float* gate, const float* up, float* out, int64_t
     const int64_t blocks = std::min<int64_t>((count + 255) / 256, 4096);
     swiglu_kernel<<<dim3((unsigned)std::max<int64_t>(blocks, 1)), dim3(256), 0, s>>>(gate, up, out, count);
     return hipGetLastError();
+}
+
+hipError_t launch_gemv_q4_k_lanes_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                       int64_t ldo, hipStream_t s, bool* handled) {
+    return launch_gemv_q4_k_lanes_rows_grouped(a, a_dtype, 1, &w, &n, &out, m, k, ldo, s, handled);
 }
 
 hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,

@@ -56,6 +56,19 @@ bool q4k_kc_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     return m >= (lhs_dtype == QMM_F32 ? 9 : 5) && n <= 4096 && k > 4096;
 }
 
+// Q4_K with 2..4 lhs rows: the decode kernel with one sub-block per lane, or the small-batch matrix-core kernel?
+bool q4k_lanes_rows_wins(int64_t n, int64_t k) {
+    // The decode kernel pays per weight (its decode runs on the vector units once per row group), the matrix-core kernel
+    // per K step and per launch.  Measured, 4 fp32 rows, decode kernel / matrix-core kernel: 512 x 4096 5.1 / 6.7 us,
+    // 1024 x 4096 5.2 / 6.7, 2048 x 4096 6.3 / 6.8, 3072 x 4096 7.7 / 6.9, 4096 x 4096 8.9 / 7.0, 14336 x 4096 20.8 / 12.3,
+    // 1024 x 8192 9.9 / 10.6, 1024 x 14336 16.2 / 17.5 (bf16 rows: 10.1 / 17.9), 4096 x 14336 42.9 / 18.0.
+    static const bool forced = [] {
+        const char* e = getenv("QMM_Q4K_LANES_ROWS");
+        return e && e[0] == '1';
+    }();
+    return forced || n <= 1024 || n * k <= ((int64_t)8 << 20);
+}
+
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     const bool f32 = lhs_dtype == QMM_F32;
     const double tiles = (double)((m + 127) / 128) * (double)((n + 255) / 256);
@@ -145,7 +158,7 @@ int static_scratch(void** ws) {
 
 extern "C" {
 
-int qmm_version(void) { return 101; }
+int qmm_version(void) { return 102; }
 
 const char* qmm_last_error(void) { return g_err; }
 
@@ -440,6 +453,14 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         return QMM_OK;
     }
 
+    // 2..4 lhs rows on a small matrix: the decode kernel with one sub-block per lane (the activations of four rows fit a
+    // lane's registers)
+    if (encoding == QMM_Q4_K && m >= 2 && m <= 4 && q4k_lanes_rows_wins(n, k)) {
+        bool handled = false;
+        hipError_t e = qmm::launch_gemv_q4_k_lanes_rows(lhs, lhs_dtype, w, (int)m, n, k, out, n, s, &handled);
+        if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K decode, 2..4 rows)");
+        if (handled) return QMM_OK;
+    }
     // 2..16 lhs rows on few weight rows and long K: the small-batch kernel that cuts K across workgroups
     if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && q4k_kc_wins(lhs_dtype, m, n, k) && qmm::gemv_q4_k_kc_supported(w, k)) {
         bool handled = false;
@@ -535,6 +556,32 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
             hipError_t e = qmm::launch_gemv_q4_k_lanes_grouped(lhs, lhs_dtype, count, ws, n, out, 1, k, 0, (hipStream_t)stream, &handled);
             if (e != hipSuccess) return hip_status(e, "qmm_matmul_grouped(Q4_K decode)");
             if (handled) return QMM_OK;
+        }
+        if (ok && total <= INT32_MAX && m >= 2 && m <= 4) {
+            // Each matrix goes to the kernel qmm_matmul would give it, so a group and separate calls agree bit for bit:
+            // the small ones as one launch of the decode kernel, the others (below) as one of the matrix-core kernel.
+            const uint8_t* small_w[qmm::kLanesMaxMats];
+            int64_t small_n[qmm::kLanesMaxMats];
+            float* small_out[qmm::kLanesMaxMats];
+            int small = 0;
+            for (int j = 0; j < count; j++)
+                if (q4k_lanes_rows_wins(n[j], k)) small_w[small] = ws[j], small_n[small] = n[j], small_out[small++] = out[j];
+            bool handled = false;
+            if (small > 0) {
+                hipError_t e = qmm::launch_gemv_q4_k_lanes_rows_grouped(lhs, lhs_dtype, small, small_w, small_n, small_out, (int)m, k, 0,
+                                                                        (hipStream_t)stream, &handled);
+                if (e != hipSuccess) return hip_status(e, "qmm_matmul_grouped(Q4_K decode, 2..4 rows)");
+            }
+            if (handled) {
+                if (small == count) return QMM_OK;
+                int rest = 0;
+                const void* rest_w[qmm::kLanesMaxMats];
+                int64_t rest_n[qmm::kLanesMaxMats];
+                float* rest_out[qmm::kLanesMaxMats];
+                for (int j = 0; j < count; j++)
+                    if (!q4k_lanes_rows_wins(n[j], k)) rest_w[rest] = rhs[j], rest_n[rest] = n[j], rest_out[rest++] = out[j];
+                return qmm_matmul_grouped(encoding, lhs, lhs_dtype, m, k, rest, rest_w, rest_n, rest_out, workspace, workspace_bytes, stream);
+            }
         }
         if (ok && total <= INT32_MAX && m >= 2 && !qmm::kernel_disabled("q4k_mm")) {
             // the lhs is narrowed once (in the kernel up to 8 rows, by the separate pass beyond) for all the matrices

@@ -11,7 +11,7 @@ namespace qmm {
 
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
-// in the dispatch order serves it.  Names: q4k_lanes, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_rows_v2,
+// in the dispatch order serves it.  Names: q4k_lanes, q4k_lanes_rows, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_rows_v2,
 // q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, gptq_mm, gptq_cols.  Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 
@@ -87,6 +87,11 @@ hipError_t launch_gemv_q4_k_lanes(const void* a, int a_dtype, const uint8_t* w, 
                                   int64_t ldo, hipStream_t s, bool* handled, bool out_bf16 = false);
 // out[i] = bf16(x[i]), i < count: round to nearest even, NaN to the canonical quiet NaN
 hipError_t launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count, hipStream_t s);
+// Two to four lhs rows through the decode kernel with one 32-column sub-block per lane (K <= 16384).
+hipError_t launch_gemv_q4_k_lanes_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
+                                       int64_t ldo, hipStream_t s, bool* handled);
+hipError_t launch_gemv_q4_k_lanes_rows_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
+                                               float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled);
 hipError_t launch_gemv_q4_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s);
 hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
