@@ -319,9 +319,10 @@ def host_cpu():
 def cpu_baseline(layer_w, m: int, budget_s: float = 10.0):
     """Port of the reference CPU path (the oracle's source) on one layer's seven projections, OpenMP over N.
 
-    Timed from a build of that source for this host (-O3 -march=native -ffast-math off, contraction on), made
-    here with `make -C oracle native`; the portable exactness-grade build that the tests check against is the
-    fallback and is named in `sample`.  Threads: the physical cores, capped at this job's share of the host."""
+    Three variants are timed and the fastest is reported (all named in `sample`): the portable exactness-grade build
+    that the tests check against, a build of the same source for this host (-O3 -march=native, contraction on, made
+    here with `make -C oracle native`), and the library's hand-vectorised AVX2 + FMA kernel with the unpack fused into
+    the dot.  Threads: the physical cores, capped at this job's share of the host."""
     import subprocess
 
     import numpy as np
@@ -331,25 +332,30 @@ def cpu_baseline(layer_w, m: int, budget_s: float = 10.0):
     model, phys = host_cpu()
     share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 16  # the job's share of the host's cores
     threads = max(1, min(phys, share, O.num_threads() if O.num_threads() > 0 else share))
-    builds = [("portable build (-march=x86-64-v3, contraction off: the one the tests check against)", O)]
+    port = lambda lib: (lambda a, w: lib.matmul_f32(O.Q4_K, a, w))  # noqa: E731
+    builds = [("portable build (-march=x86-64-v3, contraction off: the one the tests check against)", O, port(O))]
     try:
         subprocess.run(["make", "-s", "-C", os.path.join(ROOT, "oracle"), "native"], check=True, capture_output=True, timeout=120)
-        builds.append(("-O3 -march=native build of the same source", O.native()))
+        nat = O.native()
+        builds.append(("-O3 -march=native build of the same source", nat, port(nat)))
     except Exception as exc:  # no compiler, or a CPU the build does not suit: the portable library still times the port
-        builds[0] = (builds[0][0] + f"; native build unavailable: {type(exc).__name__}", O)
+        builds[0] = (builds[0][0] + f"; native build unavailable: {type(exc).__name__}",) + builds[0][1:]
     rng = np.random.Generator(np.random.PCG64(3))
     host = [(w.cpu().numpy(), n, k) for (w, (_, n, k)) in zip(layer_w, PROJ)]
     acts = {k: rng.standard_normal((m, k), dtype=np.float32) for k in (4096, 14336)}
+    # the hand-vectorised (AVX2 + FMA) fused unpack-and-dot of the same library, where the host has AVX2
+    if O.baseline_matmul_q4_k(acts[4096][:1], host[0][0][:8]) is not None:
+        builds.append(("hand-vectorised AVX2 + FMA kernel (unpack fused into the dot)", O, O.baseline_matmul_q4_k))
     nbytes = sum(alg_bytes(QE.Q4_K, m, n, k) for _, n, k in PROJ)
     results = []
-    for what, lib in builds:  # each build gets its share of the budget; the faster one is the baseline
+    for what, lib, fn in builds:  # each variant gets its share of the budget; the fastest one is the baseline
         lib.set_num_threads(threads)
         for w, n, k in host:  # warm-up pass
-            lib.matmul_f32(O.Q4_K, acts[k], w)
+            fn(acts[k], w)
         passes, t0 = 0, O.now()
         while True:
             for w, n, k in host:
-                lib.matmul_f32(O.Q4_K, acts[k], w)
+                fn(acts[k], w)
             passes += 1
             el = O.now() - t0
             if el > budget_s / len(builds) or passes >= 5000:

@@ -547,12 +547,7 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
     }
     if (tiles > 4 && !kernel_disabled("q4_0_wide")) {
         const size_t wlds = (size_t)kWWaves * kWNT * kWaveLds;
-        static bool wide_set = false;
-        if (!wide_set) {
-            hipError_t e2 = hipFuncSetAttribute((const void*)gemm_q4_0_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wlds);
-            if (e2 != hipSuccess) return e2;
-            wide_set = true;
-        }
+        if (hipError_t e2 = allow_full_lds<gemm_q4_0_wide_kernel>(); e2 != hipSuccess) return e2;
         dim3 grid((unsigned)((n + 16 * kWNT * kWWaves - 1) / (16 * kWNT * kWWaves)), (unsigned)((tiles + kWMG - 1) / kWMG));
         gemm_q4_0_wide_kernel<<<grid, dim3(64 * kWWaves), wlds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n, (int)k);
         return hipGetLastError();

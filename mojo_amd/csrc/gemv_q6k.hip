@@ -565,14 +565,10 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
 #define QMM_Q6K_GO(MT_)                                                                                              \
     do {                                                                                                             \
         if (a_dtype == QMM_F32) {                                                                                    \
-            if (lds > 64 * 1024)                                                                                     \
-                (void)hipFuncSetAttribute((const void*)gemv_q6_k_rows_kernel<MT_, float>,                            \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+            if (lds > 64 * 1024) (void)allow_full_lds<gemv_q6_k_rows_kernel<MT_, float>>();                          \
             gemv_q6_k_rows_kernel<MT_, float><<<grid, block, lds, s>>>(w, (const float*)a, out, m, (int)n, (int)k, ldo); \
         } else {                                                                                                     \
-            if (lds > 64 * 1024)                                                                                     \
-                (void)hipFuncSetAttribute((const void*)gemv_q6_k_rows_kernel<MT_, uint16_t>,                         \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
+            if (lds > 64 * 1024) (void)allow_full_lds<gemv_q6_k_rows_kernel<MT_, uint16_t>>();                       \
             gemv_q6_k_rows_kernel<MT_, uint16_t><<<grid, block, lds, s>>>(w, (const uint16_t*)a, out, m, (int)n,     \
                                                                          (int)k, ldo);                               \
         }                                                                                                            \

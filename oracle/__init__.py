@@ -256,6 +256,17 @@ def matmul_f32(enc: int, a, w, w_bf16: bool = False) -> np.ndarray:
     return out
 
 
+def baseline_matmul_q4_k(a, w, _lib=None):
+    """The hand-vectorised (AVX2) Q4_K x fp32 product that ``bench.py`` times as the CPU baseline; None where the host
+    lacks AVX2.  Agrees with matmul_f32 to rounding only (another summation order): never used as a checker."""
+    a, m, k = _rows_k(a)
+    w = _c(w, np.uint8)
+    n = w.shape[0]
+    out = np.empty((m, n), np.float32)
+    rc = (_lib or lib()).qo_baseline_matmul_q4_k(_p(a), _p(w), _i64(m), _i64(n), _i64(k), _p(out))
+    return out if rc == 0 else None
+
+
 def matmul_f64(enc: int, a, w, w_bf16: bool = False) -> np.ndarray:
     a, m, k = _rows_k(a)
     w = _c(w, np.uint8)
@@ -316,6 +327,9 @@ class _Native:
         rc = self._lib.qo_matmul_f32(C.c_int(enc), _p(a), _p(w), _i64(m), _i64(n), _i64(k), C.c_int(0), _p(out))
         assert rc == 0
         return out
+
+    def baseline_matmul_q4_k(self, a, w):
+        return baseline_matmul_q4_k(a, w, self._lib)
 
 
 def native() -> _Native:

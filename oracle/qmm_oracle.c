@@ -36,6 +36,9 @@
  *                                     int64, extreme vectors
  *   qo_matmul_* outputs               pinned: fp64 truth, closed-form special
  *                                     cases (one-hot, constant-code blocks)
+ *   qo_baseline_matmul_q4_k           timed baseline only, never a checker: held
+ *                                     to the matmul tolerance against
+ *                                     qo_matmul_f32 and the fp64 truth
  *   qo_quantize_q4_0 / qo_quantize_q8_0
  *                                     closed form pinned by properties (argmax
  *                                     -> code 0 / +-127, error bound, ties);
@@ -921,6 +924,70 @@ int qo_matmul_f32(int enc, const float* a, const uint8_t* w, int64_t m, int64_t 
     }
     return 0;
 }
+
+/* The timed CPU baseline for Q4_K with fp32 activations, hand-vectorised (AVX2 + FMA, the ISA class an x86 host of
+ * the reference dispatches on: stdlib/src/sys/info.mojo:97-162), rows of N split across threads
+ * (examples/matmul.mojo:126-141).  NOT a checker: it sums in a different order from qo_matmul_f32
+ * (sum_k a*q per sub-block first, then (d*sc) * that - (dmin*mn) * sum_k a), so it agrees with it to rounding only;
+ * the unit tests hold it to the matmul tolerance against qo_matmul_f32.  Returns -1 where the host lacks AVX2. */
+#if defined(__AVX2__) && defined(__FMA__)
+#include <immintrin.h>
+static inline float hsum8(__m256 v) {
+    __m128 s = _mm_add_ps(_mm256_castps256_ps128(v), _mm256_extractf128_ps(v, 1));
+    s = _mm_add_ps(s, _mm_movehl_ps(s, s));
+    s = _mm_add_ss(s, _mm_movehdup_ps(s));
+    return _mm_cvtss_f32(s);
+}
+int qo_baseline_matmul_q4_k(const float* a, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out) {
+    if (k % 256) return -1;
+    const int64_t nb = k / 256, nsub = k / 32;
+    float* asum = (float*)malloc(sizeof(float) * (size_t)(m * nsub));
+    for (int64_t i = 0; i < m; i++)
+        for (int64_t sb = 0; sb < nsub; sb++) {
+            const float* p = a + i * k + sb * 32;
+            __m256 t = _mm256_add_ps(_mm256_add_ps(_mm256_loadu_ps(p), _mm256_loadu_ps(p + 8)),
+                                     _mm256_add_ps(_mm256_loadu_ps(p + 16), _mm256_loadu_ps(p + 24)));
+            asum[i * nsub + sb] = hsum8(t);
+        }
+    const __m256i lo4 = _mm256_set1_epi32(0xF);
+#pragma omp parallel for schedule(static)
+    for (int64_t j = 0; j < n; j++) {
+        for (int64_t i = 0; i < m; i++) {
+            const float* ar = a + i * k;
+            const float* as = asum + i * nsub;
+            __m256 acc = _mm256_setzero_ps();
+            float macc = 0.0f;
+            for (int64_t b = 0; b < nb; b++) {
+                const uint8_t* blk = w + (j * nb + b) * 144;
+                const float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+                uint8_t sc[8], mn[8];
+                qo_unpack_scales_q4_k(blk + 4, sc, mn);
+                for (int c = 0; c < 4; c++) {
+                    const uint8_t* qs = blk + 16 + 32 * c;
+                    const float* x = ar + b * 256 + 64 * c;
+                    __m256 tl = _mm256_setzero_ps(), th = _mm256_setzero_ps();
+                    for (int g = 0; g < 4; g++) {  /* 8 code bytes: 8 weights of sub-block 2c (low nibbles), 8 of 2c + 1 */
+                        const __m256i q = _mm256_cvtepu8_epi32(_mm_loadl_epi64((const __m128i*)(qs + 8 * g)));
+                        tl = _mm256_fmadd_ps(_mm256_cvtepi32_ps(_mm256_and_si256(q, lo4)), _mm256_loadu_ps(x + 8 * g), tl);
+                        th = _mm256_fmadd_ps(_mm256_cvtepi32_ps(_mm256_srli_epi32(q, 4)), _mm256_loadu_ps(x + 32 + 8 * g), th);
+                    }
+                    acc = _mm256_fmadd_ps(_mm256_set1_ps(d * (float)sc[2 * c]), tl, acc);
+                    acc = _mm256_fmadd_ps(_mm256_set1_ps(d * (float)sc[2 * c + 1]), th, acc);
+                    macc += dmin * (float)mn[2 * c] * as[b * 8 + 2 * c] + dmin * (float)mn[2 * c + 1] * as[b * 8 + 2 * c + 1];
+                }
+            }
+            out[i * n + j] = hsum8(acc) - macc;
+        }
+    }
+    free(asum);
+    return 0;
+}
+#else
+int qo_baseline_matmul_q4_k(const float* a, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out) {
+    (void)a; (void)w; (void)m; (void)n; (void)k; (void)out;
+    return -1;
+}
+#endif
 
 int qo_matmul_f64(int enc, const float* a, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                   int w_bf16, double* out) {

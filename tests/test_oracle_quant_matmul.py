@@ -208,3 +208,19 @@ def test_rmsnorm_closed_forms_and_restatement():
     assert np.array_equal(O.rmsnorm(x, gamma, eps, to_bf16=True), O.bf16_to_f32(O.f32_to_bf16(O.rmsnorm(x, gamma, eps))))
     # a larger eps can only shrink the result
     assert np.all(np.abs(O.rmsnorm(x, gamma, 1.0)) <= np.abs(y0))
+
+
+def test_timed_cpu_baseline_kernel_agrees_with_the_checker():
+    """The hand-vectorised Q4_K kernel that the benchmark times sums in another order than matmul_f32: it is held to the
+    matmul tolerance (rtol 1e-3, atol 1e-4, symmetric) against it and against the fp64 truth, never used as a checker."""
+    rng = np.random.default_rng(11)
+    for m, n, k in ((1, 70, 4096), (3, 33, 14336), (2, 9, 256)):
+        w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+        wq = O.quantize(O.Q4_K, w)
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        got = O.baseline_matmul_q4_k(a, wq)
+        if got is None:
+            pytest.skip("host without AVX2")
+        for want in (O.matmul_f32(O.Q4_K, a, wq), O.matmul_f64(O.Q4_K, a, wq).astype(np.float32)):
+            tol = np.maximum(1e-3 * np.maximum(np.abs(got), np.abs(want)), 1e-4)
+            assert (np.abs(got - want) <= tol).all()
