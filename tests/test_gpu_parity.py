@@ -568,6 +568,7 @@ def test_q8_k_activations_only_for_k_quants():
 @pytest.mark.parametrize("enc,m,k,ns,lhs_bf16", [(QE.Q4_K, 1, 4096, (512, 130, 130), False), (QE.Q4_K, 1, 14336, (300, 77), True),
                                                  (QE.Q4_K, 1, 512, (9000, 1, 17, 4100), False),
                                                  (QE.Q4_K, 3, 1024, (64, 200), False), (QE.Q4_K, 4, 4096, (4100, 130, 130), False),
+                                                 (QE.Q4_K, 4, 14336, (300, 77), False), (QE.Q4_K, 2, 8192, (1024, 1500, 40), True),
                                                  (QE.Q4_K, 8, 2304, (20, 33, 7, 50), True), (QE.Q4_K, 12, 512, (300, 17), False),
                                                  (QE.Q6_K, 1, 1024, (96, 40), False),
                                                  (QE.Q4_0, 2, 256, (33, 64, 5), False), (QE.Q4_K, 1, 256, (8, 8, 8, 8, 8), False)])
@@ -862,6 +863,27 @@ def test_q6_k_decode_vocabulary_shapes(m, n, k, lhs_bf16):
     got = qmatmul(QE.Q6_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
     assert_close(got, want, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp32 oracle")
     assert_close(got, truth, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp64 truth")
+
+
+@pytest.mark.parametrize("m,n,lhs_bf16", [(2, 16, False), (3, 33, True), (4, 1000, False), (5, 4099, True), (8, 250, False),
+                                          (9, 47, False), (16, 530, True), (12, 9000, False), (20, 300, False), (40, 130, True),
+                                          (64, 72, False)])
+def test_q6_k_small_batch_matrix_core_kernel(m, n, lhs_bf16):
+    """Q6_K with 2..64 lhs rows on K = 4096: weight rows decoded once for all lhs rows (codes as exact fp16 integers, one
+    matrix-core instruction per 16-weight scale group and set of eight lhs rows); the 2, 4, 8 and 16 row variants, further
+    passes from 17 rows on, tiles that end past the matrix, more tiles than workgroups.  Rows of very different
+    magnitude share a pass (the lhs is scaled per row)."""
+    w, a = synth(43, n, 4096, m)
+    a[m - 1] *= 1000.0
+    a[0, :512] *= 1e-3
+    if lhs_bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q6_K, w)
+    want = O.matmul_f32(O.Q6_K, a, wq)
+    truth = O.matmul_f64(O.Q6_K, a, wq)
+    got = qmatmul(QE.Q6_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
+    assert_close(got, want, f"Q6_K {m}x{n}x4096 bf16={lhs_bf16} vs fp32 oracle")
+    assert_close(got, truth, f"Q6_K {m}x{n}x4096 bf16={lhs_bf16} vs fp64 truth")
 
 
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(200, 300, 1024, False), (64, 130, 4096, True), (17, 16, 96, False),
