@@ -651,6 +651,13 @@ def extra_timings(layers, acts, gen):
     dev_s, _ = time_graphs([g], 20, 3)
     b = alg_bytes(QE.Q6_K, 1, 128256, 4096)
     out["q6_k_lm_head"] = {"us": round(dev_s * 1e6 / 20, 2), "GB/s": round(b * 20 / dev_s / 1e9, 1)}
+    # ... and with 4 and 16 lhs rows (the small-batch matrix-core kernel: one pass over the weights for up to 16 rows)
+    for mm in (4, 16):
+        am = torch.randn((mm, 4096), dtype=torch.float32, device="cuda:0", generator=gen)
+        g = capture([Gemv(QE.Q6_K, w6, am)])
+        dev_s, _ = time_graphs([g], 10, 3)
+        b = alg_bytes(QE.Q6_K, mm, 128256, 4096)
+        out[f"q6_k_lm_head_m{mm}"] = {"us": round(dev_s * 1e6 / 10, 2), "GB/s": round(b * 10 / dev_s / 1e9, 1)}
     del w6
     # cfg5: Q4_K prefill, bf16 lhs [2048, 4096] x [14336, 4096]
     ab = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
