@@ -1,5 +1,5 @@
-// Q6_K with up to 8 lhs rows a pass (16 in two passes) on the matrix cores, K = 4096: the weight rows are decoded once
-// for all lhs rows, and the per-16 int8 scales are applied to a 16 x 16 block of results at a time.
+// Q6_K with up to 16 lhs rows a pass on the matrix cores, K a multiple of 2048 up to 16384: the weight rows are decoded
+// once for all lhs rows of a pass, and the per-16 int8 scales are applied to a 16 x 16 block of results at a time.
 //
 // Arithmetic.  A Q6_K weight is d * sc * q with q = (ql nibble | qh bits << 4) - 32 and sc an int8 per 16 weights.  The
 // matrix-core operand of a weight is q itself as fp16: a byte permute interleaves the nibble bytes with bytes that hold
@@ -13,7 +13,8 @@
 //
 // Shape of the work.  A workgroup of 8 wavefronts owns 16-row tiles t = block, block + grid, ...; wavefront w owns
 // super-blocks 2 w and 2 w + 1 of every row (K = 4096: 16 super-blocks) and keeps the lhs operands of those 512 columns
-// in registers for the whole kernel.  The 420 bytes of its super-blocks of each of the 16 rows travel global -> LDS
+// in registers for all its tiles.  Longer rows go in rounds of 16 super-blocks: operands converted again, all tiles
+// again, results added to the output of the round before (the same thread stored it).  The 420 bytes of its super-blocks of each of the 16 rows travel global -> LDS
 // directly as 27 aligned 16-byte pieces per row (a row of 3360 bytes and 420 w both are multiples of 4 past a 16-byte
 // boundary, so fields keep a compile-time byte parity and the row stride of 432 bytes spreads 16 rows over all banks)
 // into a private ring of two slots, one tile ahead.  Per tile the wavefronts' partial results meet in LDS (two
@@ -86,7 +87,8 @@ __device__ __forceinline__ void stream16_to_lds(uint32_t lane_offset, const void
 // MROWS: lhs rows of the pass, 1, 2, 4, 8 or 16 (>= m; rows past m are zero operands and their results are dropped).  Sixteen
 // rows are two sets of eight, each with its own operands and sums, multiplied with the same decoded weights.
 // Accumulator registers that hold no wanted lhs row are not computed: a lane holds rows 4 (lane / 16) + r of a set.
-template <int MROWS, typename AT>
+// ROUNDS: K beyond 4096 (or 2048), walked in rounds of 16 super-blocks; without it everything about rounds is constant.
+template <int MROWS, typename AT, bool ROUNDS>
 __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
                                                                    float* __restrict__ out, int m, int n, int k, int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -95,14 +97,15 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
     const int nn = lane & 15, kg = lane >> 4;
     constexpr int SETS = MROWS > 8 ? 2 : 1, MR1 = MROWS > 8 ? 8 : MROWS;  // sets of lhs rows, rows of a set
     constexpr int RN = MR1 < 4 ? MR1 : 4;  // accumulator registers in use per set
-    const int64_t row_bytes = (int64_t)(k >> 8) * Q6_K_BPB;  // 3360
+    const int nblk = k >> 8;                                  // a multiple of 8: rows are whole 16-byte pieces
+    const int64_t row_bytes = (int64_t)nblk * Q6_K_BPB;
     uint8_t* ring = smem + wave * (kQSlots * kQSlot);
     const uint32_t ring_lds = lds_address(ring);
     float* red = (float*)(smem + kQRing);  // [2][kQWaves][2 sets][4][64]
     const int ntiles = (n + 15) >> 4;
     const int my_tiles = (int)blockIdx.x < ntiles ? (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
-    const int part = 2 * wave * Q6_K_BPB;  // first byte of this wavefront's super-blocks in a row
-    const int lead = part & 15;            // 0, 4, 8 or 12
+    const int lead = (2 * wave * Q6_K_BPB) & 15;  // of this wavefront's super-blocks past a 16-byte boundary: 0, 4, 8 or 12
+                                                  // (the same in every round: 16 super-blocks are 3360 bytes)
 
     // piece p = lane + 64 i of an item: row p / 27, piece p % 27 of the row's aligned range
     uint32_t full[kQLoads];  // byte offset of the piece in a tile that lies inside the matrix
@@ -111,9 +114,9 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
         const int p = min(lane + 64 * i, kQPieces - 1), pr = p / kQRowPieces;
         full[i] = (uint32_t)pr * (uint32_t)row_bytes + (uint32_t)((p - pr * kQRowPieces) * 16);
     }
-    auto issue = [&](int ti, int slot) {
+    auto issue = [&](int round, int ti, int slot) {
         const int n0 = ((int)blockIdx.x + ti * (int)gridDim.x) * 16;
-        const uint8_t* base = w + (int64_t)n0 * row_bytes + (part - lead);
+        const uint8_t* base = w + (int64_t)n0 * row_bytes + ((16 * round + 2 * wave) * Q6_K_BPB - lead);
         const int last = n - 1 - n0;  // rows past the matrix repeat its last row (their results are dropped)
 #pragma unroll
         for (int i = 0; i < kQLoads; i++) {
@@ -125,17 +128,30 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
             if (i < kQLoads - 1 || lane < kQPieces - 64 * (kQLoads - 1)) stream16_to_lds(off, base, ring_lds + slot * kQSlot + i * 1024);
         }
     };
-    if (my_tiles > 0) issue(0, 0);
+    // (constants of the unpack in vector registers: an and-or in one instruction takes no literal and one scalar at most)
+    uint32_t m03 = 0x03030303u, c54 = 0x54545454u;
+    asm volatile("" : "+v"(m03), "+v"(c54));
+    const float4v zero4 = {0.f, 0.f, 0.f, 0.f};
+    const half4v off96 = {(_Float16)96.0f, (_Float16)96.0f, (_Float16)96.0f, (_Float16)96.0f};
+    float* stg = (float*)(smem + kQRing + kQRed) + 16 * wave;  // this wavefront's inverse lhs scales
+    int it = 0;  // tiles done, over all rounds: its parity picks the buffer of the partial results
+
+    // K in rounds of 16 super-blocks (4096 columns); a last round of 8 keeps wavefronts 0..3 busy.  Results of the rounds
+    // after the first are added to what the same thread stored before.
+    const int rounds = ROUNDS ? (nblk + 15) >> 4 : 1;
+    for (int round = 0; round < rounds; round++) {
+    const bool have = ROUNDS ? 16 * round + 2 * wave < nblk : true;            // this wavefront has super-blocks in the round
+    const int nw = ROUNDS ? min(kQWaves, (nblk - 16 * round) >> 1) : kQWaves;  // wavefronts that have
+    if (have && my_tiles > 0) issue(round, 0, 0);
 
     // ---- the lhs operands of this wavefront's 512 columns.  Operand row nn of set st: lhs row 8 st + nn % 8, hi part (nn < 8)
     // or residual.  The inverse scales go to LDS and are read back where a tile's sums are finished.
     half4v fa[SETS][2][16];
-    float* stg = (float*)(smem + kQRing + kQRed) + 16 * wave;  // this wavefront's inverse scales
 #pragma unroll
     for (int st = 0; st < SETS; st++) {
         const int lrow = 8 * st + (nn & 7);
         const bool live = lrow < m;
-        const AT* ar = a + (int64_t)min(lrow, m - 1) * k + 512 * wave + 4 * kg;
+        const AT* ar = a + (int64_t)min(lrow, m - 1) * k + min(4096 * round + 512 * wave, k - 512) + 4 * kg;
         // One set: all 32 loads of the lane go out together (one round trip) and the values stay in registers for the
         // conversion.  Two sets: 16 at a time, and a second round of loads for the conversion (the first set's operands
         // take 64 registers already).
@@ -178,15 +194,10 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
     }
     __builtin_amdgcn_wave_barrier();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    // (constants of the unpack in vector registers: an and-or in one instruction takes no literal and one scalar at most)
-    uint32_t m03 = 0x03030303u, c54 = 0x54545454u;
-    asm volatile("" : "+v"(m03), "+v"(c54));
-    const float4v zero4 = {0.f, 0.f, 0.f, 0.f};
-    const half4v off96 = {(_Float16)96.0f, (_Float16)96.0f, (_Float16)96.0f, (_Float16)96.0f};
-    for (int ti = 0; ti < my_tiles; ti++) {
+    for (int ti = 0; ti < my_tiles; ti++, it++) {
         const int slot = ti & 1;
-        if (ti + 1 < my_tiles) {
-            issue(ti + 1, slot ^ 1);
+        if (have && ti + 1 < my_tiles) {
+            issue(round, ti + 1, slot ^ 1);
             wait_vmcnt<kQLoads>();
         } else {
             wait_vmcnt<0>();
@@ -197,6 +208,7 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
         for (int st = 0; st < SETS; st++)
 #pragma unroll
             for (int r = 0; r < RN; r++) acc[st][r] = 0.0f;
+        if (have) {
 #pragma unroll
         for (int bb = 0; bb < 2; bb++) {
             constexpr int kBlockDw[2] = {0, (Q6_K_BPB) >> 2};  // dword of the super-block's first aligned byte: 0, 52
@@ -242,8 +254,10 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
 #pragma unroll
                 for (int r = 0; r < RN; r++) acc[st][r] = fmaf(d, u[st][r], acc[st][r]);
         }
+        }
         // partial result of the tile: lane (column nn, operand rows 4 kg + r), lhs scale undone
-        float* mine = red + ((slot * kQWaves + wave) * 8) * 64 + lane;
+        const int buf = it & 1;
+        float* mine = red + ((buf * kQWaves + wave) * 8) * 64 + lane;
 #pragma unroll
         for (int st = 0; st < SETS; st++)
 #pragma unroll
@@ -252,20 +266,25 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
         if (tid < MROWS * 16) {
             const int row = tid >> 4, col = tid & 15;  // lhs row, column of the tile
             const int n0 = ((int)blockIdx.x + ti * (int)gridDim.x) * 16;
-            const float* src = red + (slot * kQWaves * 8 + 4 * (row >> 3) + (row & 3)) * 64 + col + 16 * ((row & 7) >> 2);
+            const float* src = red + (buf * kQWaves * 8 + 4 * (row >> 3) + (row & 3)) * 64 + col + 16 * ((row & 7) >> 2);
             float v = 0.0f;
 #pragma unroll
-            for (int ww = 0; ww < kQWaves; ww++) v += src[ww * 512] + src[ww * 512 + 32];  // hi rows, residual rows (8 further)
-            if (row < m && n0 + col < n) out[(int64_t)row * ldo + n0 + col] = v;
+            for (int ww = 0; ww < kQWaves; ww++)
+                if (ww < nw) v += src[ww * 512] + src[ww * 512 + 32];  // hi rows, residual rows (8 further)
+            if (row < m && n0 + col < n) {
+                float* o = out + (int64_t)row * ldo + n0 + col;
+                *o = ROUNDS && round ? *o + v : v;
+            }
         }
+    }
     }
 }
 
 bool gemv_q6_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k) {
-    return !kernel_disabled("q6k_mm") && m >= 1 && m <= 64 && k == 4096 && n >= 1 && n <= 0x7fffffff && ((uintptr_t)w & 15) == 0;
+    return !kernel_disabled("q6k_mm") && m >= 1 && m <= 64 && k >= 2048 && k % 2048 == 0 && k <= 16384 && n >= 1 && n <= 0x7fffffff && ((uintptr_t)w & 15) == 0;
 }
 
-// Any number of lhs rows in passes of 16; out is fp32 [m, ldo].  The caller checks gemv_q6_k_mm_supported.
+// Any number of lhs rows in passes of 16 (K = 4096) or 8; out is fp32 [m, ldo].  The caller checks gemv_q6_k_mm_supported.
 hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
                                hipStream_t s) {
     static int cus = 0;
@@ -277,15 +296,24 @@ hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int
     const int64_t ntiles = (n + 15) / 16;
     const dim3 grid((unsigned)std::min<int64_t>(ntiles, cus)), block(64 * kQWaves);
     const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
-    for (int m0 = 0; m0 < m; m0 += 16) {
-        const int rows = std::min(16, m - m0);
+    // (K in rounds: the sixteen-row variant spills in its loop there, two passes of eight rows are faster: 4096 x 14336,
+    // 16 rows: 98 against 112 us)
+    const int pass = k == 4096 ? 16 : 8;
+    for (int m0 = 0; m0 < m; m0 += pass) {
+        const int rows = std::min(pass, m - m0);
         const void* am = (const char*)a + (size_t)m0 * k * esz;
         float* om = out + (int64_t)m0 * ldo;
 #define QMM_Q6MM(MR_, AT_)                                                                                          \
     do {                                                                                                            \
-        hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_>>();                                            \
-        if (e_ != hipSuccess) return e_;                                                                            \
-        gemv_q6_k_mm_kernel<MR_, AT_><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+        if (k == 4096) {                                                                                            \
+            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, false>>();                                 \
+            if (e_ != hipSuccess) return e_;                                                                        \
+            gemv_q6_k_mm_kernel<MR_, AT_, false><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+        } else {                                                                                                    \
+            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, true>>();                                  \
+            if (e_ != hipSuccess) return e_;                                                                        \
+            gemv_q6_k_mm_kernel<MR_, AT_, true><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+        }                                                                                                           \
     } while (0)
 #define QMM_Q6MM_AT(MR_)                               \
     do {                                               \

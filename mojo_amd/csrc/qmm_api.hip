@@ -69,12 +69,14 @@ bool q4k_lanes_rows_wins(int64_t n, int64_t k) {
     return forced || n <= 1024 || n * k <= ((int64_t)8 << 20);
 }
 
-// Q6_K on K = 4096: the small-batch matrix-core kernel, or passes of the decode kernel (one or two lhs rows each)?
+// Q6_K (K a multiple of 2048 up to 16384): the small-batch matrix-core kernel, or passes of the decode kernel (one or two
+// lhs rows each)?
 bool q6k_mm_wanted(int64_t m, int64_t n) {
     // Measured, small-batch kernel / decode-kernel passes, fp32 lhs: 128256 rows: 1 lhs row 87 / 78 us, 2 87 / 113, 4 95 / 225,
     // 8 98 / 449, 16 144 / 895; 14336 rows: 1 17.0 / 14.8, 2 17.5 / 20.6, 4 19.5 / 40.8, 8 21.6 / 81.7, 16 46.7 / 162;
     // 4096 rows: 2 10.3 / 9.6, 4 11.7 / 15.2, 8 13.8 / 32.9, 16 36 / 52; 1024 rows: 2 9.8 / 6.1, 4 11.2 / 7.7, 8 13.2 / 21.9,
-    // 16 29 / 38.  (Its fixed cost is the conversion of the lhs in every workgroup.)  QMM_Q6K_MM=1 sends every shape there.
+    // 16 29 / 38; 4096 x 14336 (four rounds over K): 2 33 / 24, 4 39 / 47, 8 49 / 93, 16 98 / 186.  (Its fixed cost is the
+    // conversion of the lhs in every workgroup and round.)  QMM_Q6K_MM=1 sends every shape there.
     static const bool forced = [] {
         const char* e = getenv("QMM_Q6K_MM");
         return e && e[0] == '1';
@@ -487,7 +489,7 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     if (encoding == QMM_Q4_K && m > 16)
         return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");
 
-    // Q6_K with 2..64 lhs rows on K = 4096: the small-batch matrix-core kernel (passes of 16 rows)
+    // Q6_K with 2..64 lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
     if (encoding == QMM_Q6_K && q6k_mm_wanted(m, n) && qmm::gemv_q6_k_mm_supported(w, m, n, k))
         return hip_status(qmm::launch_gemv_q6_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, s), "qmm_matmul(Q6_K small batch)");
 

@@ -865,15 +865,18 @@ def test_q6_k_decode_vocabulary_shapes(m, n, k, lhs_bf16):
     assert_close(got, truth, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp64 truth")
 
 
-@pytest.mark.parametrize("m,n,lhs_bf16", [(2, 16, False), (3, 33, True), (4, 1000, False), (5, 4099, True), (8, 250, False),
-                                          (9, 47, False), (16, 530, True), (12, 9000, False), (20, 300, False), (40, 130, True),
-                                          (64, 72, False)])
-def test_q6_k_small_batch_matrix_core_kernel(m, n, lhs_bf16):
+@pytest.mark.parametrize("m,n,k,lhs_bf16", [(2, 16, 4096, False), (3, 33, 4096, True), (4, 1000, 4096, False), (5, 4099, 4096, True),
+                                            (8, 250, 4096, False), (9, 47, 4096, False), (16, 530, 4096, True), (12, 9000, 4096, False),
+                                            (20, 300, 4096, False), (40, 130, 4096, True), (64, 72, 4096, False),
+                                            (4, 300, 14336, False), (8, 130, 8192, True), (5, 2100, 2048, False),
+                                            (16, 77, 6144, False), (6, 40, 16384, True)])
+def test_q6_k_small_batch_matrix_core_kernel(m, n, k, lhs_bf16):
     """Q6_K with 2..64 lhs rows on K = 4096: weight rows decoded once for all lhs rows (codes as exact fp16 integers, one
     matrix-core instruction per 16-weight scale group and set of eight lhs rows); the 2, 4, 8 and 16 row variants, further
-    passes from 17 rows on, tiles that end past the matrix, more tiles than workgroups.  Rows of very different
-    magnitude share a pass (the lhs is scaled per row)."""
-    w, a = synth(43, n, 4096, m)
+    passes from 17 rows on, tiles that end past the matrix, more tiles than workgroups; K in rounds of 4096 columns whose
+    results add up in the output (a last round of 2048 with half the wavefronts).  Rows of very different magnitude share
+    a pass (the lhs is scaled per row)."""
+    w, a = synth(43, n, k, m)
     a[m - 1] *= 1000.0
     a[0, :512] *= 1e-3
     if lhs_bf16:
@@ -882,8 +885,8 @@ def test_q6_k_small_batch_matrix_core_kernel(m, n, lhs_bf16):
     want = O.matmul_f32(O.Q6_K, a, wq)
     truth = O.matmul_f64(O.Q6_K, a, wq)
     got = qmatmul(QE.Q6_K, None, gpu(a).to(torch.bfloat16) if lhs_bf16 else gpu(a), gpu(wq))
-    assert_close(got, want, f"Q6_K {m}x{n}x4096 bf16={lhs_bf16} vs fp32 oracle")
-    assert_close(got, truth, f"Q6_K {m}x{n}x4096 bf16={lhs_bf16} vs fp64 truth")
+    assert_close(got, want, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp32 oracle")
+    assert_close(got, truth, f"Q6_K {m}x{n}x{k} bf16={lhs_bf16} vs fp64 truth")
 
 
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(200, 300, 1024, False), (64, 130, 4096, True), (17, 16, 96, False),
