@@ -95,7 +95,10 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nn = lane & 15, kg = lane >> 4;
-    constexpr int SETS = MROWS > 8 ? 2 : 1, MR1 = MROWS > 8 ? 8 : MROWS;  // sets of lhs rows, rows of a set
+    // Sixteen bf16 lhs rows need no residual rows (a bf16 value scaled by a power of two is an fp16 number, down to what is
+    // 2^-26 of its row's largest: far below the fp32 sums' resolution): all sixteen operand rows carry hi parts, one set.
+    constexpr bool HI16 = MROWS == 16 && sizeof(AT) == 2;
+    constexpr int SETS = MROWS > 8 && !HI16 ? 2 : 1, MR1 = MROWS > 8 ? 8 : MROWS;  // sets of lhs rows, rows of a set
     constexpr int RN = MR1 < 4 ? MR1 : 4;  // accumulator registers in use per set
     const int nblk = k >> 8;                                  // a multiple of 8: rows are whole 16-byte pieces
     const int64_t row_bytes = (int64_t)nblk * Q6_K_BPB;
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
     half4v fa[SETS][2][16];
 #pragma unroll
     for (int st = 0; st < SETS; st++) {
-        const int lrow = 8 * st + (nn & 7);
+        const int lrow = HI16 ? nn : 8 * st + (nn & 7);
         const bool live = lrow < m;
         const AT* ar = a + (int64_t)min(lrow, m - 1) * k + min(4096 * round + 512 * wave, k - 512) + 4 * kg;
         // One set: all 32 loads of the lane go out together (one round trip) and the values stay in registers for the
@@ -187,10 +190,10 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
                 // hi: the value cut to fp16 (toward zero); the residual x - hi is exact in fp32 and is cut the same way
                 const fp16x2v h01 = __builtin_amdgcn_cvt_pkrtz(x.x, x.y), h23 = __builtin_amdgcn_cvt_pkrtz(x.z, x.w);
                 const uint32_t r01 = pkrtz(x.x - (float)h01.x, x.y - (float)h01.y), r23 = pkrtz(x.z - (float)h23.x, x.w - (float)h23.y);
-                fa[st][g >> 4][g & 15] = nn < 8 ? as_half4(__builtin_bit_cast(uint32_t, h01), __builtin_bit_cast(uint32_t, h23)) : as_half4(r01, r23);
+                fa[st][g >> 4][g & 15] = HI16 || nn < 8 ? as_half4(__builtin_bit_cast(uint32_t, h01), __builtin_bit_cast(uint32_t, h23)) : as_half4(r01, r23);
             }
         }
-        if (kg == 0 && nn < 8) stg[8 * st + nn] = isc;
+        if (kg == 0 && (HI16 || nn < 8)) stg[8 * st + nn] = isc;
     }
     __builtin_amdgcn_wave_barrier();
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -261,16 +264,17 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
 #pragma unroll
         for (int st = 0; st < SETS; st++)
 #pragma unroll
-            for (int r = 0; r < RN; r++) mine[(4 * st + r) * 64] = acc[st][r] * stg[8 * st + ((4 * kg + r) & 7)];
+            for (int r = 0; r < RN; r++) mine[(4 * st + r) * 64] = acc[st][r] * stg[HI16 ? 4 * kg + r : 8 * st + ((4 * kg + r) & 7)];
         __syncthreads();
         if (tid < MROWS * 16) {
             const int row = tid >> 4, col = tid & 15;  // lhs row, column of the tile
             const int n0 = ((int)blockIdx.x + ti * (int)gridDim.x) * 16;
-            const float* src = red + (buf * kQWaves * 8 + 4 * (row >> 3) + (row & 3)) * 64 + col + 16 * ((row & 7) >> 2);
+            const float* src = HI16 ? red + (buf * kQWaves * 8 + (row & 3)) * 64 + col + 16 * (row >> 2)
+                                    : red + (buf * kQWaves * 8 + 4 * (row >> 3) + (row & 3)) * 64 + col + 16 * ((row & 7) >> 2);
             float v = 0.0f;
 #pragma unroll
             for (int ww = 0; ww < kQWaves; ww++)
-                if (ww < nw) v += src[ww * 512] + src[ww * 512 + 32];  // hi rows, residual rows (8 further)
+                if (ww < nw) v += HI16 ? src[ww * 512] : src[ww * 512 + 0] + src[ww * 512 + 32];  // hi rows, residual rows (8 further)
             if (row < m && n0 + col < n) {
                 float* o = out + (int64_t)row * ldo + n0 + col;
                 *o = ROUNDS && round ? *o + v : v;
@@ -296,9 +300,9 @@ hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int
     const int64_t ntiles = (n + 15) / 16;
     const dim3 grid((unsigned)std::min<int64_t>(ntiles, cus)), block(64 * kQWaves);
     const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
-    // (K in rounds: the sixteen-row variant spills in its loop there, two passes of eight rows are faster: 4096 x 14336,
-    // 16 rows: 98 against 112 us)
-    const int pass = k == 4096 ? 16 : 8;
+    // (K in rounds: the sixteen-row fp32 variant spills in its loop there, two passes of eight rows are faster: 4096 x 14336,
+    // 16 rows: 98 against 112 us; sixteen bf16 rows are one operand set and go as one pass everywhere)
+    const int pass = k == 4096 || a_dtype != QMM_F32 ? 16 : 8;
     for (int m0 = 0; m0 < m; m0 += pass) {
         const int rows = std::min(pass, m - m0);
         const void* am = (const char*)a + (size_t)m0 * k * esz;

@@ -869,10 +869,11 @@ def test_q6_k_decode_vocabulary_shapes(m, n, k, lhs_bf16):
                                             (8, 250, 4096, False), (9, 47, 4096, False), (16, 530, 4096, True), (12, 9000, 4096, False),
                                             (20, 300, 4096, False), (40, 130, 4096, True), (64, 72, 4096, False),
                                             (4, 300, 14336, False), (8, 130, 8192, True), (5, 2100, 2048, False),
-                                            (16, 77, 6144, False), (6, 40, 16384, True)])
+                                            (16, 77, 6144, False), (6, 40, 16384, True), (16, 300, 14336, True), (13, 50, 2048, True)])
 def test_q6_k_small_batch_matrix_core_kernel(m, n, k, lhs_bf16):
     """Q6_K with 2..64 lhs rows on K = 4096: weight rows decoded once for all lhs rows (codes as exact fp16 integers, one
-    matrix-core instruction per 16-weight scale group and set of eight lhs rows); the 2, 4, 8 and 16 row variants, further
+    matrix-core instruction per 16-weight scale group and set of eight lhs rows; sixteen bf16 rows are one set without
+    residual rows); the 2, 4, 8 and 16 row variants, further
     passes from 17 rows on, tiles that end past the matrix, more tiles than workgroups; K in rounds of 4096 columns whose
     results add up in the output (a last round of 2048 with half the wavefronts).  Rows of very different magnitude share
     a pass (the lhs is scaled per row)."""
