@@ -84,6 +84,19 @@ bool q6k_mm_wanted(int64_t m, int64_t n) {
     return forced || m >= 5 || (m >= 3 && n >= 2048) || (m == 2 && n >= 8192);
 }
 
+// Q5_K: the small-batch matrix-core kernel, or passes of the decode kernel (up to four lhs rows each)?
+bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
+    // Measured, small-batch kernel / decode-kernel passes, fp32 lhs (bf16 lhs: the small-batch kernel is 10-20 % faster, and
+    // sixteen bf16 rows cost what eight do): 14336 x 4096: 2 lhs rows 17.5 / 17.5 us, 4 19.2 / 27.2, 8 20.9 / 53.6, 16 41.5 / 106;
+    // 4096 x 4096: 4 11.9 / 11.4, 8 14.3 / 22.1; 1024 x 4096: 4 11.6 / 7.8, 8 13.9 / 15.3; 4096 x 14336: 2 34.4 / 33.1, 4 40.4 / 65.4,
+    // 8 50.2 / 130.  QMM_Q5K_MM=1 sends every shape the kernel takes there.
+    static const bool forced = [] {
+        const char* e = getenv("QMM_Q5K_MM");
+        return e && e[0] == '1';
+    }();
+    return forced || m >= 5 || (m >= 3 && n * k >= ((int64_t)32 << 20));
+}
+
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     const bool f32 = lhs_dtype == QMM_F32;
     const double tiles = (double)((m + 127) / 128) * (double)((n + 255) / 256);
@@ -430,6 +443,9 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     // Q5_K and Q6_K with many lhs rows: weights to fp16 integer planes in the workspace, then the matrix cores
     if (qmm::gemm_planes_wanted(encoding, m, n, k))
         return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
+    // Q5_K with several lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
+    if (encoding == QMM_Q5_K && q5k_mm_wanted(m, n, k) && qmm::gemv_q5_k_mm_supported(w, m, n, k))
+        return hip_status(qmm::launch_gemv_q5_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, s), "qmm_matmul(Q5_K small batch)");
     if (encoding == QMM_Q5_K) {
         // a decode-shaped kernel; a pass takes as many lhs rows as fit its LDS copy of the lhs
         const int64_t ngroups = (k / 256 + 15) / 16;

@@ -20,6 +20,7 @@ CASES = {
              (40, 300, 1024, True), (1, 70, 32768, False), (200, 260, 512, True), (3, 1100, 8192, False)],
     "Q4_0": [(1, 200, 4096, False), (4, 200, 4096, True), (9, 72, 1056, False), (16, 200, 4096, False), (80, 136, 1024, True)],
     "Q6_K": [(1, 8200, 2048, False), (1, 300, 4096, True), (4, 200, 4096, False), (16, 72, 512, False), (70, 136, 1024, True), (8, 600, 4096, False)],
+    "Q5_K": [(2, 300, 4096, False), (6, 200, 4096, True), (16, 72, 1024, False)],
     "GPTQ": [(1, 264, 1024, False), (4, 264, 1024, True), (16, 264, 1024, False), (40, 264, 1024, True)],
 }
 
@@ -42,7 +43,8 @@ def main() -> int:
                 got = qmatmul(QE.GPTQ, QuantizationConfig(), lhs, torch.from_numpy(qw).to(dev),
                               torch.from_numpy(sc.view(np.float16)).to(dev), torch.from_numpy(qz).to(dev))
             else:
-                enc, oenc = {"Q4_K": (QE.Q4_K, O.Q4_K), "Q4_0": (QE.Q4_0, O.Q4_0), "Q6_K": (QE.Q6_K, O.Q6_K)}[name]
+                enc, oenc = {"Q4_K": (QE.Q4_K, O.Q4_K), "Q4_0": (QE.Q4_0, O.Q4_0), "Q6_K": (QE.Q6_K, O.Q6_K),
+                             "Q5_K": (QE.Q5_K, O.Q5_K)}[name]
                 wq = O.quantize(oenc, w)
                 want = O.matmul_q4_0(a, wq) if name == "Q4_0" else O.matmul_f32(oenc, a, wq)
                 got = qmatmul(enc, None, lhs, torch.from_numpy(wq).to(dev))

@@ -1,5 +1,5 @@
 """Every kernel that only runs when another one is switched off (QMM_DISABLE) or when QMM_Q4K_TILE / QMM_Q4K_PLANES /
-QMM_Q4_0_PLANES / QMM_Q4K_LANES_ROWS / QMM_Q6K_MM force it: each
+QMM_Q4_0_PLANES / QMM_Q4K_LANES_ROWS / QMM_Q6K_MM / QMM_Q5K_MM force it: each
 setting gets a child process (the library reads its environment once), which checks a fixed set of shapes of all
 four encodings against the oracle."""
 import os
@@ -21,10 +21,10 @@ SETTINGS = [
                     "q6k_staged,kquant_planes,gptq_mm,gptq_cols"},
     # the tile kernel on shapes it does not get by itself
     {"QMM_Q4K_TILE": "1"},
-    # the plane GEMMs of Q4_K and Q4_0, the 2..4-row decode kernel of Q4_K and the small-batch kernel of Q6_K likewise
-    {"QMM_Q4K_PLANES": "1", "QMM_Q4_0_PLANES": "1", "QMM_Q4K_LANES_ROWS": "1", "QMM_Q6K_MM": "1"},
-    # the kernels that the 2..4-row decode kernel of Q4_K and the small-batch kernel of Q6_K take small batches from
-    {"QMM_DISABLE": "q4k_lanes_rows,q6k_mm"},
+    # the plane GEMMs of Q4_K and Q4_0, the 2..4-row decode kernel of Q4_K and the small-batch kernels of Q6_K and Q5_K likewise
+    {"QMM_Q4K_PLANES": "1", "QMM_Q4_0_PLANES": "1", "QMM_Q4K_LANES_ROWS": "1", "QMM_Q6K_MM": "1", "QMM_Q5K_MM": "1"},
+    # the kernels that the 2..4-row decode kernel of Q4_K and the small-batch kernels of Q6_K and Q5_K take small batches from
+    {"QMM_DISABLE": "q4k_lanes_rows,q6k_mm,q5k_mm"},
 ]
 
 
@@ -35,4 +35,4 @@ def test_fallback_kernels_match_the_oracle(setting):
     proc = subprocess.run([sys.executable, os.path.join(HERE, "fallback_child.py")], env=env, capture_output=True, text=True,
                           timeout=600)
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
-    assert proc.stdout.count(": ok") == 24, proc.stdout
+    assert proc.stdout.count(": ok") == 27, proc.stdout

@@ -309,6 +309,37 @@ def test_q5_k_decode_shapes(m, n, k, bf16):
     assert_close(got, truth, f"Q5_K {m}x{n}x{k} bf16={bf16}")
 
 
+@pytest.mark.parametrize("m,n,k,bf16", [(5, 16, 4096, False), (8, 1000, 4096, True), (16, 4099, 4096, False), (16, 530, 4096, True),
+                                        (12, 9000, 512, False), (7, 300, 8192, False), (16, 77, 14336, True), (9, 40, 32768, False),
+                                        (20, 130, 4608, True), (32, 72, 1024, False)])
+def test_q5_k_small_batch_matrix_core_kernel(m, n, k, bf16):
+    """Q5_K with 5..32 lhs rows, K a multiple of 512: weight rows decoded once for the lhs rows of a pass (codes as exact fp16
+    integers, one matrix-core instruction per 32-weight sub-block, the min term through the lhs sub-block sums); 8-row passes
+    (fp32) and 16-row passes (bf16: no residual rows), tiles that end past the matrix, more tiles than workgroups, K in
+    rounds of 4096 columns with a last round in which only some wavefronts have a share; a third of the blocks carry random
+    bytes (every fifth-bit / nibble / scale combination); rows of very different magnitude share a pass."""
+    w, a = synth(44, n, k, m)
+    a[m - 1] *= 10.0  # (not more: the random blocks make large weights, and fp32 sums of 1e4 carry 1e-3 of noise)
+    a[0] *= 1e-4
+    a[1, :512] *= 1e-3
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(O.Q5_K, w)
+    rng = np.random.default_rng(45)
+    blocks = wq.reshape(-1, 176)
+    rnd = rng.integers(0, 256, blocks.shape, dtype=np.uint8)
+    rnd[:, 0:4] = blocks[:, 0:4]
+    blocks[::3] = rnd[::3]
+    truth = O.matmul_f64(O.Q5_K, a, wq)
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    got = qmatmul(QE.Q5_K, None, lhs, gpu(wq))
+    assert_close(got, truth, f"Q5_K {m}x{n}x{k} bf16={bf16} vs fp64 truth")
+    # (against the fp32 oracle only where cancellation leaves something to compare: both are fp32 sums in different orders)
+    want = O.matmul_f32(O.Q5_K, a, wq)
+    big = np.abs(truth) > 1e-3 * np.abs(truth).max(axis=1, keepdims=True)
+    assert O.isclose(got.cpu().numpy()[big], want[big], RTOL, ATOL).all()
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256), (1, 14336, 4096), (3, 200, 14336)])
 def test_gptq_matmul(m, n, k):
     w, a = synth(5, n, k, m)
