@@ -726,7 +726,16 @@ def extra_timings(layers, acts, gen):
     dev_s, _ = time_graphs([g], 20, 3)
     us = dev_s * 1e6 / (20 * 8)
     out["q5_k_m1_14336x4096"] = {"us": round(us, 3), "GB/s": round(alg_bytes(QE.Q5_K, 1, 14336, 4096) / us / 1e3, 1)}
+    # ... and with 8 fp32 / 16 bf16 lhs rows (one pass of the small-batch matrix-core kernel each)
+    w5 = [c.w for c in cs]
     del cs
+    for mm, dt, tag in ((8, torch.float32, "m8"), (16, torch.bfloat16, "m16_bf16")):
+        am = torch.randn((mm, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(dt)
+        g = capture([Gemv(QE.Q5_K, w_, am) for w_ in w5])
+        dev_s, _ = time_graphs([g], 20, 3)
+        us = dev_s * 1e6 / (20 * 8)
+        out[f"q5_k_{tag}_14336x4096"] = {"us": round(us, 3)}
+    del w5
     # Q4_0 prefill, same shape as cfg5: Q8_0 lhs codes and q - 8 as exact fp16 integers on the fp16 matrix cores (the time
     # includes the lhs quantisation and the weight plane conversion)
     ab32 = torch.randn((2048, 4096), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
