@@ -350,13 +350,13 @@ def test_gptq_matmul(m, n, k):
 
 
 @pytest.mark.parametrize("enc", [QE.Q4_0, QE.Q4_K, QE.Q5_K, QE.Q6_K])
-@pytest.mark.parametrize("m", [1, 4, 40])
+@pytest.mark.parametrize("m", [1, 4, 8, 40])
 def test_non_finite_lhs_values_stay_in_their_row(enc, m):
     """A NaN in the lhs gives the oracle's outputs, NaN for NaN (Q4_0: the Q8_0 quantiser's maximum search drops it on
     both sides).  An infinity makes its whole output row non-finite on both sides; the kind may differ: the K-quant
     kernels add the offset / min terms as separate sums, so they report NaN (inf - inf) where the element-wise
     oracle reports +-inf.  Rows without such a value are not touched by it."""
-    w, a = synth(5, 64, 1024, m)
+    w, a = synth(5, 64, 2048, m)
     wq = O.quantize(ENC[enc], w)
     for val in (np.nan, np.inf, -np.inf):
         a2 = a.copy()
