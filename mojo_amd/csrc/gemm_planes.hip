@@ -100,10 +100,22 @@ __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quart
             for (int q = 0; q < 8; q++) q4k_scale_min(q, s3, sc5[q], mn5[q]);
             if constexpr (ENC == QMM_Q5_K) fifth = *(const uint2*)(blk + 16 + 8 * f);  // fifth bits of elements 8 f .. 8 f + 7 of every sub-block
         }
+        // Codes to fp16 without a conversion instruction: the nibble byte (nibble in its high half) under a byte that holds the
+        // remaining code bits below 0x54 reads as 0x5400 + (code << 4) = 64 + code; two byte permutes per dword put the eight
+        // codes in the piece's element order (0, 2, 1, 3, 4, 6, 5, 7), a packed subtraction takes the 64 (and Q6_K's 32) off and
+        // a packed multiplication by the scale gives the plane values, all exact small integers.
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        auto pair = [](uint32_t x) __attribute__((always_inline)) { return __builtin_bit_cast(half2v, x); };
+        auto bits = [](half2v x) __attribute__((always_inline)) { return __builtin_bit_cast(uint32_t, x); };
+        auto both = [](float x) __attribute__((always_inline)) {
+            half2v r = {(_Float16)x, (_Float16)x};
+            return r;
+        };
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             // the eight weights 64 c + 32 g + 8 f + (0..7) of the super-block: their code bytes are eight neighbours
-            int v0[8], v1[8];
+            uint2 lo4, hi4;
+            half2v off, s0, s1 = both(0.0f);
             if constexpr (ENC == QMM_Q6_K) {
                 const int h = c >> 1, quad = (2 * c + g) & 3;
                 // (columns are 212 bytes apart in the stage: four-byte reads)
@@ -111,36 +123,29 @@ __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quart
                 const uint32_t* qhp = (const uint32_t*)(blk + 128 + 32 * h + 8 * f);
                 const uint2 ql = make_uint2(qlp[0], qlp[1]), qh = make_uint2(qhp[0], qhp[1]);
                 const int sc = (int)(int8_t)blk[192 + 8 * h + 2 * quad + (f >> 1)];
-                const int hi16 = (sc >> 4) * 16, lo = sc & 15;  // sc = 16 hi + lo
-                const int nsh = (quad & 2) ? 4 : 0, hsh = 2 * quad;
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const int e = kPerm[i];
-                    const uint32_t lw = e < 4 ? ql.x : ql.y, hw = e < 4 ? qh.x : qh.y;
-                    const int q = (int)(((lw >> (8 * (e & 3) + nsh)) & 15u) | (((hw >> (8 * (e & 3) + hsh)) & 3u) << 4)) - 32;
-                    v0[i] = live ? hi16 * q : 0;
-                    v1[i] = live ? lo * q : 0;
-                }
+                s0 = both(live ? (float)((sc >> 4) * 16) : 0.0f);  // sc = 16 hi + lo
+                s1 = both(live ? (float)(sc & 15) : 0.0f);
+                lo4 = (quad & 2) ? make_uint2(ql.x & 0xF0F0F0F0u, ql.y & 0xF0F0F0F0u) : make_uint2((ql.x << 4) & 0xF0F0F0F0u, (ql.y << 4) & 0xF0F0F0F0u);
+                hi4 = make_uint2(((qh.x >> (2 * quad)) & 0x03030303u) | 0x54545454u, ((qh.y >> (2 * quad)) & 0x03030303u) | 0x54545454u);
+                off = both(96.0f);
             } else {
                 const int sb = 2 * c + g;
                 const uint2 qs = *(const uint2*)(blk + (ENC == QMM_Q5_K ? 48 : 16) + 32 * c + 8 * f);
-                const int scale = live ? (int)sc5[sb] : 0;
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const int e = kPerm[i];
-                    const uint32_t lw = e < 4 ? qs.x : qs.y;
-                    int q = (int)((lw >> (8 * (e & 3) + 4 * g)) & 15u);
-                    if constexpr (ENC == QMM_Q5_K) q |= (int)((((e < 4 ? fifth.x : fifth.y) >> (8 * (e & 3) + sb)) & 1u) << 4);
-                    v0[i] = scale * q;
-                    v1[i] = 0;
-                }
+                s0 = both(live ? (float)sc5[sb] : 0.0f);
+                lo4 = g ? make_uint2(qs.x & 0xF0F0F0F0u, qs.y & 0xF0F0F0F0u) : make_uint2((qs.x << 4) & 0xF0F0F0F0u, (qs.y << 4) & 0xF0F0F0F0u);
+                if constexpr (ENC == QMM_Q5_K) hi4 = make_uint2(((fifth.x >> sb) & 0x01010101u) | 0x54545454u, ((fifth.y >> sb) & 0x01010101u) | 0x54545454u);
+                else hi4 = make_uint2(0x54545454u, 0x54545454u);
+                off = both(64.0f);
             }
+            // elements (0, 2), (1, 3) of the first dword, (4, 6), (5, 7) of the second
+            const half2v q0 = pair(__builtin_amdgcn_perm(hi4.x, lo4.x, 0x06020400u)) - off, q1 = pair(__builtin_amdgcn_perm(hi4.x, lo4.x, 0x07030501u)) - off;
+            const half2v q2 = pair(__builtin_amdgcn_perm(hi4.y, lo4.y, 0x06020400u)) - off, q3 = pair(__builtin_amdgcn_perm(hi4.y, lo4.y, 0x07030501u)) - off;
             const int64_t step = (int64_t)rb * 4 + c;
 #pragma unroll
             for (int pl = 0; pl < NPL; pl++) {
-                const int* v = pl == 0 ? v0 : v1;
+                const half2v sp = pl == 0 ? s0 : s1;
                 uint8_t* tile = planes + (((int64_t)tile_n * NPL + pl) * steps_row + step) * kBBuf;
-                *(uint4*)(tile + dst_in_tile) = make_uint4(pack_ints(v[0], v[1]), pack_ints(v[2], v[3]), pack_ints(v[4], v[5]), pack_ints(v[6], v[7]));
+                *(uint4*)(tile + dst_in_tile) = make_uint4(bits(q0 * sp), bits(q1 * sp), bits(q2 * sp), bits(q3 * sp));
             }
         }
         // tables: one thread per column
