@@ -60,6 +60,17 @@ __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float1
     }
 }
 
+// acc *= g in place, for the same reasons (and with the same idle states in front).
+__device__ __forceinline__ void rescale_mul(float16v& acc, float g) {
+    asm volatile("s_nop 7\n\ts_nop 3");
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        float t = acc[r];
+        asm volatile("v_mul_f32 %0, %0, %1" : "+v"(t) : "v"(g));
+        acc[r] = t;
+    }
+}
+
 // Operand orders inside every 64-wide chunk of a row; position f*16 + g*8 + slot holds column
 //   kLhsOrderQ4K : 32*(f/2) + 16*g + 8*(f%2) + (0,2,1,3,4,6,5,7)[slot]
 //   kLhsOrderGPTQ: 16*f + 8*g + (0,4,1,5,2,6,3,7)[slot], odd columns pre-multiplied by 1/16
@@ -71,9 +82,15 @@ __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float1
 constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1, kLhsOrderQ4K16 = 2, kLhsOrderTile = 3;
 
 // One lhs row by one workgroup of 256 threads.
+// With next > 0 the rows of a16 / a16_lo are lda = k + 256 next halfs long and the sub-block sums go behind the row's k
+// columns instead of into asum, as `next` further blocks of 256 operand positions: the 32 positions of super-block b are
+// 8 hi, 8 lo, 8 hi, 8 lo parts of its sums (what multiplies a weight-side block of 8 hi, 8 hi, 8 lo, 8 lo table parts to the
+// full hi/lo product), zeros beyond the last super-block.
 template <typename AT, int ORDER>
 __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
-                                             _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum, float* __restrict__ inv) {
+                                             _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum, float* __restrict__ inv,
+                                             int64_t lda = 0, int next = 0) {
+    if (lda == 0) lda = k;
     __shared__ uint32_t wmax[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const AT* ar = a + (int64_t)row * k;
@@ -98,21 +115,21 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
         if constexpr (ORDER == kLhsOrderQ4K) {
             const int hin = kl >> 5, gg = (kl >> 4) & 1, odd = (kl >> 3) & 1;
             const int pos = (2 * hin + odd) * 16 + gg * 8 + (kl & 4);
-            const int64_t o = (int64_t)row * k + (i & ~63) + pos;
+            const int64_t o = (int64_t)row * lda + (i & ~63) + pos;
             *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
             if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
         } else if constexpr (ORDER == kLhsOrderTile) {
             const int gg = kl >> 5, f = (kl >> 3) & 3;
-            const int64_t o = (int64_t)row * k + (i & ~63) + f * 16 + gg * 8 + (kl & 4);
+            const int64_t o = (int64_t)row * lda + (i & ~63) + f * 16 + gg * 8 + (kl & 4);
             *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
             if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
         } else if constexpr (ORDER == kLhsOrderQ4K16) {
-            const int64_t o = (int64_t)row * k + i;
+            const int64_t o = (int64_t)row * lda + i;
             *(uint2*)(a16 + o) = make_uint2(pack_half2(h0, h2), pack_half2(h1, h3));
             if (a16_lo) *(uint2*)(a16_lo + o) = make_uint2(pack_half2(x0 - h0, x2 - h2), pack_half2(x1 - h1, x3 - h3));
         } else {
             // columns kl..kl+3 of an 8-group go to slots 0,2,4,6 (kl % 8 == 0) or 1,3,5,7 (kl % 8 == 4)
-            const int64_t o = (int64_t)row * k + (i & ~63) + (kl & ~7) + ((kl >> 2) & 1);
+            const int64_t o = (int64_t)row * lda + (i & ~63) + (kl & ~7) + ((kl >> 2) & 1);
             const float sixteenth = 0.0625f;
             a16[o] = (_Float16)h0;
             a16[o + 2] = (_Float16)(h1 * sixteenth);
@@ -129,11 +146,18 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
         if ((lane & 7) == 0) {
             const int blk = i >> 8, j = (i >> 5) & 7;
             const float sh = h2f(f2h(sum));
-            _Float16* as = asum + ((int64_t)row * (k >> 8) + blk) * 16;
-            as[j] = (_Float16)sh;
-            as[8 + j] = (_Float16)(sum - sh);
+            if (next > 0) {
+                _Float16* as = a16 + (int64_t)row * lda + k + blk * 32;
+                as[j] = as[16 + j] = (_Float16)sh;
+                as[8 + j] = as[24 + j] = (_Float16)(sum - sh);
+            } else {
+                _Float16* as = asum + ((int64_t)row * (k >> 8) + blk) * 16;
+                as[j] = (_Float16)sh;
+                as[8 + j] = (_Float16)(sum - sh);
+            }
         }
     }
+    for (int i = (k >> 8) * 32 + tid; i < next * 256; i += 256) a16[(int64_t)row * lda + k + i] = (_Float16)0.0f;
 }
 
 template <typename AT, int ORDER>
@@ -153,9 +177,11 @@ struct LhsPlanes {
 
 // row_pad: the planes are sized for m rounded up to a multiple of it (kernels that read whole row tiles past the
 // last row; the pass leaves those rows unwritten, and nothing computed from them is ever stored).
-inline LhsPlanes lhs_planes(void* workspace, int lhs_dtype, int64_t m, int64_t k, int64_t row_pad = 1) {
+inline LhsPlanes lhs_planes(void* workspace, int lhs_dtype, int64_t m, int64_t k, int64_t row_pad = 1, int64_t lda = 0) {
     auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
     m = (m + row_pad - 1) / row_pad * row_pad;
+    const int64_t k_sums = k;
+    if (lda > k) k = lda;  // rows with extension blocks (see prep_lhs_row)
     LhsPlanes p;
     char* ws = (char*)workspace;
     int64_t off = 0;
@@ -167,7 +193,7 @@ inline LhsPlanes lhs_planes(void* workspace, int lhs_dtype, int64_t m, int64_t k
         off += up(m * k * 2);
     }
     p.asum = (_Float16*)(ws + off);
-    off += up(m * (k / 256) * 32);
+    off += up(m * (k_sums / 256) * 32);
     p.inv = (float*)(ws + off);
     off += up(m * 4);
     p.bytes = off;

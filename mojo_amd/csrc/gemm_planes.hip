@@ -38,7 +38,6 @@ constexpr int kABuf = TM * 128, kBBuf = TN * 128, kSBuf = TM * 32, kMBuf = TN * 
 constexpr int kOffA = 0, kOffB = kOffA + 3 * kABuf, kOffS = kOffB + 3 * kBBuf, kOffM = kOffS + kSBuf, kOffD = kOffM + kMBuf;
 constexpr int kOffInv = kOffD + kDBuf, kPlanesLds = kOffInv + TM * 4;
 static_assert(kPlanesLds <= kLdsPerCu, "planes kernel LDS");
-constexpr int kPerm[8] = {0, 2, 1, 3, 4, 6, 5, 7};
 
 struct PlaneSpace {
     uint8_t* planes;  // [tiles_n][nplanes * steps][16 KB]
@@ -46,19 +45,36 @@ struct PlaneSpace {
     uint8_t* mtab;    // [tiles_n][nblk][128][32 bytes]   (Q5_K)
     int64_t bytes;
 };
-PlaneSpace plane_space(void* base, int64_t n, int64_t k, int nplanes, bool with_min) {
+// nblk_tile: blocks of four steps per 128-column tile and plane (the super-blocks, plus the wide GEMM's extension blocks)
+// dblocks: scale blocks per tile (GPTQ groups of 128: two per 256 k)
+PlaneSpace plane_space(void* base, int64_t n, int64_t k, int nplanes, bool with_mtab, int64_t nblk_tile, int64_t dblocks = 0) {
     auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
     const int64_t tiles_n = (n + TN - 1) / TN, nblk = k / 256;
     PlaneSpace p;
     int64_t off = 0;
     p.planes = (uint8_t*)base + off;
-    off += up(tiles_n * nplanes * nblk * 4 * kBBuf);
+    off += up(tiles_n * nplanes * nblk_tile * 4 * kBBuf);
     p.dtab = (float*)((uint8_t*)base + off);
-    off += up(tiles_n * nblk * kDBuf);
+    off += up(tiles_n * (dblocks ? dblocks : nblk_tile) * kDBuf);
     p.mtab = (uint8_t*)base + off;
-    off += with_min ? up(tiles_n * nblk * kMBuf) : 0;
+    off += with_mtab ? up(tiles_n * nblk * kMBuf) : 0;
     p.bytes = off;
     return p;
+}
+
+// Which GEMM serves a single-plane encoding: the 256 x 256 tiles from this many of them on (fewer leave compute units idle
+// where the 256 x 128 kernel still has work for them).
+constexpr int kWideMinTiles = 128;
+constexpr int kOptionalPlanesMinRows = 1024;  // Q4_K and GPTQ have GEMM kernels that need no conversion pass: planes from here on
+bool wide_tiles(int encoding, int64_t m, int64_t n) {
+    if (encoding == QMM_Q6_K || kernel_disabled("planes_wide")) return false;
+    const int64_t tiles_m = (m + TM - 1) / TM, tiles_nw = (n + 2 * TN - 1) / (2 * TN);
+    return tiles_m * tiles_nw >= kWideMinTiles;
+}
+// blocks per tile: with the wide GEMM, Q4_K / Q5_K carry their min operands as one extension block per eight super-blocks
+int64_t blocks_per_tile(int encoding, int64_t m, int64_t n, int64_t k) {
+    const int64_t nblk = k / 256;
+    return wide_tiles(encoding, m, n) ? nblk + (nblk + 7) / 8 : nblk;
 }
 
 __device__ __forceinline__ uint32_t pack_ints(int a, int b) { return pack_half2((float)a, (float)b); }
@@ -69,9 +85,14 @@ __device__ __forceinline__ uint32_t pack_ints(int a, int b) { return pack_half2(
 // columns are first copied into LDS (16-byte loads where the rows allow it, two-byte loads otherwise: rows of Q6_K blocks start
 // on even addresses only) at a stride that is a multiple of four bytes, so that the code bytes can be read eight at a time; thread t then takes piece
 // t % 8 of column t / 8 of each of the four steps, so that eight neighbouring threads write one 128-byte row of the tile.
+// nblk_tile > nblk (the wide GEMM's layout for Q4_K / Q5_K): every 128-column tile has nblk_tile - nblk further blocks of four
+// steps behind its nblk super-blocks, with scale 1, that hold the min operands: the 32 positions of super-block b in them are
+// -(dmin * mn) of its eight sub-blocks as 8 hi, 8 hi, 8 lo, 8 lo parts (lhs side: the sub-block sums as hi, lo, hi, lo), zeros
+// beyond the last super-block; no mtab then.  Blocks with d = 0 get a plane of zeros (the wide GEMM keeps no unit for them).
 template <int ENC>
 __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quarter, const uint8_t* __restrict__ w, int n, int nblk,
-                                                   uint8_t* __restrict__ planes, float* __restrict__ dtab, uint8_t* __restrict__ mtab) {
+                                                   int nblk_tile, uint8_t* __restrict__ planes, float* __restrict__ dtab,
+                                                   uint8_t* __restrict__ mtab) {
     constexpr int BPB = ENC == QMM_Q6_K ? Q6_K_BPB : ENC == QMM_Q5_K ? Q5_K_BPB : Q4_K_BPB;
     constexpr int STRIDE = (BPB + 3) / 4 * 4;  // 212 for Q6_K
     constexpr int NPL = ENC == QMM_Q6_K ? 2 : 1;
@@ -110,11 +131,12 @@ __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quart
     }
     __syncthreads();
     const int piece = tid & 7, g = piece & 1, f = piece >> 1;
-    const int64_t steps_row = (int64_t)nblk * 4;
+    const int64_t steps_row = (int64_t)nblk_tile * 4;
     {
         const int col = col0 + (tid >> 3), ncol = tile_n * TN + col;
-        const bool live = ncol < n;
         const uint8_t* blk = (const uint8_t*)stage + (tid >> 3) * STRIDE;
+        const uint16_t dbits = *(const uint16_t*)(blk + (ENC == QMM_Q6_K ? 208 : 0));
+        const bool in_n = ncol < n, live = in_n && (dbits & 0x7fffu) != 0;  // live: the column exists and its block has a scale
         const uint32_t dst_in_tile = (uint32_t)(col * 128 + ((piece ^ ((col >> 1) & 7)) << 4));
         // Q4_K / Q5_K header fields of this column's block
         uint32_t sc5[8], mn5[8];
@@ -175,21 +197,39 @@ __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quart
         }
         // tables: one thread per column
         if (piece == 0) {
-            const int64_t tb = (int64_t)tile_n * nblk + rb;
-            const uint16_t dbits = *(const uint16_t*)(blk + (ENC == QMM_Q6_K ? 208 : 0));
-            dtab[tb * TN + col] = live ? h2f(dbits) : 0.0f;
+            const int64_t tb = (int64_t)tile_n * nblk_tile + rb;
+            dtab[tb * TN + col] = in_n ? h2f(dbits) : 0.0f;
             if constexpr (ENC != QMM_Q6_K) {
                 const uint32_t ndm = ((uint32_t)(*(const uint16_t*)(blk + 2)) ^ 0x8000u) * 0x00010001u;  // (-dmin, -dmin)
                 uint32_t hi[4], lo[4];
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const uint32_t mp = live ? pack_half2((float)mn5[2 * q], (float)mn5[2 * q + 1]) : 0u;
+                    const uint32_t mp = in_n ? pack_half2((float)mn5[2 * q], (float)mn5[2 * q + 1]) : 0u;
                     hi[q] = pk_mul(ndm, mp);
                     lo[q] = pk_fma(ndm, mp, hi[q] ^ 0x80008000u);
                 }
-                uint8_t* mt = mtab + (tb * TN + col) * 32;
-                *(uint4*)mt = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-                *(uint4*)(mt + 16) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                if (nblk_tile > nblk) {
+                    // pieces 4 (rb % 2) + (0, 1, 2, 3) of step (rb % 8) / 2 of the extension block rb / 8
+                    const int xb = rb >> 3;
+                    uint8_t* tile = planes + ((int64_t)tile_n * steps_row + (nblk + xb) * 4 + ((rb & 7) >> 1)) * kBBuf + col * 128;
+                    const int sw = (col >> 1) & 7, p0 = (rb & 1) * 4;
+                    const uint4 vh = make_uint4(hi[0], hi[1], hi[2], hi[3]), vl = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                    *(uint4*)(tile + (((p0 + 0) ^ sw) << 4)) = vh;
+                    *(uint4*)(tile + (((p0 + 1) ^ sw) << 4)) = vh;
+                    *(uint4*)(tile + (((p0 + 2) ^ sw) << 4)) = vl;
+                    *(uint4*)(tile + (((p0 + 3) ^ sw) << 4)) = vl;
+                    if ((rb & 7) == 0) dtab[((int64_t)tile_n * nblk_tile + nblk + xb) * TN + col] = 1.0f;
+                    if (rb == nblk - 1) {  // the rest of the last extension block
+                        for (int b2 = rb + 1; b2 < (xb + 1) * 8; b2++) {
+                            uint8_t* t2 = planes + ((int64_t)tile_n * steps_row + (nblk + xb) * 4 + ((b2 & 7) >> 1)) * kBBuf + col * 128;
+                            for (int q = 0; q < 4; q++) *(uint4*)(t2 + ((((b2 & 1) * 4 + q) ^ sw) << 4)) = make_uint4(0, 0, 0, 0);
+                        }
+                    }
+                } else {
+                    uint8_t* mt = mtab + (tb * TN + col) * 32;
+                    *(uint4*)mt = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                    *(uint4*)(mt + 16) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                }
             }
         }
     }
@@ -198,15 +238,16 @@ __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quart
 // Everything the GEMM needs done first, in one launch of 256-thread workgroups: [0, conv) convert weights (the long part,
 // so it starts first), the next m narrow one lhs row each, the rest zero the output tiles that the GEMM fills with atomic adds.
 template <int ENC, typename AT>
-__global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __restrict__ w, int nblk, uint8_t* __restrict__ planes,
-                                                              float* __restrict__ dtab, uint8_t* __restrict__ mtab, int conv,
-                                                              const AT* __restrict__ a, int k, LhsPlanes p, SplitTiles z) {
+__global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __restrict__ w, int nblk, int nblk_tile, int tiles_n128,
+                                                              uint8_t* __restrict__ planes, float* __restrict__ dtab,
+                                                              uint8_t* __restrict__ mtab, int conv, const AT* __restrict__ a, int k,
+                                                              LhsPlanes p, SplitTiles z) {
     const int b = (int)blockIdx.x;
     if (b < conv) {
-        const int t = b >> 2, rb = t / z.tiles_n;
-        planes_from_kquant<ENC>(t - rb * z.tiles_n, rb, b & 3, w, z.n, nblk, planes, dtab, mtab);
+        const int t = b >> 2, rb = t / tiles_n128;
+        planes_from_kquant<ENC>(t - rb * tiles_n128, rb, b & 3, w, z.n, nblk, nblk_tile, planes, dtab, mtab);
     } else if (b < conv + z.m) {
-        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv);
+        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv, (int64_t)k + (nblk_tile - nblk) * 256, nblk_tile - nblk);
     } else {
         const int e = b - conv - z.m;
         zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
@@ -696,11 +737,316 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
     }
 }
 
+// The GEMM over one plane on 256 x 256 output tiles: the two-plane kernel's structure (32 KB of lhs and 2 x 16 KB of weights per
+// step, two buffers each, 32 matrix-core instructions per wavefront and step, six operand reads for eight of them), with the second
+// 16 KB being the neighbouring 128-column tile instead of a second plane, and one set of 128 accumulators per lane and no second
+// set for the running super-block: the accumulators are kept in units of the current super-block's scale,
+//     acc <- acc * (d_prev / d_cur)   at each super-block boundary,   acc <- acc * d_last   at the end,
+// so that the matrix cores add each super-block's exact integer products directly onto them.  A zero scale keeps the unit of the
+// block before it (its plane holds zeros, see the conversion).
+namespace {
+constexpr int kwOffA = 0, kwOffB = 2 * kABuf, kwOffD = kwOffB + 4 * kBBuf, kwOffInv = kwOffD + 2 * kDBuf, kPlanesWLds = kwOffInv + TM * 4;
+static_assert(kPlanesWLds <= kLdsPerCu, "wide kernel LDS");
+}  // namespace
+
+template <int SPB>  // steps (of 64 k) per scale block: 4 for the K-quants, 2 for GPTQ groups of 128
+__global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t* __restrict__ planes, const float* __restrict__ dtab,
+                                                                 const _Float16* __restrict__ a16, const float* __restrict__ inv,
+                                                                 float* __restrict__ out, int m, int n, int lda, int nblk_walk,
+                                                                 int nblk_tile, int tiles_m, int tiles_n, int tiles_n128, int accumulate,
+                                                                 int allow_split) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const uint32_t lds0 = lds_address(smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int nl = lane & 31, g = lane >> 5;
+    const int nblk_row = nblk_walk;  // blocks of a full unit; nblk_tile: blocks per 128-column tile in the planes and tables
+    const uint32_t fa0 = (uint32_t)(kwOffA + (wm * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
+    const uint32_t fb0 = (uint32_t)(kwOffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
+    const uint32_t lane16 = (uint32_t)(lane * 16);
+
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
+    const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
+    int full;
+    const int units = xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
+    for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
+        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_row);
+        const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * SPB;  // this unit's share of K
+        const int kb0 = __builtin_amdgcn_readfirstlane(unit.kb0), unit_half = __builtin_amdgcn_readfirstlane(unit.half);
+        int tile_m, tile_n;
+        tile_order(unit.tile, tiles_m, tiles_n, kTileGm, tile_m, tile_n);
+        tile_m = __builtin_amdgcn_readfirstlane(tile_m);
+        tile_n = __builtin_amdgcn_readfirstlane(tile_n);
+        const int m0 = tile_m * TM, n0 = tile_n * 2 * TN;
+        // the second half of the tile is the next 128-column tile of the planes (the same one again at a ragged edge: its columns
+        // lie beyond n and are not stored)
+        const int second = __builtin_amdgcn_readfirstlane(min(tile_n * 2 + 1, tiles_n128 - 1) - tile_n * 2);
+
+        const uint8_t* a_base = (const uint8_t*)a16 + ((int64_t)(m0 + wave * 32) * lda + (int64_t)kb0 * (SPB * 64)) * 2;
+        const int64_t plane_bytes = (int64_t)nblk_tile * SPB * kBBuf;  // the plane of one 128-column tile
+        const uint8_t* b_base = planes + (int64_t)tile_n * 2 * plane_bytes + (int64_t)kb0 * SPB * kBBuf;
+        const int64_t dtile = (int64_t)nblk_tile * kDBuf;
+        const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * 2 * dtile + (int64_t)kb0 * kDBuf;
+
+        auto issue_A1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            const uint32_t a_off = (uint32_t)((l >> 3) * (lda * 2) + (((l & 7) ^ ((4 * i + (l >> 4)) & 7)) << 4));
+            const uint32_t dst = lds0 + kwOffA + buf * kABuf + wave * 4096;
+            load16_to_lds(a_off, a_base + (int64_t)min(step, ns - 1) * 128 + (int64_t)i * 16 * lda,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
+        };
+        // the i-th (0..3) of this wavefront's four 1 KB pieces of the two weight tiles of step `step`: half i / 2, piece 2 wave + i % 2
+        auto issue_B1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
+            const int pl = i >> 1, piece = (wave * 2 + (i & 1)) * 1024;
+            load16_to_lds(lane16, b_base + pl * second * plane_bytes + (int64_t)min(step, ns - 1) * kBBuf + piece,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kwOffB + (buf * 2 + pl) * kBBuf + piece)));
+        };
+        // the 256 scales of super-block blk: lanes 0..3 bring this wavefront's sixteen of the first half, lanes 4..7 of the second
+        auto issue_D = [&](int blk) __attribute__((always_inline)) {
+            if (lane < 8) {
+                int l = lane;
+                asm volatile("" : "+v"(l));
+                load16_to_lds((uint32_t)((l & 3) * 16) + (uint32_t)((l >> 2) * second) * (uint32_t)dtile,
+                              d_base + (int64_t)min(blk, nblk - 1) * kDBuf + wave * 64,
+                              (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kwOffD + wave * 128)));
+            }
+        };
+        // scale of column c (0..127) of half pl, as issue_D leaves them: [c / 16][pl][c % 16]
+        auto d_at = [&](int pl, int ni) __attribute__((always_inline)) {
+            const int c = wn * 64 + ni * 32 + nl;
+            return *(const float*)(smem + kwOffD + ((c >> 4) * 32 + pl * 16 + (c & 15)) * 4);
+        };
+
+        float16v acc[2][2][2];  // [half][row group][column group]
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t >> 2][(t >> 1) & 1][t & 1][r] = 0.0f;
+        half8 afr[2][2], bfr[2][2][2];  // [slot][row group], [slot][half][column group]
+        float unit_d[2][2] = {{1.f, 1.f}, {1.f, 1.f}}, ratio[2][2] = {{1.f, 1.f}, {1.f, 1.f}};
+
+        // ---- tile prologue
+        __syncthreads();  // every wavefront is done with the previous tile's LDS contents
+        issue_D(0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_A1(0, 0, i);
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_B1(0, 0, i);
+        if (tid < TM) *(float*)(smem + kwOffInv + tid * 4) = inv[min(m0 + tid, m - 1)];
+        wait_vmcnt<0>();
+        __syncthreads();
+
+        uint32_t fa = 0, fb = 0;
+        auto step_bases = [&](int buf) __attribute__((always_inline)) {
+            int ao = buf * kABuf, bo = buf * 2 * kBBuf;
+            asm volatile("" : "+s"(ao), "+s"(bo));
+            fa = fa0 + (uint32_t)ao;
+            fb = fb0 + (uint32_t)bo;
+        };
+        auto read_frags = [&](int f, int slot) __attribute__((always_inline)) {
+            const uint32_t xa = fa ^ (uint32_t)(f << 5), xb = fb ^ (uint32_t)(f << 5);
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + xa + mi * 4096);
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++)
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + xb + pl * kBBuf + ni * 4096);
+        };
+        auto mfma_slice = [&](int slot, auto&& between) __attribute__((always_inline)) {
+#pragma unroll
+            for (int pl = 0; pl < 2; pl++)
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++) {
+                        acc[pl][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][pl][ni], acc[pl][mi][ni], 0, 0, 0);
+                        between(pl * 4 + mi * 2 + ni);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+        };
+
+        // FIRST: the first step of the unit (nothing to finish, nothing to rescale), a variant of its own so that the loop body
+        // has no branches around matrix-core instructions (the compiler copies accumulators where they meet).
+        auto phase = [&](int blk, auto CC, auto FF) __attribute__((always_inline)) {
+            constexpr int c = decltype(CC)::value, cur = c & 1, nxt = cur ^ 1;
+            constexpr bool FIRST = decltype(FF)::value;
+            const int s = blk * SPB + c;
+            step_bases(cur);
+            read_frags(0, 0);
+            if (c == 0) {
+                // the new super-block's unit: its scale, or the previous unit where the scale is zero
+#pragma unroll
+                for (int pl = 0; pl < 2; pl++)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++) {
+                        const float dn = d_at(pl, ni), un = dn != 0.0f ? dn : unit_d[pl][ni];
+                        ratio[pl][ni] = unit_d[pl][ni] / un;
+                        unit_d[pl][ni] = un;
+                    }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (!FIRST) {
+                mfma_slice(1, [&](int i) __attribute__((always_inline)) {  // last slice of step s - 1
+                    if (i & 1) issue_A1(s + 1, nxt, i >> 1);
+                });
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) issue_A1(s + 1, nxt, i);
+            }
+            if constexpr (c == 1) issue_D(blk + 1);  // (the current scales were read in phase 0)
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (c == 0 && !FIRST) {
+                // the accumulators change unit, sub-tile by sub-tile, in front of the new super-block's first instruction on each
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    const int pl = t >> 2, mi = (t >> 1) & 1, ni = t & 1;
+                    rescale_mul(acc[pl][mi][ni], ratio[pl][ni]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc[pl][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][mi], bfr[0][pl][ni], acc[pl][mi][ni], 0, 0, 0);
+                    if (t < 4) issue_B1(s + 1, nxt, t);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < 4) issue_B1(s + 1, nxt, i); });
+            }
+            read_frags(2, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_slice(1, [](int) __attribute__((always_inline)) {});
+            read_frags(3, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_slice(0, [](int) __attribute__((always_inline)) {});
+            wait_vmcnt<0>();  // lhs and weights of step s + 1 (and, in phase 1, the next scales) have landed
+            __syncthreads();
+        };
+        // (the first block apart from the loop: see FIRST)
+        phase(0, std::integral_constant<int, 0>{}, std::true_type{});
+        phase(0, std::integral_constant<int, 1>{}, std::false_type{});
+        if constexpr (SPB == 4) {
+            phase(0, std::integral_constant<int, 2>{}, std::false_type{});
+            phase(0, std::integral_constant<int, 3>{}, std::false_type{});
+        }
+        for (int blk = 1; blk < nblk; blk++) {
+            phase(blk, std::integral_constant<int, 0>{}, std::false_type{});
+            phase(blk, std::integral_constant<int, 1>{}, std::false_type{});
+            if constexpr (SPB == 4) {
+                phase(blk, std::integral_constant<int, 2>{}, std::false_type{});
+                phase(blk, std::integral_constant<int, 3>{}, std::false_type{});
+            }
+        }
+        mfma_slice(1, [](int) __attribute__((always_inline)) {});  // last slice of the last step
+
+        // ---- tile epilogue: back to true units (last super-block's scale, row scale), store
+#pragma unroll
+        for (int pl = 0; pl < 2; pl++) {
+            const int col0 = n0 + pl * TN + wn * 64 + nl, col1 = col0 + 32;
+            const bool c0_ok = col0 < n, c1_ok = col1 < n;
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+                float4 iv[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) iv[j] = *(const float4*)(smem + kwOffInv + (wm * 64 + mi * 32 + 8 * j + 4 * g) * 4);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    const float4 q = iv[r >> 2];
+                    const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
+                    if (row < m) {
+                        float* o_ = out + (int64_t)row * n;
+                        const float v0 = acc[pl][mi][0][r] * unit_d[pl][0] * is, v1 = acc[pl][mi][1][r] * unit_d[pl][1] * is;
+                        if (unit_half) {  // one of the two K parts of this tile: out holds zero or the other part
+                            if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
+                            if (c1_ok) unsafeAtomicAdd(o_ + col1, v1);
+                        } else if (accumulate) {
+                            if (c0_ok) o_[col0] += v0;
+                            if (c1_ok) o_[col1] += v1;
+                        } else {
+                            if (c0_ok) __builtin_nontemporal_store(v0, o_ + col0);
+                            if (c1_ok) __builtin_nontemporal_store(v1, o_ + col1);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// GPTQ (4-bit, [K/8, N] int32 words of eight consecutive k, zero point = stored + 1) to one plane of q - zero in [-16, 14],
+// the scale blocks being the groups: one workgroup per (128-column tile, 256 k).  The 32 x 128 words come in coalesced,
+// through LDS, and leave as 16-byte pieces, eight neighbouring threads writing one 128-byte row of the tile; a word is exactly
+// one piece (k = 64 step + 32 g + 8 f + 0..7).  Nibble n under the byte 0x64 reads as fp16 1024 + n; the packed subtraction of
+// 1024 + zero leaves the exact difference.
+__device__ __forceinline__ void planes_from_gptq(int tile_n, int rb, const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
+                                                 const uint32_t* __restrict__ qzeros, int n, int k, int group, uint8_t* __restrict__ planes,
+                                                 float* __restrict__ dtab) {
+    __shared__ uint32_t stage[32 * 129];
+    const int tid = (int)threadIdx.x, n0 = tile_n * TN;
+    for (int i = tid; i < 32 * 128; i += 256) {
+        const int row = i >> 7, col = i & 127;
+        stage[row * 129 + col] = n0 + col < n ? qweight[(int64_t)(rb * 32 + row) * n + n0 + col] : 0u;
+    }
+    __syncthreads();
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    auto pair = [](uint32_t x) __attribute__((always_inline)) { return __builtin_bit_cast(half2v, x); };
+    auto bits = [](half2v x) __attribute__((always_inline)) { return __builtin_bit_cast(uint32_t, x); };
+    const int piece = tid & 7, g = piece & 1, f = piece >> 1;
+    const int64_t steps_tile = k / 64, groups = k / group;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int col = j * 32 + (tid >> 3), ncol = min(n0 + col, n - 1);
+        const bool in_n = n0 + col < n;
+        const uint32_t dst = (uint32_t)(col * 128 + ((piece ^ ((col >> 1) & 7)) << 4));
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int64_t gi = ((int64_t)rb * 256 + c * 64) / group;
+            const uint32_t zero = ((qzeros[gi * (n >> 3) + (ncol >> 3)] >> (4 * (ncol & 7))) & 0xFu) + 1u;
+            const uint16_t sbits = scales[gi * n + ncol];
+            const bool live = in_n && (sbits & 0x7fffu) != 0;
+            const uint32_t x = stage[(8 * c + 4 * g + f) * 129 + col];
+            const uint32_t y = x & 0x0F0F0F0Fu, z = (x >> 4) & 0x0F0F0F0Fu;  // nibbles 0, 2, 4, 6 and 1, 3, 5, 7
+            const _Float16 o = (_Float16)(float)(1024u + zero);
+            const half2v off = {o, o};
+            uint4 v;
+            v.x = bits(pair(__builtin_amdgcn_perm(0x64646464u, y, 0x04010400u)) - off);  // k 0, 2
+            v.y = bits(pair(__builtin_amdgcn_perm(0x64646464u, z, 0x04010400u)) - off);  // k 1, 3
+            v.z = bits(pair(__builtin_amdgcn_perm(0x64646464u, y, 0x04030402u)) - off);  // k 4, 6
+            v.w = bits(pair(__builtin_amdgcn_perm(0x64646464u, z, 0x04030402u)) - off);  // k 5, 7
+            if (!live) v = make_uint4(0u, 0u, 0u, 0u);
+            *(uint4*)(planes + ((int64_t)tile_n * steps_tile + rb * 4 + c) * kBBuf + dst) = v;
+            if (piece == 0 && ((rb * 256 + c * 64) % group) == 0) dtab[((int64_t)tile_n * groups + gi) * TN + col] = in_n ? h2f(sbits) : 0.0f;
+        }
+    }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(256) void gptq_planes_prologue_kernel(const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
+                                                                   const uint32_t* __restrict__ qzeros, int group, int tiles_n128,
+                                                                   uint8_t* __restrict__ planes, float* __restrict__ dtab, int conv,
+                                                                   const AT* __restrict__ a, int k, LhsPlanes p, SplitTiles z) {
+    const int b = (int)blockIdx.x;
+    if (b < conv) {
+        const int rb = b / tiles_n128;
+        planes_from_gptq(b - rb * tiles_n128, rb, qweight, scales, qzeros, z.n, k, group, planes, dtab);
+    } else if (b < conv + z.m) {
+        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv);
+    } else {
+        const int e = b - conv - z.m;
+        zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
+    }
+}
+
 bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     if (kernel_disabled("kquant_planes") || k % 256 || k < 256) return false;
-    if (encoding == QMM_Q4_K) {  // QMM_Q4K_PLANES=1 (read once) sends every Q4_K prefill shape here, for tests and comparisons
+    if (encoding == QMM_Q4_K) {
+        // From this many lhs rows on the conversion pass costs less than the plane GEMM on 256 x 256 tiles gains on the tile
+        // kernel that unpacks as it goes (14336 x 4096 with 2048 rows: 235 + 34 us against 285 + 11 us).  QMM_Q4K_PLANES=1 (read
+        // once) sends every Q4_K prefill shape here, for tests and comparisons.
         static const bool force = getenv("QMM_Q4K_PLANES") != nullptr && atoi(getenv("QMM_Q4K_PLANES")) == 1;
-        return force && m > 16;
+        return m > 16 && (force || (m >= kOptionalPlanesMinRows && wide_tiles(encoding, m, n) && !kernel_disabled("q4k_planes")));
     }
     if (encoding != QMM_Q5_K && encoding != QMM_Q6_K) return false;
     // Below these row counts the passes of the decode kernels (16 lhs rows a pass for Q6_K, 1 to 4 for Q5_K) cost less than
@@ -709,20 +1055,24 @@ bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
 }
 
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    const bool q6 = encoding == QMM_Q6_K;
-    const int64_t lhs = (lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes + 255) / 256 * 256;
-    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6).bytes;
+    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
+    const int64_t nblk_tile = blocks_per_tile(encoding, m, n, k);
+    const int64_t lhs = (lhs_planes(nullptr, lhs_dtype, m, k, TM, nblk_tile * 256).bytes + 255) / 256 * 256;
+    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile).bytes;
 }
 
 hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                               float* out, void* workspace, hipStream_t s) {
-    const bool q6 = encoding == QMM_Q6_K;
+    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
     const int nplanes = q6 ? 2 : 1;
-    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
-    const PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, nplanes, !q6);
-    hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : allow_full_lds<gemm_planes_kernel>();
+    const int nblk = (int)(k / 256), nblk_tile = (int)blocks_per_tile(encoding, m, n, k);
+    const int64_t lda = (int64_t)nblk_tile * 256;
+    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM, lda);
+    const PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, nplanes, !q6 && !wide, nblk_tile);
+    hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : wide ? allow_full_lds<gemm_planes_wide_kernel<4>>() : allow_full_lds<gemm_planes_kernel>();
     if (e != hipSuccess) return e;
-    const int tiles_m = (int)((m + TM - 1) / TM), tiles_n = (int)((n + TN - 1) / TN), nblk = (int)(k / 256);
+    const int tiles_m = (int)((m + TM - 1) / TM), tiles_n128 = (int)((n + TN - 1) / TN);
+    const int tiles_n = wide ? (tiles_n128 + 1) / 2 : tiles_n128;  // the GEMM's column tiles
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
     static int cus = 0;
     if (!cus) {
@@ -731,17 +1081,19 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
             cus = 256;
     }
     const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
-    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, nblk, wg);
+    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, nblk_tile, wg, wide ? 2 * TN : TN);
     const int max_split = z.max_split;
-    const int64_t conv = (int64_t)tiles_n * nblk * 4, blocks = conv + m + (int64_t)max_split * 64;
-    if (blocks > INT32_MAX) return hipErrorInvalidValue;
+    const int64_t conv = (int64_t)tiles_n128 * nblk * 4, blocks = conv + m + (int64_t)max_split * 64;
+    if (blocks > INT32_MAX || lda * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
     const dim3 pgrid((unsigned)blocks);
     auto prologue = [&](auto enc_c) {
         constexpr int ENC = decltype(enc_c)::value;
         if (lhs_dtype == QMM_F32)
-            planes_prologue_kernel<ENC, float><<<pgrid, dim3(256), 0, s>>>(w, nblk, ps.planes, ps.dtab, ps.mtab, (int)conv, (const float*)lhs, (int)k, p, z);
+            planes_prologue_kernel<ENC, float><<<pgrid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv,
+                                                                          (const float*)lhs, (int)k, p, z);
         else
-            planes_prologue_kernel<ENC, uint16_t><<<pgrid, dim3(256), 0, s>>>(w, nblk, ps.planes, ps.dtab, ps.mtab, (int)conv, (const uint16_t*)lhs, (int)k, p, z);
+            planes_prologue_kernel<ENC, uint16_t><<<pgrid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv,
+                                                                             (const uint16_t*)lhs, (int)k, p, z);
     };
     if (q6) prologue(std::integral_constant<int, QMM_Q6_K>{});
     else if (encoding == QMM_Q4_K) prologue(std::integral_constant<int, QMM_Q4_K>{});
@@ -755,9 +1107,66 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
         if (q6)
             gemm_planes2_kernel<<<dim3((unsigned)wg), dim3(512), kPlanes2Lds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k,
                                                                                  tiles_m, tiles_n, pass, split);
+        else if (wide)
+            gemm_planes_wide_kernel<4><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)lda,
+                                                                                         pass == 0 ? nblk_tile : nblk, nblk_tile, tiles_m,
+                                                                                         tiles_n, tiles_n128, pass, split);
         else
             gemm_planes_kernel<<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m, (int)n,
                                                                                (int)k, tiles_m, tiles_n, pass == 0, pass, split);
+    }
+    return hipGetLastError();
+}
+
+// GPTQ through the plane GEMM: groups of 128 or 256 (a scale block is two or four steps), plain groups (no act-order), and
+// enough 256 x 256 tiles that the conversion pass (the weights once) costs less than the GEMM gains.
+bool gemm_gptq_planes_wanted(int64_t m, int64_t n, int64_t k, int group) {
+    if (kernel_disabled("gptq_planes") || (group != 128 && group != 256) || k % 256 || n % 8) return false;
+    return m >= kOptionalPlanesMinRows && wide_tiles(QMM_GPTQ, m, n);
+}
+
+int64_t gemm_gptq_planes_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    const int64_t lhs = (lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes + 255) / 256 * 256;
+    return lhs + plane_space(nullptr, n, k, 1, false, k / 256, k / 128).bytes;  // (tables sized for the smaller group)
+}
+
+hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros,
+                                   int64_t m, int64_t n, int64_t k, int group, float* out, void* workspace, hipStream_t s) {
+    const int groups = (int)(k / group), nblk256 = (int)(k / 256);
+    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
+    // (steps per tile k / 64 = 4 blocks of 256: the plane array is sized in those; the tables in groups)
+    PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, 1, false, nblk256, k / 128);
+    hipError_t e = group == 128 ? allow_full_lds<gemm_planes_wide_kernel<2>>() : allow_full_lds<gemm_planes_wide_kernel<4>>();
+    if (e != hipSuccess) return e;
+    const int tiles_m = (int)((m + TM - 1) / TM), tiles_n128 = (int)((n + TN - 1) / TN), tiles_n = (tiles_n128 + 1) / 2;
+    const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
+    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, groups, wg, 2 * TN);
+    const int64_t conv = (int64_t)tiles_n128 * nblk256, blocks = conv + m + (int64_t)z.max_split * 64;
+    if (blocks > INT32_MAX || k * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
+    if (lhs_dtype == QMM_F32)
+        gptq_planes_prologue_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(qweight, scales, qzeros, group, tiles_n128, ps.planes, ps.dtab,
+                                                                                       (int)conv, (const float*)lhs, (int)k, p, z);
+    else
+        gptq_planes_prologue_kernel<uint16_t><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(qweight, scales, qzeros, group, tiles_n128, ps.planes, ps.dtab,
+                                                                                          (int)conv, (const uint16_t*)lhs, (int)k, p, z);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    for (int pass = 0; pass < (p.a16_lo ? 2 : 1); pass++) {
+        const _Float16* a = pass == 0 ? p.a16 : p.a16_lo;
+        const int split = pass == 0 && z.max_split > 0 ? 1 : 0;
+        if (group == 128)
+            gemm_planes_wide_kernel<2><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k, groups,
+                                                                                         groups, tiles_m, tiles_n, tiles_n128, pass, split);
+        else
+            gemm_planes_wide_kernel<4><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k, groups,
+                                                                                         groups, tiles_m, tiles_n, tiles_n128, pass, split);
     }
     return hipGetLastError();
 }

@@ -1,4 +1,4 @@
-// Pieces shared by the prefill kernels that work on 256 x 128 output tiles with one persistent workgroup per compute
+// Pieces shared by the prefill kernels that work on 256 x 128 (or 256 x 256) output tiles with one persistent workgroup per compute
 // unit: the tile order inside an XCD, and the work units that balance a last, partly filled round of tiles.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -54,9 +54,11 @@ struct SplitTiles {
     float* out;
     int m, n, tiles_m, tiles_n, k_blocks, wgs_per_xcd;
     int max_split;  // largest number of split tiles on any XCD: the zeroing takes max_split * 64 workgroups
+    int tn;         // columns of a tile: 128 or 256
 };
 __device__ __forceinline__ void zero_split_tile_part(const SplitTiles& z, int j, int x, int part) {
-    constexpr int TM = 256, TN = 128;
+    constexpr int TM = 256;
+    const int TN = z.tn;
     const int total = z.tiles_m * z.tiles_n, per_xcd = (total + 7) / 8;
     const int xcd_base = x * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
     int full;
@@ -65,9 +67,10 @@ __device__ __forceinline__ void zero_split_tile_part(const SplitTiles& z, int j,
     int tile_m, tile_n;
     tile_order(xcd_base + full + j, z.tiles_m, z.tiles_n, kTileGm, tile_m, tile_n);
     const int m0 = tile_m * TM + part * (TM / 8), n0 = tile_n * TN;
-    const int col = n0 + ((int)threadIdx.x & 31) * 4;
+    const int per_row = TN / 4;  // threads that cover a row of the tile: 32 or 64
+    const int col = n0 + ((int)threadIdx.x & (per_row - 1)) * 4;
     const bool wide = (z.n & 3) == 0;  // rows start on 16-byte boundaries
-    for (int r = (int)threadIdx.x >> 5; r < TM / 8; r += 8) {
+    for (int r = (int)threadIdx.x / per_row; r < TM / 8; r += 256 / per_row) {
         const int row = m0 + r;
         if (row >= z.m) break;
         float* o = z.out + (int64_t)row * z.n + col;
@@ -80,8 +83,8 @@ __device__ __forceinline__ void zero_split_tile_part(const SplitTiles& z, int j,
     }
 }
 // The split tiles of a launch with `wg` persistent workgroups (host side).
-inline SplitTiles split_tiles(float* out, int64_t m, int64_t n, int tiles_m, int tiles_n, int k_blocks, int wg) {
-    SplitTiles z{out, (int)m, (int)n, tiles_m, tiles_n, k_blocks, wg / 8, 0};
+inline SplitTiles split_tiles(float* out, int64_t m, int64_t n, int tiles_m, int tiles_n, int k_blocks, int wg, int tn = 128) {
+    SplitTiles z{out, (int)m, (int)n, tiles_m, tiles_n, k_blocks, wg / 8, 0, tn};
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
     for (int x = 0; x < 8; x++) {
         const int n_x = per_xcd < total - x * per_xcd ? per_xcd : (total - x * per_xcd > 0 ? total - x * per_xcd : 0);

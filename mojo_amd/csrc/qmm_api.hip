@@ -186,7 +186,7 @@ int static_scratch(void** ws) {
 
 extern "C" {
 
-int qmm_version(void) { return 102; }
+int qmm_version(void) { return 103; }
 
 const char* qmm_last_error(void) { return g_err; }
 
@@ -269,9 +269,25 @@ int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int
         "qmm_quantize_gptq");
 }
 
+// Q4_K and GPTQ have prefill kernels that need no weight planes: the plane GEMM serves them only when the caller's
+// workspace holds the planes (what qmm_matmul_workspace_bytes reports); a smaller workspace gets the other kernel.  The
+// switch is per call and thread: set at the top of qmm_matmul, read by the dispatch and by the size queries under it.
+static thread_local bool g_skip_optional_planes = false;
+struct OptionalPlanesScope {
+    bool prev;
+    explicit OptionalPlanesScope(bool skip) : prev(g_skip_optional_planes) { g_skip_optional_planes = skip; }
+    ~OptionalPlanesScope() { g_skip_optional_planes = prev; }
+};
+static bool kquant_planes(int encoding, int64_t m, int64_t n, int64_t k) {
+    return qmm::gemm_planes_wanted(encoding, m, n, k) && !(encoding == QMM_Q4_K && g_skip_optional_planes);
+}
+static bool gptq_planes(int64_t m, int64_t n, int64_t k, int group) {
+    return !g_skip_optional_planes && qmm::gemm_gptq_planes_wanted(m, n, k, group);
+}
+
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || k <= 0) return 0;
-    if (qmm::gemm_planes_wanted(encoding, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    if (kquant_planes(encoding, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (encoding == QMM_Q4_0) {
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         const int64_t c = qmm::gemm_q4_0_planes_wanted(m, n, k) ? qmm::gemm_q4_0_planes_workspace_bytes(m, n, k) : 0;
@@ -284,7 +300,8 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
         const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k) : 0;
-        return a > b ? a : b;
+        const int64_t c = gptq_planes(m, n, k, 128) ? qmm::gemm_gptq_planes_workspace_bytes(lhs_dtype, m, n, k) : 0;  // (the group size is not known here)
+        return std::max(std::max(a, b), c);
     }
     return 0;
 }
@@ -316,6 +333,10 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
 int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
                int flags, void* stream) {
+    // the plane GEMM for Q4_K / GPTQ only with a workspace that holds the planes
+    const bool optional = (encoding == QMM_Q4_K || encoding == QMM_GPTQ) && m > 0 && n > 0 && k > 0 && !g_skip_optional_planes;
+    const OptionalPlanesScope scope(g_skip_optional_planes ||
+                                    (optional && (!workspace || workspace_bytes < qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags))));
     if (!(flags & QMM_FLAG_OUT_BF16) || (flags & ~(QMM_FLAG_W_BF16 | QMM_FLAG_ACT_Q8K | QMM_FLAG_OUT_BF16)))
         return matmul_f32(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, out, workspace, workspace_bytes, flags, stream);
     // bf16 output
@@ -383,6 +404,10 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
             return QMM_OK;
         }
         // GEMM (128 x 256 tiles) or passes of the small-batch kernel (16 rows each)?
+        if (gptq_planes(m, n, k, cfg->group_size))
+            return hip_status(qmm::launch_gemm_gptq_planes(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1], (const uint32_t*)rhs[2],
+                                                           m, n, k, cfg->group_size, out, workspace, s),
+                              "qmm_matmul(GPTQ planes GEMM)");
         const bool gemm_wins = !gptq_small_batch_wins(lhs_dtype, m, n, k);
         if (m > 16 && qmm::gemm_gptq_supported(k, cfg->group_size) &&
             (gemm_wins || !qmm::gemv_gptq_mm_supported(rhs[0], n, k, cfg->group_size)))
@@ -441,7 +466,7 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         return matmul_f32(encoding, cfg, y, QMM_F32, m, k, rhs, n_rhs, n, out, (char*)workspace + ybytes, workspace_bytes - ybytes, 0, stream);
     }
     // Q5_K and Q6_K with many lhs rows: weights to fp16 integer planes in the workspace, then the matrix cores
-    if (qmm::gemm_planes_wanted(encoding, m, n, k))
+    if (kquant_planes(encoding, m, n, k))
         return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
     // Q5_K with several lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
     if (encoding == QMM_Q5_K && q5k_mm_wanted(m, n, k) && qmm::gemv_q5_k_mm_supported(w, m, n, k))
@@ -555,7 +580,11 @@ int qmm_matmul_rmsnorm(int encoding, const qmm_gptq_config* cfg, const void* x, 
 
 int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                       const void* const* rhs, int n_rhs, int64_t n, float* out, int flags, void* stream) {
-    const int64_t need = qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags);
+    int64_t need = qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags);
+    if (need > (int64_t)QMM_STATIC_SCRATCH_BYTES && (encoding == QMM_Q4_K || encoding == QMM_GPTQ)) {
+        const OptionalPlanesScope no_planes(true);  // the kernels that need no weight planes
+        need = qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags);
+    }
     if (need > (int64_t)QMM_STATIC_SCRATCH_BYTES)
         return fail(QMM_ERR_WORKSPACE,
                     "qmm_matmul_static: this problem needs %lld bytes of scratch and the static buffer holds %lld; "

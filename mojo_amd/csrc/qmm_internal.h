@@ -156,6 +156,11 @@ hipError_t launch_gemm_q4_k_tile(const void* lhs, int lhs_dtype, const uint8_t* 
 // Q5_K and Q6_K (Q4_K on request) on the matrix cores: a pass that turns the weights into fp16 integer planes in the
 // workspace, then a tile GEMM over them.
 bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k);
+// GPTQ through the same GEMM (plain groups of 128 or 256 and large problems only)
+bool gemm_gptq_planes_wanted(int64_t m, int64_t n, int64_t k, int group);
+int64_t gemm_gptq_planes_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k);
+hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros,
+                                   int64_t m, int64_t n, int64_t k, int group, float* out, void* workspace, hipStream_t s);
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                               float* out, void* workspace, hipStream_t s);

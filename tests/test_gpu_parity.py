@@ -727,6 +727,46 @@ def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
     assert torch.equal(got, again)
 
 
+@pytest.mark.parametrize("kind,m,n,k,bf16", [
+    ("Q5_K", 1030, 8200, 2304, False), ("Q4_K", 1600, 8200, 768, True), ("Q4_K", 1540, 4100, 2304, False),
+    ("GPTQ128", 1600, 8200, 768, True), ("GPTQ256", 1540, 8200, 768, False), ("GPTQ128", 1536, 4104, 1280, False)])
+def test_plane_gemm_on_256_wide_tiles(kind, m, n, k, bf16):
+    """Large problems of the single-plane encodings (from 128 tiles of 256 x 256; Q4_K and GPTQ from 1536 lhs rows): the plane GEMM
+    that keeps its accumulators in units of the current scale block's scale.  Q4_K / Q5_K carry their min term as extension
+    blocks (K = 2304: nine super-blocks, a full extension block and one with a single super-block and zeros); GPTQ's scale
+    blocks are its groups (two or four steps; K = 1280 with groups of 128 ends on half a 256-block); ragged m and n; an fp32
+    lhs (second pass on the residual); 233 and 119 tiles (a last round cut in K halves or not).  Every fifth K-quant block has
+    d = 0 with its codes, scales and dmin in place (the weights are then -dmin * mn), every third carries random code and scale bytes."""
+    w, a = synth(81, n, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    if kind.startswith("GPTQ"):
+        group = int(kind[4:])
+        qw, sc, qz, gi = O.quantize_gptq(w, group)
+        sc[::2, ::7] = 0  # groups with a zero scale
+        truth = O.matmul_gptq(a, qw, sc, qz, group=group, f64=True)
+        args = (QE.GPTQ, QuantizationConfig(group_size=group), lhs, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    else:
+        enc = QE[kind]
+        e = ENC[enc]
+        bpb = 176 if enc == QE.Q5_K else 144
+        wq = O.quantize(e, w)
+        blocks = wq.reshape(-1, bpb)
+        rnd = np.random.default_rng(82).integers(0, 256, blocks.shape, dtype=np.uint8)
+        rnd[:, 0:4] = blocks[:, 0:4]  # the fp16 super-block scales stay finite
+        blocks[::3] = rnd[::3]
+        blocks[::5, 0:2] = 0
+        truth = O.matmul_f64(e, a, wq)
+        args = (enc, None, lhs, gpu(wq))
+    got = qmatmul(*args)
+    assert_close(got, truth, f"{kind} wide plane GEMM {m}x{n}x{k} bf16={bf16}")
+    again = qmatmul(*args)
+    assert torch.equal(got, again)
+    # a workspace too small for the planes: Q4_K and GPTQ then run their other prefill kernels, Q5_K has none (64 MiB hold its planes here)
+    assert_close(qmatmul(*args, static_scratch=True), truth, f"{kind} {m}x{n}x{k} with the static scratch")
+
+
 def test_q6_k_prefill_equals_the_decode_kernel_passes():
     """The same product through the planes GEMM (72 rows at once) and through the decode kernel (the rows in three calls
     of at most 64): two summation orders of the same exact products."""
