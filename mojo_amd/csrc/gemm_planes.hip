@@ -528,7 +528,6 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
     // operand reads: row (column) nl of the wavefront's 32-row groups, piece 2 f + g, swizzled; slice f: the address xor f << 5
     const uint32_t fa0 = (uint32_t)(k2OffA + (wm * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const uint32_t fb0 = (uint32_t)(k2OffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
-    const float16v zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const uint32_t lane16 = (uint32_t)(lane * 16);
 
     const int total = tiles_m * tiles_n;
@@ -574,18 +573,17 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
                               (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + k2OffD + wave * 64)));
         };
 
-        float16v acc[2][2], P[2][2];
+        // The accumulators are kept in units of the current super-block's scale (see gemm_planes_wide_kernel below): no second
+        // set for the running super-block.
+        float16v acc[2][2];
 #pragma unroll
         for (int mi = 0; mi < 2; mi++)
 #pragma unroll
             for (int ni = 0; ni < 2; ni++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    acc[mi][ni][r] = 0.0f;
-                    P[mi][ni][r] = 0.0f;
-                }
+                for (int r = 0; r < 16; r++) acc[mi][ni][r] = 0.0f;
         half8 afr[2][2], bfr[2][2][2];  // [slot][row group], [slot][plane][column group]
-        float dcur[2] = {0.f, 0.f};
+        float unit_d[2] = {1.f, 1.f}, ratio[2] = {1.f, 1.f};
 
         // ---- tile prologue
         __syncthreads();  // every wavefront is done with the previous tile's LDS contents
@@ -625,26 +623,31 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
                 for (int mi = 0; mi < 2; mi++)
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
-                        P[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][pl][ni], P[mi][ni], 0, 0, 0);
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][pl][ni], acc[mi][ni], 0, 0, 0);
                         between(pl * 4 + mi * 2 + ni);
                         __builtin_amdgcn_sched_barrier(0);
                     }
         };
-        auto rescale_tile = [&](int t) __attribute__((always_inline)) {
-            const int mi = t >> 1, ni = t & 1;
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[mi][ni][r] = fmaf(dcur[ni], P[mi][ni][r], acc[mi][ni][r]);
-        };
 
         // One phase = from the barrier inside step s - 1 to the barrier inside step s; the buffers of step s are those of index s % 2 = c % 2.
         // All loads of step s + 1 are issued in the first half of the phase, into the buffers that step s - 1 used.
-        auto phase = [&](int blk, auto CC) __attribute__((always_inline)) {
+        // FIRST: the first step of the unit, a variant of its own (see gemm_planes_wide_kernel)
+        auto phase = [&](int blk, auto CC, auto FF) __attribute__((always_inline)) {
             constexpr int c = decltype(CC)::value, cur = c & 1, nxt = cur ^ 1;
+            constexpr bool FIRST = decltype(FF)::value;
             const int s = blk * 4 + c;
             step_bases(cur);
             read_frags(0, 0);
+            if (c == 0) {
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++) {
+                    const float dn = *(const float*)(smem + k2OffD + (wn * 64 + ni * 32 + nl) * 4), un = dn != 0.0f ? dn : unit_d[ni];
+                    ratio[ni] = unit_d[ni] / un;
+                    unit_d[ni] = un;
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
-            if (s > 0) {
+            if constexpr (!FIRST) {
                 mfma_slice(1, [&](int i) __attribute__((always_inline)) {  // last slice of step s - 1
                     if (i & 1) issue_A1(s + 1, nxt, i >> 1);
                 });
@@ -656,33 +659,23 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
             __builtin_amdgcn_sched_barrier(0);
             read_frags(1, 1);
             __builtin_amdgcn_sched_barrier(0);
-            if (c == 0 && s > 0) {
-                // the finished super-block's rescale, sub-tile by sub-tile, in front of the instruction that restarts its P
+            if constexpr (c == 0 && !FIRST) {
+                // the accumulators change unit, sub-tile by sub-tile, in front of the new super-block's first instruction on each
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    rescale_tile(t);
+                    rescale_mul(acc[t >> 1][t & 1], ratio[t & 1]);
                     __builtin_amdgcn_sched_barrier(0);
-                    P[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][0][t & 1], zero16, 0, 0, 0);
+                    acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][0][t & 1], acc[t >> 1][t & 1], 0, 0, 0);
                     issue_B1(s + 1, nxt, t);
                     __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    P[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][1][t & 1], P[t >> 1][t & 1], 0, 0, 0);
+                    acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][1][t & 1], acc[t >> 1][t & 1], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
-                if (c == 0) {  // the first step of the unit: P starts from zero
-#pragma unroll
-                    for (int t = 0; t < 4; t++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) P[t >> 1][t & 1][r] = 0.0f;
-                }
                 mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < 4) issue_B1(s + 1, nxt, i); });
-            }
-            if (c == 0) {
-#pragma unroll
-                for (int ni = 0; ni < 2; ni++) dcur[ni] = *(const float*)(smem + k2OffD + (wn * 64 + ni * 32 + nl) * 4);
             }
             read_frags(2, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -693,15 +686,17 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
             wait_vmcnt<0>();  // lhs and weights of step s + 1 (and, in phase 2, the next scales) have landed
             __syncthreads();
         };
-        for (int blk = 0; blk < nblk; blk++) {
-            phase(blk, std::integral_constant<int, 0>{});
-            phase(blk, std::integral_constant<int, 1>{});
-            phase(blk, std::integral_constant<int, 2>{});
-            phase(blk, std::integral_constant<int, 3>{});
+        phase(0, std::integral_constant<int, 0>{}, std::true_type{});
+        phase(0, std::integral_constant<int, 1>{}, std::false_type{});
+        phase(0, std::integral_constant<int, 2>{}, std::false_type{});
+        phase(0, std::integral_constant<int, 3>{}, std::false_type{});
+        for (int blk = 1; blk < nblk; blk++) {
+            phase(blk, std::integral_constant<int, 0>{}, std::false_type{});
+            phase(blk, std::integral_constant<int, 1>{}, std::false_type{});
+            phase(blk, std::integral_constant<int, 2>{}, std::false_type{});
+            phase(blk, std::integral_constant<int, 3>{}, std::false_type{});
         }
         mfma_slice(1, [](int) __attribute__((always_inline)) {});  // last slice of the last step
-#pragma unroll
-        for (int t = 0; t < 4; t++) rescale_tile(t);
 
         // ---- tile epilogue: undo the row scale, store
         {
@@ -719,7 +714,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
                     const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
                     if (row < m) {
                         float* o_ = out + (int64_t)row * n;
-                        const float v0 = acc[mi][0][r] * is, v1 = acc[mi][1][r] * is;
+                        const float v0 = acc[mi][0][r] * unit_d[0] * is, v1 = acc[mi][1][r] * unit_d[1] * is;
                         if (unit_half) {  // one of the two K halves of this tile: out holds zero or the other half
                             if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
                             if (c1_ok) unsafeAtomicAdd(o_ + col1, v1);
