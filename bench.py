@@ -36,7 +36,7 @@ from mojo_amd import _lib, qmatmul, quantize, quantize_gptq  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
 BF16_PEAK_TFLOPS = 2500.0
-PREFILL_KERNEL = "gemm_q4_k_tile_kernel"
+PREFILL_KERNEL = "planes_prologue_kernel + gemm_planes_wide_kernel"
 
 # (name, N, K) of the Llama-3-8B projections
 PROJ = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
@@ -502,7 +502,7 @@ def prefill_roofline(gen, cus: int, nominal_mhz: float):
             "peak_at_measured_clock": round(peak_at_clock, 1) if peak_at_clock else None,
             "frac_at_measured_clock": round(tf / peak_at_clock, 4) if peak_at_clock else None,
             "workload": f"Q4_K prefill GEMM, bf16 lhs [{mm}, {k}] x Q4_K weights [{n}, {k}], fp32 out; launch_us covers the "
-                        "lhs preparation kernel and the GEMM"}
+                        "preparation kernel (lhs narrowing, weights to fp16 integer planes) and the GEMM"}
 
 
 def calib_main() -> int:
@@ -529,14 +529,14 @@ def prefill_main(args, gen) -> int:
     if args.workload == "prefill":
         call, name, kern = Gemv(QE.Q4_K, make_weight(QE.Q4_K, n, k, gen), ab), "Q4_K", PREFILL_KERNEL
     elif args.workload == "q6k_prefill":
-        call, name, kern = Gemv(QE.Q6_K, make_weight(QE.Q6_K, n, k, gen), ab), "Q6_K", "planes_prologue_kernel + gemm_planes_kernel"
+        call, name, kern = Gemv(QE.Q6_K, make_weight(QE.Q6_K, n, k, gen), ab), "Q6_K", "planes_prologue_kernel + gemm_planes2_kernel"
     elif args.workload == "q40_prefill":
         call, name, kern = Gemv(QE.Q4_0, make_weight(QE.Q4_0, n, k, gen), ab), "Q4_0", "q4_0_planes_prologue_kernel + gemm_q4_0_planes_kernel"
     elif args.workload == "q5k_prefill":
-        call, name, kern = Gemv(QE.Q5_K, make_weight(QE.Q5_K, n, k, gen), ab), "Q5_K", "planes_prologue_kernel + gemm_planes_kernel"
+        call, name, kern = Gemv(QE.Q5_K, make_weight(QE.Q5_K, n, k, gen), ab), "Q5_K", "planes_prologue_kernel + gemm_planes_wide_kernel"
     else:
         wg = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
-        call, name, kern = GptqMatmul(wg, ab), "GPTQ g128", "gemm_gptq_kernel"
+        call, name, kern = GptqMatmul(wg, ab), "GPTQ g128", "gptq_planes_prologue_kernel + gemm_planes_wide_kernel"
     g = capture([call])
     dev_s, wall_s = time_graphs([g], steps, warmup)
     us = dev_s * 1e6 / steps
@@ -547,11 +547,11 @@ def prefill_main(args, gen) -> int:
         "steps": steps, "warmup": warmup, "ms_per_step": round(us / 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 products, f32 sums", "data": "synthetic",
         "config": {"workload": f"{name} prefill GEMM, bf16 lhs [{mm}, {k}] x weights [{n}, {k}], fp32 out; one step = "
-                               f"lhs preparation (for Q5_K / Q6_K also the weight conversion) + one GEMM launch", "m": mm, "n": n, "k": k},
+                               f"one preparation launch (lhs narrowing, weights to fp16 integer planes) + one GEMM launch", "m": mm, "n": n, "k": k},
         "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": None, "kernel": kern,
                      "flops_per_launch": flops, "launch_us": round(us, 2),
-                     "note": "launch_us includes the preparation kernel (lhs narrowing; for Q5_K / Q6_K also the weight planes)"},
+                     "note": "launch_us includes the preparation kernel (lhs narrowing, weight planes)"},
         "cpu_baseline": None,
     }))
     return 0
