@@ -60,17 +60,6 @@ __device__ __forceinline__ void rescale_add(float16v& acc, float g, const float1
     }
 }
 
-// acc *= g in place, for the same reasons (and with the same idle states in front).
-__device__ __forceinline__ void rescale_mul(float16v& acc, float g) {
-    asm volatile("s_nop 7\n\ts_nop 3");
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        float t = acc[r];
-        asm volatile("v_mul_f32 %0, %0, %1" : "+v"(t) : "v"(g));
-        acc[r] = t;
-    }
-}
-
 // Operand orders inside every 64-wide chunk of a row; position f*16 + g*8 + slot holds column
 //   kLhsOrderQ4K : 32*(f/2) + 16*g + 8*(f%2) + (0,2,1,3,4,6,5,7)[slot]
 //   kLhsOrderGPTQ: 16*f + 8*g + (0,4,1,5,2,6,3,7)[slot], odd columns pre-multiplied by 1/16

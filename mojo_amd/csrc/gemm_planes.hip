@@ -529,6 +529,12 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
     const uint32_t fa0 = (uint32_t)(k2OffA + (wm * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const uint32_t fb0 = (uint32_t)(k2OffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const uint32_t lane16 = (uint32_t)(lane * 16);
+    uint32_t fax[4], fbx[4];
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        fax[f] = fa0 ^ (uint32_t)(f << 5);
+        fbx[f] = fb0 ^ (uint32_t)(f << 5);
+    }
 
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
@@ -551,12 +557,12 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
         const uint8_t* d_base = (const uint8_t*)dtab + ((int64_t)tile_n * nblk_row + kb0) * kDBuf;
 
         // the i-th of the four loads that bring this wavefront's 32 rows of the lhs of step `step` into buffer `buf`
+        // lhs rows wave * 32 + 8 i + lane / 8; LDS position lane % 8 of a row holds piece (lane % 8) ^ ((row / 2) % 8)
+        uint32_t a_offs[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) a_offs[i] = (uint32_t)((lane >> 3) * (k * 2) + (((lane & 7) ^ ((4 * i + (lane >> 4)) & 7)) << 4));
         auto issue_A1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
-            // lhs rows wave * 32 + 8 i + lane / 8; LDS position lane % 8 of a row holds piece (lane % 8) ^ ((row / 2) % 8).  The lane
-            // offset is recomputed at every use (behind an empty asm statement): kept in a register of its own it gets spilled.
-            int l = lane;
-            asm volatile("" : "+v"(l));
-            const uint32_t a_off = (uint32_t)((l >> 3) * (k * 2) + (((l & 7) ^ ((4 * i + (l >> 4)) & 7)) << 4));
+            const uint32_t a_off = a_offs[i & 1];
             const uint32_t dst = lds0 + k2OffA + buf * kABuf + wave * 4096;
             load16_to_lds(a_off, a_base + (int64_t)min(step, ns - 1) * 128 + (int64_t)i * 16 * k,
                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
@@ -596,24 +602,15 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
         wait_vmcnt<0>();
         __syncthreads();
 
-        // Operand addresses of the current step: recomputed every phase from the buffer offsets behind an empty asm statement
-        // (left to itself the compiler keeps the addresses of every (phase, slice, operand) in registers of their own, spills them
-        // and reloads them inside the loop, and every reload waits for all outstanding global -> LDS loads).
-        uint32_t fa = 0, fb = 0;
-        auto step_bases = [&](int buf) __attribute__((always_inline)) {
-            int ao = buf * kABuf, bo = buf * 2 * kBBuf;
-            asm volatile("" : "+s"(ao), "+s"(bo));
-            fa = fa0 + (uint32_t)ao;
-            fb = fb0 + (uint32_t)bo;
-        };
-        auto read_frags = [&](int f, int slot) __attribute__((always_inline)) {
-            const uint32_t xa = fa ^ (uint32_t)(f << 5), xb = fb ^ (uint32_t)(f << 5);
+        // operand addresses of the four slices (the slice index is xor-ed into the swizzled piece index), buffer 0: eight registers;
+        // buffer, row group, plane and column group are immediate offsets of the reads
+        auto read_frags = [&](int buf, int f, int slot) __attribute__((always_inline)) {
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + xa + mi * 4096);
+            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + fax[f] + (buf * kABuf + mi * 4096));
 #pragma unroll
             for (int pl = 0; pl < 2; pl++)
 #pragma unroll
-                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + xb + pl * kBBuf + ni * 4096);
+                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + fbx[f] + (buf * 2 * kBBuf + pl * kBBuf + ni * 4096));
         };
         // the eight matrix-core instructions of one slice (both planes); `between(i)` is placed after the i-th of them
         auto mfma_slice = [&](int slot, auto&& between) __attribute__((always_inline)) {
@@ -636,13 +633,12 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
             constexpr int c = decltype(CC)::value, cur = c & 1, nxt = cur ^ 1;
             constexpr bool FIRST = decltype(FF)::value;
             const int s = blk * 4 + c;
-            step_bases(cur);
-            read_frags(0, 0);
+            read_frags(cur, 0, 0);
             if (c == 0) {
 #pragma unroll
                 for (int ni = 0; ni < 2; ni++) {
                     const float dn = *(const float*)(smem + k2OffD + (wn * 64 + ni * 32 + nl) * 4), un = dn != 0.0f ? dn : unit_d[ni];
-                    ratio[ni] = unit_d[ni] / un;
+                    ratio[ni] = unit_d[ni] * __builtin_amdgcn_rcpf(un);  // (one ulp off at most: 2e-7 relative per super-block)
                     unit_d[ni] = un;
                 }
             }
@@ -657,13 +653,14 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
             }
             if constexpr (c == 2) issue_D(blk + 1);  // (the current scales were read in phase 0)
             __builtin_amdgcn_sched_barrier(0);
-            read_frags(1, 1);
+            read_frags(cur, 1, 1);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (c == 0 && !FIRST) {
                 // the accumulators change unit, sub-tile by sub-tile, in front of the new super-block's first instruction on each
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    rescale_mul(acc[t >> 1][t & 1], ratio[t & 1]);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[t >> 1][t & 1][r] *= ratio[t & 1];
                     __builtin_amdgcn_sched_barrier(0);
                     acc[t >> 1][t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][t >> 1], bfr[0][0][t & 1], acc[t >> 1][t & 1], 0, 0, 0);
                     issue_B1(s + 1, nxt, t);
@@ -677,10 +674,10 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
             } else {
                 mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < 4) issue_B1(s + 1, nxt, i); });
             }
-            read_frags(2, 0);
+            read_frags(cur, 2, 0);
             __builtin_amdgcn_sched_barrier(0);
             mfma_slice(1, [](int) __attribute__((always_inline)) {});
-            read_frags(3, 1);
+            read_frags(cur, 3, 1);
             __builtin_amdgcn_sched_barrier(0);
             mfma_slice(0, [](int) __attribute__((always_inline)) {});
             wait_vmcnt<0>();  // lhs and weights of step s + 1 (and, in phase 2, the next scales) have landed
@@ -760,6 +757,12 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
     const uint32_t fa0 = (uint32_t)(kwOffA + (wm * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const uint32_t fb0 = (uint32_t)(kwOffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const uint32_t lane16 = (uint32_t)(lane * 16);
+    uint32_t fax[4], fbx[4];
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        fax[f] = fa0 ^ (uint32_t)(f << 5);
+        fbx[f] = fb0 ^ (uint32_t)(f << 5);
+    }
 
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
@@ -785,10 +788,11 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
         const int64_t dtile = (int64_t)nblk_tile * kDBuf;
         const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * 2 * dtile + (int64_t)kb0 * kDBuf;
 
+        uint32_t a_offs[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) a_offs[i] = (uint32_t)((lane >> 3) * (lda * 2) + (((lane & 7) ^ ((4 * i + (lane >> 4)) & 7)) << 4));
         auto issue_A1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
-            int l = lane;
-            asm volatile("" : "+v"(l));
-            const uint32_t a_off = (uint32_t)((l >> 3) * (lda * 2) + (((l & 7) ^ ((4 * i + (l >> 4)) & 7)) << 4));
+            const uint32_t a_off = a_offs[i & 1];
             const uint32_t dst = lds0 + kwOffA + buf * kABuf + wave * 4096;
             load16_to_lds(a_off, a_base + (int64_t)min(step, ns - 1) * 128 + (int64_t)i * 16 * lda,
                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
@@ -834,21 +838,15 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
         wait_vmcnt<0>();
         __syncthreads();
 
-        uint32_t fa = 0, fb = 0;
-        auto step_bases = [&](int buf) __attribute__((always_inline)) {
-            int ao = buf * kABuf, bo = buf * 2 * kBBuf;
-            asm volatile("" : "+s"(ao), "+s"(bo));
-            fa = fa0 + (uint32_t)ao;
-            fb = fb0 + (uint32_t)bo;
-        };
-        auto read_frags = [&](int f, int slot) __attribute__((always_inline)) {
-            const uint32_t xa = fa ^ (uint32_t)(f << 5), xb = fb ^ (uint32_t)(f << 5);
+        // operand addresses of the four slices (the slice index is xor-ed into the swizzled piece index), buffer 0: eight registers;
+        // buffer, row group, half and column group are immediate offsets of the reads
+        auto read_frags = [&](int buf, int f, int slot) __attribute__((always_inline)) {
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + xa + mi * 4096);
+            for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + fax[f] + (buf * kABuf + mi * 4096));
 #pragma unroll
             for (int pl = 0; pl < 2; pl++)
 #pragma unroll
-                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + xb + pl * kBBuf + ni * 4096);
+                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + fbx[f] + (buf * 2 * kBBuf + pl * kBBuf + ni * 4096));
         };
         auto mfma_slice = [&](int slot, auto&& between) __attribute__((always_inline)) {
 #pragma unroll
@@ -869,8 +867,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
             constexpr int c = decltype(CC)::value, cur = c & 1, nxt = cur ^ 1;
             constexpr bool FIRST = decltype(FF)::value;
             const int s = blk * SPB + c;
-            step_bases(cur);
-            read_frags(0, 0);
+            read_frags(cur, 0, 0);
             if (c == 0) {
                 // the new super-block's unit: its scale, or the previous unit where the scale is zero
 #pragma unroll
@@ -878,7 +875,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
 #pragma unroll
                     for (int ni = 0; ni < 2; ni++) {
                         const float dn = d_at(pl, ni), un = dn != 0.0f ? dn : unit_d[pl][ni];
-                        ratio[pl][ni] = unit_d[pl][ni] / un;
+                        ratio[pl][ni] = unit_d[pl][ni] * __builtin_amdgcn_rcpf(un);  // (one ulp off at most: 2e-7 relative per block)
                         unit_d[pl][ni] = un;
                     }
             }
@@ -893,14 +890,15 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
             }
             if constexpr (c == 1) issue_D(blk + 1);  // (the current scales were read in phase 0)
             __builtin_amdgcn_sched_barrier(0);
-            read_frags(1, 1);
+            read_frags(cur, 1, 1);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (c == 0 && !FIRST) {
                 // the accumulators change unit, sub-tile by sub-tile, in front of the new super-block's first instruction on each
 #pragma unroll
                 for (int t = 0; t < 8; t++) {
                     const int pl = t >> 2, mi = (t >> 1) & 1, ni = t & 1;
-                    rescale_mul(acc[pl][mi][ni], ratio[pl][ni]);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[pl][mi][ni][r] *= ratio[pl][ni];
                     __builtin_amdgcn_sched_barrier(0);
                     acc[pl][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][mi], bfr[0][pl][ni], acc[pl][mi][ni], 0, 0, 0);
                     if (t < 4) issue_B1(s + 1, nxt, t);
@@ -909,10 +907,10 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
             } else {
                 mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < 4) issue_B1(s + 1, nxt, i); });
             }
-            read_frags(2, 0);
+            read_frags(cur, 2, 0);
             __builtin_amdgcn_sched_barrier(0);
             mfma_slice(1, [](int) __attribute__((always_inline)) {});
-            read_frags(3, 1);
+            read_frags(cur, 3, 1);
             __builtin_amdgcn_sched_barrier(0);
             mfma_slice(0, [](int) __attribute__((always_inline)) {});
             wait_vmcnt<0>();  // lhs and weights of step s + 1 (and, in phase 1, the next scales) have landed
