@@ -741,12 +741,16 @@ constexpr int kwOffA = 0, kwOffB = 2 * kABuf, kwOffD = kwOffB + 4 * kBBuf, kwOff
 static_assert(kPlanesWLds <= kLdsPerCu, "wide kernel LDS");
 }  // namespace
 
-template <int SPB>  // steps (of 64 k) per scale block: 4 for the K-quants, 2 for GPTQ groups of 128
+// SPB: steps (of 64 k) per scale block: 4 for the K-quants, 2 for GPTQ groups of 128.  NG: 32-column groups per wavefront: 4 for
+// the 256 x 256 tile, 3 for a 256 x 192 tile (a launch of those finishes a problem whose last round of 256 x 256 tiles would
+// leave a quarter or more of the compute units idle).  The launch covers the columns from n_begin (a multiple of 64) on.
+template <int SPB, int NG>
 __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t* __restrict__ planes, const float* __restrict__ dtab,
                                                                  const _Float16* __restrict__ a16, const float* __restrict__ inv,
                                                                  float* __restrict__ out, int m, int n, int lda, int nblk_walk,
-                                                                 int nblk_tile, int tiles_m, int tiles_n, int tiles_n128, int accumulate,
-                                                                 int allow_split) {
+                                                                 int nblk_tile, int tiles_m, int tiles_n, int tiles_n128, int n_begin,
+                                                                 int accumulate, int allow_split) {
+    constexpr int TW = NG * 64;  // columns of a tile
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = lds_address(smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -754,8 +758,10 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
     const int wm = wave >> 1, wn = wave & 1;
     const int nl = lane & 31, g = lane >> 5;
     const int nblk_row = nblk_walk;  // blocks of a full unit; nblk_tile: blocks per 128-column tile in the planes and tables
+    // operand reads: row (column) nl of the wavefront's 32-row groups, piece 2 f + g, swizzled; slice f: the address xor f << 5.
+    // The weight tile sits in LDS as TW rows of 128 bytes; the wavefront's columns are wn * 32 NG + 32 j + nl.
     const uint32_t fa0 = (uint32_t)(kwOffA + (wm * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
-    const uint32_t fb0 = (uint32_t)(kwOffB + (wn * 64 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
+    const uint32_t fb0 = (uint32_t)(kwOffB + (wn * NG * 32 + nl) * 128 + ((g ^ ((nl >> 1) & 7)) << 4));
     const uint32_t lane16 = (uint32_t)(lane * 16);
     uint32_t fax[4], fbx[4];
 #pragma unroll
@@ -763,6 +769,8 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
         fax[f] = fa0 ^ (uint32_t)(f << 5);
         fbx[f] = fb0 ^ (uint32_t)(f << 5);
     }
+    const int64_t plane_bytes = (int64_t)nblk_tile * SPB * kBBuf;  // the plane of one 128-column tile
+    const int64_t dtile = (int64_t)nblk_tile * kDBuf;             // its scales
 
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
@@ -777,17 +785,9 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
         tile_order(unit.tile, tiles_m, tiles_n, kTileGm, tile_m, tile_n);
         tile_m = __builtin_amdgcn_readfirstlane(tile_m);
         tile_n = __builtin_amdgcn_readfirstlane(tile_n);
-        const int m0 = tile_m * TM, n0 = tile_n * 2 * TN;
-        // the second half of the tile is the next 128-column tile of the planes (the same one again at a ragged edge: its columns
-        // lie beyond n and are not stored)
-        const int second = __builtin_amdgcn_readfirstlane(min(tile_n * 2 + 1, tiles_n128 - 1) - tile_n * 2);
+        const int m0 = tile_m * TM, n0 = n_begin + tile_n * TW;
 
         const uint8_t* a_base = (const uint8_t*)a16 + ((int64_t)(m0 + wave * 32) * lda + (int64_t)kb0 * (SPB * 64)) * 2;
-        const int64_t plane_bytes = (int64_t)nblk_tile * SPB * kBBuf;  // the plane of one 128-column tile
-        const uint8_t* b_base = planes + (int64_t)tile_n * 2 * plane_bytes + (int64_t)kb0 * SPB * kBBuf;
-        const int64_t dtile = (int64_t)nblk_tile * kDBuf;
-        const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * 2 * dtile + (int64_t)kb0 * kDBuf;
-
         uint32_t a_offs[2];
 #pragma unroll
         for (int i = 0; i < 2; i++) a_offs[i] = (uint32_t)((lane >> 3) * (lda * 2) + (((lane & 7) ^ ((4 * i + (lane >> 4)) & 7)) << 4));
@@ -797,35 +797,40 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
             load16_to_lds(a_off, a_base + (int64_t)min(step, ns - 1) * 128 + (int64_t)i * 16 * lda,
                           (uint32_t)__builtin_amdgcn_readfirstlane((int)(dst + i * 1024)));
         };
-        // the i-th (0..3) of this wavefront's four 1 KB pieces of the two weight tiles of step `step`: half i / 2, piece 2 wave + i % 2
+        // This wavefront's NG pieces of 1 KB (eight columns) of the weight tile: piece NG wave + i.  A piece lies inside one
+        // 128-column tile of the planes (at a ragged edge the last one again: those columns lie beyond n and are not stored).
+        const uint8_t* b_src[NG];
+#pragma unroll
+        for (int i = 0; i < NG; i++) {
+            const int c = n0 + (wave * NG + i) * 8;
+            b_src[i] = planes + (int64_t)min(c >> 7, tiles_n128 - 1) * plane_bytes + (int64_t)kb0 * SPB * kBBuf + (c & 127) * 128;
+        }
         auto issue_B1 = [&](int step, int buf, int i) __attribute__((always_inline)) {
-            const int pl = i >> 1, piece = (wave * 2 + (i & 1)) * 1024;
-            load16_to_lds(lane16, b_base + pl * second * plane_bytes + (int64_t)min(step, ns - 1) * kBBuf + piece,
-                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kwOffB + (buf * 2 + pl) * kBBuf + piece)));
+            load16_to_lds(lane16, b_src[i] + (int64_t)min(step, ns - 1) * kBBuf,
+                          (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kwOffB + buf * 2 * kBBuf + (wave * NG + i) * 1024)));
         };
-        // the 256 scales of super-block blk: lanes 0..3 bring this wavefront's sixteen of the first half, lanes 4..7 of the second
+        // the TW scales of block blk, in column order: lanes 0..7 of the first 2 NG wavefronts bring 32 each
+        const uint32_t d_voff = [&] {
+            const int c = n0 + wave * 32 + (lane & 7) * 4;
+            return (uint32_t)min(c >> 7, tiles_n128 - 1) * (uint32_t)dtile + (uint32_t)((c & 127) * 4);
+        }();
+        const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)kb0 * kDBuf;
         auto issue_D = [&](int blk) __attribute__((always_inline)) {
-            if (lane < 8) {
-                int l = lane;
-                asm volatile("" : "+v"(l));
-                load16_to_lds((uint32_t)((l & 3) * 16) + (uint32_t)((l >> 2) * second) * (uint32_t)dtile,
-                              d_base + (int64_t)min(blk, nblk - 1) * kDBuf + wave * 64,
+            if (wave < 2 * NG && lane < 8)
+                load16_to_lds(d_voff, d_base + (int64_t)min(blk, nblk - 1) * kDBuf,
                               (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + kwOffD + wave * 128)));
-            }
         };
-        // scale of column c (0..127) of half pl, as issue_D leaves them: [c / 16][pl][c % 16]
-        auto d_at = [&](int pl, int ni) __attribute__((always_inline)) {
-            const int c = wn * 64 + ni * 32 + nl;
-            return *(const float*)(smem + kwOffD + ((c >> 4) * 32 + pl * 16 + (c & 15)) * 4);
-        };
+        auto d_at = [&](int j) __attribute__((always_inline)) { return *(const float*)(smem + kwOffD + (wn * NG * 32 + j * 32 + nl) * 4); };
 
-        float16v acc[2][2][2];  // [half][row group][column group]
+        float16v acc[NG][2];  // [column group][row group]
 #pragma unroll
-        for (int t = 0; t < 8; t++)
+        for (int t = 0; t < 2 * NG; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[t >> 2][(t >> 1) & 1][t & 1][r] = 0.0f;
-        half8 afr[2][2], bfr[2][2][2];  // [slot][row group], [slot][half][column group]
-        float unit_d[2][2] = {{1.f, 1.f}, {1.f, 1.f}}, ratio[2][2] = {{1.f, 1.f}, {1.f, 1.f}};
+            for (int r = 0; r < 16; r++) acc[t >> 1][t & 1][r] = 0.0f;
+        half8 afr[2][2], bfr[2][NG];  // [slot][row group], [slot][column group]
+        float unit_d[NG], ratio[NG];
+#pragma unroll
+        for (int j = 0; j < NG; j++) unit_d[j] = ratio[j] = 1.0f;
 
         // ---- tile prologue
         __syncthreads();  // every wavefront is done with the previous tile's LDS contents
@@ -833,34 +838,33 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
 #pragma unroll
         for (int i = 0; i < 4; i++) issue_A1(0, 0, i);
 #pragma unroll
-        for (int i = 0; i < 4; i++) issue_B1(0, 0, i);
+        for (int i = 0; i < NG; i++) issue_B1(0, 0, i);
         if (tid < TM) *(float*)(smem + kwOffInv + tid * 4) = inv[min(m0 + tid, m - 1)];
         wait_vmcnt<0>();
         __syncthreads();
 
         // operand addresses of the four slices (the slice index is xor-ed into the swizzled piece index), buffer 0: eight registers;
-        // buffer, row group, half and column group are immediate offsets of the reads
+        // buffer, row group and column group are immediate offsets of the reads
         auto read_frags = [&](int buf, int f, int slot) __attribute__((always_inline)) {
 #pragma unroll
             for (int mi = 0; mi < 2; mi++) afr[slot][mi] = *(const half8*)(smem + fax[f] + (buf * kABuf + mi * 4096));
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++)
-#pragma unroll
-                for (int ni = 0; ni < 2; ni++) bfr[slot][pl][ni] = *(const half8*)(smem + fbx[f] + (buf * 2 * kBBuf + pl * kBBuf + ni * 4096));
+            for (int j = 0; j < NG; j++) bfr[slot][j] = *(const half8*)(smem + fbx[f] + (buf * 2 * kBBuf + j * 4096));
         };
+        // the 2 NG matrix-core instructions of one slice; `between(i)` is placed after the i-th of them
         auto mfma_slice = [&](int slot, auto&& between) __attribute__((always_inline)) {
 #pragma unroll
-            for (int pl = 0; pl < 2; pl++)
+            for (int j = 0; j < NG; j++)
 #pragma unroll
-                for (int mi = 0; mi < 2; mi++)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ni++) {
-                        acc[pl][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][pl][ni], acc[pl][mi][ni], 0, 0, 0);
-                        between(pl * 4 + mi * 2 + ni);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+                for (int mi = 0; mi < 2; mi++) {
+                    acc[j][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[slot][mi], bfr[slot][j], acc[j][mi], 0, 0, 0);
+                    between(j * 2 + mi);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
         };
 
+        // One phase = from the barrier inside step s - 1 to the barrier inside step s; the buffers of step s are those of index s % 2.
+        // All loads of step s + 1 are issued in the first half of the phase, into the buffers that step s - 1 used.
         // FIRST: the first step of the unit (nothing to finish, nothing to rescale), a variant of its own so that the loop body
         // has no branches around matrix-core instructions (the compiler copies accumulators where they meet).
         auto phase = [&](int blk, auto CC, auto FF) __attribute__((always_inline)) {
@@ -869,20 +873,25 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
             const int s = blk * SPB + c;
             read_frags(cur, 0, 0);
             if (c == 0) {
-                // the new super-block's unit: its scale, or the previous unit where the scale is zero
+                // the new block's unit: its scale, or the previous unit where the scale is zero
 #pragma unroll
-                for (int pl = 0; pl < 2; pl++)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ni++) {
-                        const float dn = d_at(pl, ni), un = dn != 0.0f ? dn : unit_d[pl][ni];
-                        ratio[pl][ni] = unit_d[pl][ni] * __builtin_amdgcn_rcpf(un);  // (one ulp off at most: 2e-7 relative per block)
-                        unit_d[pl][ni] = un;
-                    }
+                for (int j = 0; j < NG; j++) {
+                    const float dn = d_at(j), un = dn != 0.0f ? dn : unit_d[j];
+                    ratio[j] = unit_d[j] * __builtin_amdgcn_rcpf(un);  // (one ulp off at most: 2e-7 relative per block)
+                    unit_d[j] = un;
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (!FIRST) {
                 mfma_slice(1, [&](int i) __attribute__((always_inline)) {  // last slice of step s - 1
-                    if (i & 1) issue_A1(s + 1, nxt, i >> 1);
+                    if constexpr (NG == 4) {
+                        if (i & 1) issue_A1(s + 1, nxt, i >> 1);
+                    } else {
+                        if (i == 0) issue_A1(s + 1, nxt, 0);
+                        if (i == 2) issue_A1(s + 1, nxt, 1);
+                        if (i == 3) issue_A1(s + 1, nxt, 2);
+                        if (i == 5) issue_A1(s + 1, nxt, 3);
+                    }
                 });
             } else {
 #pragma unroll
@@ -893,19 +902,19 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
             read_frags(cur, 1, 1);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (c == 0 && !FIRST) {
-                // the accumulators change unit, sub-tile by sub-tile, in front of the new super-block's first instruction on each
+                // the accumulators change unit, sub-tile by sub-tile, in front of the new block's first instruction on each
 #pragma unroll
-                for (int t = 0; t < 8; t++) {
-                    const int pl = t >> 2, mi = (t >> 1) & 1, ni = t & 1;
+                for (int t = 0; t < 2 * NG; t++) {
+                    const int j = t >> 1, mi = t & 1;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) acc[pl][mi][ni][r] *= ratio[pl][ni];
+                    for (int r = 0; r < 16; r++) acc[j][mi][r] *= ratio[j];
                     __builtin_amdgcn_sched_barrier(0);
-                    acc[pl][mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][mi], bfr[0][pl][ni], acc[pl][mi][ni], 0, 0, 0);
-                    if (t < 4) issue_B1(s + 1, nxt, t);
+                    acc[j][mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afr[0][mi], bfr[0][j], acc[j][mi], 0, 0, 0);
+                    if (t < NG) issue_B1(s + 1, nxt, t);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
-                mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < 4) issue_B1(s + 1, nxt, i); });
+                mfma_slice(0, [&](int i) __attribute__((always_inline)) { if (i < NG) issue_B1(s + 1, nxt, i); });
             }
             read_frags(cur, 2, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -933,39 +942,102 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_wide_kernel(const uint8_t*
         }
         mfma_slice(1, [](int) __attribute__((always_inline)) {});  // last slice of the last step
 
-        // ---- tile epilogue: back to true units (last super-block's scale, row scale), store
+        // ---- tile epilogue: back to true units (last block's scale, row scale), store
 #pragma unroll
-        for (int pl = 0; pl < 2; pl++) {
-            const int col0 = n0 + pl * TN + wn * 64 + nl, col1 = col0 + 32;
-            const bool c0_ok = col0 < n, c1_ok = col1 < n;
+        for (int mi = 0; mi < 2; mi++) {
+            float4 iv[4];
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++) {
-                float4 iv[4];
+            for (int q = 0; q < 4; q++) iv[q] = *(const float4*)(smem + kwOffInv + (wm * 64 + mi * 32 + 8 * q + 4 * g) * 4);
 #pragma unroll
-                for (int j = 0; j < 4; j++) iv[j] = *(const float4*)(smem + kwOffInv + (wm * 64 + mi * 32 + 8 * j + 4 * g) * 4);
+            for (int j = 0; j < NG; j++) {
+                const int col = n0 + wn * NG * 32 + j * 32 + nl;
+                const bool col_ok = col < n;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
                     const float4 q = iv[r >> 2];
                     const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
-                    if (row < m) {
-                        float* o_ = out + (int64_t)row * n;
-                        const float v0 = acc[pl][mi][0][r] * unit_d[pl][0] * is, v1 = acc[pl][mi][1][r] * unit_d[pl][1] * is;
-                        if (unit_half) {  // one of the two K parts of this tile: out holds zero or the other part
-                            if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
-                            if (c1_ok) unsafeAtomicAdd(o_ + col1, v1);
-                        } else if (accumulate) {
-                            if (c0_ok) o_[col0] += v0;
-                            if (c1_ok) o_[col1] += v1;
-                        } else {
-                            if (c0_ok) __builtin_nontemporal_store(v0, o_ + col0);
-                            if (c1_ok) __builtin_nontemporal_store(v1, o_ + col1);
-                        }
+                    if (row < m && col_ok) {
+                        float* o_ = out + (int64_t)row * n + col;
+                        const float v = acc[j][mi][r] * unit_d[j] * is;
+                        if (unit_half) unsafeAtomicAdd(o_, v);  // one of the two K parts of this tile: out holds zero or the other part
+                        else if (accumulate) *o_ += v;
+                        else __builtin_nontemporal_store(v, o_);
                     }
                 }
             }
         }
     }
+}
+
+// How a problem is cut into launches of the wide kernel.  All 256 x 256 tiles, unless the last round of those would leave
+// a quarter or more of the compute units idle while 256 x 192 tiles over the remaining columns fit one round: then the
+// first launch takes whole rounds of 256 x 256 tiles (`wide_strips` column strips), the second the rest as 256 x 192 tiles.
+struct WidePlan {
+    int wide_strips;    // 256-column strips of the first launch
+    int narrow_strips;  // 192-column strips of the second launch (0: one launch)
+};
+WidePlan wide_plan(int64_t m, int64_t n, int cus) {
+    const int tiles_m = (int)((m + TM - 1) / TM), strips = (int)((n + 2 * TN - 1) / (2 * TN));
+    const int total = tiles_m * strips, rounds = total / cus, rem = total - rounds * cus;
+    WidePlan p{strips, 0};
+    if (rounds == 0 || rem == 0 || 4 * rem > 3 * cus || (rounds * cus) % tiles_m != 0 || kernel_disabled("planes_192")) return p;
+    const int first = rounds * cus / tiles_m;
+    const int64_t rest = n - (int64_t)first * 2 * TN;
+    const int narrow = (int)((rest + 191) / 192);
+    if (rest <= 0 || tiles_m * narrow > cus) return p;
+    p.wide_strips = first;
+    p.narrow_strips = narrow;
+    return p;
+}
+
+int compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    return cus;
+}
+
+// The launches of the wide kernel for one lhs plane.  `z` is what the preparation launch zeroes (split tiles of a single launch;
+// a problem cut into two launches splits none).
+struct WideLaunch {
+    WidePlan plan;
+    int tiles_m, tiles_n128, wg;
+    SplitTiles z;
+};
+WideLaunch wide_launch(float* out, int64_t m, int64_t n, int blocks_walked) {
+    WideLaunch L;
+    const int cus = compute_units();
+    L.plan = wide_plan(m, n, cus);
+    L.tiles_m = (int)((m + TM - 1) / TM);
+    L.tiles_n128 = (int)((n + TN - 1) / TN);
+    const int total = L.tiles_m * L.plan.wide_strips;
+    L.wg = 8 * std::min((total + 7) / 8, std::max(1, cus / 8));
+    L.z = split_tiles(out, m, n, L.tiles_m, L.plan.wide_strips, blocks_walked, L.wg, 2 * TN);
+    if (L.plan.narrow_strips) L.z.max_split = 0;
+    return L;
+}
+template <int SPB>
+hipError_t run_wide(const WideLaunch& L, const uint8_t* planes, const float* dtab, const _Float16* a, const float* inv, float* out, int64_t m,
+                    int64_t n, int64_t lda, int nblk_walk, int nblk_tile, int pass, hipStream_t s) {
+    hipError_t e = allow_full_lds<gemm_planes_wide_kernel<SPB, 4>>();
+    if (e == hipSuccess && L.plan.narrow_strips) e = allow_full_lds<gemm_planes_wide_kernel<SPB, 3>>();
+    if (e != hipSuccess) return e;
+    const int split = pass == 0 && L.z.max_split > 0 ? 1 : 0;
+    gemm_planes_wide_kernel<SPB, 4><<<dim3((unsigned)L.wg), dim3(512), kPlanesWLds, s>>>(planes, dtab, a, inv, out, (int)m, (int)n, (int)lda, nblk_walk,
+                                                                                        nblk_tile, L.tiles_m, L.plan.wide_strips, L.tiles_n128, 0,
+                                                                                        pass, split);
+    if (L.plan.narrow_strips) {
+        const int total = L.tiles_m * L.plan.narrow_strips;
+        const int wg = 8 * std::min((total + 7) / 8, std::max(1, compute_units() / 8));
+        gemm_planes_wide_kernel<SPB, 3><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(planes, dtab, a, inv, out, (int)m, (int)n, (int)lda, nblk_walk,
+                                                                                          nblk_tile, L.tiles_m, L.plan.narrow_strips, L.tiles_n128,
+                                                                                          L.plan.wide_strips * 2 * TN, pass, 0);
+    }
+    return hipGetLastError();
 }
 
 // GPTQ (4-bit, [K/8, N] int32 words of eight consecutive k, zero point = stored + 1) to one plane of q - zero in [-16, 14],
@@ -1062,19 +1134,14 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
     const int64_t lda = (int64_t)nblk_tile * 256;
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM, lda);
     const PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, nplanes, !q6 && !wide, nblk_tile);
-    hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : wide ? allow_full_lds<gemm_planes_wide_kernel<4>>() : allow_full_lds<gemm_planes_kernel>();
+    hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : wide ? hipSuccess : allow_full_lds<gemm_planes_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n128 = (int)((n + TN - 1) / TN);
-    const int tiles_n = wide ? (tiles_n128 + 1) / 2 : tiles_n128;  // the GEMM's column tiles
+    const int tiles_n = tiles_n128;  // the column tiles of the 256 x 128 kernels
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-    }
-    const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
-    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, nblk_tile, wg, wide ? 2 * TN : TN);
+    const int wg = 8 * std::min(per_xcd, std::max(1, compute_units() / 8));
+    const WideLaunch L = wide ? wide_launch(out, m, n, nblk_tile) : WideLaunch{};
+    const SplitTiles z = wide ? L.z : split_tiles(out, m, n, tiles_m, tiles_n, nblk_tile, wg, TN);
     const int max_split = z.max_split;
     const int64_t conv = (int64_t)tiles_n128 * nblk * 4, blocks = conv + m + (int64_t)max_split * 64;
     if (blocks > INT32_MAX || lda * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
@@ -1100,11 +1167,10 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
         if (q6)
             gemm_planes2_kernel<<<dim3((unsigned)wg), dim3(512), kPlanes2Lds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k,
                                                                                  tiles_m, tiles_n, pass, split);
-        else if (wide)
-            gemm_planes_wide_kernel<4><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)lda,
-                                                                                         pass == 0 ? nblk_tile : nblk, nblk_tile, tiles_m,
-                                                                                         tiles_n, tiles_n128, pass, split);
-        else
+        else if (wide) {
+            e = run_wide<4>(L, ps.planes, ps.dtab, a, p.inv, out, m, n, lda, pass == 0 ? nblk_tile : nblk, nblk_tile, pass, s);
+            if (e != hipSuccess) return e;
+        } else
             gemm_planes_kernel<<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m, (int)n,
                                                                                (int)k, tiles_m, tiles_n, pass == 0, pass, split);
     }
@@ -1129,18 +1195,10 @@ hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_
     const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
     // (steps per tile k / 64 = 4 blocks of 256: the plane array is sized in those; the tables in groups)
     PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, 1, false, nblk256, k / 128);
-    hipError_t e = group == 128 ? allow_full_lds<gemm_planes_wide_kernel<2>>() : allow_full_lds<gemm_planes_wide_kernel<4>>();
-    if (e != hipSuccess) return e;
-    const int tiles_m = (int)((m + TM - 1) / TM), tiles_n128 = (int)((n + TN - 1) / TN), tiles_n = (tiles_n128 + 1) / 2;
-    const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-    }
-    const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
-    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, groups, wg, 2 * TN);
+    const WideLaunch L = wide_launch(out, m, n, groups);
+    const SplitTiles& z = L.z;
+    const int tiles_n128 = L.tiles_n128;
+    hipError_t e = hipSuccess;
     const int64_t conv = (int64_t)tiles_n128 * nblk256, blocks = conv + m + (int64_t)z.max_split * 64;
     if (blocks > INT32_MAX || k * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
     if (lhs_dtype == QMM_F32)
@@ -1153,13 +1211,9 @@ hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_
     if (e != hipSuccess) return e;
     for (int pass = 0; pass < (p.a16_lo ? 2 : 1); pass++) {
         const _Float16* a = pass == 0 ? p.a16 : p.a16_lo;
-        const int split = pass == 0 && z.max_split > 0 ? 1 : 0;
-        if (group == 128)
-            gemm_planes_wide_kernel<2><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k, groups,
-                                                                                         groups, tiles_m, tiles_n, tiles_n128, pass, split);
-        else
-            gemm_planes_wide_kernel<4><<<dim3((unsigned)wg), dim3(512), kPlanesWLds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k, groups,
-                                                                                         groups, tiles_m, tiles_n, tiles_n128, pass, split);
+        e = group == 128 ? run_wide<2>(L, ps.planes, ps.dtab, a, p.inv, out, m, n, k, groups, groups, pass, s)
+                         : run_wide<4>(L, ps.planes, ps.dtab, a, p.inv, out, m, n, k, groups, groups, pass, s);
+        if (e != hipSuccess) return e;
     }
     return hipGetLastError();
 }

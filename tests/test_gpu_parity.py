@@ -729,13 +729,16 @@ def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
 
 @pytest.mark.parametrize("kind,m,n,k,bf16", [
     ("Q5_K", 1030, 8200, 2304, False), ("Q4_K", 1600, 8200, 768, True), ("Q4_K", 1540, 4100, 2304, False),
-    ("GPTQ128", 1600, 8200, 768, True), ("GPTQ256", 1540, 8200, 768, False), ("GPTQ128", 1536, 4104, 1280, False)])
+    ("GPTQ128", 1600, 8200, 768, True), ("GPTQ256", 1540, 8200, 768, False), ("GPTQ128", 1536, 4104, 1280, False),
+    ("Q4_K", 2000, 14192, 512, True), ("GPTQ128", 1990, 14192, 512, False), ("Q5_K", 1800, 14000, 256, True)])
 def test_plane_gemm_on_256_wide_tiles(kind, m, n, k, bf16):
     """Large problems of the single-plane encodings (from 128 tiles of 256 x 256; Q4_K and GPTQ from 1536 lhs rows): the plane GEMM
     that keeps its accumulators in units of the current scale block's scale.  Q4_K / Q5_K carry their min term as extension
     blocks (K = 2304: nine super-blocks, a full extension block and one with a single super-block and zeros); GPTQ's scale
     blocks are its groups (two or four steps; K = 1280 with groups of 128 ends on half a 256-block); ragged m and n; an fp32
-    lhs (second pass on the residual); 233 and 119 tiles (a last round cut in K halves or not).  Every fifth K-quant block has
+    lhs (second pass on the residual); 233 and 119 tiles (a last round cut in K halves or not); 8 x 56 tiles on 256 compute units
+    (one round of 256 x 256 tiles, then the remaining 6000 / 5808 columns as 256 x 192 tiles in a launch of their own, the last
+    of them ragged and reaching past the last 128-column tile of the planes).  Every fifth K-quant block has
     d = 0 with its codes, scales and dmin in place (the weights are then -dmin * mn), every third carries random code and scale bytes."""
     w, a = synth(81, n, k, m)
     if bf16:
