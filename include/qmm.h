@@ -109,7 +109,7 @@ int qmm_quantize_gptq(const qmm_gptq_config* cfg, const float* w, int64_t n, int
 
 /* Bytes of device scratch qmm_matmul needs for this problem (may be 0); the second form for a call with `flags`
  * (QMM_FLAG_OUT_BF16 adds room for an fp32 result wherever the kernel does not store bf16 itself).  For large
- * Q4_K / GPTQ prefill problems (1024 lhs rows or more) the figure includes fp16 planes of the weights (2 bytes per
+ * Q4_K / GPTQ prefill problems (more than 512 lhs rows) the figure includes fp16 planes of the weights (2 bytes per
  * weight) for the faster of two kernels; qmm_matmul given less than that, but enough for the lhs planes, runs the other one. */
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags);

@@ -65,7 +65,7 @@ PlaneSpace plane_space(void* base, int64_t n, int64_t k, int nplanes, bool with_
 // Which GEMM serves a single-plane encoding: the 256 x 256 tiles from this many of them on (fewer leave compute units idle
 // where the 256 x 128 kernel still has work for them).
 constexpr int kWideMinTiles = 128;
-constexpr int kOptionalPlanesMinRows = 1024;  // Q4_K and GPTQ have GEMM kernels that need no conversion pass: planes from here on
+constexpr int kOptionalPlanesMinRows = 513;  // Q4_K and GPTQ have GEMM kernels that need no conversion pass: planes from three row tiles on
 bool wide_tiles(int encoding, int64_t m, int64_t n) {
     if (encoding == QMM_Q6_K || kernel_disabled("planes_wide")) return false;
     const int64_t tiles_m = (m + TM - 1) / TM, tiles_nw = (n + 2 * TN - 1) / (2 * TN);
@@ -1107,8 +1107,9 @@ __global__ __launch_bounds__(256) void gptq_planes_prologue_kernel(const uint32_
 bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     if (kernel_disabled("kquant_planes") || k % 256 || k < 256) return false;
     if (encoding == QMM_Q4_K) {
-        // From this many lhs rows on the conversion pass costs less than the plane GEMM on 256 x 256 tiles gains on the tile
-        // kernel that unpacks as it goes (14336 x 4096 with 2048 rows: 235 + 34 us against 285 + 11 us).  QMM_Q4K_PLANES=1 (read
+        // From three row tiles on (and 128 tiles of 256 x 256) the conversion pass costs less than the plane GEMM gains on the
+        // tile kernel that unpacks as it goes (14336 x 4096 with 2048 rows: 226 + 34 us against 285 + 11 us; 768 rows: 126
+        // against 132 us, GPTQ 113 against 137 us; 512 rows: 119 against 88 us).  QMM_Q4K_PLANES=1 (read
         // once) sends every Q4_K prefill shape here, for tests and comparisons.
         static const bool force = getenv("QMM_Q4K_PLANES") != nullptr && atoi(getenv("QMM_Q4K_PLANES")) == 1;
         return m > 16 && (force || (m >= kOptionalPlanesMinRows && wide_tiles(encoding, m, n) && !kernel_disabled("q4k_planes")));
