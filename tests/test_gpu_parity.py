@@ -771,6 +771,31 @@ def test_plane_gemm_on_256_wide_tiles(kind, m, n, k, bf16):
     assert_close(qmatmul(*args, static_scratch=True), truth, f"{kind} {m}x{n}x{k} with the static scratch")
 
 
+@pytest.mark.parametrize("enc,m,n,k", [(QE.Q4_K, 520, 16500, 512), (QE.Q6_K, 70, 300, 1024)])
+def test_plane_gemm_non_finite_super_block_scale(enc, m, n, k):
+    """A super-block scale of +inf or NaN makes every output of its weight row non-finite (as in the oracle, whose sums
+    then hold inf - inf or 0 * inf) and leaves the other columns alone: the plane GEMMs carry their accumulators in units
+    of the running scale, per column."""
+    e = ENC[enc]
+    bpb, doff = (144, 0) if enc == QE.Q4_K else (210, 208)
+    w, a = synth(91, n, k, m)
+    a = O.bf16_to_f32(O.f32_to_bf16(a))
+    wq = O.quantize(e, w)
+    rows = wq.reshape(n, k // 256, bpb)
+    bad = {5: (0, 0x7C00), n - 3: (k // 256 - 1, 0x7E00), 130: (1, 0xFC00)}  # column: (super-block, fp16 bits)
+    for col, (blk, bits16) in bad.items():
+        rows[col, blk, doff:doff + 2] = np.frombuffer(np.uint16(bits16).tobytes(), dtype=np.uint8)
+    want = O.matmul_f32(e, a, wq)
+    got = qmatmul(enc, None, gpu(a).to(torch.bfloat16), gpu(wq)).cpu().numpy()
+    good = np.ones(n, dtype=bool)
+    for col in bad:
+        good[col] = False
+        assert not np.isfinite(want[:, col]).any()
+        assert not np.isfinite(got[:, col]).any(), f"column {col}: finite outputs under a non-finite scale"
+    assert np.isfinite(got[:, good]).all()
+    assert O.isclose(got[:, good], want[:, good], RTOL, ATOL).all()
+
+
 def test_q6_k_prefill_equals_the_decode_kernel_passes():
     """The same product through the planes GEMM (72 rows at once) and through the decode kernel (the rows in three calls
     of at most 64): two summation orders of the same exact products."""
