@@ -1,24 +1,31 @@
-// Prefill (m > 16 lhs rows) for Q5_K and Q6_K on the matrix cores, in two steps: a conversion pass turns the
-// packed weights into planes of exact small integers in fp16, already in the LDS image of the matrix-core operand
-// tiles, and a GEMM that is the Q4_K tile kernel without the unpack streams lhs and plane tiles global -> LDS
-// directly and applies the fp32 super-block scales in the lanes.
+// Prefill on the matrix cores through weight planes, in two steps: a conversion pass turns the packed weights into planes
+// of exact small integers in fp16, already in the LDS image of the matrix-core operand tiles, and a GEMM streams lhs and
+// plane tiles global -> LDS directly and applies the fp32 scales of the scale blocks (K-quant super-blocks, GPTQ groups) in
+// the lanes.  Q5_K (more than 32 lhs rows) and Q6_K (more than 64) always come here; Q4_K and GPTQ (plain groups of 128 or
+// 256) from 513 rows on large matrices, when the caller's workspace holds the planes.
 //
-// Arithmetic (exact products, fp32 sums, as in gemm_q4k_tile.hip):
-//   Q5_K  w = d * (sc * q) - dmin * mn,  q = nibble | fifth bit << 4 <= 31, sc <= 63: one plane, sc * q <= 1953 (an
-//         fp16 integer); the min term as two extra matrix-core products per super-block over the lhs sub-block sums.
+// Arithmetic (exact products, fp32 sums):
+//   Q4_K / Q5_K  w = d * (sc * q) - dmin * mn,  q <= 15 / 31, sc <= 63: one plane, sc * q <= 1953 (an fp16 integer); the min
+//         term as matrix-core products of the lhs sub-block sums with -(dmin * mn), both split into fp16 hi + lo parts:
+//         extra instructions per super-block in gemm_planes_kernel, extension blocks of K in gemm_planes_wide_kernel.
 //   Q6_K  w = d * (sc * q),  q in [-32, 31], sc an int8 per 16 weights: sc * q reaches 4096 and odd values above
 //         2048 are no fp16 numbers, so sc = 16 hi + lo (hi = sc >> 4 in [-8, 7], lo = sc & 15) gives two planes,
 //         (16 hi) * q (a multiple of 16 with at most 9 significant bits) and lo * q (<= 480), both exact.  Its GEMM
-//         (gemm_planes2_kernel) multiplies both planes of a K step with the same lhs operands and scales the sum of the
-//         two partial products of a super-block by d.
+//         (gemm_planes2_kernel) multiplies both planes of a K step with the same lhs operands.
+//   GPTQ  w = s * (q - zero),  q - zero in [-16, 14]: one plane, no zero-point term left.
 // The planes cost workspace (2 bytes per weight and plane) and one pass over the weights (tens of microseconds at
-// the sizes this path is chosen for); they buy a GEMM whose only vector-ALU work is the rescale.
+// the sizes this path is chosen for); they buy a GEMM whose only vector-ALU work is the change of scale.
+//
+// Three GEMM kernels: gemm_planes_wide_kernel (one plane, 256 x 256 or 256 x 192 tiles, accumulators in units of the
+// current block's scale; large problems), gemm_planes2_kernel (two planes, 256 x 128 tiles, the same accumulator scheme),
+// gemm_planes_kernel (one plane, 256 x 128 tiles, a second accumulator set per super-block and the min term in the kernel;
+// problems with fewer than 128 tiles of 256 x 256).
 //
 // Plane layout: [n_tile][plane * steps + step][128 columns][64 halfs] with the 16-byte pieces of a column's row at
 // piece index p ^ ((column / 2) % 8) (the swizzle of the tile kernel's LDS buffers), piece p = 2 f + g holding the
 // weights k = 64 step + 32 g + 8 f + (0,2,1,3,4,6,5,7)[slot] (the lhs order kLhsOrderTile): one (tile, step) is 16 KB
-// of contiguous memory that goes to LDS as it is.  Tables per (n_tile, super-block): d as fp32 [128], and for Q5_K
-// the min operands -(dmin * mn) split exactly into fp16 hi + lo, [128 columns][8 hi, 8 lo].
+// of contiguous memory that goes to LDS as it is.  Tables per (n_tile, scale block): the scale as fp32 [128], and for
+// gemm_planes_kernel the min operands -(dmin * mn) split exactly into fp16 hi + lo, [128 columns][8 hi, 8 lo].
 #include <stdlib.h>
 
 #include <algorithm>
