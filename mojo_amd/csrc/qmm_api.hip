@@ -465,7 +465,8 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q8_K round trip)");
         return matmul_f32(encoding, cfg, y, QMM_F32, m, k, rhs, n_rhs, n, out, (char*)workspace + ybytes, workspace_bytes - ybytes, 0, stream);
     }
-    // Q5_K and Q6_K with many lhs rows: weights to fp16 integer planes in the workspace, then the matrix cores
+    // Q5_K and Q6_K with many lhs rows, Q4_K with more than 512 on large matrices: weights to fp16 integer planes in the workspace,
+    // then the matrix cores
     if (kquant_planes(encoding, m, n, k))
         return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
     // Q5_K with several lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
