@@ -108,6 +108,25 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.qmm_matmul_rmsnorm_workspace_bytes(1, 1, 3, 8, 4096, 0) == 3 * 4096 * 2
 
 
+def test_workspace_figures_of_the_optional_weight_planes():
+    """Host arithmetic only.  Large Q4_K / GPTQ prefill problems (more than 512 lhs rows, 128 or more tiles of 256 x 256)
+    are quoted with room for fp16 weight planes, 2 bytes per weight; the same matrices with fewer rows, and small matrices,
+    are quoted for the kernels that unpack as they go (lhs planes only).  Q5_K / Q6_K always need their planes beyond 32 / 64
+    rows (Q6_K two of them)."""
+    lib = _lib.load()
+    n, k = 14336, 4096
+    bf16 = _lib.QMM_BF16
+    for enc in (QE.Q4_K, QE.GPTQ):
+        big = lib.qmm_matmul_workspace_bytes(enc.code, bf16, 2048, n, k)
+        mid = lib.qmm_matmul_workspace_bytes(enc.code, bf16, 512, n, k)
+        small_matrix = lib.qmm_matmul_workspace_bytes(enc.code, bf16, 2048, 2048, k)  # 8 x 8 tiles
+        assert big >= 2 * n * k + 2048 * k * 2, enc
+        assert mid < 32 << 20 and small_matrix < 64 << 20, enc
+    assert lib.qmm_matmul_workspace_bytes(QE.Q5_K.code, bf16, 40, n, k) >= 2 * n * k
+    assert lib.qmm_matmul_workspace_bytes(QE.Q6_K.code, bf16, 70, n, k) >= 4 * n * k
+    assert lib.qmm_matmul_workspace_bytes(QE.Q6_K.code, bf16, 64, n, k) == 0
+
+
 def test_quantization_encoding_metadata():
     assert QE.Q4_0.block_parameters == mojo_amd.BlockParameters(32, 18)
     assert QE.Q4_K.block_parameters.block_size == 144 and QE.Q6_K.block_parameters.block_size == 210
