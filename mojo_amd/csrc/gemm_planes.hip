@@ -19,7 +19,7 @@
 // Three GEMM kernels: gemm_planes_wide_kernel (one plane, 256 x 256 or 256 x 192 tiles, accumulators in units of the
 // current block's scale; large problems), gemm_planes2_kernel (two planes, 256 x 128 tiles, the same accumulator scheme),
 // gemm_planes_kernel (one plane, 256 x 128 tiles, a second accumulator set per super-block and the min term in the kernel;
-// problems with fewer than 128 tiles of 256 x 256).
+// problems with fewer than 160 tiles of 256 x 256).
 //
 // Plane layout: [n_tile][plane * steps + step][128 columns][64 halfs] with the 16-byte pieces of a column's row at
 // piece index p ^ ((column / 2) % 8) (the swizzle of the tile kernel's LDS buffers), piece p = 2 f + g holding the
@@ -69,9 +69,10 @@ PlaneSpace plane_space(void* base, int64_t n, int64_t k, int nplanes, bool with_
     return p;
 }
 
-// Which GEMM serves a single-plane encoding: the 256 x 256 tiles from this many of them on (fewer leave compute units idle
-// where the 256 x 128 kernel still has work for them).
-constexpr int kWideMinTiles = 128;
+// Which GEMM serves a single-plane encoding: the 256 x 256 tiles from this many of them on.  Up to 256 tiles the wide kernel
+// takes one round whatever their number, the 256 x 128 kernels' time grows with it (K halves balance their last round):
+// 2048 rows x 4096 columns x 4096 (128 tiles) 105.8 against 92.5 us (Q5_K), 5120 columns (160 tiles) 112.5 against 132.7 us.
+constexpr int kWideMinTiles = 160;
 constexpr int kOptionalPlanesMinRows = 513;  // Q4_K and GPTQ have GEMM kernels that need no conversion pass: planes from three row tiles on
 bool wide_tiles(int encoding, int64_t m, int64_t n) {
     if (encoding == QMM_Q6_K || kernel_disabled("planes_wide")) return false;
@@ -1114,7 +1115,7 @@ __global__ __launch_bounds__(256) void gptq_planes_prologue_kernel(const uint32_
 bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     if (kernel_disabled("kquant_planes") || k % 256 || k < 256) return false;
     if (encoding == QMM_Q4_K) {
-        // From three row tiles on (and 128 tiles of 256 x 256) the conversion pass costs less than the plane GEMM gains on the
+        // From three row tiles on (and 160 tiles of 256 x 256) the conversion pass costs less than the plane GEMM gains on the
         // tile kernel that unpacks as it goes (14336 x 4096 with 2048 rows: 226 + 34 us against 285 + 11 us; 768 rows: 126
         // against 132 us, GPTQ 113 against 137 us; 512 rows: 119 against 88 us).  QMM_Q4K_PLANES=1 (read
         // once) sends every Q4_K prefill shape here, for tests and comparisons.

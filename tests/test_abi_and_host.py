@@ -109,7 +109,7 @@ def test_argument_validation_happens_before_any_launch():
 
 
 def test_workspace_figures_of_the_optional_weight_planes():
-    """Host arithmetic only.  Large Q4_K / GPTQ prefill problems (more than 512 lhs rows, 128 or more tiles of 256 x 256)
+    """Host arithmetic only.  Large Q4_K / GPTQ prefill problems (more than 512 lhs rows, 160 or more tiles of 256 x 256)
     are quoted with room for fp16 weight planes, 2 bytes per weight; the same matrices with fewer rows, and small matrices,
     are quoted for the kernels that unpack as they go (lhs planes only).  Q5_K / Q6_K always need their planes beyond 32 / 64
     rows (Q6_K two of them)."""

@@ -675,7 +675,7 @@ def test_q4_k_gemm_f32_lhs(m, n, k):
 @pytest.mark.parametrize("m,n,k,bf16", [(512, 16384, 512, True), (500, 18600, 768, True), (300, 32768, 256, True),
                                         (520, 8200, 512, False)])
 def test_q4_k_gemm_tile_kernel(m, n, k, bf16):
-    """Shapes with at least 256 output tiles of 256 x 128 (and no more than 512 lhs rows or fewer than 128 tiles of
+    """Shapes with at least 256 output tiles of 256 x 128 (and no more than 512 lhs rows or fewer than 160 tiles of
     256 x 256: beyond, the plane GEMM takes over) go to the kernel that unpacks each weight tile once per
     workgroup into LDS: whole rounds of tiles (256), a last round cut in two K halves that meet through atomic adds
     (292 tiles: 37 per XCD, 5 in the last round; K = 768 gives halves of 1 and 2 super-blocks), a single super-block
@@ -729,15 +729,15 @@ def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
 
 
 @pytest.mark.parametrize("kind,m,n,k,bf16", [
-    ("Q5_K", 1030, 8200, 2304, False), ("Q4_K", 1600, 8200, 768, True), ("Q4_K", 1540, 4100, 2304, False),
-    ("GPTQ128", 1600, 8200, 768, True), ("GPTQ256", 1540, 8200, 768, False), ("GPTQ128", 1536, 4104, 1280, False),
+    ("Q5_K", 1030, 8200, 2304, False), ("Q4_K", 1600, 8200, 768, True), ("Q4_K", 1540, 10300, 2304, False),
+    ("GPTQ128", 1600, 8200, 768, True), ("GPTQ256", 1540, 8200, 768, False), ("GPTQ128", 1536, 11016, 1280, False),
     ("Q4_K", 2000, 14192, 512, True), ("GPTQ128", 1990, 14192, 512, False), ("Q5_K", 1800, 14000, 256, True)])
 def test_plane_gemm_on_256_wide_tiles(kind, m, n, k, bf16):
-    """Large problems of the single-plane encodings (from 128 tiles of 256 x 256; Q4_K and GPTQ from 513 lhs rows): the plane GEMM
+    """Large problems of the single-plane encodings (from 160 tiles of 256 x 256; Q4_K and GPTQ from 513 lhs rows): the plane GEMM
     that keeps its accumulators in units of the current scale block's scale.  Q4_K / Q5_K carry their min term as extension
     blocks (K = 2304: nine super-blocks, a full extension block and one with a single super-block and zeros); GPTQ's scale
     blocks are its groups (two or four steps; K = 1280 with groups of 128 ends on half a 256-block); ragged m and n; an fp32
-    lhs (second pass on the residual); 233 and 119 tiles (a last round cut in K halves or not); 8 x 56 tiles on 256 compute units
+    lhs (second pass on the residual); 231, 287 and 264 tiles (one round; a second round of few tiles cut in K halves); 8 x 56 tiles on 256 compute units
     (one round of 256 x 256 tiles, then the remaining 6000 / 5808 columns as 256 x 192 tiles in a launch of their own, the last
     of them ragged and reaching past the last 128-column tile of the planes).  Every fifth K-quant block has
     d = 0 with its codes, scales and dmin in place (the weights are then -dmin * mn), every third carries random code and scale bytes."""
