@@ -177,6 +177,29 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
                        int64_t workspace_bytes, void* stream);
 
 /*
+ * Weight planes kept across calls.  MAX's graph compiler folds a weight repack step ahead of its quantized matmul
+ * kernels into model load (the packed layout is contractual on disk only; MAX itself is not in the reference
+ * snapshot, see the top of this file); this pair of calls is the explicit form of it for the prefill GEMMs here:
+ * qmm_repack converts the packed weights of one matrix once into the fp16 integer planes and scale tables that the
+ * matrix-core GEMMs read (2 bytes per weight, Q6_K 4, plus tables: qmm_repack_bytes, 0 if the encoding or shape has
+ * no plane GEMM: Q4_0, GPTQ with act-order or groups other than 128 / 256, K not a multiple of 256), into a buffer
+ * the caller owns, 256-byte aligned; the buffer depends on the weights only.  qmm_matmul_repacked is qmm_matmul with
+ * that buffer at hand: row counts for which the plane GEMMs are the faster route (Q6_K above 64 rows, Q5_K above
+ * 32, Q4_K / GPTQ above 256 on matrices with at least 160 output tiles of 256 x 256) skip the conversion that
+ * qmm_matmul repeats per call (same kernels, same planes: where qmm_matmul takes the planes too the results are equal
+ * bit for bit); other row counts are handed to qmm_matmul with `rhs`.  rhs = NULL (a caller that dropped the packed tensors): every row count goes through the planes.
+ * flags must be 0.  Workspace: qmm_matmul_repacked_workspace_bytes (the lhs planes, or what qmm_matmul needs for the
+ * kernels that read the packed tensors).
+ */
+int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k);
+int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs, int n_rhs, int64_t n, int64_t k,
+               void* packed, int64_t packed_bytes, void* stream);
+int64_t qmm_matmul_repacked_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
+int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
+                        const void* const* rhs, int n_rhs, const void* packed, int64_t packed_bytes, int64_t n, float* out,
+                        void* workspace, int64_t workspace_bytes, int flags, void* stream);
+
+/*
  * The gated-MLP step either side of ops.qmatmul in a Llama block (no counterpart in the reference's op set: there the
  * graph holds two qmatmul nodes, a SiLU and a multiply):
  *     out fp32[m, n] = silu(lhs . dequant(gate)^T) * (lhs . dequant(up)^T),   silu(x) = x / (1 + exp(-x)).

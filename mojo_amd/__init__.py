@@ -12,10 +12,13 @@ from .ops import (
     dequantize,
     qmatmul,
     qmatmul_grouped,
+    qmatmul_repacked,
     qmatmul_rmsnorm,
     qmatmul_swiglu,
     quantize,
     quantize_gptq,
+    repack_weights,
+    RepackedWeights,
 )
 from .weights import GGUFWeights, load_gptq_config, load_gptq_linear
 
@@ -25,6 +28,9 @@ __all__ = [
     "QuantizationEncoding",
     "qmatmul",
     "qmatmul_grouped",
+    "qmatmul_repacked",
+    "repack_weights",
+    "RepackedWeights",
     "qmatmul_rmsnorm",
     "qmatmul_swiglu",
     "dequantize",

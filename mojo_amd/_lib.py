@@ -37,6 +37,11 @@ SIGNATURES = {
                           _i64, _int, _vp]),
     "qmm_matmul_static": (_int, [_int, C.POINTER(GptqConfig), _vp, _int, _i64, _i64, C.POINTER(_vp), _int, _i64, _vp, _int,
                                  _vp]),
+    "qmm_repack_bytes": (_i64, [_int, C.POINTER(GptqConfig), _i64, _i64]),
+    "qmm_repack": (_int, [_int, C.POINTER(GptqConfig), C.POINTER(_vp), _int, _i64, _i64, _vp, _i64, _vp]),
+    "qmm_matmul_repacked_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64]),
+    "qmm_matmul_repacked": (_int, [_int, C.POINTER(GptqConfig), _vp, _int, _i64, _i64, C.POINTER(_vp), _int, _vp, _i64, _i64, _vp,
+                                   _vp, _i64, _int, _vp]),
     "qmm_matmul_grouped": (_int, [_int, _vp, _int, _i64, _i64, _int, C.POINTER(_vp), C.POINTER(_i64), C.POINTER(_vp), _vp,
                                   _i64, _vp]),
     "qmm_matmul_swiglu_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64]),

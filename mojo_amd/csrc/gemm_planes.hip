@@ -63,7 +63,7 @@ PlaneSpace plane_space(void* base, int64_t n, int64_t k, int nplanes, bool with_
     off += up(tiles_n * nplanes * nblk_tile * 4 * kBBuf);
     p.dtab = (float*)((uint8_t*)base + off);
     off += up(tiles_n * (dblocks ? dblocks : nblk_tile) * kDBuf);
-    p.mtab = (uint8_t*)base + off;
+    p.mtab = with_mtab ? (uint8_t*)base + off : nullptr;
     off += with_mtab ? up(tiles_n * nblk * kMBuf) : 0;
     p.bytes = off;
     return p;
@@ -233,8 +233,9 @@ __device__ __forceinline__ void planes_from_kquant(int tile_n, int rb, int quart
                             for (int q = 0; q < 4; q++) *(uint4*)(t2 + ((((b2 & 1) * 4 + q) ^ sw) << 4)) = make_uint4(0, 0, 0, 0);
                         }
                     }
-                } else {
-                    uint8_t* mt = mtab + (tb * TN + col) * 32;
+                }
+                if (mtab) {  // (planes kept across calls carry both forms of the min operands)
+                    uint8_t* mt = mtab + (((int64_t)tile_n * nblk + rb) * TN + col) * 32;
                     *(uint4*)mt = make_uint4(hi[0], hi[1], hi[2], hi[3]);
                     *(uint4*)(mt + 16) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
                 }
@@ -249,15 +250,16 @@ template <int ENC, typename AT>
 __global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __restrict__ w, int nblk, int nblk_tile, int tiles_n128,
                                                               uint8_t* __restrict__ planes, float* __restrict__ dtab,
                                                               uint8_t* __restrict__ mtab, int conv, const AT* __restrict__ a, int k,
-                                                              LhsPlanes p, SplitTiles z) {
+                                                              int lhs_ext, int lhs_rows, LhsPlanes p, SplitTiles z) {
     const int b = (int)blockIdx.x;
     if (b < conv) {
         const int t = b >> 2, rb = t / tiles_n128;
         planes_from_kquant<ENC>(t - rb * tiles_n128, rb, b & 3, w, z.n, nblk, nblk_tile, planes, dtab, mtab);
-    } else if (b < conv + z.m) {
-        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv, (int64_t)k + (nblk_tile - nblk) * 256, nblk_tile - nblk);
+    } else if (b < conv + lhs_rows) {
+        // (lhs_ext: extension blocks behind each lhs row, as many as the planes have when the wide GEMM follows, else none)
+        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv, (int64_t)k + lhs_ext * 256, lhs_ext);
     } else {
-        const int e = b - conv - z.m;
+        const int e = b - conv - lhs_rows;
         zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
     }
 }
@@ -269,7 +271,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
                                                             const uint8_t* __restrict__ mtab, const _Float16* __restrict__ a16,
                                                             const _Float16* __restrict__ asum, const float* __restrict__ inv,
                                                             float* __restrict__ out, int m, int n, int k, int tiles_m,
-                                                            int tiles_n, int with_min, int accumulate, int allow_split) {
+                                                            int tiles_n, int nblk_tile, int with_min, int accumulate, int allow_split) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = lds_address(smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -306,8 +308,10 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
         const uint8_t* a_base = (const uint8_t*)a16 + (int64_t)(m0 + wave * 32) * k * 2;
         const uint32_t s_off = (uint32_t)((wave * 32 + (lane >> 1)) * (nblk_row * 32) + (lane & 1) * 16);
         const uint8_t* s_base = (const uint8_t*)asum + (int64_t)m0 * nblk_row * 32;
-        const uint8_t* b_base = planes + ((int64_t)tile_n * nblk_row + kb0) * 4 * kBBuf;
-        const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * nblk_row * kDBuf;
+        // (nblk_tile: blocks of four steps a tile holds in planes and dtab; more than the super-blocks where the planes also
+        // carry the wide GEMM's extension blocks)
+        const uint8_t* b_base = planes + ((int64_t)tile_n * nblk_tile + kb0) * 4 * kBBuf;
+        const uint8_t* d_base = (const uint8_t*)dtab + (int64_t)tile_n * nblk_tile * kDBuf;
         const uint8_t* m_base = mtab + (int64_t)tile_n * nblk_row * kMBuf;
         auto real_blk = [&](int blk) __attribute__((always_inline)) { return kb0 + min(blk, nblk - 1); };  // super-block of the row
 
@@ -1099,15 +1103,15 @@ template <typename AT>
 __global__ __launch_bounds__(256) void gptq_planes_prologue_kernel(const uint32_t* __restrict__ qweight, const uint16_t* __restrict__ scales,
                                                                    const uint32_t* __restrict__ qzeros, int group, int tiles_n128,
                                                                    uint8_t* __restrict__ planes, float* __restrict__ dtab, int conv,
-                                                                   const AT* __restrict__ a, int k, LhsPlanes p, SplitTiles z) {
+                                                                   const AT* __restrict__ a, int k, int lhs_rows, LhsPlanes p, SplitTiles z) {
     const int b = (int)blockIdx.x;
     if (b < conv) {
         const int rb = b / tiles_n128;
         planes_from_gptq(b - rb * tiles_n128, rb, qweight, scales, qzeros, z.n, k, group, planes, dtab);
-    } else if (b < conv + z.m) {
+    } else if (b < conv + lhs_rows) {
         prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv);
     } else {
-        const int e = b - conv - z.m;
+        const int e = b - conv - lhs_rows;
         zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
     }
 }
@@ -1123,9 +1127,12 @@ bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
         return m > 16 && (force || (m >= kOptionalPlanesMinRows && wide_tiles(encoding, m, n) && !kernel_disabled("q4k_planes")));
     }
     if (encoding != QMM_Q5_K && encoding != QMM_Q6_K) return false;
-    // Below these row counts the passes of the decode kernels (16 lhs rows a pass for Q6_K, 1 to 4 for Q5_K) cost less than
-    // the conversion pass plus a GEMM whose 256-row tiles are mostly empty.
-    return encoding == QMM_Q6_K ? m > 64 : m > 32;
+    // Up to these row counts the passes of the small-batch kernels (16 lhs rows a pass) cost less than the conversion pass plus
+    // a GEMM whose 256-row tiles are mostly empty (14336 x 4096, Q5_K: 48 rows 52 us, 64 rows 69 us, the planes 65 us; Q6_K:
+    // 64 rows 88 us, the planes 118 us; beyond 64 rows neither encoding has a kernel that takes more than four rows a pass).
+    // Q5_K with 33 to 64 rows where that kernel does not apply (K not a multiple of 512 or beyond 32768) also comes here.
+    if (encoding == QMM_Q5_K && m > 32 && (k % 512 || k > 32768 || kernel_disabled("q5k_mm"))) return true;
+    return m > 64;
 }
 
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
@@ -1135,34 +1142,45 @@ int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int6
     return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile).bytes;
 }
 
-hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
-                              float* out, void* workspace, hipStream_t s) {
-    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
-    const int nplanes = q6 ? 2 : 1;
-    const int nblk = (int)(k / 256), nblk_tile = (int)blocks_per_tile(encoding, m, n, k);
-    const int64_t lda = (int64_t)nblk_tile * 256;
-    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM, lda);
-    const PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, nplanes, !q6 && !wide, nblk_tile);
+namespace {
+
+// One launch of the preparation kernel and the GEMM launches behind it.  `ps` holds the planes, nblk_tile blocks of four steps
+// per tile (the super-blocks, then extension blocks if any); convert: they are made from `w` in the preparation launch,
+// otherwise they were made earlier.  wide (not Q6_K): the 256 x 256 tiles, which walk the extension blocks for the min term;
+// the 256 x 128 kernel reads the min operands from ps.mtab and skips the extension blocks if the planes have them.
+hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, bool convert, int64_t m, int64_t n, int64_t k,
+                             float* out, void* lhs_space, const PlaneSpace& ps, int nblk_tile, bool wide, hipStream_t s) {
+    const bool q6 = encoding == QMM_Q6_K;
+    const int nblk = (int)(k / 256), lhs_ext = wide ? nblk_tile - nblk : 0;
+    const int64_t lda = (int64_t)(nblk + lhs_ext) * 256;
+    const LhsPlanes p = lhs_planes(lhs_space, lhs_dtype, m, k, TM, lda);
     hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : wide ? hipSuccess : allow_full_lds<gemm_planes_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n128 = (int)((n + TN - 1) / TN);
     const int tiles_n = tiles_n128;  // the column tiles of the 256 x 128 kernels
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-    const int wg = 8 * std::min(per_xcd, std::max(1, compute_units() / 8));
+    // Tiles for no more than half of the compute units: the launch still takes a workgroup per compute unit, and the unit
+    // arithmetic then cuts every tile in two K halves.  A tile's time is set by K, so up to 96 tiles this takes a quarter to
+    // a third off the call (14336 x 4096 Q6_K, 65 lhs rows: 160 -> 118 us; 4096 x 4096 Q5_K, 256 rows: 66 -> 48 us); from 112
+    // tiles on the zeroing and the atomic adds cost what the halves gain (4096 x 4096, 1024 rows: 63 -> 72 us), unless K is long
+    // (4096 x 14336, 1024 rows: 188 -> 159 us).
+    const int per_xcd_cus = std::max(1, compute_units() / 8);
+    const bool halve_all = 2 * per_xcd <= per_xcd_cus && nblk >= 2 && (total <= 96 || nblk >= 32);
+    const int wg = 8 * (halve_all ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
     const WideLaunch L = wide ? wide_launch(out, m, n, nblk_tile) : WideLaunch{};
-    const SplitTiles z = wide ? L.z : split_tiles(out, m, n, tiles_m, tiles_n, nblk_tile, wg, TN);
+    const SplitTiles z = wide ? L.z : split_tiles(out, m, n, tiles_m, tiles_n, nblk, wg, TN);
     const int max_split = z.max_split;
-    const int64_t conv = (int64_t)tiles_n128 * nblk * 4, blocks = conv + m + (int64_t)max_split * 64;
+    const int64_t conv = convert ? (int64_t)tiles_n128 * nblk * 4 : 0, blocks = conv + m + (int64_t)max_split * 64;
     if (blocks > INT32_MAX || lda * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
     const dim3 pgrid((unsigned)blocks);
     auto prologue = [&](auto enc_c) {
         constexpr int ENC = decltype(enc_c)::value;
         if (lhs_dtype == QMM_F32)
             planes_prologue_kernel<ENC, float><<<pgrid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv,
-                                                                          (const float*)lhs, (int)k, p, z);
+                                                                          (const float*)lhs, (int)k, lhs_ext, (int)m, p, z);
         else
             planes_prologue_kernel<ENC, uint16_t><<<pgrid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv,
-                                                                             (const uint16_t*)lhs, (int)k, p, z);
+                                                                             (const uint16_t*)lhs, (int)k, lhs_ext, (int)m, p, z);
     };
     if (q6) prologue(std::integral_constant<int, QMM_Q6_K>{});
     else if (encoding == QMM_Q4_K) prologue(std::integral_constant<int, QMM_Q4_K>{});
@@ -1181,9 +1199,76 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
             if (e != hipSuccess) return e;
         } else
             gemm_planes_kernel<<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m, (int)n,
-                                                                               (int)k, tiles_m, tiles_n, pass == 0, pass, split);
+                                                                               (int)k, tiles_m, tiles_n, nblk_tile, pass == 0, pass, split);
     }
     return hipGetLastError();
+}
+
+// Planes that outlive a call serve every row count, so Q4_K / Q5_K carry the min operands in both forms: extension blocks for
+// the wide GEMM and the table for the 256 x 128 kernel.
+int repacked_blocks_per_tile(int encoding, int64_t k) {
+    const int nblk = (int)(k / 256);
+    return encoding == QMM_Q6_K ? nblk : nblk + (nblk + 7) / 8;
+}
+PlaneSpace repacked_space(int encoding, void* base, int64_t n, int64_t k) {
+    const bool q6 = encoding == QMM_Q6_K;
+    return plane_space(base, n, k, q6 ? 2 : 1, !q6, repacked_blocks_per_tile(encoding, k));
+}
+
+}  // namespace
+
+hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
+                              float* out, void* workspace, hipStream_t s) {
+    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
+    const int nblk_tile = (int)blocks_per_tile(encoding, m, n, k);
+    const int64_t lhs_bytes = (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)nblk_tile * 256).bytes + 255) / 256 * 256;
+    const PlaneSpace ps = plane_space((uint8_t*)workspace + lhs_bytes, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile);
+    return run_kquant_planes(encoding, lhs, lhs_dtype, w, true, m, n, k, out, workspace, ps, nblk_tile, wide, s);
+}
+
+// Weight planes kept across calls (the weights of a model are converted once, at load time): the conversion alone, and the
+// GEMM over planes made by it.
+int64_t repacked_planes_bytes(int encoding, int64_t n, int64_t k) { return repacked_space(encoding, nullptr, n, k).bytes; }
+
+hipError_t launch_repack_planes(int encoding, const uint8_t* w, int64_t n, int64_t k, void* packed, hipStream_t s) {
+    const int nblk = (int)(k / 256), nblk_tile = repacked_blocks_per_tile(encoding, k);
+    const PlaneSpace ps = repacked_space(encoding, packed, n, k);
+    const int tiles_n128 = (int)((n + TN - 1) / TN);
+    const int64_t conv = (int64_t)tiles_n128 * nblk * 4;
+    if (conv > INT32_MAX) return hipErrorInvalidValue;
+    SplitTiles z{};
+    z.n = (int)n;
+    const LhsPlanes none{};
+    const dim3 grid((unsigned)conv);
+    if (encoding == QMM_Q6_K)
+        planes_prologue_kernel<QMM_Q6_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z);
+    else if (encoding == QMM_Q4_K)
+        planes_prologue_kernel<QMM_Q4_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z);
+    else
+        planes_prologue_kernel<QMM_Q5_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z);
+    return hipGetLastError();
+}
+
+// With the conversion out of the way the plane GEMMs pay from fewer rows on than inside qmm_matmul.
+// 14336 x 4096: Q5_K 40 lhs rows 39.5 us against 52 us for three passes of the small-batch kernel, Q6_K 53 us against 44 / 66 us
+// for two / three passes of its decode kernel; 4096 x 4096: Q5_K 36 us against 30 us (48 rows) / 40 us (64), Q6_K 45 against 38 / 53.
+// Q4_K against its kernels that unpack as they go: 14336 x 4096, 160 / 256 / 512 rows 53 / 62 / 75 against 68 / 78 / 88 us;
+// 4096 x 4096, 256 / 512 / 1024 rows 41 / 49 / 63 against 35 / 59 / 60 us; 4096 x 14336, 256 / 512 / 1024: 104 / 114 / 159 against 81 / 116 / 180.
+bool repacked_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
+    if (k % 256 || k < 256) return false;
+    if (encoding == QMM_Q6_K || encoding == QMM_Q5_K) return m > 48 || (m > 32 && n * k >= ((int64_t)48 << 20));
+    if (encoding != QMM_Q4_K) return false;
+    const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
+    return m > 128 && tiles >= 64;
+}
+int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t k) {
+    return (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)repacked_blocks_per_tile(encoding, k) * 256).bytes + 255) / 256 * 256;
+}
+hipError_t launch_gemm_planes_repacked(int encoding, const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k,
+                                       float* out, void* workspace, hipStream_t s) {
+    const PlaneSpace ps = repacked_space(encoding, const_cast<void*>(packed), n, k);
+    return run_kquant_planes(encoding, lhs, lhs_dtype, nullptr, false, m, n, k, out, workspace, ps, repacked_blocks_per_tile(encoding, k),
+                             wide_tiles(encoding, m, n), s);
 }
 
 // GPTQ through the plane GEMM: groups of 128 or 256 (a scale block is two or four steps), plain groups (no act-order), and
@@ -1198,24 +1283,24 @@ int64_t gemm_gptq_planes_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, in
     return lhs + plane_space(nullptr, n, k, 1, false, k / 256, k / 128).bytes;  // (tables sized for the smaller group)
 }
 
-hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros,
-                                   int64_t m, int64_t n, int64_t k, int group, float* out, void* workspace, hipStream_t s) {
+namespace {
+// convert: the planes in `ps` are made from the checkpoint tensors in the preparation launch; otherwise they were made earlier.
+hipError_t run_gptq_planes(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros, bool convert,
+                           int64_t m, int64_t n, int64_t k, int group, float* out, void* lhs_space, const PlaneSpace& ps, hipStream_t s) {
     const int groups = (int)(k / group), nblk256 = (int)(k / 256);
-    const LhsPlanes p = lhs_planes(workspace, lhs_dtype, m, k, TM);
-    // (steps per tile k / 64 = 4 blocks of 256: the plane array is sized in those; the tables in groups)
-    PlaneSpace ps = plane_space((uint8_t*)workspace + (p.bytes + 255) / 256 * 256, n, k, 1, false, nblk256, k / 128);
+    const LhsPlanes p = lhs_planes(lhs_space, lhs_dtype, m, k, TM);
     const WideLaunch L = wide_launch(out, m, n, groups);
     const SplitTiles& z = L.z;
     const int tiles_n128 = L.tiles_n128;
     hipError_t e = hipSuccess;
-    const int64_t conv = (int64_t)tiles_n128 * nblk256, blocks = conv + m + (int64_t)z.max_split * 64;
+    const int64_t conv = convert ? (int64_t)tiles_n128 * nblk256 : 0, blocks = conv + m + (int64_t)z.max_split * 64;
     if (blocks > INT32_MAX || k * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
     if (lhs_dtype == QMM_F32)
         gptq_planes_prologue_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(qweight, scales, qzeros, group, tiles_n128, ps.planes, ps.dtab,
-                                                                                       (int)conv, (const float*)lhs, (int)k, p, z);
+                                                                                       (int)conv, (const float*)lhs, (int)k, (int)m, p, z);
     else
         gptq_planes_prologue_kernel<uint16_t><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(qweight, scales, qzeros, group, tiles_n128, ps.planes, ps.dtab,
-                                                                                          (int)conv, (const uint16_t*)lhs, (int)k, p, z);
+                                                                                          (int)conv, (const uint16_t*)lhs, (int)k, (int)m, p, z);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     for (int pass = 0; pass < (p.a16_lo ? 2 : 1); pass++) {
@@ -1225,6 +1310,38 @@ hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_
         if (e != hipSuccess) return e;
     }
     return hipGetLastError();
+}
+// (steps per tile k / 64 = 4 blocks of 256: the plane array is sized in those; the tables in groups of 128, the smaller size)
+PlaneSpace gptq_space(void* base, int64_t n, int64_t k) { return plane_space(base, n, k, 1, false, k / 256, k / 128); }
+}  // namespace
+
+hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros,
+                                   int64_t m, int64_t n, int64_t k, int group, float* out, void* workspace, hipStream_t s) {
+    const int64_t lhs_bytes = (lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes + 255) / 256 * 256;
+    return run_gptq_planes(lhs, lhs_dtype, qweight, scales, qzeros, true, m, n, k, group, out, workspace,
+                           gptq_space((uint8_t*)workspace + lhs_bytes, n, k), s);
+}
+
+// GPTQ planes kept across calls.
+bool gptq_planes_supported(int64_t n, int64_t k, int group) { return (group == 128 || group == 256) && k % 256 == 0 && k >= 256 && n % 8 == 0; }
+int64_t repacked_gptq_bytes(int64_t n, int64_t k) { return gptq_space(nullptr, n, k).bytes; }
+hipError_t launch_repack_gptq(const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros, int64_t n, int64_t k, int group, void* packed,
+                              hipStream_t s) {
+    const PlaneSpace ps = gptq_space(packed, n, k);
+    const int tiles_n128 = (int)((n + TN - 1) / TN);
+    const int64_t conv = (int64_t)tiles_n128 * (k / 256);
+    if (conv > INT32_MAX) return hipErrorInvalidValue;
+    SplitTiles z{};
+    z.n = (int)n;
+    gptq_planes_prologue_kernel<uint16_t><<<dim3((unsigned)conv), dim3(256), 0, s>>>(qweight, scales, qzeros, group, tiles_n128, ps.planes, ps.dtab, (int)conv,
+                                                                                    nullptr, (int)k, 0, LhsPlanes{}, z);
+    return hipGetLastError();
+}
+bool repacked_gptq_wanted(int64_t m, int64_t n) { return m > 256 && wide_tiles(QMM_GPTQ, m, n); }
+int64_t repacked_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return (lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes + 255) / 256 * 256; }
+hipError_t launch_gemm_gptq_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, int group, float* out,
+                                     void* workspace, hipStream_t s) {
+    return run_gptq_planes(lhs, lhs_dtype, nullptr, nullptr, nullptr, false, m, n, k, group, out, workspace, gptq_space(const_cast<void*>(packed), n, k), s);
 }
 
 }  // namespace qmm

@@ -186,7 +186,7 @@ int static_scratch(void** ws) {
 
 extern "C" {
 
-int qmm_version(void) { return 103; }
+int qmm_version(void) { return 104; }
 
 const char* qmm_last_error(void) { return g_err; }
 
@@ -594,6 +594,84 @@ int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     void* ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;
     return qmm_matmul(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, out, ws, (int64_t)QMM_STATIC_SCRATCH_BYTES, flags, stream);
+}
+
+// Weight planes kept across calls.
+static bool repackable(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
+    if (n <= 0 || k < 256 || k % 256 || n > INT32_MAX || k > INT32_MAX) return false;
+    if (encoding == QMM_GPTQ) return cfg && cfg->bits == 4 && !cfg->desc_act && qmm::gptq_planes_supported(n, k, cfg->group_size);
+    return encoding == QMM_Q4_K || encoding == QMM_Q5_K || encoding == QMM_Q6_K;
+}
+
+int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
+    if (!repackable(encoding, cfg, n, k)) return 0;
+    return encoding == QMM_GPTQ ? qmm::repacked_gptq_bytes(n, k) : qmm::repacked_planes_bytes(encoding, n, k);
+}
+
+int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs, int n_rhs, int64_t n, int64_t k, void* packed,
+               int64_t packed_bytes, void* stream) {
+    if (!rhs || !packed) return fail(QMM_ERR_INVALID, "qmm_repack: null pointer");
+    if (!repackable(encoding, cfg, n, k))
+        return fail(QMM_ERR_UNSUPPORTED, "qmm_repack: no weight planes for encoding %d with N=%lld K=%lld (Q4_K, Q5_K, Q6_K, and 4-bit GPTQ with "
+                                         "plain groups of 128 or 256; K a multiple of 256)", encoding, (long long)n, (long long)k);
+    const int64_t need = qmm_repack_bytes(encoding, cfg, n, k);
+    if (packed_bytes < need) return fail(QMM_ERR_WORKSPACE, "qmm_repack: %lld bytes required (qmm_repack_bytes), %lld given", (long long)need, (long long)packed_bytes);
+    if (!aligned(packed, 256)) return fail(QMM_ERR_INVALID, "qmm_repack: the buffer must be 256-byte aligned");
+    if (encoding == QMM_GPTQ) {
+        if (n_rhs != 3 && n_rhs != 4) return fail(QMM_ERR_INVALID, "qmm_repack: GPTQ takes rhs = (qweight, scales, qzeros[, g_idx]), got %d", n_rhs);
+        if (int rc = check_gptq(cfg, n, k)) return rc;
+        for (int i = 0; i < 3; i++)
+            if (!rhs[i] || !aligned(rhs[i], 4)) return fail(QMM_ERR_INVALID, "qmm_repack: GPTQ rhs[%d] null or misaligned", i);
+        return hip_status(qmm::launch_repack_gptq((const uint32_t*)rhs[0], (const uint16_t*)rhs[1], (const uint32_t*)rhs[2], n, k, cfg->group_size,
+                                                  packed, (hipStream_t)stream), "qmm_repack(GPTQ)");
+    }
+    if (n_rhs != 1 || !rhs[0]) return fail(QMM_ERR_INVALID, "qmm_repack: GGUF encodings take exactly one rhs tensor");
+    if (!aligned(rhs[0], encoding == QMM_Q6_K ? 2 : 16)) return fail(QMM_ERR_INVALID, "qmm_repack: rhs misaligned (Q4_K / Q5_K 16 bytes, Q6_K 2)");
+    return hip_status(qmm::launch_repack_planes(encoding, (const uint8_t*)rhs[0], n, k, packed, (hipStream_t)stream), "qmm_repack");
+}
+
+// Does a call with these rows go through the planes?  Without the packed tensors every row count does.
+static bool repacked_path(int encoding, int64_t m, int64_t n, int64_t k, bool have_rhs) {
+    if (!have_rhs) return true;
+    return encoding == QMM_GPTQ ? qmm::repacked_gptq_wanted(m, n) : qmm::repacked_planes_wanted(encoding, m, n, k);
+}
+
+int64_t qmm_matmul_repacked_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    if (m <= 0 || n <= 0 || k < 256 || k % 256) return 0;
+    const int64_t planes = encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
+                                                : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
+    if (repacked_path(encoding, m, n, k, true)) return planes;
+    const OptionalPlanesScope no_planes(true);  // the other route: qmm_matmul's kernels on the packed tensors (or, without those, the planes)
+    return std::max(planes, qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k));
+}
+
+int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
+                        const void* const* rhs, int n_rhs, const void* packed, int64_t packed_bytes, int64_t n, float* out,
+                        void* workspace, int64_t workspace_bytes, int flags, void* stream) {
+    if (!lhs || !packed || !out) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: null pointer");
+    if (flags) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul_repacked: flags must be 0 (0x%x given)", flags);
+    if (m <= 0 || m > INT32_MAX) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: M=%lld", (long long)m);
+    if (!repackable(encoding, cfg, n, k))
+        return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul_repacked: no weight planes for encoding %d with N=%lld K=%lld", encoding, (long long)n, (long long)k);
+    if (packed_bytes < qmm_repack_bytes(encoding, cfg, n, k) || !aligned(packed, 256))
+        return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: the packed buffer must be 256-byte aligned and hold qmm_repack_bytes = %lld bytes (%lld given)",
+                    (long long)qmm_repack_bytes(encoding, cfg, n, k), (long long)packed_bytes);
+    if (!repacked_path(encoding, m, n, k, rhs != nullptr)) {
+        const OptionalPlanesScope no_planes(true);
+        return qmm_matmul(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, out, workspace, workspace_bytes, 0, stream);
+    }
+    if (lhs_dtype != QMM_F32 && lhs_dtype != QMM_BF16) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs dtype must be f32 or bf16");
+    if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs must be 16-byte aligned");
+    const int64_t need = encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
+                                              : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
+    if (!workspace || workspace_bytes < need)
+        return fail(QMM_ERR_WORKSPACE, "qmm_matmul_repacked: workspace of %lld bytes required, %lld given", (long long)need, (long long)workspace_bytes);
+    if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: workspace must be 256-byte aligned");
+    if (encoding == QMM_GPTQ)
+        return hip_status(qmm::launch_gemm_gptq_repacked(lhs, lhs_dtype, packed, m, n, k, cfg->group_size, out, workspace, (hipStream_t)stream),
+                          "qmm_matmul_repacked(GPTQ)");
+    return hip_status(qmm::launch_gemm_planes_repacked(encoding, lhs, lhs_dtype, packed, m, n, k, out, workspace, (hipStream_t)stream),
+                      "qmm_matmul_repacked");
 }
 
 int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, int count,

@@ -164,6 +164,23 @@ hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                               float* out, void* workspace, hipStream_t s);
+// Weight planes kept across calls: the conversion alone into a buffer of *_bytes, and the plane GEMMs over such a buffer (workspace:
+// the lhs planes only).  *_wanted: the row counts from which the planes beat the kernels that read the packed weights, the
+// conversion no longer counting.  The K-quant layout serves both plane GEMMs (Q4_K / Q5_K: min operands in both forms).
+int64_t repacked_planes_bytes(int encoding, int64_t n, int64_t k);
+hipError_t launch_repack_planes(int encoding, const uint8_t* w, int64_t n, int64_t k, void* packed, hipStream_t s);
+bool repacked_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k);
+int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t k);
+hipError_t launch_gemm_planes_repacked(int encoding, const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k,
+                                       float* out, void* workspace, hipStream_t s);
+bool gptq_planes_supported(int64_t n, int64_t k, int group);
+int64_t repacked_gptq_bytes(int64_t n, int64_t k);
+hipError_t launch_repack_gptq(const uint32_t* qweight, const uint16_t* scales, const uint32_t* qzeros, int64_t n, int64_t k, int group, void* packed,
+                              hipStream_t s);
+bool repacked_gptq_wanted(int64_t m, int64_t n);
+int64_t repacked_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
+hipError_t launch_gemm_gptq_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, int group, float* out,
+                                     void* workspace, hipStream_t s);
 
 hipError_t launch_block_dots_q4_0(const uint8_t* a_q8, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                   int32_t* out, hipStream_t s);

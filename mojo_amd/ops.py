@@ -148,6 +148,84 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
     return out.reshape(*lead, n)
 
 
+class RepackedWeights:
+    """The weights of one matrix as the plane GEMMs read them, made once by :func:`repack_weights` (the weight repack
+    step that MAX's graph compiler folds into model load).  ``rhs`` are the packed tensors the planes were made from, or
+    an empty tuple if the caller does not keep them (then every row count goes through the planes)."""
+
+    __slots__ = ("encoding", "config", "n", "k", "packed", "rhs")
+
+    def __init__(self, encoding, config, n, k, packed, rhs):
+        self.encoding, self.config, self.n, self.k, self.packed, self.rhs = encoding, config, n, k, packed, tuple(rhs)
+
+
+def _k_of(encoding: QuantizationEncoding, rhs) -> int:
+    if encoding == QuantizationEncoding.GPTQ:
+        return rhs[0].shape[0] * 8
+    bp = encoding.block_parameters
+    return rhs[0].shape[1] // bp.block_size * bp.elements_per_block
+
+
+def repack_weights(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], *rhs: torch.Tensor,
+                   keep_rhs: bool = True) -> RepackedWeights:
+    """Converts the packed weights of one matrix (the ``rhs`` of :func:`qmatmul`) into fp16 integer planes and scale tables,
+    once, for :func:`qmatmul_repacked`.  Q4_K, Q5_K, Q6_K and GPTQ with plain groups of 128 or 256 (K a multiple of 256);
+    other encodings raise ``NotImplementedError``.  The planes take 2 bytes per weight (Q6_K 4)."""
+    if not isinstance(encoding, QuantizationEncoding):
+        raise TypeError("encoding must be a QuantizationEncoding")
+    if not rhs or not isinstance(rhs[0], torch.Tensor) or rhs[0].dim() != 2:
+        raise TypeError("repack_weights takes the rhs tensors of qmatmul")
+    if not (encoding.is_gguf or encoding == QuantizationEncoding.GPTQ):
+        raise ValueError(f"{encoding.name} is not a weight encoding of qmatmul")
+    k = _k_of(encoding, rhs)
+    n, cfg_p = _check_rhs(encoding, config, k, rhs)
+    lib = _lib.load()
+    size = lib.qmm_repack_bytes(encoding.code, cfg_p, n, k)
+    if size <= 0:
+        raise NotImplementedError(f"repack_weights: no weight planes for {encoding.name} with N={n}, K={k}")
+    packed = torch.empty((size,), dtype=torch.uint8, device=rhs[0].device)
+    ptrs = (C.c_void_p * len(rhs))(*[t.data_ptr() for t in rhs])
+    _lib.check(lib.qmm_repack(encoding.code, cfg_p, ptrs, len(rhs), n, k, _ptr(packed), size, _stream(rhs[0])), "repack_weights")
+    return RepackedWeights(encoding, config, n, k, packed, rhs if keep_rhs else ())
+
+
+def qmatmul_repacked(lhs: torch.Tensor, weights: RepackedWeights, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """:func:`qmatmul` on weights converted beforehand: the same fp32 result, without the conversion pass that the prefill
+    GEMMs of :func:`qmatmul` run per call.  Row counts that the decode kernels serve go to them (on ``weights.rhs``)."""
+    if not isinstance(weights, RepackedWeights):
+        raise TypeError("weights must come from repack_weights")
+    _require_gpu(lhs, "lhs")
+    if lhs.dtype not in _DTYPES:
+        raise TypeError(f"lhs must be float32 or bfloat16, got {lhs.dtype}")
+    if lhs.dim() < 1 or lhs.shape[-1] != weights.k:
+        raise ValueError(f"lhs must end in K={weights.k}")
+    if lhs.device != weights.packed.device:
+        raise ValueError("lhs and the repacked weights must be on one device")
+    lead = lhs.shape[:-1]
+    m = 1
+    for d in lead:
+        m *= d
+    if m == 0:
+        raise ValueError("qmatmul of an empty tensor")
+    n, k, enc = weights.n, weights.k, weights.encoding
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+    else:
+        _require_gpu(out, "out")
+        if out.dtype != torch.float32 or out.numel() != m * n or out.device != lhs.device:
+            raise TypeError(f"out must be a contiguous float32 tensor of {m} x {n} elements on the device of lhs")
+    lib = _lib.load()
+    cfg_p = C.byref(_gptq_cfg(weights.config)) if enc == QuantizationEncoding.GPTQ else None
+    lhs_dt = _DTYPES[lhs.dtype]
+    need = lib.qmm_matmul_repacked_workspace_bytes(enc.code, lhs_dt, m, n, k)
+    ws = torch.empty((need,), dtype=torch.uint8, device=lhs.device) if need > 0 else None
+    ptrs = (C.c_void_p * len(weights.rhs))(*[t.data_ptr() for t in weights.rhs]) if weights.rhs else None
+    rc = lib.qmm_matmul_repacked(enc.code, cfg_p, _ptr(lhs), lhs_dt, m, k, ptrs, len(weights.rhs), _ptr(weights.packed),
+                                 weights.packed.numel(), n, _ptr(out), _ptr(ws), need, 0, _stream(lhs))
+    _lib.check(rc, "qmatmul_repacked")
+    return out.reshape(*lead, n)
+
+
 def qmatmul_rmsnorm(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], x: torch.Tensor,
                     gamma: torch.Tensor, eps: float, *rhs: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """``qmatmul(encoding, config, rms_norm(x, gamma, eps), *rhs)`` as one call: the normalisation in front of the

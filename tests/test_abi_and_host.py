@@ -111,8 +111,9 @@ def test_argument_validation_happens_before_any_launch():
 def test_workspace_figures_of_the_optional_weight_planes():
     """Host arithmetic only.  Large Q4_K / GPTQ prefill problems (more than 512 lhs rows, 160 or more tiles of 256 x 256)
     are quoted with room for fp16 weight planes, 2 bytes per weight; the same matrices with fewer rows, and small matrices,
-    are quoted for the kernels that unpack as they go (lhs planes only).  Q5_K / Q6_K always need their planes beyond 32 / 64
-    rows (Q6_K two of them)."""
+    are quoted for the kernels that unpack as they go (lhs planes only).  Q5_K / Q6_K always need their planes beyond 64
+    rows (Q6_K two of them; Q5_K from 33 rows where K is no multiple of 512).  Planes kept across calls: the buffer holds
+    them with both forms of the Q4_K / Q5_K min operands, and a call's workspace then only the lhs."""
     lib = _lib.load()
     n, k = 14336, 4096
     bf16 = _lib.QMM_BF16
@@ -122,9 +123,27 @@ def test_workspace_figures_of_the_optional_weight_planes():
         small_matrix = lib.qmm_matmul_workspace_bytes(enc.code, bf16, 2048, 2048, k)  # 8 x 8 tiles
         assert big >= 2 * n * k + 2048 * k * 2, enc
         assert mid < 32 << 20 and small_matrix < 64 << 20, enc
-    assert lib.qmm_matmul_workspace_bytes(QE.Q5_K.code, bf16, 40, n, k) >= 2 * n * k
+    assert lib.qmm_matmul_workspace_bytes(QE.Q5_K.code, bf16, 65, n, k) >= 2 * n * k
+    assert lib.qmm_matmul_workspace_bytes(QE.Q5_K.code, bf16, 40, n, k) == 0
+    assert lib.qmm_matmul_workspace_bytes(QE.Q5_K.code, bf16, 40, n, 4096 + 256) >= 2 * n * (4096 + 256)
     assert lib.qmm_matmul_workspace_bytes(QE.Q6_K.code, bf16, 70, n, k) >= 4 * n * k
     assert lib.qmm_matmul_workspace_bytes(QE.Q6_K.code, bf16, 64, n, k) == 0
+    for enc, per_weight in ((QE.Q4_K, 2), (QE.Q5_K, 2), (QE.Q6_K, 4)):
+        held = lib.qmm_repack_bytes(enc.code, None, n, k)
+        assert per_weight * n * k * (1.125 if per_weight == 2 else 1) <= held < per_weight * n * k * 1.2, enc  # (one extension block per eight)
+        ws = lib.qmm_matmul_repacked_workspace_bytes(enc.code, bf16, 2048, n, k)
+        assert 2048 * k * 2 <= ws < 2048 * k * 2 * 1.2 + (1 << 20), enc
+    cfg = _lib.GptqConfig(4, 128, 0, 1)
+    assert 2 * n * k <= lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(cfg), n, k) < 2.1 * n * k
+    assert lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(_lib.GptqConfig(4, 64, 0, 1)), n, k) == 0      # groups of 64: no plane GEMM
+    assert lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(_lib.GptqConfig(4, 128, 1, 1)), n, k) == 0     # act-order
+    assert lib.qmm_repack_bytes(QE.Q4_0.code, None, n, k) == 0 and lib.qmm_repack_bytes(QE.Q4_K.code, None, n, 4096 + 32) == 0
+    fake = C.c_void_p(0x1000)
+    assert lib.qmm_repack(QE.Q4_0.code, None, (C.c_void_p * 1)(0x1000), 1, n, k, fake, 1 << 40, None) == -2
+    assert lib.qmm_repack(QE.Q4_K.code, None, (C.c_void_p * 1)(0x1000), 1, n, k, fake, 16, None) == -4
+    assert lib.qmm_matmul_repacked(QE.Q4_K.code, None, fake, bf16, 2048, k, None, 0, fake, 1 << 40, n, fake, None, 0, 1, None) == -2  # flags
+    assert lib.qmm_matmul_repacked(QE.Q4_K.code, None, fake, bf16, 2048, k, None, 0, fake, 16, n, fake, None, 0, 0, None) == -1      # buffer too small
+    assert lib.qmm_matmul_repacked(QE.Q4_K.code, None, fake, bf16, 2048, k, None, 0, C.c_void_p(0x1000), 1 << 40, n, fake, None, 0, 0, None) == -4  # no workspace
 
 
 def test_quantization_encoding_metadata():

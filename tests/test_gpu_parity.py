@@ -695,10 +695,10 @@ def test_q4_k_gemm_tile_kernel(m, n, k, bf16):
 
 @pytest.mark.parametrize("enc,m,n,k,bf16", [
     (QE.Q6_K, 65, 130, 512, True), (QE.Q6_K, 300, 257, 1024, False), (QE.Q6_K, 1000, 9300, 768, True), (QE.Q6_K, 256, 128, 256, True),
-    (QE.Q5_K, 33, 130, 512, True), (QE.Q5_K, 300, 257, 1024, False), (QE.Q5_K, 1000, 9300, 768, True), (QE.Q5_K, 520, 8200, 256, False),
+    (QE.Q5_K, 65, 130, 512, True), (QE.Q5_K, 33, 130, 768, True), (QE.Q5_K, 300, 257, 1024, False), (QE.Q5_K, 1000, 9300, 768, True), (QE.Q5_K, 520, 8200, 256, False),
     (QE.Q5_K, 40, 24, 36864, True)])
 def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
-    """Q5_K above 32 and Q6_K above 64 lhs rows: the weights become fp16 integer planes (Q5_K sc * q; Q6_K two planes,
+    """Q5_K and Q6_K above 64 lhs rows (Q5_K above 32 where its small-batch kernel does not take K): the weights become fp16 integer planes (Q5_K sc * q; Q6_K two planes,
     (16 hi) * q and lo * q with sc = 16 hi + lo) and a tile GEMM multiplies them.  Ragged edges in m and n, one super-block,
     a last round of tiles cut in two K halves (292 tiles; for Q6_K the cut falls between or inside the planes), fp32 lhs
     (second pass on the residual), a K beyond what the Q5_K decode kernel takes; a third of the blocks carry random bytes

@@ -1,0 +1,125 @@
+"""GPU parity of the weight planes kept across calls (repack_weights / qmatmul_repacked) against the CPU oracle and against
+qmatmul, which converts per call.
+
+Bars: fp32 outputs within rtol 1e-3 / atol 1e-4 under the reference's symmetric isclose
+(stdlib/src/math/math.mojo:1023-1030); bit-identical to qmatmul wherever both run the same GEMM over the same planes.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from conftest import synth
+from mojo_amd import QuantizationConfig, QuantizationEncoding as QE
+from mojo_amd import qmatmul, qmatmul_repacked, repack_weights
+from test_gpu_parity import ENC, assert_close, gpu
+
+pytestmark = pytest.mark.gpu
+
+
+def kquant_weights(enc, n, k, seed):
+    """Quantised weights with every third block random bytes (finite scales) and every fifth with d = 0."""
+    e = ENC[enc]
+    bpb = {QE.Q4_K: 144, QE.Q5_K: 176, QE.Q6_K: 210}[enc]
+    w, _ = synth(seed, n, k, 1)
+    wq = O.quantize(e, w)
+    blocks = wq.reshape(-1, bpb)
+    rnd = np.random.default_rng(seed + 1).integers(0, 256, blocks.shape, dtype=np.uint8)
+    keep = slice(208, 210) if enc == QE.Q6_K else slice(0, 4)
+    rnd[:, keep] = blocks[:, keep]
+    blocks[::3] = rnd[::3]
+    blocks[::5, keep.start:keep.start + 2] = 0
+    return wq
+
+
+def lhs_rows(seed, m, k, bf16):
+    _, a = synth(seed, 1, k, m)
+    if bf16:
+        a = O.bf16_to_f32(O.f32_to_bf16(a))
+    return a, (gpu(a).to(torch.bfloat16) if bf16 else gpu(a))
+
+
+@pytest.mark.parametrize("enc,n,k,rows", [
+    # (row count, bf16 lhs, same route as qmatmul)
+    (QE.Q6_K, 300, 1024, [(70, True, True), (300, False, True), (3, True, True)]),
+    (QE.Q6_K, 9300, 768, [(1000, True, True)]),
+    (QE.Q5_K, 8200, 2304, [(1030, False, True), (40, True, True), (700, True, True), (2, False, True)]),
+    (QE.Q5_K, 257, 512, [(33, True, True), (300, False, True)]),
+    (QE.Q4_K, 14080, 768, [(520, True, True), (1600, False, True), (300, True, False), (64, True, True)]),
+    (QE.Q4_K, 20600, 256, [(2000, True, True), (300, True, False)]),
+])
+def test_repacked_kquant_matches_oracle_and_qmatmul(enc, n, k, rows):
+    """One conversion, many calls.  Q4_K / Q5_K planes carry their min operands both as extension blocks (wide GEMM: 1030 x 8200,
+    520 and 1600 x 14080, 2000 x 20600 in two launches) and as the table of the 256 x 128 kernel (40, 700 x 8200 and the small
+    matrix), which then steps over the extension blocks (K = 2304: two of them, one with a single super-block); Q6_K has one
+    layout.  Row counts of the decode kernels are served from the packed tensors.  300 x 20600 (162 tiles of 256 x 256) takes the wide tiles
+    here, 300 x 14080 the 256 x 128 plane kernel, and inside qmatmul both take kernels that unpack as they go: close, not identical."""
+    wq = kquant_weights(enc, n, k, 7 + n % 5)
+    wq_d = gpu(wq)
+    weights = repack_weights(enc, None, wq_d)
+    assert weights.n == n and weights.k == k
+    for m, bf16, same in rows:
+        a, lhs = lhs_rows(m, m, k, bf16)
+        truth = O.matmul_f64(ENC[enc], a, wq)
+        got = qmatmul_repacked(lhs, weights)
+        assert_close(got, truth, f"{enc.name} repacked {m}x{n}x{k} bf16={bf16}")
+        assert torch.equal(got, qmatmul_repacked(lhs, weights))
+        if same:
+            assert torch.equal(got, qmatmul(enc, None, lhs, wq_d)), f"{enc.name} {m}x{n}x{k}: differs from qmatmul"
+
+
+@pytest.mark.parametrize("group,n,k,rows", [
+    (128, 8200, 768, [(1600, True, True), (1540, False, True), (300, True, True), (5, True, True)]),
+    (256, 14192, 512, [(1990, False, True)]),
+    (128, 11016, 1280, [(1536, True, True)]),
+])
+def test_repacked_gptq_matches_oracle_and_qmatmul(group, n, k, rows):
+    """GPTQ planes (q - zero, scale blocks = groups) made once; groups with a zero scale; one and two launches of the wide GEMM, a
+    last round of tiles cut in K halves (1536 x 11016), K ending on half a 256-block."""
+    w, _ = synth(21, n, k, 1)
+    qw, sc, qz, gi = O.quantize_gptq(w, group)
+    sc[::2, ::7] = 0
+    cfg = QuantizationConfig(group_size=group)
+    rhs = (gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    weights = repack_weights(QE.GPTQ, cfg, *rhs)
+    for m, bf16, same in rows:
+        a, lhs = lhs_rows(30 + m, m, k, bf16)
+        truth = O.matmul_gptq(a, qw, sc, qz, group=group, f64=True)
+        got = qmatmul_repacked(lhs, weights)
+        assert_close(got, truth, f"GPTQ g{group} repacked {m}x{n}x{k} bf16={bf16}")
+        if same:
+            assert torch.equal(got, qmatmul(QE.GPTQ, cfg, lhs, *rhs)), f"GPTQ {m}x{n}x{k}: differs from qmatmul"
+
+
+@pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q5_K, QE.Q6_K, QE.GPTQ])
+def test_repacked_without_the_packed_tensors(enc):
+    """keep_rhs=False: the planes are all the caller holds, and every row count goes through the plane GEMMs (one lhs row, a
+    few, a ragged row tile; small matrices run the 256 x 128 kernel, GPTQ the wide one)."""
+    n, k = 264, 1024
+    if enc == QE.GPTQ:
+        w, _ = synth(41, n, k, 1)
+        qw, sc, qz, gi = O.quantize_gptq(w, 128)
+        cfg = QuantizationConfig(group_size=128)
+        weights = repack_weights(enc, cfg, gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi), keep_rhs=False)
+        truth_of = lambda a: O.matmul_gptq(a, qw, sc, qz, group=128, f64=True)
+    else:
+        wq = kquant_weights(enc, n, k, 43)
+        weights = repack_weights(enc, None, gpu(wq), keep_rhs=False)
+        truth_of = lambda a: O.matmul_f64(ENC[enc], a, wq)
+    assert weights.rhs == ()
+    for m, bf16 in [(1, True), (5, False), (270, True)]:
+        a, lhs = lhs_rows(50 + m, m, k, bf16)
+        assert_close(qmatmul_repacked(lhs, weights), truth_of(a), f"{enc.name} planes only, {m} rows")
+
+
+def test_repack_refusals():
+    w = torch.zeros((8, 18 * 8), dtype=torch.uint8, device="cuda:0")
+    with pytest.raises(NotImplementedError):
+        repack_weights(QE.Q4_0, None, w)  # no plane GEMM over kept planes for Q4_0
+    n, k = 64, 512
+    wq, _ = synth(3, n, k, 1)
+    qw, sc, qz, gi = O.quantize_gptq(wq, 64)
+    with pytest.raises(NotImplementedError):
+        repack_weights(QE.GPTQ, QuantizationConfig(group_size=64), gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
+    with pytest.raises(TypeError):
+        qmatmul_repacked(torch.zeros((1, 256), device="cuda:0"), "weights")
