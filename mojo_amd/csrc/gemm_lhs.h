@@ -83,10 +83,26 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
     __shared__ uint32_t wmax[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const AT* ar = a + (int64_t)row * k;
+    // Rows of up to 8192 elements stay in registers between the maximum search and the conversion (one read of the row).
+    constexpr int kHeld = 8;
+    float held[kHeld][4];
+    const bool hold = k <= kHeld * 1024;
     float mx = 0.0f;
-    for (int i = tid * 4; i < k; i += 1024) {
-        float x0 = load_f32(ar, i), x1 = load_f32(ar, i + 1), x2 = load_f32(ar, i + 2), x3 = load_f32(ar, i + 3);
-        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3))));
+    if (hold) {
+#pragma unroll
+        for (int it = 0; it < kHeld; it++) {
+            const int i = tid * 4 + it * 1024;
+            if (i < k) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) held[it][q] = load_f32(ar, i + q);
+                mx = fmaxf(mx, fmaxf(fmaxf(fabsf(held[it][0]), fabsf(held[it][1])), fmaxf(fabsf(held[it][2]), fabsf(held[it][3]))));
+            }
+        }
+    } else {
+        for (int i = tid * 4; i < k; i += 1024) {
+            float x0 = load_f32(ar, i), x1 = load_f32(ar, i + 1), x2 = load_f32(ar, i + 2), x3 = load_f32(ar, i + 3);
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3))));
+        }
     }
     const uint32_t mb = wave_max_nonneg_bits(mx);
     if (lane == 0) wmax[wave] = mb;
@@ -96,9 +112,7 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
     if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite row: leave unscaled
     const float s = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
     if (tid == 0) inv[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
-    for (int i = tid * 4; i < k; i += 1024) {
-        const float x0 = load_f32(ar, i) * s, x1 = load_f32(ar, i + 1) * s, x2 = load_f32(ar, i + 2) * s,
-                    x3 = load_f32(ar, i + 3) * s;
+    auto emit = [&](int i, float x0, float x1, float x2, float x3) __attribute__((always_inline)) {
         const float h0 = h2f(f2h(x0)), h1 = h2f(f2h(x1)), h2 = h2f(f2h(x2)), h3 = h2f(f2h(x3));
         const int kl = i & 63;
         if constexpr (ORDER == kLhsOrderQ4K) {
@@ -145,6 +159,15 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
                 as[8 + j] = (_Float16)(sum - sh);
             }
         }
+    };
+    if (hold) {
+#pragma unroll
+        for (int it = 0; it < kHeld; it++) {
+            const int i = tid * 4 + it * 1024;
+            if (i < k) emit(i, held[it][0] * s, held[it][1] * s, held[it][2] * s, held[it][3] * s);
+        }
+    } else {
+        for (int i = tid * 4; i < k; i += 1024) emit(i, load_f32(ar, i) * s, load_f32(ar, i + 1) * s, load_f32(ar, i + 2) * s, load_f32(ar, i + 3) * s);
     }
     for (int i = (k >> 8) * 32 + tid; i < next * 256; i += 256) a16[(int64_t)row * lda + k + i] = (_Float16)0.0f;
 }

@@ -1165,7 +1165,9 @@ hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const
     // tiles on the zeroing and the atomic adds cost what the halves gain (4096 x 4096, 1024 rows: 63 -> 72 us), unless K is long
     // (4096 x 14336, 1024 rows: 188 -> 159 us).
     const int per_xcd_cus = std::max(1, compute_units() / 8);
-    const bool halve_all = 2 * per_xcd <= per_xcd_cus && nblk >= 2 && (total <= 96 || nblk >= 32);
+    // (A single row tile with at most 192 rows leaves a wavefront row without work, and the halves pay up to 128 tiles:
+    // 14336 x 4096 with 65 rows, Q6_K 160 -> 118 us; with 256 rows 60 -> 62 us.)
+    const bool halve_all = 2 * per_xcd <= per_xcd_cus && nblk >= 2 && (total <= 96 || nblk >= 32 || m <= 192);
     const int wg = 8 * (halve_all ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
     const WideLaunch L = wide ? wide_launch(out, m, n, nblk_tile) : WideLaunch{};
     const SplitTiles z = wide ? L.z : split_tiles(out, m, n, tiles_m, tiles_n, nblk, wg, TN);
