@@ -182,10 +182,11 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
  * snapshot, see the top of this file); this pair of calls is the explicit form of it for the prefill GEMMs here:
  * qmm_repack converts the packed weights of one matrix once into the fp16 integer planes and scale tables that the
  * matrix-core GEMMs read (2 bytes per weight, Q6_K 4, plus tables: qmm_repack_bytes, 0 if the encoding or shape has
- * no plane GEMM: Q4_0, GPTQ with act-order or groups other than 128 / 256, K not a multiple of 256), into a buffer
+ * no plane GEMM: GPTQ with act-order or groups other than 128 / 256, K not a multiple of 256; Q4_0: the plane of q - 8 and
+ * its block scales, the lhs is still quantised to Q8_0 per call), into a buffer
  * the caller owns, 256-byte aligned; the buffer depends on the weights only.  qmm_matmul_repacked is qmm_matmul with
- * that buffer at hand: row counts for which the plane GEMMs are the faster route (Q6_K above 64 rows, Q5_K above
- * 32, Q4_K / GPTQ above 256 on matrices with at least 160 output tiles of 256 x 256) skip the conversion that
+ * that buffer at hand: row counts for which the plane GEMMs are the faster route (Q5_K / Q6_K from 49 rows, 33 on large matrices; Q4_0 from 49; Q4_K from
+ * 129 with at least 64 tiles of 256 x 128; GPTQ from 257 with at least 160 tiles of 256 x 256) skip the conversion that
  * qmm_matmul repeats per call (same kernels, same planes: where qmm_matmul takes the planes too the results are equal
  * bit for bit); other row counts are handed to qmm_matmul with `rhs`.  rhs = NULL (a caller that dropped the packed tensors): every row count goes through the planes.
  * flags must be 0.  Workspace: qmm_matmul_repacked_workspace_bytes (the lhs planes, or what qmm_matmul needs for the

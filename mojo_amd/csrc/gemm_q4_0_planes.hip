@@ -48,18 +48,20 @@ struct Q40Space {
     uint16_t* dw;     // [tiles_n][k / 256][128][8] weight block scales (fp16 bits)
     int64_t bytes;
 };
-Q40Space q40_space(void* base, int64_t m, int64_t n, int64_t k) {
+// The lhs part at `lhs_base`, the weight part at `w_base` (directly behind the lhs part if null: one workspace holds both).
+Q40Space q40_space(void* lhs_base, int64_t m, int64_t n, int64_t k, void* w_base = nullptr) {
     auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
     const int64_t m_pad = (m + TM - 1) / TM * TM, tiles_n = (n + TN - 1) / TN;
     Q40Space p;
     int64_t off = 0;
-    p.a16 = (_Float16*)((uint8_t*)base + off);
+    p.a16 = (_Float16*)((uint8_t*)lhs_base + off);
     off += up(m_pad * k * 2);
-    p.da = (uint16_t*)((uint8_t*)base + off);
+    p.da = (uint16_t*)((uint8_t*)lhs_base + off);
     off += up(m_pad * (k / 32) * 2);
-    p.planes = (uint8_t*)base + off;
+    uint8_t* wb = w_base ? (uint8_t*)w_base - off : (uint8_t*)lhs_base;
+    p.planes = wb + off;
     off += up(tiles_n * (k / 64) * kBBuf);
-    p.dw = (uint16_t*)((uint8_t*)base + off);
+    p.dw = (uint16_t*)(wb + off);
     off += up(tiles_n * (k / 256) * kDwBuf);
     p.bytes = off;
     return p;
@@ -136,15 +138,15 @@ __device__ __forceinline__ void q4_0_lhs_row(int row, const AT* __restrict__ a, 
 
 template <typename AT>
 __global__ __launch_bounds__(256) void q4_0_planes_prologue_kernel(const uint8_t* __restrict__ w, int nblk32, Q40Space sp, int conv,
-                                                                   const AT* __restrict__ a, int k, SplitTiles z) {
+                                                                   const AT* __restrict__ a, int k, int lhs_rows, SplitTiles z) {
     const int b = (int)blockIdx.x;
     if (b < conv) {
         const int t = b >> 2, grp = t / z.tiles_n;
         q4_0_plane_part(t - grp * z.tiles_n, grp, b & 3, w, z.n, nblk32, sp.planes, sp.dw);
-    } else if (b < conv + z.m) {
+    } else if (b < conv + lhs_rows) {
         q4_0_lhs_row<AT>(b - conv, a, k, sp.a16, sp.da);
     } else {
-        const int e = b - conv - z.m;
+        const int e = b - conv - lhs_rows;
         zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
     }
 }
@@ -407,33 +409,57 @@ bool gemm_q4_0_planes_wanted(int64_t m, int64_t n, int64_t k) {
 
 int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k) { return q40_space(nullptr, m, n, k).bytes; }
 
-hipError_t launch_gemm_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out,
-                                   void* workspace, hipStream_t s) {
-    const Q40Space sp = q40_space(workspace, m, n, k);
+namespace {
+// convert: the weight plane in `sp` is made from `w` in the preparation launch; otherwise it was made earlier.
+hipError_t run_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, bool convert, int64_t m, int64_t n, int64_t k, float* out,
+                           const Q40Space& sp, hipStream_t s) {
     hipError_t e = allow_full_lds<gemm_q4_0_planes_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n = (int)((n + TN - 1) / TN), ngrp = (int)(k / 256);
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-    }
-    const int wg = 8 * std::min(per_xcd, std::max(1, cus / 8));
-    const SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, ngrp, wg);
-    const int64_t conv = (int64_t)tiles_n * ngrp * 4, blocks = conv + m + (int64_t)z.max_split * 64;
+    // Tiles for no more than half of the compute units: a workgroup per compute unit all the same, and the unit arithmetic cuts
+    // every tile in two K halves (a tile's time is set by K).
+    const int per_xcd_cus = std::max(1, compute_units() / 8);
+    const bool halve_all = 2 * per_xcd <= per_xcd_cus && ngrp >= 2;
+    const int wg = 8 * (halve_all ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
+    SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, ngrp, wg);
+    const int64_t conv = convert ? (int64_t)tiles_n * ngrp * 4 : 0, blocks = conv + m + (int64_t)z.max_split * 64;
     if (blocks > INT32_MAX) return hipErrorInvalidValue;
     const dim3 pgrid((unsigned)blocks);
     if (lhs_dtype == QMM_F32)
-        q4_0_planes_prologue_kernel<float><<<pgrid, dim3(256), 0, s>>>(w, (int)(k / 32), sp, (int)conv, (const float*)lhs, (int)k, z);
+        q4_0_planes_prologue_kernel<float><<<pgrid, dim3(256), 0, s>>>(w, (int)(k / 32), sp, (int)conv, (const float*)lhs, (int)k, (int)m, z);
     else
-        q4_0_planes_prologue_kernel<uint16_t><<<pgrid, dim3(256), 0, s>>>(w, (int)(k / 32), sp, (int)conv, (const uint16_t*)lhs, (int)k, z);
+        q4_0_planes_prologue_kernel<uint16_t><<<pgrid, dim3(256), 0, s>>>(w, (int)(k / 32), sp, (int)conv, (const uint16_t*)lhs, (int)k, (int)m, z);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     gemm_q4_0_planes_kernel<<<dim3((unsigned)wg), dim3(512), kQ40Lds, s>>>(sp.planes, sp.dw, sp.a16, sp.da, out, (int)m, (int)n, (int)k,
                                                                          tiles_m, tiles_n, z.max_split > 0 ? 1 : 0);
     return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_gemm_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out,
+                                   void* workspace, hipStream_t s) {
+    return run_q4_0_planes(lhs, lhs_dtype, w, true, m, n, k, out, q40_space(workspace, m, n, k), s);
+}
+
+// The weight plane kept across calls: the conversion alone, and the GEMM over a plane made by it (workspace: the lhs part).
+int64_t repacked_q4_0_bytes(int64_t n, int64_t k) { return q40_space(nullptr, 0, n, k).bytes; }
+hipError_t launch_repack_q4_0(const uint8_t* w, int64_t n, int64_t k, void* packed, hipStream_t s) {
+    const Q40Space sp = q40_space(nullptr, 0, n, k, packed);
+    const int tiles_n = (int)((n + TN - 1) / TN);
+    const int64_t conv = (int64_t)tiles_n * (k / 256) * 4;
+    if (conv > INT32_MAX) return hipErrorInvalidValue;
+    SplitTiles z{};
+    z.n = (int)n;
+    z.tiles_n = tiles_n;
+    q4_0_planes_prologue_kernel<uint16_t><<<dim3((unsigned)conv), dim3(256), 0, s>>>(w, (int)(k / 32), sp, (int)conv, nullptr, (int)k, 0, z);
+    return hipGetLastError();
+}
+int64_t repacked_q4_0_workspace_bytes(int64_t m, int64_t k) { return q40_space(nullptr, m, 0, k).bytes; }
+hipError_t launch_gemm_q4_0_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, float* out,
+                                     void* workspace, hipStream_t s) {
+    return run_q4_0_planes(lhs, lhs_dtype, nullptr, false, m, n, k, out, q40_space(workspace, m, n, k, const_cast<void*>(packed)), s);
 }
 
 }  // namespace qmm

@@ -600,11 +600,12 @@ int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs,
 static bool repackable(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
     if (n <= 0 || k < 256 || k % 256 || n > INT32_MAX || k > INT32_MAX) return false;
     if (encoding == QMM_GPTQ) return cfg && cfg->bits == 4 && !cfg->desc_act && qmm::gptq_planes_supported(n, k, cfg->group_size);
-    return encoding == QMM_Q4_K || encoding == QMM_Q5_K || encoding == QMM_Q6_K;
+    return encoding == QMM_Q4_K || encoding == QMM_Q5_K || encoding == QMM_Q6_K || encoding == QMM_Q4_0;
 }
 
 int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
     if (!repackable(encoding, cfg, n, k)) return 0;
+    if (encoding == QMM_Q4_0) return qmm::repacked_q4_0_bytes(n, k);
     return encoding == QMM_GPTQ ? qmm::repacked_gptq_bytes(n, k) : qmm::repacked_planes_bytes(encoding, n, k);
 }
 
@@ -612,7 +613,7 @@ int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs,
                int64_t packed_bytes, void* stream) {
     if (!rhs || !packed) return fail(QMM_ERR_INVALID, "qmm_repack: null pointer");
     if (!repackable(encoding, cfg, n, k))
-        return fail(QMM_ERR_UNSUPPORTED, "qmm_repack: no weight planes for encoding %d with N=%lld K=%lld (Q4_K, Q5_K, Q6_K, and 4-bit GPTQ with "
+        return fail(QMM_ERR_UNSUPPORTED, "qmm_repack: no weight planes for encoding %d with N=%lld K=%lld (Q4_0, Q4_K, Q5_K, Q6_K, and 4-bit GPTQ with "
                                          "plain groups of 128 or 256; K a multiple of 256)", encoding, (long long)n, (long long)k);
     const int64_t need = qmm_repack_bytes(encoding, cfg, n, k);
     if (packed_bytes < need) return fail(QMM_ERR_WORKSPACE, "qmm_repack: %lld bytes required (qmm_repack_bytes), %lld given", (long long)need, (long long)packed_bytes);
@@ -626,20 +627,26 @@ int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs,
                                                   packed, (hipStream_t)stream), "qmm_repack(GPTQ)");
     }
     if (n_rhs != 1 || !rhs[0]) return fail(QMM_ERR_INVALID, "qmm_repack: GGUF encodings take exactly one rhs tensor");
-    if (!aligned(rhs[0], encoding == QMM_Q6_K ? 2 : 16)) return fail(QMM_ERR_INVALID, "qmm_repack: rhs misaligned (Q4_K / Q5_K 16 bytes, Q6_K 2)");
+    if (!aligned(rhs[0], encoding == QMM_Q6_K || encoding == QMM_Q4_0 ? 2 : 16))
+        return fail(QMM_ERR_INVALID, "qmm_repack: rhs misaligned (Q4_K / Q5_K 16 bytes, Q4_0 / Q6_K 2)");
+    if (encoding == QMM_Q4_0)
+        return hip_status(qmm::launch_repack_q4_0((const uint8_t*)rhs[0], n, k, packed, (hipStream_t)stream), "qmm_repack(Q4_0)");
     return hip_status(qmm::launch_repack_planes(encoding, (const uint8_t*)rhs[0], n, k, packed, (hipStream_t)stream), "qmm_repack");
 }
 
 // Does a call with these rows go through the planes?  Without the packed tensors every row count does.
+constexpr int64_t kQ40RepackedMinRows = 48;  // 14336 x 4096: the plane GEMM 55 us, the int8 kernels 57 us at 48 rows, 59 at 64 (4096 x 4096: 49 against 52 at 64)
 static bool repacked_path(int encoding, int64_t m, int64_t n, int64_t k, bool have_rhs) {
     if (!have_rhs) return true;
+    if (encoding == QMM_Q4_0) return m > kQ40RepackedMinRows;
     return encoding == QMM_GPTQ ? qmm::repacked_gptq_wanted(m, n) : qmm::repacked_planes_wanted(encoding, m, n, k);
 }
 
 int64_t qmm_matmul_repacked_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || n <= 0 || k < 256 || k % 256) return 0;
-    const int64_t planes = encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
-                                                : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
+    const int64_t planes = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, k)
+                           : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
+                                                  : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
     if (repacked_path(encoding, m, n, k, true)) return planes;
     const OptionalPlanesScope no_planes(true);  // the other route: qmm_matmul's kernels on the packed tensors (or, without those, the planes)
     return std::max(planes, qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k));
@@ -662,11 +669,14 @@ int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lh
     }
     if (lhs_dtype != QMM_F32 && lhs_dtype != QMM_BF16) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs dtype must be f32 or bf16");
     if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs must be 16-byte aligned");
-    const int64_t need = encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
-                                              : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
+    const int64_t need = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, k)
+                         : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
+                                                : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
     if (!workspace || workspace_bytes < need)
         return fail(QMM_ERR_WORKSPACE, "qmm_matmul_repacked: workspace of %lld bytes required, %lld given", (long long)need, (long long)workspace_bytes);
     if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: workspace must be 256-byte aligned");
+    if (encoding == QMM_Q4_0)
+        return hip_status(qmm::launch_gemm_q4_0_repacked(lhs, lhs_dtype, packed, m, n, k, out, workspace, (hipStream_t)stream), "qmm_matmul_repacked(Q4_0)");
     if (encoding == QMM_GPTQ)
         return hip_status(qmm::launch_gemm_gptq_repacked(lhs, lhs_dtype, packed, m, n, k, cfg->group_size, out, workspace, (hipStream_t)stream),
                           "qmm_matmul_repacked(GPTQ)");

@@ -164,6 +164,13 @@ hipError_t launch_gemm_gptq_planes(const void* lhs, int lhs_dtype, const uint32_
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                               float* out, void* workspace, hipStream_t s);
+int compute_units();  // of the current device, read once (gemm_planes.hip)
+// The Q4_0 weight plane kept across calls (gemm_q4_0_planes.hip)
+int64_t repacked_q4_0_bytes(int64_t n, int64_t k);
+hipError_t launch_repack_q4_0(const uint8_t* w, int64_t n, int64_t k, void* packed, hipStream_t s);
+int64_t repacked_q4_0_workspace_bytes(int64_t m, int64_t k);
+hipError_t launch_gemm_q4_0_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, float* out,
+                                     void* workspace, hipStream_t s);
 // Weight planes kept across calls: the conversion alone into a buffer of *_bytes, and the plane GEMMs over such a buffer (workspace:
 // the lhs planes only).  *_wanted: the row counts from which the planes beat the kernels that read the packed weights, the
 // conversion no longer counting.  The K-quant layout serves both plane GEMMs (Q4_K / Q5_K: min operands in both forms).

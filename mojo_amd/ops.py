@@ -169,7 +169,7 @@ def _k_of(encoding: QuantizationEncoding, rhs) -> int:
 def repack_weights(encoding: QuantizationEncoding, config: Optional[QuantizationConfig], *rhs: torch.Tensor,
                    keep_rhs: bool = True) -> RepackedWeights:
     """Converts the packed weights of one matrix (the ``rhs`` of :func:`qmatmul`) into fp16 integer planes and scale tables,
-    once, for :func:`qmatmul_repacked`.  Q4_K, Q5_K, Q6_K and GPTQ with plain groups of 128 or 256 (K a multiple of 256);
+    once, for :func:`qmatmul_repacked`.  Q4_0, Q4_K, Q5_K, Q6_K and GPTQ with plain groups of 128 or 256 (K a multiple of 256);
     other encodings raise ``NotImplementedError``.  The planes take 2 bytes per weight (Q6_K 4)."""
     if not isinstance(encoding, QuantizationEncoding):
         raise TypeError("encoding must be a QuantizationEncoding")

@@ -137,9 +137,10 @@ def test_workspace_figures_of_the_optional_weight_planes():
     assert 2 * n * k <= lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(cfg), n, k) < 2.1 * n * k
     assert lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(_lib.GptqConfig(4, 64, 0, 1)), n, k) == 0      # groups of 64: no plane GEMM
     assert lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(_lib.GptqConfig(4, 128, 1, 1)), n, k) == 0     # act-order
-    assert lib.qmm_repack_bytes(QE.Q4_0.code, None, n, k) == 0 and lib.qmm_repack_bytes(QE.Q4_K.code, None, n, 4096 + 32) == 0
+    assert 2 * n * k <= lib.qmm_repack_bytes(QE.Q4_0.code, None, n, k) < 2.1 * n * k
+    assert lib.qmm_repack_bytes(QE.Q8_0.code, None, n, k) == 0 and lib.qmm_repack_bytes(QE.Q4_K.code, None, n, 4096 + 32) == 0
     fake = C.c_void_p(0x1000)
-    assert lib.qmm_repack(QE.Q4_0.code, None, (C.c_void_p * 1)(0x1000), 1, n, k, fake, 1 << 40, None) == -2
+    assert lib.qmm_repack(QE.Q8_0.code, None, (C.c_void_p * 1)(0x1000), 1, n, k, fake, 1 << 40, None) == -2
     assert lib.qmm_repack(QE.Q4_K.code, None, (C.c_void_p * 1)(0x1000), 1, n, k, fake, 16, None) == -4
     assert lib.qmm_matmul_repacked(QE.Q4_K.code, None, fake, bf16, 2048, k, None, 0, fake, 1 << 40, n, fake, None, 0, 1, None) == -2  # flags
     assert lib.qmm_matmul_repacked(QE.Q4_K.code, None, fake, bf16, 2048, k, None, 0, fake, 16, n, fake, None, 0, 0, None) == -1      # buffer too small

@@ -91,6 +91,25 @@ def test_repacked_gptq_matches_oracle_and_qmatmul(group, n, k, rows):
             assert torch.equal(got, qmatmul(QE.GPTQ, cfg, lhs, *rhs)), f"GPTQ {m}x{n}x{k}: differs from qmatmul"
 
 
+@pytest.mark.parametrize("n,k,rows", [(300, 1024, [(70, True), (300, False), (16, True)]), (9300, 768, [(1000, True)])])
+def test_repacked_q4_0_matches_oracle_and_qmatmul(n, k, rows):
+    """Q4_0: the plane of q - 8 and the block scales made once.  The lhs is quantised to Q8_0 per call as everywhere, so the
+    result is that of the integer block dots: bit-identical with qmatmul above 64 rows (same GEMM), within the bar of the
+    oracle's Q8_0 x Q4_0 product at every row count; without the packed tensor few rows run over the plane too."""
+    w, _ = synth(17, n, k, 1)
+    wq = O.quantize(O.Q4_0, w)
+    wq_d = gpu(wq)
+    weights = repack_weights(QE.Q4_0, None, wq_d)
+    alone = repack_weights(QE.Q4_0, None, wq_d, keep_rhs=False)
+    for m, bf16 in rows:
+        a, lhs = lhs_rows(60 + m, m, k, bf16)
+        want = O.matmul_q4_0(a, wq)
+        got = qmatmul_repacked(lhs, weights)
+        assert_close(got, want, f"Q4_0 repacked {m}x{n}x{k} bf16={bf16}")
+        assert torch.equal(got, qmatmul(QE.Q4_0, None, lhs, wq_d)), f"Q4_0 {m}x{n}x{k}: differs from qmatmul"
+        assert_close(qmatmul_repacked(lhs, alone), want, f"Q4_0 plane only {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("enc", [QE.Q4_K, QE.Q5_K, QE.Q6_K, QE.GPTQ])
 def test_repacked_without_the_packed_tensors(enc):
     """keep_rhs=False: the planes are all the caller holds, and every row count goes through the plane GEMMs (one lhs row, a
@@ -113,9 +132,9 @@ def test_repacked_without_the_packed_tensors(enc):
 
 
 def test_repack_refusals():
-    w = torch.zeros((8, 18 * 8), dtype=torch.uint8, device="cuda:0")
+    w = torch.zeros((8, 18 * 4), dtype=torch.uint8, device="cuda:0")
     with pytest.raises(NotImplementedError):
-        repack_weights(QE.Q4_0, None, w)  # no plane GEMM over kept planes for Q4_0
+        repack_weights(QE.Q4_0, None, w)  # K = 128: the plane GEMMs take multiples of 256
     n, k = 64, 512
     wq, _ = synth(3, n, k, 1)
     qw, sc, qz, gi = O.quantize_gptq(wq, 64)
