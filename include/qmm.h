@@ -186,7 +186,7 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
  * its block scales, the lhs is still quantised to Q8_0 per call), into a buffer
  * the caller owns, 256-byte aligned; the buffer depends on the weights only.  qmm_matmul_repacked is qmm_matmul with
  * that buffer at hand: row counts for which the plane GEMMs are the faster route (Q5_K / Q6_K from 49 rows, 33 on large matrices; Q4_0 from 49; Q4_K from
- * 129 with at least 64 tiles of 256 x 128; GPTQ from 257 with at least 160 tiles of 256 x 256) skip the conversion that
+ * 129 with at least 64 tiles of 256 x 128; GPTQ from 257 with at least 160 tiles of 256 x 256, or from 97 with at most 64) skip the conversion that
  * qmm_matmul repeats per call (same kernels, same planes: where qmm_matmul takes the planes too the results are equal
  * bit for bit); other row counts are handed to qmm_matmul with `rhs`.  rhs = NULL (a caller that dropped the packed tensors): every row count goes through the planes.
  * flags must be 0.  Workspace: qmm_matmul_repacked_workspace_bytes (the lhs planes, or what qmm_matmul needs for the
