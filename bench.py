@@ -746,7 +746,31 @@ def extra_timings(layers, acts, gen):
     us = dev_s * 1e6 / 20
     tf = 2 * 2048 * 14336 * 4096 / us / 1e6
     out["gptq_prefill_m2048"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
-    del wg
+    kept = RepackedGemv(QE.GPTQ, wg[:3], ab)
+    dev_s, _ = time_graphs([capture([kept])], 20, 3)
+    us = dev_s * 1e6 / 20
+    tf = 2 * 2048 * 14336 * 4096 / us / 1e6
+    out["gptq_prefill_m2048_repacked"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
+    del wg, kept
+    # a prefill step of one layer: the seven Q4_K projections with 2048 / 512 lhs rows (bf16), as qmm_matmul calls and over
+    # weight planes made once (qmm_repack; the planes of a layer take 0.5 GB)
+    ws = [make_weight(QE.Q4_K, n, k, gen) for _, n, k in PROJ]
+    for rows in (2048, 512):
+        acts = {k: torch.randn((rows, k), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16) for k in (4096, 14336)}
+        flops = sum(2.0 * rows * n * k for _, n, k in PROJ)
+        res = {}
+        qkv = torch.cat(ws[0:3])  # rows of packed blocks are independent: q | k | v as one matrix of 6144 rows
+        for name, calls in (("qmm_matmul", [Gemv(QE.Q4_K, w, acts[k]) for w, (_, n, k) in zip(ws, PROJ)]),
+                            ("qmm_matmul_repacked", [RepackedGemv(QE.Q4_K, (w,), acts[k]) for w, (_, n, k) in zip(ws, PROJ)]),
+                            ("qmm_matmul_repacked_qkv_as_one_matrix", [RepackedGemv(QE.Q4_K, (qkv,), acts[4096])] +
+                             [RepackedGemv(QE.Q4_K, (w,), acts[k]) for w, (_, n, k) in list(zip(ws, PROJ))[3:]])):
+            dev_s, _ = time_graphs([capture(calls)], 10, 2)
+            us = dev_s * 1e6 / 10
+            res[name] = {"us_per_step": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1), "frac_of_2500": round(flops / us / 1e6 / BF16_PEAK_TFLOPS, 4)}
+            del calls
+        del qkv
+        out[f"q4_k_prefill_layer_m{rows}"] = res
+    del ws
     # cfg1 / cfg2: Q4_0 with Q8_0 activations
     for tag, mm, n, k, copies in (("q4_0_m1_4096x4096", 1, 4096, 4096, 32), ("q4_0_m16_14336x4096", 16, 14336, 4096, 10)):
         am = torch.randn((mm, k), dtype=torch.float32, device="cuda:0", generator=gen)
