@@ -439,7 +439,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path runs on a single MI355X and --gpus {args.gpus} is not "
-              "supported (sharding by N is described in DESIGN.md).", file=sys.stderr)
+              "supported (the path would shard by output columns N across GPUs; that is not built).", file=sys.stderr)
         return 2
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
