@@ -260,8 +260,15 @@ __global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __r
         prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv, (int64_t)k + lhs_ext * 256, lhs_ext);
     } else {
         const int e = b - conv - lhs_rows;
-        zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
+        if (z.part) zero_flat(z.out, z.part, (int64_t)z.m * z.n, e);
+        else zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
     }
+}
+
+// out += part (the second pair of K quarters of gemm_planes_kernel's quarter mode)
+__global__ __launch_bounds__(256) void add_part_kernel(float* __restrict__ out, const float* __restrict__ part, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) out[i] += part[i];
 }
 
 // The GEMM over the planes.  Structure, buffers and schedule are those of gemm_q4_k_tile_kernel (see there); what differs:
@@ -271,7 +278,8 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
                                                             const uint8_t* __restrict__ mtab, const _Float16* __restrict__ a16,
                                                             const _Float16* __restrict__ asum, const float* __restrict__ inv,
                                                             float* __restrict__ out, int m, int n, int k, int tiles_m,
-                                                            int tiles_n, int nblk_tile, int with_min, int accumulate, int allow_split) {
+                                                            int tiles_n, int nblk_tile, int with_min, int accumulate, int allow_split,
+                                                            float* __restrict__ part) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = lds_address(smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -286,10 +294,19 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
     const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
+    // part != null: every tile in four K quarters, one unit each.  Quarters 0 and 1 meet in `out`, 2 and 3 in `part` (both zeroed
+    // beforehand; two terms per element each, so neither sum depends on the order), and a launch behind this one adds `part` to `out`.
     int full;
-    const int units = xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
+    const int units = part ? 4 * n_x : xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
     for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
-        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_row);
+        TileUnit unit;
+        if (part) {
+            const int q = u & 3, b0 = q * nblk_row / 4, b1 = (q + 1) * nblk_row / 4;
+            unit.tile = xcd_base + (u >> 2); unit.kb0 = b0; unit.nb = b1 - b0; unit.half = 1;
+        } else {
+            unit = xcd_unit(u, xcd_base, full, nblk_row);
+        }
+        float* __restrict__ dst = part && (u & 2) ? part : out;
         // (uniform values that come out of integer divisions live in vector registers unless told otherwise; everything
         // below that is derived from them, the base pointers above all, would follow them there)
         const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * 4;  // this unit's share of K
@@ -497,9 +514,9 @@ __global__ __launch_bounds__(512, 1) void gemm_planes_kernel(const uint8_t* __re
                     const float4 q = iv[r >> 2];
                     const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
                     if (row < m) {
-                        float* o_ = out + (int64_t)row * n;
+                        float* o_ = dst + (int64_t)row * n;
                         const float v0 = acc[mi][0][r] * is, v1 = acc[mi][1][r] * is;
-                        if (unit_half) {  // one of the two K halves of this tile: out holds zero or the other half
+                        if (unit_half) {  // one of the two K parts of this tile that meet here: zero or the other part is there
                             if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
                             if (c1_ok) unsafeAtomicAdd(o_ + col1, v1);
                         } else if (accumulate) {
@@ -1138,11 +1155,24 @@ bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     return m > 64;
 }
 
+// Very few tiles, or few on a long K: the 256 x 128 one-plane kernel cuts every tile in four K quarters (bf16 lhs: one pass), which
+// takes a second m x n buffer behind everything else in the workspace, zeroing of both and a launch that adds them.  Against K halves,
+// over kept planes: 4096 x 4096 with 65 rows (16 tiles) 36 -> 27 us, 1024 x 4096 with 512 rows 40 -> 35 us, 4096 x 14336 with 256 / 512
+// rows (32 / 64 tiles) 104 -> 74 / 113 -> 103 us; but 4096 x 4096 with 256 rows (32 tiles) 41 -> 41 us, with 512 rows (64 tiles) 49 -> 60 us.
+bool quarter_mode(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    if (encoding == QMM_Q6_K || lhs_dtype != QMM_BF16 || wide_tiles(encoding, m, n) || kernel_disabled("planes_quarters")) return false;
+    const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN), nblk = k / 256;
+    return tiles <= std::min<int64_t>(64, nblk + nblk / 4) && nblk >= 8 && 4 * ((tiles + 7) / 8) <= std::max(1, compute_units() / 8);
+}
+int64_t quarter_part_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    return quarter_mode(encoding, lhs_dtype, m, n, k) ? (m * n * 4 + 255) / 256 * 256 : 0;
+}
+
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
     const int64_t nblk_tile = blocks_per_tile(encoding, m, n, k);
     const int64_t lhs = (lhs_planes(nullptr, lhs_dtype, m, k, TM, nblk_tile * 256).bytes + 255) / 256 * 256;
-    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile).bytes;
+    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile).bytes + quarter_part_bytes(encoding, lhs_dtype, m, n, k);
 }
 
 namespace {
@@ -1152,8 +1182,9 @@ namespace {
 // otherwise they were made earlier.  wide (not Q6_K): the 256 x 256 tiles, which walk the extension blocks for the min term;
 // the 256 x 128 kernel reads the min operands from ps.mtab and skips the extension blocks if the planes have them.
 hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, bool convert, int64_t m, int64_t n, int64_t k,
-                             float* out, void* lhs_space, const PlaneSpace& ps, int nblk_tile, bool wide, hipStream_t s) {
+                             float* out, void* lhs_space, const PlaneSpace& ps, int nblk_tile, bool wide, float* part, hipStream_t s) {
     const bool q6 = encoding == QMM_Q6_K;
+    if (!quarter_mode(encoding, lhs_dtype, m, n, k)) part = nullptr;
     const int nblk = (int)(k / 256), lhs_ext = wide ? nblk_tile - nblk : 0;
     const int64_t lda = (int64_t)(nblk + lhs_ext) * 256;
     const LhsPlanes p = lhs_planes(lhs_space, lhs_dtype, m, k, TM, lda);
@@ -1171,11 +1202,16 @@ hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const
     // (A single row tile with at most 192 rows leaves a wavefront row without work, and the halves pay up to 128 tiles:
     // 14336 x 4096 with 65 rows, Q6_K 160 -> 118 us; with 256 rows 60 -> 62 us.)
     const bool halve_all = 2 * per_xcd <= per_xcd_cus && nblk >= 2 && (total <= 96 || nblk >= 32 || m <= 192);
-    const int wg = 8 * (halve_all ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
+    const int wg = 8 * (halve_all || part ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
     const WideLaunch L = wide ? wide_launch(out, m, n, nblk_tile) : WideLaunch{};
-    const SplitTiles z = wide ? L.z : split_tiles(out, m, n, tiles_m, tiles_n, nblk, wg, TN);
+    SplitTiles z = wide ? L.z : split_tiles(out, m, n, tiles_m, tiles_n, nblk, wg, TN);
+    if (part) {  // quarter mode: no halves, the whole of out and part zeroed
+        z.max_split = 0;
+        z.part = part;
+    }
     const int max_split = z.max_split;
-    const int64_t conv = convert ? (int64_t)tiles_n128 * nblk * 4 : 0, blocks = conv + m + (int64_t)max_split * 64;
+    const int64_t zero_blocks = part ? (m * n + kZeroFlatFloats - 1) / kZeroFlatFloats : (int64_t)max_split * 64;
+    const int64_t conv = convert ? (int64_t)tiles_n128 * nblk * 4 : 0, blocks = conv + m + zero_blocks;
     if (blocks > INT32_MAX || lda * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
     const dim3 pgrid((unsigned)blocks);
     auto prologue = [&](auto enc_c) {
@@ -1204,8 +1240,9 @@ hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const
             if (e != hipSuccess) return e;
         } else
             gemm_planes_kernel<<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m, (int)n,
-                                                                               (int)k, tiles_m, tiles_n, nblk_tile, pass == 0, pass, split);
+                                                                               (int)k, tiles_m, tiles_n, nblk_tile, pass == 0, pass, split, part);
     }
+    if (part) add_part_kernel<<<dim3((unsigned)((m * n + 255) / 256)), dim3(256), 0, s>>>(out, part, m * n);
     return hipGetLastError();
 }
 
@@ -1228,7 +1265,8 @@ hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, cons
     const int nblk_tile = (int)blocks_per_tile(encoding, m, n, k);
     const int64_t lhs_bytes = (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)nblk_tile * 256).bytes + 255) / 256 * 256;
     const PlaneSpace ps = plane_space((uint8_t*)workspace + lhs_bytes, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile);
-    return run_kquant_planes(encoding, lhs, lhs_dtype, w, true, m, n, k, out, workspace, ps, nblk_tile, wide, s);
+    float* part = (float*)((uint8_t*)workspace + lhs_bytes + ps.bytes);
+    return run_kquant_planes(encoding, lhs, lhs_dtype, w, true, m, n, k, out, workspace, ps, nblk_tile, wide, part, s);
 }
 
 // Weight planes kept across calls (the weights of a model are converted once, at load time): the conversion alone, and the
@@ -1266,14 +1304,18 @@ bool repacked_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
     return m > 128 && tiles >= 64;
 }
-int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t k) {
+static int64_t repacked_lhs_bytes(int encoding, int lhs_dtype, int64_t m, int64_t k) {
     return (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)repacked_blocks_per_tile(encoding, k) * 256).bytes + 255) / 256 * 256;
+}
+int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    return repacked_lhs_bytes(encoding, lhs_dtype, m, k) + quarter_part_bytes(encoding, lhs_dtype, m, n, k);
 }
 hipError_t launch_gemm_planes_repacked(int encoding, const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k,
                                        float* out, void* workspace, hipStream_t s) {
     const PlaneSpace ps = repacked_space(encoding, const_cast<void*>(packed), n, k);
+    float* part = (float*)((uint8_t*)workspace + repacked_lhs_bytes(encoding, lhs_dtype, m, k));
     return run_kquant_planes(encoding, lhs, lhs_dtype, nullptr, false, m, n, k, out, workspace, ps, repacked_blocks_per_tile(encoding, k),
-                             wide_tiles(encoding, m, n), s);
+                             wide_tiles(encoding, m, n), part, s);
 }
 
 // GPTQ through the plane GEMM: groups of 128 or 256 (a scale block is two or four steps), plain groups (no act-order), and

@@ -55,7 +55,19 @@ struct SplitTiles {
     int m, n, tiles_m, tiles_n, k_blocks, wgs_per_xcd;
     int max_split;  // largest number of split tiles on any XCD: the zeroing takes max_split * 64 workgroups
     int tn;         // columns of a tile: 128 or 256
+    float* part;    // not null: no tiles are split in halves; the whole of `out` and of this second m x n buffer is zeroed instead
 };
+constexpr int kZeroFlatFloats = 8192;  // per workgroup of 256 threads
+__device__ __forceinline__ void zero_flat(float* a, float* b, int64_t count, int e) {
+    const int64_t i0 = (int64_t)e * kZeroFlatFloats + threadIdx.x;
+    for (int j = 0; j < kZeroFlatFloats / 256; j++) {
+        const int64_t i = i0 + j * 256;
+        if (i < count) {
+            a[i] = 0.0f;
+            b[i] = 0.0f;
+        }
+    }
+}
 __device__ __forceinline__ void zero_split_tile_part(const SplitTiles& z, int j, int x, int part) {
     constexpr int TM = 256;
     const int TN = z.tn;
@@ -84,7 +96,7 @@ __device__ __forceinline__ void zero_split_tile_part(const SplitTiles& z, int j,
 }
 // The split tiles of a launch with `wg` persistent workgroups (host side).
 inline SplitTiles split_tiles(float* out, int64_t m, int64_t n, int tiles_m, int tiles_n, int k_blocks, int wg, int tn = 128) {
-    SplitTiles z{out, (int)m, (int)n, tiles_m, tiles_n, k_blocks, wg / 8, 0, tn};
+    SplitTiles z{out, (int)m, (int)n, tiles_m, tiles_n, k_blocks, wg / 8, 0, tn, nullptr};
     const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
     for (int x = 0; x < 8; x++) {
         const int n_x = per_xcd < total - x * per_xcd ? per_xcd : (total - x * per_xcd > 0 ? total - x * per_xcd : 0);

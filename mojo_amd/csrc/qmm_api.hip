@@ -646,7 +646,7 @@ int64_t qmm_matmul_repacked_workspace_bytes(int encoding, int lhs_dtype, int64_t
     if (m <= 0 || n <= 0 || k < 256 || k % 256) return 0;
     const int64_t planes = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, k)
                            : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
-                                                  : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
+                                                  : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (repacked_path(encoding, m, n, k, true)) return planes;
     const OptionalPlanesScope no_planes(true);  // the other route: qmm_matmul's kernels on the packed tensors (or, without those, the planes)
     return std::max(planes, qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k));
@@ -671,7 +671,7 @@ int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lh
     if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs must be 16-byte aligned");
     const int64_t need = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, k)
                          : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
-                                                : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, k);
+                                                : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (!workspace || workspace_bytes < need)
         return fail(QMM_ERR_WORKSPACE, "qmm_matmul_repacked: workspace of %lld bytes required, %lld given", (long long)need, (long long)workspace_bytes);
     if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: workspace must be 256-byte aligned");

@@ -12,7 +12,8 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_lanes_rows, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, gptq_mm, gptq_cols.  Nothing is disabled by default.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
+// Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 
 hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
@@ -177,7 +178,7 @@ hipError_t launch_gemm_q4_0_repacked(const void* lhs, int lhs_dtype, const void*
 int64_t repacked_planes_bytes(int encoding, int64_t n, int64_t k);
 hipError_t launch_repack_planes(int encoding, const uint8_t* w, int64_t n, int64_t k, void* packed, hipStream_t s);
 bool repacked_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k);
-int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t k);
+int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_planes_repacked(int encoding, const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k,
                                        float* out, void* workspace, hipStream_t s);
 bool gptq_planes_supported(int64_t n, int64_t k, int group);
