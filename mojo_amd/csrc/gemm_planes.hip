@@ -546,7 +546,7 @@ static_assert(kPlanes2Lds <= kLdsPerCu, "two-plane kernel LDS");
 __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __restrict__ planes, const float* __restrict__ dtab,
                                                              const _Float16* __restrict__ a16, const float* __restrict__ inv,
                                                              float* __restrict__ out, int m, int n, int k, int tiles_m, int tiles_n,
-                                                             int accumulate, int allow_split) {
+                                                             int accumulate, int allow_split, float* __restrict__ part) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = lds_address(smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -568,10 +568,18 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
     const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
+    // (part != null: every tile in four K quarters that meet pairwise in `out` and `part`, as in gemm_planes_kernel)
     int full;
-    const int units = xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
+    const int units = part ? 4 * n_x : xcd_units(n_x, wgs_per_xcd, nblk_row, allow_split, full);
     for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
-        const TileUnit unit = xcd_unit(u, xcd_base, full, nblk_row);
+        TileUnit unit;
+        if (part) {
+            const int q = u & 3, b0 = q * nblk_row / 4, b1 = (q + 1) * nblk_row / 4;
+            unit.tile = xcd_base + (u >> 2); unit.kb0 = b0; unit.nb = b1 - b0; unit.half = 1;
+        } else {
+            unit = xcd_unit(u, xcd_base, full, nblk_row);
+        }
+        float* __restrict__ dst = part && (u & 2) ? part : out;
         const int nblk = __builtin_amdgcn_readfirstlane(unit.nb), ns = nblk * 4;  // this unit's share of K
         const int kb0 = __builtin_amdgcn_readfirstlane(unit.kb0), unit_half = __builtin_amdgcn_readfirstlane(unit.half);
         int tile_m, tile_n;
@@ -739,7 +747,7 @@ __global__ __launch_bounds__(512, 1) void gemm_planes2_kernel(const uint8_t* __r
                     const float4 q = iv[r >> 2];
                     const float is = (r & 3) == 0 ? q.x : (r & 3) == 1 ? q.y : (r & 3) == 2 ? q.z : q.w;
                     if (row < m) {
-                        float* o_ = out + (int64_t)row * n;
+                        float* o_ = dst + (int64_t)row * n;
                         const float v0 = acc[mi][0][r] * unit_d[0] * is, v1 = acc[mi][1][r] * unit_d[1] * is;
                         if (unit_half) {  // one of the two K halves of this tile: out holds zero or the other half
                             if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
@@ -1155,14 +1163,16 @@ bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     return m > 64;
 }
 
-// Very few tiles, or few on a long K: the 256 x 128 one-plane kernel cuts every tile in four K quarters (bf16 lhs: one pass), which
+// Very few tiles, or few on a long K: the 256 x 128 plane kernels (one plane, and Q6_K's two) cut every tile in four K quarters (bf16 lhs: one pass), which
 // takes a second m x n buffer behind everything else in the workspace, zeroing of both and a launch that adds them.  Against K halves,
 // over kept planes: 4096 x 4096 with 65 rows (16 tiles) 36 -> 27 us, 1024 x 4096 with 512 rows 40 -> 35 us, 4096 x 14336 with 256 / 512
 // rows (32 / 64 tiles) 104 -> 74 / 113 -> 103 us; but 4096 x 4096 with 256 rows (32 tiles) 41 -> 41 us, with 512 rows (64 tiles) 49 -> 60 us.
 bool quarter_mode(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    if (encoding == QMM_Q6_K || lhs_dtype != QMM_BF16 || wide_tiles(encoding, m, n) || kernel_disabled("planes_quarters")) return false;
+    if (lhs_dtype != QMM_BF16 || wide_tiles(encoding, m, n) || kernel_disabled("planes_quarters")) return false;
     const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN), nblk = k / 256;
-    return tiles <= std::min<int64_t>(64, nblk + nblk / 4) && nblk >= 8 && 4 * ((tiles + 7) / 8) <= std::max(1, compute_units() / 8);
+    // (up to 128 lhs rows half of a tile's wavefront rows have no work, and the quarters pay up to 64 tiles: 4096 x 4096, 65 rows)
+    const bool few = tiles <= std::min<int64_t>(64, nblk + nblk / 4) || (m <= 128 && tiles <= 64);
+    return few && nblk >= 8 && 4 * ((tiles + 7) / 8) <= std::max(1, compute_units() / 8);
 }
 int64_t quarter_part_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     return quarter_mode(encoding, lhs_dtype, m, n, k) ? (m * n * 4 + 255) / 256 * 256 : 0;
@@ -1234,7 +1244,7 @@ hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const
         const int split = pass == 0 && max_split > 0 ? 1 : 0;
         if (q6)
             gemm_planes2_kernel<<<dim3((unsigned)wg), dim3(512), kPlanes2Lds, s>>>(ps.planes, ps.dtab, a, p.inv, out, (int)m, (int)n, (int)k,
-                                                                                 tiles_m, tiles_n, pass, split);
+                                                                                 tiles_m, tiles_n, pass, split, part);
         else if (wide) {
             e = run_wide<4>(L, ps.planes, ps.dtab, a, p.inv, out, m, n, lda, pass == 0 ? nblk_tile : nblk, nblk_tile, pass, s);
             if (e != hipSuccess) return e;

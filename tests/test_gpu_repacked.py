@@ -46,6 +46,7 @@ def lhs_rows(seed, m, k, bf16):
     (QE.Q5_K, 8200, 2304, [(1030, False, True), (40, True, True), (700, True, True), (2, False, True)]),
     (QE.Q5_K, 257, 512, [(33, True, True), (300, False, True)]),
     (QE.Q5_K, 1100, 2560, [(300, True, True), (70, True, True), (300, False, True)]),
+    (QE.Q6_K, 1100, 2560, [(300, True, True), (70, True, True), (300, False, True)]),
     (QE.Q4_K, 14080, 768, [(520, True, True), (1600, False, True), (300, True, False), (64, True, True)]),
     (QE.Q4_K, 20600, 256, [(2000, True, True), (300, True, False)]),
 ])
