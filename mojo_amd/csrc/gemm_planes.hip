@@ -1167,12 +1167,19 @@ bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
 // takes a second m x n buffer behind everything else in the workspace, zeroing of both and a launch that adds them.  Against K halves,
 // over kept planes: 4096 x 4096 with 65 rows (16 tiles) 36 -> 27 us, 1024 x 4096 with 512 rows 40 -> 35 us, 4096 x 14336 with 256 / 512
 // rows (32 / 64 tiles) 104 -> 74 / 113 -> 103 us; but 4096 x 4096 with 256 rows (32 tiles) 41 -> 41 us, with 512 rows (64 tiles) 49 -> 60 us.
-bool quarter_mode(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    if (lhs_dtype != QMM_BF16 || wide_tiles(encoding, m, n) || kernel_disabled("planes_quarters")) return false;
+bool few_tiles_for_quarters(int64_t m, int64_t n, int64_t k) {
     const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN), nblk = k / 256;
     // (up to 128 lhs rows half of a tile's wavefront rows have no work, and the quarters pay up to 64 tiles: 4096 x 4096, 65 rows)
     const bool few = tiles <= std::min<int64_t>(64, nblk + nblk / 4) || (m <= 128 && tiles <= 64);
     return few && nblk >= 8 && 4 * ((tiles + 7) / 8) <= std::max(1, compute_units() / 8);
+}
+hipError_t launch_add_part(float* out, const float* part, int64_t count, hipStream_t s) {
+    add_part_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s>>>(out, part, count);
+    return hipGetLastError();
+}
+bool quarter_mode(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    if (lhs_dtype != QMM_BF16 || wide_tiles(encoding, m, n) || kernel_disabled("planes_quarters")) return false;
+    return few_tiles_for_quarters(m, n, k);
 }
 int64_t quarter_part_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     return quarter_mode(encoding, lhs_dtype, m, n, k) ? (m * n * 4 + 255) / 256 * 256 : 0;

@@ -145,6 +145,8 @@ __global__ __launch_bounds__(256) void q4_0_planes_prologue_kernel(const uint8_t
         q4_0_plane_part(t - grp * z.tiles_n, grp, b & 3, w, z.n, nblk32, sp.planes, sp.dw);
     } else if (b < conv + lhs_rows) {
         q4_0_lhs_row<AT>(b - conv, a, k, sp.a16, sp.da);
+    } else if (z.part) {
+        zero_flat(z.out, z.part, (int64_t)z.m * z.n, b - conv - lhs_rows);
     } else {
         const int e = b - conv - lhs_rows;
         zero_split_tile_part(z, e >> 6, (e >> 3) & 7, e & 7);
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(256) void q4_0_planes_prologue_kernel(const uint8_t
 __global__ __launch_bounds__(512, 1) void gemm_q4_0_planes_kernel(const uint8_t* __restrict__ planes, const uint16_t* __restrict__ dw,
                                                                  const _Float16* __restrict__ a16, const uint16_t* __restrict__ da,
                                                                  float* __restrict__ out, int m, int n, int k, int tiles_m, int tiles_n,
-                                                                 int allow_split) {
+                                                                 int allow_split, float* __restrict__ part) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const uint32_t lds0 = lds_address(smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -175,10 +177,19 @@ __global__ __launch_bounds__(512, 1) void gemm_q4_0_planes_kernel(const uint8_t*
     const int total = tiles_m * tiles_n;
     const int per_xcd = (total + 7) / 8, wgs_per_xcd = (int)(gridDim.x >> 3);
     const int xcd_base = (int)(blockIdx.x & 7) * per_xcd, n_x = max(0, min(per_xcd, total - xcd_base));
+    // part != null: every tile in four K quarters, one unit each.  Quarters 0 and 1 meet in `out`, 2 and 3 in `part` (both zeroed
+    // beforehand; two terms per element each, so neither sum depends on the order), and a launch behind this one adds `part` to `out`.
     int full;
-    const int units = xcd_units(n_x, wgs_per_xcd, ngrp_row, allow_split, full);
+    const int units = part ? 4 * n_x : xcd_units(n_x, wgs_per_xcd, ngrp_row, allow_split, full);
     for (int u = (int)(blockIdx.x >> 3); u < units; u += wgs_per_xcd) {
-        const TileUnit unit = xcd_unit(u, xcd_base, full, ngrp_row);
+        TileUnit unit;
+        if (part) {
+            const int q = u & 3, b0 = q * ngrp_row / 4, b1 = (q + 1) * ngrp_row / 4;
+            unit.tile = xcd_base + (u >> 2); unit.kb0 = b0; unit.nb = b1 - b0; unit.half = 1;
+        } else {
+            unit = xcd_unit(u, xcd_base, full, ngrp_row);
+        }
+        float* __restrict__ dst = part && (u & 2) ? part : out;
         const int ngrp = __builtin_amdgcn_readfirstlane(unit.nb), ns = ngrp * 4;  // this unit's share of K: groups, steps
         const int kg0 = __builtin_amdgcn_readfirstlane(unit.kb0), unit_half = __builtin_amdgcn_readfirstlane(unit.half);
         int tile_m, tile_n;
@@ -381,7 +392,7 @@ __global__ __launch_bounds__(512, 1) void gemm_q4_0_planes_kernel(const uint8_t*
                 for (int r = 0; r < 16; r++) {
                     const int row = m0 + wm * 64 + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
                     if (row < m) {
-                        float* o_ = out + (int64_t)row * n;
+                        float* o_ = dst + (int64_t)row * n;
                         const float v0 = acc[mi][0][r], v1 = acc[mi][1][r];
                         if (unit_half) {  // one of the two K halves of this tile: out holds zero or the other half
                             if (c0_ok) unsafeAtomicAdd(o_ + col0, v0);
@@ -407,12 +418,16 @@ bool gemm_q4_0_planes_wanted(int64_t m, int64_t n, int64_t k) {
     return m > 64;
 }
 
-int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k) { return q40_space(nullptr, m, n, k).bytes; }
+int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k);
 
 namespace {
+bool quarters_wanted(int64_t m, int64_t n, int64_t k) { return !kernel_disabled("planes_quarters") && few_tiles_for_quarters(m, n, k); }
+int64_t part_bytes(int64_t m, int64_t n, int64_t k) { return quarters_wanted(m, n, k) ? (m * n * 4 + 255) / 256 * 256 : 0; }
 // convert: the weight plane in `sp` is made from `w` in the preparation launch; otherwise it was made earlier.
+// part: room for a second m x n result (quarter mode), used where few_tiles_for_quarters says so.
 hipError_t run_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, bool convert, int64_t m, int64_t n, int64_t k, float* out,
-                           const Q40Space& sp, hipStream_t s) {
+                           const Q40Space& sp, float* part, hipStream_t s) {
+    if (!quarters_wanted(m, n, k)) part = nullptr;
     hipError_t e = allow_full_lds<gemm_q4_0_planes_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n = (int)((n + TN - 1) / TN), ngrp = (int)(k / 256);
@@ -421,9 +436,14 @@ hipError_t run_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, boo
     // every tile in two K halves (a tile's time is set by K).
     const int per_xcd_cus = std::max(1, compute_units() / 8);
     const bool halve_all = 2 * per_xcd <= per_xcd_cus && ngrp >= 2;
-    const int wg = 8 * (halve_all ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
+    const int wg = 8 * (halve_all || part ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
     SplitTiles z = split_tiles(out, m, n, tiles_m, tiles_n, ngrp, wg);
-    const int64_t conv = convert ? (int64_t)tiles_n * ngrp * 4 : 0, blocks = conv + m + (int64_t)z.max_split * 64;
+    if (part) {
+        z.max_split = 0;
+        z.part = part;
+    }
+    const int64_t zero_blocks = part ? (m * n + kZeroFlatFloats - 1) / kZeroFlatFloats : (int64_t)z.max_split * 64;
+    const int64_t conv = convert ? (int64_t)tiles_n * ngrp * 4 : 0, blocks = conv + m + zero_blocks;
     if (blocks > INT32_MAX) return hipErrorInvalidValue;
     const dim3 pgrid((unsigned)blocks);
     if (lhs_dtype == QMM_F32)
@@ -433,15 +453,18 @@ hipError_t run_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, boo
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     gemm_q4_0_planes_kernel<<<dim3((unsigned)wg), dim3(512), kQ40Lds, s>>>(sp.planes, sp.dw, sp.a16, sp.da, out, (int)m, (int)n, (int)k,
-                                                                         tiles_m, tiles_n, z.max_split > 0 ? 1 : 0);
+                                                                         tiles_m, tiles_n, z.max_split > 0 ? 1 : 0, part);
+    if (part) return launch_add_part(out, part, m * n, s);
     return hipGetLastError();
 }
 }  // namespace
 
 hipError_t launch_gemm_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k, float* out,
                                    void* workspace, hipStream_t s) {
-    return run_q4_0_planes(lhs, lhs_dtype, w, true, m, n, k, out, q40_space(workspace, m, n, k), s);
+    const Q40Space sp = q40_space(workspace, m, n, k);
+    return run_q4_0_planes(lhs, lhs_dtype, w, true, m, n, k, out, sp, (float*)((uint8_t*)workspace + sp.bytes), s);
 }
+int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k) { return q40_space(nullptr, m, n, k).bytes + part_bytes(m, n, k); }
 
 // The weight plane kept across calls: the conversion alone, and the GEMM over a plane made by it (workspace: the lhs part).
 int64_t repacked_q4_0_bytes(int64_t n, int64_t k) { return q40_space(nullptr, 0, n, k).bytes; }
@@ -456,10 +479,11 @@ hipError_t launch_repack_q4_0(const uint8_t* w, int64_t n, int64_t k, void* pack
     q4_0_planes_prologue_kernel<uint16_t><<<dim3((unsigned)conv), dim3(256), 0, s>>>(w, (int)(k / 32), sp, (int)conv, nullptr, (int)k, 0, z);
     return hipGetLastError();
 }
-int64_t repacked_q4_0_workspace_bytes(int64_t m, int64_t k) { return q40_space(nullptr, m, 0, k).bytes; }
+int64_t repacked_q4_0_workspace_bytes(int64_t m, int64_t n, int64_t k) { return q40_space(nullptr, m, 0, k).bytes + part_bytes(m, n, k); }
 hipError_t launch_gemm_q4_0_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, float* out,
                                      void* workspace, hipStream_t s) {
-    return run_q4_0_planes(lhs, lhs_dtype, nullptr, false, m, n, k, out, q40_space(workspace, m, n, k, const_cast<void*>(packed)), s);
+    float* part = (float*)((uint8_t*)workspace + q40_space(nullptr, m, 0, k).bytes);
+    return run_q4_0_planes(lhs, lhs_dtype, nullptr, false, m, n, k, out, q40_space(workspace, m, n, k, const_cast<void*>(packed)), part, s);
 }
 
 }  // namespace qmm

@@ -644,7 +644,7 @@ static bool repacked_path(int encoding, int64_t m, int64_t n, int64_t k, bool ha
 
 int64_t qmm_matmul_repacked_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || n <= 0 || k < 256 || k % 256) return 0;
-    const int64_t planes = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, k)
+    const int64_t planes = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, n, k)
                            : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
                                                   : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (repacked_path(encoding, m, n, k, true)) return planes;
@@ -669,7 +669,7 @@ int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lh
     }
     if (lhs_dtype != QMM_F32 && lhs_dtype != QMM_BF16) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs dtype must be f32 or bf16");
     if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs must be 16-byte aligned");
-    const int64_t need = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, k)
+    const int64_t need = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, n, k)
                          : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
                                                 : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (!workspace || workspace_bytes < need)

@@ -166,10 +166,13 @@ int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int6
 hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                               float* out, void* workspace, hipStream_t s);
 int compute_units();  // of the current device, read once (gemm_planes.hip)
+// The 256 x 128 plane kernels' quarter mode (gemm_planes.hip): the shapes with few enough tiles, and out += part behind the GEMM.
+bool few_tiles_for_quarters(int64_t m, int64_t n, int64_t k);
+hipError_t launch_add_part(float* out, const float* part, int64_t count, hipStream_t s);
 // The Q4_0 weight plane kept across calls (gemm_q4_0_planes.hip)
 int64_t repacked_q4_0_bytes(int64_t n, int64_t k);
 hipError_t launch_repack_q4_0(const uint8_t* w, int64_t n, int64_t k, void* packed, hipStream_t s);
-int64_t repacked_q4_0_workspace_bytes(int64_t m, int64_t k);
+int64_t repacked_q4_0_workspace_bytes(int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemm_q4_0_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, float* out,
                                      void* workspace, hipStream_t s);
 // Weight planes kept across calls: the conversion alone into a buffer of *_bytes, and the plane GEMMs over such a buffer (workspace:

@@ -39,4 +39,4 @@ def test_fallback_kernels_match_the_oracle(setting):
     proc = subprocess.run([sys.executable, os.path.join(HERE, "fallback_child.py")], env=env, capture_output=True, text=True,
                           timeout=600)
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
-    assert proc.stdout.count(": ok") == 32, proc.stdout
+    assert proc.stdout.count(": ok") == 33, proc.stdout

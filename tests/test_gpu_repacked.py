@@ -96,11 +96,13 @@ def test_repacked_gptq_matches_oracle_and_qmatmul(group, n, k, rows):
             assert torch.equal(got, qmatmul(QE.GPTQ, cfg, lhs, *rhs)), f"GPTQ {m}x{n}x{k}: differs from qmatmul"
 
 
-@pytest.mark.parametrize("n,k,rows", [(300, 1024, [(70, True), (300, False), (16, True)]), (9300, 768, [(1000, True)])])
+@pytest.mark.parametrize("n,k,rows", [(300, 1024, [(70, True), (300, False), (16, True)]), (9300, 768, [(1000, True)]),
+                                      (1100, 2560, [(300, True), (70, False)])])
 def test_repacked_q4_0_matches_oracle_and_qmatmul(n, k, rows):
     """Q4_0: the plane of q - 8 and the block scales made once.  The lhs is quantised to Q8_0 per call as everywhere, so the
     result is that of the integer block dots: bit-identical with qmatmul above 64 rows (same GEMM), within the bar of the
-    oracle's Q8_0 x Q4_0 product at every row count; without the packed tensor few rows run over the plane too."""
+    oracle's Q8_0 x Q4_0 product at every row count; without the packed tensor few rows run over the plane too.  1100 x 2560:
+    few tiles on ten groups of 256, cut in four K quarters that meet pairwise in two buffers."""
     w, _ = synth(17, n, k, 1)
     wq = O.quantize(O.Q4_0, w)
     wq_d = gpu(wq)
