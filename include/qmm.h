@@ -177,20 +177,24 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
                        int64_t workspace_bytes, void* stream);
 
 /*
- * Weight planes kept across calls.  MAX's graph compiler folds a weight repack step ahead of its quantized matmul
- * kernels into model load (the packed layout is contractual on disk only; MAX itself is not in the reference
- * snapshot, see the top of this file); this pair of calls is the explicit form of it for the prefill GEMMs here:
- * qmm_repack converts the packed weights of one matrix once into the fp16 integer planes and scale tables that the
- * matrix-core GEMMs read (2 bytes per weight, Q6_K 4, plus tables: qmm_repack_bytes, 0 if the encoding or shape has
- * no plane GEMM: GPTQ with act-order or groups other than 128 / 256, K not a multiple of 256; Q4_0: the plane of q - 8 and
- * its block scales, the lhs is still quantised to Q8_0 per call), into a buffer
- * the caller owns, 256-byte aligned; the buffer depends on the weights only.  qmm_matmul_repacked is qmm_matmul with
- * that buffer at hand: row counts for which the plane GEMMs are the faster route (Q5_K / Q6_K from 49 rows, 33 on large matrices; Q4_0 from 49; Q4_K from
- * 129 with at least 64 tiles of 256 x 128; GPTQ from 257 with at least 160 tiles of 256 x 256, or from 97 with at most 64) skip the conversion that
- * qmm_matmul repeats per call (same kernels, same planes: where qmm_matmul takes the planes too the results are equal
- * bit for bit); other row counts are handed to qmm_matmul with `rhs`.  rhs = NULL (a caller that dropped the packed tensors): every row count goes through the planes.
- * flags must be 0.  Workspace: qmm_matmul_repacked_workspace_bytes (the lhs planes, or what qmm_matmul needs for the
- * kernels that read the packed tensors).
+ * Weight planes kept across calls.  MAX's graph compiler folds a weight repack step ahead of its quantized
+ * matmul kernels into model load (the packed layout is contractual on disk only; MAX itself is not in the
+ * reference snapshot, see the top of this file).  This pair of calls is the explicit form of that step for the
+ * prefill GEMMs here.
+ *   qmm_repack converts the packed weights of one matrix, once, into the fp16 integer planes and scale tables
+ *   that the matrix-core GEMMs read: 2 bytes per weight (Q6_K 4) plus tables, qmm_repack_bytes in all, into a
+ *   256-byte aligned buffer the caller owns.  The buffer depends on the weights only.  Encodings: Q4_K, Q5_K,
+ *   Q6_K; GPTQ with plain groups of 128 or 256; Q4_0 (the plane of q - 8 and its block scales: the lhs is still
+ *   quantised to Q8_0 in every call).  K must be a multiple of 256.  qmm_repack_bytes returns 0, and qmm_repack
+ *   QMM_ERR_UNSUPPORTED, for anything else (act-order GPTQ, other groups, other K).
+ *   qmm_matmul_repacked is qmm_matmul with that buffer at hand.  Row counts for which the plane GEMMs are the
+ *   faster route skip the conversion that qmm_matmul repeats per call: Q5_K / Q6_K from 49 rows (33 on matrices
+ *   of 48 Mi weights or more), Q4_0 from 49, Q4_K from 129 with at least 64 tiles of 256 x 128, GPTQ from 257
+ *   with at least 160 tiles of 256 x 256 or from 97 with at most 64.  Same kernels, same planes: where qmm_matmul
+ *   takes the planes too, the results are equal bit for bit.  Other row counts are handed to qmm_matmul with
+ *   `rhs`.  rhs = NULL (a caller that dropped the packed tensors): every row count goes through the planes.
+ *   flags must be 0.  Workspace: qmm_matmul_repacked_workspace_bytes (the lhs planes, or what qmm_matmul needs
+ *   for the kernels that read the packed tensors).
  */
 int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k);
 int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs, int n_rhs, int64_t n, int64_t k,
