@@ -49,14 +49,16 @@ __device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ub
 // HALF: a lane owns one 32-column sub-block instead of a 64-column chunk (lane l: super-block l / 8, chunk (l / 2) % 4, low nibbles
 // for even l, high nibbles for odd l), which halves the activations a lane keeps per lhs row and so makes room for four lhs
 // rows; a wavefront then covers 8 super-blocks, a row of 4096 columns takes two wavefronts (WPR up to 8, parts of up to 8).
-template <int MT, int WPR, int L, typename AT, bool HALF>
-__global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const LanesMats mats, const AT* __restrict__ a,
-                                                                        int m, int k, int64_t ldo, int ring_slots,
-                                                                        int streams, int rows_each, int rows_extra) {
+// PLAIN: one matrix, one lhs row, no pairing, two ring slots, all known at compile time: the row-to-matrix lookup, the
+// pair walk and the run-time slot arithmetic fall away, which shortens the scalar code in front of the first loads (a
+// launch spends its first microsecond there; the weights of a short launch arrive that much later).
+template <int MT, int WPR, int L, typename AT, bool HALF, bool PLAIN>
+__device__ __forceinline__ void lanes_body(const LanesMats& mats, const AT* __restrict__ a, int m, int k, int64_t ldo, int ring_slots,
+                                           int streams, int rows_each, int rows_extra) {
     // One matrix (the plain call) needs nothing from the argument block per row.  With several, the row's matrix is
     // looked up in the block: a dependent scalar load per row, a round trip to memory while the scalar cache is
     // cold, which a short launch cannot hide; the grouped launches are long enough.
-    const bool single = mats.count == 1;
+    const bool single = PLAIN || mats.count == 1;
     const uint8_t* const w0 = mats.w[0];
     float* const o0 = mats.out[0];
     const int e0 = mats.end[0];
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     const int bpw = (nblk + WPR - 1) / WPR;                       // super-blocks per part (<= 16)
     const int blk0 = min(part * bpw, nblk - 1);
     const int nb = max(0, min(bpw, nblk - part * bpw));           // super-blocks of this part
-    const int kRing = ring_slots;
+    const int kRing = PLAIN ? 2 : ring_slots;
     const int pieces = bpw * 9;       // 16-byte pieces of a full row part
     const int kSlot = pieces * 16;    // bytes of a slot
     uint8_t* ring = smem + wave * (kRing * kSlot);
@@ -79,7 +81,7 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     const int gs = (int)blockIdx.x * (kWaves / WPR) + wave / WPR, GS = streams;  // streams = workgroups * kWaves / WPR
     // Rows of this row stream.  Plain: gs, gs + GS, ...  Gated pair (mats.swiglu): the stream owns the row PAIRS
     // gs, gs + GS, ... and walks gate row, up row, gate row, ...: both results of a pair end up in its own slots.
-    const bool paired = mats.swiglu != 0;
+    const bool paired = !PLAIN && mats.swiglu != 0;
     const int np = paired ? e0 : n;
     // rows (or pairs) of this stream: np / GS, one more for the first np % GS streams (the host did the division)
     const int my_rows = (rows_each + (gs < rows_extra ? 1 : 0)) * (paired ? 2 : 1);
@@ -320,6 +322,34 @@ __global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_
     }
 }
 
+template <int MT, int WPR, int L, typename AT, bool HALF>
+__global__ __launch_bounds__(64 * kWaves, MT == 1 ? 4 : 2) void gemv_q4_k_lanes_kernel(const LanesMats mats, const AT* __restrict__ a,
+                                                                        int m, int k, int64_t ldo, int ring_slots,
+                                                                        int streams, int rows_each, int rows_extra) {
+    lanes_body<MT, WPR, L, AT, HALF, false>(mats, a, m, k, ldo, ring_slots, streams, rows_each, rows_extra);
+}
+
+// The plain call: one matrix [n, k], one lhs row, dense fp32 or bf16 output.  Twelve dwords of arguments.
+template <int WPR, int L, typename AT>
+__global__ __launch_bounds__(64 * kWaves, 4) void gemv_q4_k_lanes_plain_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                                               float* __restrict__ out, int n, int k, int out_bf16,
+                                                                               int streams, int rows_each, int rows_extra) {
+    // every argument is fetched in the first batch of scalar loads (left alone, the compiler fetches a pointer where it is first
+    // used: another round trip in front of the loads that need it)
+    asm volatile("" ::"s"(w), "s"(a), "s"(out), "s"(k), "s"(streams), "s"(rows_each), "s"(rows_extra));
+    LanesMats mats;
+#pragma unroll
+    for (int j = 0; j < kLanesMaxMats; j++) {
+        mats.w[j] = w;
+        mats.out[j] = out;
+        mats.end[j] = n;
+    }
+    mats.count = 1;
+    mats.swiglu = 0;
+    mats.out_bf16 = out_bf16;
+    lanes_body<1, WPR, L, AT, false, true>(mats, a, 1, k, 0, 2, streams, rows_each, rows_extra);
+}
+
 // Takes K <= 16384 and m = 1 (reports other shapes through *handled = false).  count matrices [n[j], k] share the
 // lhs; out[j] is fp32 [m, n[j]] (ldo = 0: dense; a single matrix may give its own leading dimension).
 hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
@@ -375,8 +405,18 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     if (wgs < min_wgs) wgs = min_wgs;  // no wavefront owns more rows than it has result slots
     dim3 grid((unsigned)wgs), block(64 * kWaves);
     const int total_streams = (int)wgs * streams;
+    const bool plain = count == 1 && !swiglu && (ldo == 0 || ldo == ns[0]) && !kernel_disabled("q4k_lanes_plain");
 #define QMM_GO3(MT_, WPR_, L_, AT_)                                                                                   \
     do {                                                                                                              \
+        if (plain) {                                                                                                  \
+            hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_plain_kernel<WPR_, L_, AT_>>();                            \
+            if (e_ != hipSuccess) return e_;                                                                          \
+            gemv_q4_k_lanes_plain_kernel<WPR_, L_, AT_><<<grid, block, lds, s>>>(ws[0], (const AT_*)a, outs[0], (int)n, (int)k,  \
+                                                                                 out_bf16 ? 1 : 0, total_streams,     \
+                                                                                 (int)(units / total_streams),       \
+                                                                                 (int)(units % total_streams));      \
+            break;                                                                                                    \
+        }                                                                                                             \
         hipError_t e_ = allow_full_lds<gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_, false>>();                         \
         if (e_ != hipSuccess) return e_;                                                                              \
         gemv_q4_k_lanes_kernel<MT_, WPR_, L_, AT_, false><<<grid, block, lds, s>>>(mats, (const AT_*)a, m, (int)k, ldo, ring, \
