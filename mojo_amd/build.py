@@ -31,6 +31,13 @@ FLAGS = [
 ]
 
 
+# Per-file additions.  Kernel-argument preloading (the first dwords of the argument block arrive in scalar registers
+# with the wavefront instead of through a scalar load) for the decode kernels whose first microsecond decides a launch.
+PER_FILE_FLAGS = {
+    "gemv_q4k_lanes.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
+}
+
+
 def sources() -> list[str]:
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
@@ -41,7 +48,7 @@ def _headers_mtime() -> float:
 
 
 def _compile(src: str, obj: str, verbose: bool) -> None:
-    cmd = [HIPCC, *FLAGS, "-c", "-o", obj, src]
+    cmd = [HIPCC, *FLAGS, *PER_FILE_FLAGS.get(os.path.basename(src), []), "-c", "-o", obj, src]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
