@@ -35,6 +35,7 @@ FLAGS = [
 # with the wavefront instead of through a scalar load) for the decode kernels whose first microsecond decides a launch.
 PER_FILE_FLAGS = {
     "gemv_q4k_lanes.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
+    "gemv_q4k_mm.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
 }
 
 

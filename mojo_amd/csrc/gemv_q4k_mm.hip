@@ -66,12 +66,11 @@ __device__ __forceinline__ half8 zero_half8() { return pack4(0u, 0u, 0u, 0u); }
 // INLINE: lhs converted in the kernel (m <= 8, AT = float or bf16 bits); otherwise a16 / a16_lo / asum /
 // inv come from prep_lhs_kernel<.., kLhsOrderQ4K16>.
 // MROWS (INLINE): lhs rows converted, 1, 2, 4 or 8 (>= m; rows past m repeat the last one and their results are dropped).
-template <int NPART, bool INLINE, int MROWS, typename AT>
-__global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, const AT* __restrict__ a,
-                                                           const _Float16* __restrict__ a16,
-                                                           const _Float16* __restrict__ a16_lo,
-                                                           const _Float16* __restrict__ asum, const float* __restrict__ inv,
-                                                           int m, int k) {
+// PLAIN: one matrix, known at compile time: no matrix lookup per item, a short argument block.
+template <int NPART, bool INLINE, int MROWS, typename AT, bool PLAIN>
+__device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict__ a, const _Float16* __restrict__ a16,
+                                        const _Float16* __restrict__ a16_lo, const _Float16* __restrict__ asum,
+                                        const float* __restrict__ inv, int m, int k) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -84,7 +83,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
     const int ntiles = mats.tile_end[kLanesMaxMats - 1];  // 16-row tiles, numbered through the matrices (entries past count repeat the last)
     // One matrix (the plain call) needs nothing from the argument block per item; with several, the tile's matrix is
     // looked up there (dependent scalar loads per item).
-    const bool single = mats.count == 1;
+    const bool single = PLAIN || mats.count == 1;
     const uint8_t* const w_first = mats.w[0];
     float* const out_first = mats.out[0];
     const int n_first = mats.n[0];
@@ -100,6 +99,30 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
         first = min(first, nblk - 1);  // (no share: a valid address, the data is not used)
     };
 
+    int last_issued = -1;  // newest item whose loads into LDS have been issued
+    int x_after = -1;      // the item that was newest when the last load_x was issued
+    // INLINE: raw lhs values of the wavefront's two super-blocks of the next group to convert; lane holds
+    // columns 4 lane .. 4 lane + 3 of each.  Loaded a group ahead; the first ones are the first loads of the kernel
+    // (the conversion waits for them while the first weights are on their way).
+    constexpr int RP = MROWS < 4 ? MROWS : 4;  // rows converted together (they share the free ring slot as staging)
+    constexpr int NX = INLINE ? kRunBlk * MROWS : 0;  // load instructions of one load_x
+    typedef typename std::conditional<sizeof(AT) == 4, u32x4, u32x2>::type xraw_t;
+    xraw_t xr[kRunBlk][MROWS];
+    auto load_x = [&](int g) {
+        int b0, cnt;
+        group_share(g, b0, cnt);
+#pragma unroll
+        for (int bb = 0; bb < kRunBlk; bb++) {
+            const int blk = min(b0 + bb, nblk - 1);
+#pragma unroll
+            for (int mi = 0; mi < MROWS; mi++)
+                hidden_load(xr[bb][mi], a + (int64_t)min(mi, m - 1) * k + (int64_t)blk * 256 + 4 * lane);
+        }
+        x_after = last_issued;
+    };
+    if constexpr (INLINE) {
+        if (total > 0) load_x(0);
+    }
     // piece p = lane + 64 i of an item: row p / 18, 16-byte piece p % 18
     int prow[kLoads], pidx[kLoads];
 #pragma unroll
@@ -132,8 +155,6 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
         }
     };
 
-    int last_issued = -1;  // newest item whose loads into LDS have been issued
-    int x_after = -1;      // the item that was newest when the last load_x was issued
     // items in flight: it + 1 and it + 2
     int ig = 0, it_t = 0, islot = 0;  // next item to issue
     auto issue_next = [&]() {
@@ -142,31 +163,10 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
         islot = islot == kSlots - 1 ? 0 : islot + 1;
         if (++it_t == my_tiles) { it_t = 0; ig++; }
     };
-    // INLINE: raw lhs values of the wavefront's two super-blocks of the next group to convert; lane holds
-    // columns 4 lane .. 4 lane + 3 of each.  Loaded a group ahead (the first ones before the first weights).
-    constexpr int RP = MROWS < 4 ? MROWS : 4;  // rows converted together (they share the free ring slot as staging)
-    constexpr int NX = INLINE ? kRunBlk * MROWS : 0;  // load instructions of one load_x
-    typedef typename std::conditional<sizeof(AT) == 4, u32x4, u32x2>::type xraw_t;
-    xraw_t xr[kRunBlk][MROWS];
-    auto load_x = [&](int g) {
-        int b0, cnt;
-        group_share(g, b0, cnt);
-#pragma unroll
-        for (int bb = 0; bb < kRunBlk; bb++) {
-            const int blk = min(b0 + bb, nblk - 1);
-#pragma unroll
-            for (int mi = 0; mi < MROWS; mi++)
-                hidden_load(xr[bb][mi], a + (int64_t)min(mi, m - 1) * k + (int64_t)blk * 256 + 4 * lane);
-        }
-        x_after = last_issued;
-    };
-    if constexpr (INLINE) {
-        if (total > 0) load_x(0);
-    }
-    // one item before the conversion: its loads keep the memory system busy while the lhs is converted, and
-    // the wavefront is not held up in the issue of more loads before it gets to the conversion
+    // two items before the conversion (the third slot is its staging area): their loads keep the memory system busy while
+    // the lhs is converted
     if (total > 0) issue_next();
-    if (!INLINE && total > 1) issue_next();
+    if (total > 1) issue_next();
 
     // lhs operand row of this lane: INLINE: row nn % 8, hi plane for nn < 8, residual for nn >= 8
     const int mrow = min(INLINE ? (nn & 7) : nn, m - 1);
@@ -220,28 +220,42 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
                             x2 = __uint_as_float(raw.y << 16); x3 = __uint_as_float(raw.y & 0xffff0000u);
                         }
                     };
-                    // largest magnitude of every (super-block, row) over the wavefront, all of them in one go
+                    // largest magnitude of every (super-block, row), lane-local
                     uint32_t mxs[kRunBlk * RP];
+                    uint32_t lane_max = 0;
+                    bool floor_ok = true;
 #pragma unroll
                     for (int bb = 0; bb < kRunBlk; bb++)
 #pragma unroll
                         for (int j = 0; j < RP; j++) {
                             float x0, x1, x2, x3;
                             widen(xr[bb][ps * RP + j], x0, x1, x2, x3);
-                            mxs[bb * RP + j] = max_abs_bits(x0, x1, x2, x3);
+                            const uint32_t mx = max_abs_bits(x0, x1, x2, x3);
+                            mxs[bb * RP + j] = mx;
+                            lane_max = max(lane_max, mx);
+                            floor_ok = floor_ok && __builtin_amdgcn_ballot_w64(mx >= 0x3C800000u) != 0;  // some value of it reaches 2^-6
                         }
-                    wave_umax_many(mxs);
+                    // Every one of them between 2^-6 and 2^15 (activations of ordinary size): the values go to fp16 as they are,
+                    // hi + residual carry 22 bits of each, and what is below fp16's normal range (2^-14) is small against the
+                    // largest value of its row and super-block.  Otherwise a power of two per row and super-block brings the
+                    // largest value to 2^9 first (maxima over the wavefront, all of them in one go).
+                    const bool as_is = floor_ok && __builtin_amdgcn_ballot_w64(lane_max >= 0x47000000u) == 0;
+                    if (!as_is) wave_umax_many(mxs);
 #pragma unroll
                     for (int bb = 0; bb < kRunBlk; bb++) {
 #pragma unroll
                         for (int j = 0; j < RP; j++) {
                             float x0, x1, x2, x3;
                             widen(xr[bb][ps * RP + j], x0, x1, x2, x3);
-                            const uint32_t mxb = mxs[bb * RP + j];
-                            int e = (int)((mxb >> 23) & 0xffu) - 127;
-                            if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite: leave unscaled
-                            const float sc = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
-                            isc[bb][j] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+                            float sc = 1.0f;
+                            isc[bb][j] = 1.0f;
+                            if (!as_is) {
+                                const uint32_t mxb = mxs[bb * RP + j];
+                                int e = (int)((mxb >> 23) & 0xffu) - 127;
+                                if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite: leave unscaled
+                                sc = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
+                                isc[bb][j] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+                            }
                             x0 *= sc; x1 *= sc; x2 *= sc; x3 *= sc;
                             // hi part: the value cut to fp16 (toward zero: one instruction converts and packs two);
                             // the residual x - hi is exact in fp32 and is cut to fp16 the same way
@@ -407,6 +421,32 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
     }
 }
 
+template <int NPART, bool INLINE, int MROWS, typename AT>
+__global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, const AT* __restrict__ a,
+                                                           const _Float16* __restrict__ a16,
+                                                           const _Float16* __restrict__ a16_lo,
+                                                           const _Float16* __restrict__ asum, const float* __restrict__ inv,
+                                                           int m, int k) {
+    mm_body<NPART, INLINE, MROWS, AT, false>(mats, a, a16, a16_lo, asum, inv, m, k);
+}
+
+// The plain call with up to 8 lhs rows: one matrix [n, k], lhs converted in the kernel.  Nine dwords of arguments.
+template <int MROWS, typename AT>
+__global__ __launch_bounds__(512) void gemv_q4_k_mm_plain_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
+                                                                 float* __restrict__ out, int n, int m, int k) {
+    asm volatile("" ::"s"(w), "s"(a), "s"(out), "s"(n), "s"(m), "s"(k));  // (all arguments in the first batch of scalar loads)
+    MmMats mats;
+#pragma unroll
+    for (int j = 0; j < kLanesMaxMats; j++) {
+        mats.w[j] = w;
+        mats.out[j] = out;
+        mats.n[j] = n;
+        mats.tile_end[j] = (n + 15) >> 4;
+    }
+    mats.count = 1;
+    mm_body<1, true, MROWS, AT, true>(mats, a, nullptr, nullptr, nullptr, nullptr, m, k);
+}
+
 int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) {
     return m <= 8 ? 0 : lhs_planes(nullptr, lhs_dtype, m, k).bytes;
 }
@@ -436,6 +476,14 @@ hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count
     hipError_t e = hipSuccess;
     static bool lds_set = false;
     if (!lds_set) {
+        const void* pfns[8] = {(const void*)gemv_q4_k_mm_plain_kernel<1, float>, (const void*)gemv_q4_k_mm_plain_kernel<2, float>,
+                               (const void*)gemv_q4_k_mm_plain_kernel<4, float>, (const void*)gemv_q4_k_mm_plain_kernel<8, float>,
+                               (const void*)gemv_q4_k_mm_plain_kernel<1, uint16_t>, (const void*)gemv_q4_k_mm_plain_kernel<2, uint16_t>,
+                               (const void*)gemv_q4_k_mm_plain_kernel<4, uint16_t>, (const void*)gemv_q4_k_mm_plain_kernel<8, uint16_t>};
+        for (const void* fn : pfns) {
+            e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return e;
+        }
         const void* fns[10] = {(const void*)gemv_q4_k_mm_kernel<1, true, 1, float>, (const void*)gemv_q4_k_mm_kernel<1, true, 2, float>,
                                (const void*)gemv_q4_k_mm_kernel<1, true, 4, float>, (const void*)gemv_q4_k_mm_kernel<1, true, 8, float>,
                                (const void*)gemv_q4_k_mm_kernel<1, true, 1, uint16_t>, (const void*)gemv_q4_k_mm_kernel<1, true, 2, uint16_t>,
@@ -453,9 +501,14 @@ hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count
     const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
     dim3 grid((unsigned)wgs), block(64 * kWaves);
     if (m <= 8) {
+        const bool plain = count == 1 && !kernel_disabled("q4k_mm_plain");
 #define QMM_MM_INLINE(MR_)                                                                                            \
     do {                                                                                                              \
-        if (lhs_dtype == QMM_F32)                                                                                     \
+        if (plain && lhs_dtype == QMM_F32)                                                                            \
+            gemv_q4_k_mm_plain_kernel<MR_, float><<<grid, block, kLdsBytes, s>>>(ws[0], (const float*)lhs, outs[0], (int)ns[0], (int)m, (int)k); \
+        else if (plain)                                                                                               \
+            gemv_q4_k_mm_plain_kernel<MR_, uint16_t><<<grid, block, kLdsBytes, s>>>(ws[0], (const uint16_t*)lhs, outs[0], (int)ns[0], (int)m, (int)k); \
+        else if (lhs_dtype == QMM_F32)                                                                                \
             gemv_q4_k_mm_kernel<1, true, MR_, float><<<grid, block, kLdsBytes, s>>>(                                  \
                 mats, (const float*)lhs, nullptr, nullptr, nullptr, nullptr, (int)m, (int)k);                         \
         else                                                                                                          \
