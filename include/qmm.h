@@ -177,10 +177,10 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
                        int64_t workspace_bytes, void* stream);
 
 /*
- * Weight planes kept across calls.  MAX's graph compiler folds a weight repack step ahead of its quantized
- * matmul kernels into model load (the packed layout is contractual on disk only; MAX itself is not in the
- * reference snapshot, see the top of this file).  This pair of calls is the explicit form of that step for the
- * prefill GEMMs here.
+ * Weight planes kept across calls.  (External knowledge, not verifiable from the reference snapshot, which holds no
+ * MAX code: MAX is understood to fold a weight repack step ahead of its quantized matmul kernels into model load; the
+ * packed layout is contractual on disk only.)  These calls are an explicit form of such a step for the prefill GEMMs
+ * here; nothing in the reference's op interface corresponds to them.
  *   qmm_repack converts the packed weights of one matrix, once, into the fp16 integer planes and scale tables
  *   that the matrix-core GEMMs read: 2 bytes per weight (Q6_K 4) plus tables, qmm_repack_bytes in all, into a
  *   256-byte aligned buffer the caller owns.  The buffer depends on the weights only.  Encodings: Q4_K, Q5_K,
@@ -195,10 +195,22 @@ int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, 
  *   `rhs`.  rhs = NULL (a caller that dropped the packed tensors): every row count goes through the planes.
  *   flags must be 0.  Workspace: qmm_matmul_repacked_workspace_bytes (the lhs planes, or what qmm_matmul needs
  *   for the kernels that read the packed tensors).
+ *   The price is memory: the buffer is 4.25 x the packed tensor for Q4_K / Q5_K (2 bytes per weight plus one extension
+ *   block per eight super-blocks and the tables: 140 MB for 14336 x 4096), 3.9 x for GPTQ, 4.9 x for Q6_K (two planes),
+ *   3.6 x for Q4_0.  A host that keeps planes for every matrix holds an fp16-sized model; a host that does not pays the
+ *   conversion in every qmm_matmul call that takes the plane GEMM, inside a workspace of that size.
+ *   The buffer begins with a 256-byte record (encoding, N, K, GPTQ group, layout version) that qmm_repack writes.  Every
+ *   qmm_matmul_repacked call that reads the planes compares the record with its own arguments on the device, behind its
+ *   kernels: on a mismatch the whole result is set to NaN (planes of equal size made for another matrix shape, encoding
+ *   or group would otherwise give plausible garbage).  qmm_repack_check does the same comparison on the host (it copies
+ *   the record back and synchronises the stream: for load time, not for the hot path) and returns QMM_ERR_INVALID with
+ *   both descriptions in qmm_last_error.  Neither can tell two matrices of the same encoding and shape apart.
  */
 int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k);
 int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs, int n_rhs, int64_t n, int64_t k,
                void* packed, int64_t packed_bytes, void* stream);
+int qmm_repack_check(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k, const void* packed, int64_t packed_bytes,
+                     void* stream);
 int64_t qmm_matmul_repacked_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                         const void* const* rhs, int n_rhs, const void* packed, int64_t packed_bytes, int64_t n, float* out,

@@ -39,6 +39,7 @@ SIGNATURES = {
                                  _vp]),
     "qmm_repack_bytes": (_i64, [_int, C.POINTER(GptqConfig), _i64, _i64]),
     "qmm_repack": (_int, [_int, C.POINTER(GptqConfig), C.POINTER(_vp), _int, _i64, _i64, _vp, _i64, _vp]),
+    "qmm_repack_check": (_int, [_int, C.POINTER(GptqConfig), _i64, _i64, _vp, _i64, _vp]),
     "qmm_matmul_repacked_workspace_bytes": (_i64, [_int, _int, _i64, _i64, _i64]),
     "qmm_matmul_repacked": (_int, [_int, C.POINTER(GptqConfig), _vp, _int, _i64, _i64, C.POINTER(_vp), _int, _vp, _i64, _i64, _vp,
                                    _vp, _i64, _int, _vp]),

@@ -186,7 +186,7 @@ int static_scratch(void** ws) {
 
 extern "C" {
 
-int qmm_version(void) { return 104; }
+int qmm_version(void) { return 105; }
 
 const char* qmm_last_error(void) { return g_err; }
 
@@ -352,7 +352,8 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
         if (handled) return QMM_OK;
     }
     if (m <= 0 || n <= 0) return fail(QMM_ERR_INVALID, "qmm_matmul: M=%lld N=%lld must be positive", (long long)m, (long long)n);
-    const int64_t base = up256(qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k)), need = base + up256(m * n * 4);
+    // (the fp32 result sits behind everything the inner call needs, the Q8_K round trip of the lhs included)
+    const int64_t base = up256(qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, inner)), need = base + up256(m * n * 4);
     if (!workspace || workspace_bytes < need)
         return fail(QMM_ERR_WORKSPACE, "qmm_matmul: bf16 output of this problem goes through an fp32 result in the workspace: %lld bytes required "
                                        "(qmm_matmul_workspace_bytes_flags), %lld given", (long long)need, (long long)workspace_bytes);
@@ -596,17 +597,82 @@ int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     return qmm_matmul(encoding, cfg, lhs, lhs_dtype, m, k, rhs, n_rhs, n, out, ws, (int64_t)QMM_STATIC_SCRATCH_BYTES, flags, stream);
 }
 
-// Weight planes kept across calls.
+// Weight planes kept across calls.  The buffer starts with a 256-byte record of what it was made for; the planes follow.
+namespace {
+constexpr int64_t kPackHeaderBytes = 256;
+constexpr uint32_t kPackMagic = 0x504D4D51u;  // "QMMP"
+constexpr uint32_t kPackLayout = 1;           // bumped whenever the plane layouts change
+struct PackHeader {
+    uint32_t magic, layout;
+    int32_t encoding, group;
+    int64_t n, k, bytes;
+};
+static_assert(sizeof(PackHeader) <= kPackHeaderBytes, "header fits its 256 bytes");
+__host__ __device__ inline bool same_header(const PackHeader& a, const PackHeader& b) {
+    return a.magic == b.magic && a.layout == b.layout && a.encoding == b.encoding && a.group == b.group && a.n == b.n && a.k == b.k &&
+           a.bytes == b.bytes;
+}
+PackHeader make_header(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k, int64_t bytes) {
+    PackHeader h;
+    h.magic = kPackMagic;
+    h.layout = kPackLayout;
+    h.encoding = encoding;
+    h.group = encoding == QMM_GPTQ && cfg ? cfg->group_size : 0;
+    h.n = n;
+    h.k = k;
+    h.bytes = bytes;
+    return h;
+}
+__global__ void pack_header_write_kernel(PackHeader* at, const PackHeader h) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) *at = h;
+}
+// Runs behind the kernels of a qmm_matmul_repacked call.  A buffer whose record says another encoding, shape or group than the
+// call (planes of the same size made for something else pass every host-side check) turns the whole result into NaN: a
+// wrong buffer cannot pass for a right one.
+__global__ __launch_bounds__(256) void pack_header_check_kernel(const PackHeader* at, const PackHeader want, float* out, int64_t count) {
+    const PackHeader have = *at;
+    if (same_header(have, want)) return;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) out[i] = __uint_as_float(0x7fc00000u);
+}
+}  // namespace
+
 static bool repackable(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
     if (n <= 0 || k < 256 || k % 256 || n > INT32_MAX || k > INT32_MAX) return false;
     if (encoding == QMM_GPTQ) return cfg && cfg->bits == 4 && !cfg->desc_act && qmm::gptq_planes_supported(n, k, cfg->group_size);
     return encoding == QMM_Q4_K || encoding == QMM_Q5_K || encoding == QMM_Q6_K || encoding == QMM_Q4_0;
 }
 
-int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
-    if (!repackable(encoding, cfg, n, k)) return 0;
+static int64_t repack_plane_bytes(int encoding, int64_t n, int64_t k) {
     if (encoding == QMM_Q4_0) return qmm::repacked_q4_0_bytes(n, k);
     return encoding == QMM_GPTQ ? qmm::repacked_gptq_bytes(n, k) : qmm::repacked_planes_bytes(encoding, n, k);
+}
+
+int64_t qmm_repack_bytes(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k) {
+    if (!repackable(encoding, cfg, n, k)) return 0;
+    return kPackHeaderBytes + repack_plane_bytes(encoding, n, k);
+}
+
+int qmm_repack_check(int encoding, const qmm_gptq_config* cfg, int64_t n, int64_t k, const void* packed, int64_t packed_bytes,
+                     void* stream) {
+    if (!packed) return fail(QMM_ERR_INVALID, "qmm_repack_check: null pointer");
+    if (!repackable(encoding, cfg, n, k))
+        return fail(QMM_ERR_UNSUPPORTED, "qmm_repack_check: no weight planes for encoding %d with N=%lld K=%lld", encoding, (long long)n, (long long)k);
+    const int64_t need = qmm_repack_bytes(encoding, cfg, n, k);
+    if (packed_bytes < need || !aligned(packed, 256))
+        return fail(QMM_ERR_INVALID, "qmm_repack_check: the packed buffer must be 256-byte aligned and hold qmm_repack_bytes = %lld bytes (%lld given)",
+                    (long long)need, (long long)packed_bytes);
+    PackHeader have;
+    hipError_t e = hipMemcpyAsync(&have, packed, sizeof(have), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return hip_status(e, "qmm_repack_check");
+    const PackHeader want = make_header(encoding, cfg, n, k, need);
+    if (have.magic != kPackMagic) return fail(QMM_ERR_INVALID, "qmm_repack_check: the buffer does not start with the record qmm_repack writes");
+    if (!same_header(have, want))
+        return fail(QMM_ERR_INVALID, "qmm_repack_check: the buffer holds planes of encoding %d, N=%lld, K=%lld, group %d, layout %u; the call names "
+                                     "encoding %d, N=%lld, K=%lld, group %d, layout %u", have.encoding, (long long)have.n, (long long)have.k, have.group,
+                    have.layout, want.encoding, (long long)want.n, (long long)want.k, want.group, want.layout);
+    return QMM_OK;
 }
 
 int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs, int n_rhs, int64_t n, int64_t k, void* packed,
@@ -618,20 +684,26 @@ int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs,
     const int64_t need = qmm_repack_bytes(encoding, cfg, n, k);
     if (packed_bytes < need) return fail(QMM_ERR_WORKSPACE, "qmm_repack: %lld bytes required (qmm_repack_bytes), %lld given", (long long)need, (long long)packed_bytes);
     if (!aligned(packed, 256)) return fail(QMM_ERR_INVALID, "qmm_repack: the buffer must be 256-byte aligned");
+    void* const planes = (char*)packed + kPackHeaderBytes;
+    auto finish = [&](hipError_t e, const char* what) {
+        if (e != hipSuccess) return hip_status(e, what);
+        pack_header_write_kernel<<<dim3(1), dim3(64), 0, (hipStream_t)stream>>>((PackHeader*)packed, make_header(encoding, cfg, n, k, need));
+        return hip_status(hipGetLastError(), "qmm_repack(record)");
+    };
     if (encoding == QMM_GPTQ) {
         if (n_rhs != 3 && n_rhs != 4) return fail(QMM_ERR_INVALID, "qmm_repack: GPTQ takes rhs = (qweight, scales, qzeros[, g_idx]), got %d", n_rhs);
         if (int rc = check_gptq(cfg, n, k)) return rc;
         for (int i = 0; i < 3; i++)
             if (!rhs[i] || !aligned(rhs[i], 4)) return fail(QMM_ERR_INVALID, "qmm_repack: GPTQ rhs[%d] null or misaligned", i);
-        return hip_status(qmm::launch_repack_gptq((const uint32_t*)rhs[0], (const uint16_t*)rhs[1], (const uint32_t*)rhs[2], n, k, cfg->group_size,
-                                                  packed, (hipStream_t)stream), "qmm_repack(GPTQ)");
+        return finish(qmm::launch_repack_gptq((const uint32_t*)rhs[0], (const uint16_t*)rhs[1], (const uint32_t*)rhs[2], n, k, cfg->group_size,
+                                              planes, (hipStream_t)stream), "qmm_repack(GPTQ)");
     }
     if (n_rhs != 1 || !rhs[0]) return fail(QMM_ERR_INVALID, "qmm_repack: GGUF encodings take exactly one rhs tensor");
     if (!aligned(rhs[0], encoding == QMM_Q6_K || encoding == QMM_Q4_0 ? 2 : 16))
         return fail(QMM_ERR_INVALID, "qmm_repack: rhs misaligned (Q4_K / Q5_K 16 bytes, Q4_0 / Q6_K 2)");
     if (encoding == QMM_Q4_0)
-        return hip_status(qmm::launch_repack_q4_0((const uint8_t*)rhs[0], n, k, packed, (hipStream_t)stream), "qmm_repack(Q4_0)");
-    return hip_status(qmm::launch_repack_planes(encoding, (const uint8_t*)rhs[0], n, k, packed, (hipStream_t)stream), "qmm_repack");
+        return finish(qmm::launch_repack_q4_0((const uint8_t*)rhs[0], n, k, planes, (hipStream_t)stream), "qmm_repack(Q4_0)");
+    return finish(qmm::launch_repack_planes(encoding, (const uint8_t*)rhs[0], n, k, planes, (hipStream_t)stream), "qmm_repack");
 }
 
 // Does a call with these rows go through the planes?  Without the packed tensors every row count does.
@@ -675,13 +747,17 @@ int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lh
     if (!workspace || workspace_bytes < need)
         return fail(QMM_ERR_WORKSPACE, "qmm_matmul_repacked: workspace of %lld bytes required, %lld given", (long long)need, (long long)workspace_bytes);
     if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: workspace must be 256-byte aligned");
-    if (encoding == QMM_Q4_0)
-        return hip_status(qmm::launch_gemm_q4_0_repacked(lhs, lhs_dtype, packed, m, n, k, out, workspace, (hipStream_t)stream), "qmm_matmul_repacked(Q4_0)");
-    if (encoding == QMM_GPTQ)
-        return hip_status(qmm::launch_gemm_gptq_repacked(lhs, lhs_dtype, packed, m, n, k, cfg->group_size, out, workspace, (hipStream_t)stream),
-                          "qmm_matmul_repacked(GPTQ)");
-    return hip_status(qmm::launch_gemm_planes_repacked(encoding, lhs, lhs_dtype, packed, m, n, k, out, workspace, (hipStream_t)stream),
-                      "qmm_matmul_repacked");
+    const void* const planes = (const char*)packed + kPackHeaderBytes;
+    hipError_t e;
+    if (encoding == QMM_Q4_0) e = qmm::launch_gemm_q4_0_repacked(lhs, lhs_dtype, planes, m, n, k, out, workspace, (hipStream_t)stream);
+    else if (encoding == QMM_GPTQ) e = qmm::launch_gemm_gptq_repacked(lhs, lhs_dtype, planes, m, n, k, cfg->group_size, out, workspace, (hipStream_t)stream);
+    else e = qmm::launch_gemm_planes_repacked(encoding, lhs, lhs_dtype, planes, m, n, k, out, workspace, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_status(e, "qmm_matmul_repacked");
+    // the record at the head of the buffer against this call, on the device (the host never reads the buffer here)
+    const int64_t count = m * n;
+    pack_header_check_kernel<<<dim3((unsigned)std::min<int64_t>((count + 255) / 256, 1024)), dim3(256), 0, (hipStream_t)stream>>>(
+        (const PackHeader*)packed, make_header(encoding, cfg, n, k, qmm_repack_bytes(encoding, cfg, n, k)), out, count);
+    return hip_status(hipGetLastError(), "qmm_matmul_repacked(record check)");
 }
 
 int qmm_matmul_grouped(int encoding, const void* lhs, int lhs_dtype, int64_t m, int64_t k, int count,

@@ -149,8 +149,9 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
 
 
 class RepackedWeights:
-    """The weights of one matrix as the plane GEMMs read them, made once by :func:`repack_weights` (the weight repack
-    step that MAX's graph compiler folds into model load).  ``rhs`` are the packed tensors the planes were made from, or
+    """The weights of one matrix as the plane GEMMs read them, made once by :func:`repack_weights` (an explicit form
+    of the weight repack step that MAX is understood to fold into model load: external knowledge, the reference snapshot
+    holds no MAX code).  ``rhs`` are the packed tensors the planes were made from, or
     an empty tuple if the caller does not keep them (then every row count goes through the planes)."""
 
     __slots__ = ("encoding", "config", "n", "k", "packed", "rhs")

@@ -97,6 +97,17 @@ def test_argument_validation_happens_before_any_launch():
     ws = C.c_void_p(0x100000)
     assert lib.qmm_matmul(0, None, fake, 0, 1, 4096, rhs, 1, 8, fake, ws, 1 << 30, _lib.QMM_FLAG_ACT_Q8K, None) == -2
     assert lib.qmm_matmul(1, None, fake, 0, 1, 4096, rhs, 1, 8, fake, None, 0, 8, None) == -1 and b"flag" in lib.qmm_last_error()
+    # Q8_K activations and a bf16 result together: a workspace of exactly the quoted size passes the size check of the outer and
+    # of the inner call (encodings 4, 2, 1 = Q5_K, Q6_K, Q4_K at 8 rows go through the fp32 round trip of the lhs); one byte less
+    # is refused.  K = 100 makes a call that got past the size checks fail on the block size instead of reaching a launch.
+    both = _lib.QMM_FLAG_ACT_Q8K | _lib.QMM_FLAG_OUT_BF16
+    for enc in (4, 2, 1):
+        need = f(enc, 0, 8, 512, 4096, both)
+        assert need >= 8 * 4096 * 4 + 8 * 512 * 4
+        assert lib.qmm_matmul(enc, None, fake, 0, 8, 4096, rhs, 1, 512, fake, ws, need - 1, both, None) == -4
+        assert f(enc, 0, 8, 512, 100, both) >= 8 * 100 * 4 + 8 * 512 * 4
+        assert lib.qmm_matmul(enc, None, fake, 0, 8, 100, rhs, 1, 512, fake, ws, f(enc, 0, 8, 512, 100, both), both, None) == -1
+        assert b"block size" in lib.qmm_last_error()
     # the normalisation prologue
     g = C.c_void_p(0x3000)
     rn = lib.qmm_matmul_rmsnorm

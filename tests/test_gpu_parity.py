@@ -589,6 +589,21 @@ def test_kquant_matmul_with_q8_k_activations(enc, m, n, k, lhs_bf16):
         assert not O.isclose(got, O.matmul_f32(ENC[enc], a, wq), 1e-4, 1e-5).all()
 
 
+@pytest.mark.parametrize("enc,m", [(QE.Q6_K, 8), (QE.Q4_K, 8), (QE.Q5_K, 3), (QE.Q4_K, 2)])
+def test_q8_k_activations_with_bf16_output(enc, m):
+    """Both flags in one call: the bf16 result is the rounding of the fp32 result of the same call (the Q4_K integer kernel
+    for up to four rows, the fp32 round trip of the lhs otherwise), also through the static scratch."""
+    n, k = 300, 2048
+    w, a = synth(74, n, k, m)
+    wq = O.quantize(ENC[enc], w)
+    f32 = qmatmul(enc, None, gpu(a), gpu(wq), act_q8k=True)
+    want = O.f32_to_bf16(f32.cpu().numpy())
+    for static in (False, True):
+        got = qmatmul(enc, None, gpu(a), gpu(wq), act_q8k=True, out_dtype=torch.bfloat16, static_scratch=static)
+        assert got.dtype == torch.bfloat16
+        assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want), (enc, m, static)
+
+
 def test_q8_k_activations_only_for_k_quants():
     w, a = synth(72, 8, 256, 1)
     with pytest.raises(NotImplementedError):

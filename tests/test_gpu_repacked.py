@@ -149,3 +149,60 @@ def test_repack_refusals():
         repack_weights(QE.GPTQ, QuantizationConfig(group_size=64), gpu(qw), gpu(sc.view(np.float16)), gpu(qz), gpu(gi))
     with pytest.raises(TypeError):
         qmatmul_repacked(torch.zeros((1, 256), device="cuda:0"), "weights")
+
+
+def test_a_buffer_made_for_something_else_is_caught():
+    """Planes of the same size made for another encoding or GPTQ group pass every size check.  The record at the head of the
+    buffer does not: the call's result is all NaN, and qmm_repack_check names both descriptions; the right buffer passes both."""
+    import ctypes as C
+
+    from mojo_amd import _lib
+
+    lib = _lib.load()
+    n, k, m = 512, 1024, 300
+    w, a = synth(5, n, k, m)
+    lhs = gpu(O.bf16_to_f32(O.f32_to_bf16(a))).to(torch.bfloat16)
+    s = torch.cuda.current_stream().cuda_stream
+    w4, w5 = gpu(O.quantize(O.Q4_K, w)), gpu(O.quantize(O.Q5_K, w))
+    size = lib.qmm_repack_bytes(QE.Q4_K.code, None, n, k)
+    assert size == lib.qmm_repack_bytes(QE.Q5_K.code, None, n, k)  # same planes, other contents
+    packed = torch.empty((size,), dtype=torch.uint8, device="cuda:0")
+    out = torch.zeros((m, n), dtype=torch.float32, device="cuda:0")
+    need = lib.qmm_matmul_repacked_workspace_bytes(QE.Q4_K.code, _lib.QMM_BF16, m, n, k)
+    ws = torch.empty((max(need, 1),), dtype=torch.uint8, device="cuda:0")
+
+    def repack(enc, t):
+        _lib.check(lib.qmm_repack(enc.code, None, (C.c_void_p * 1)(t.data_ptr()), 1, n, k, C.c_void_p(packed.data_ptr()), size, C.c_void_p(s)), "qmm_repack")
+
+    def matmul(enc):
+        return lib.qmm_matmul_repacked(enc.code, None, C.c_void_p(lhs.data_ptr()), _lib.QMM_BF16, m, k, None, 0, C.c_void_p(packed.data_ptr()), size,
+                                       n, C.c_void_p(out.data_ptr()), C.c_void_p(ws.data_ptr()), need, 0, C.c_void_p(s))
+
+    def check(enc):
+        return lib.qmm_repack_check(enc.code, None, n, k, C.c_void_p(packed.data_ptr()), size, C.c_void_p(s))
+
+    packed.zero_()
+    assert check(QE.Q4_K) == -1 and b"record" in lib.qmm_last_error()  # never written
+    repack(QE.Q5_K, w5)
+    assert check(QE.Q5_K) == 0
+    assert check(QE.Q4_K) == -1 and b"encoding 4" in lib.qmm_last_error() and b"encoding 1" in lib.qmm_last_error()
+    assert matmul(QE.Q4_K) == 0
+    assert torch.isnan(out).all()
+    repack(QE.Q4_K, w4)
+    assert check(QE.Q4_K) == 0
+    assert matmul(QE.Q4_K) == 0
+    torch.cuda.synchronize()
+    assert_close(out, O.matmul_f64(O.Q4_K, O.bf16_to_f32(O.f32_to_bf16(a)), O.quantize(O.Q4_K, w)), "Q4_K over its own planes")
+    # GPTQ: groups of 128 and of 256 give buffers of one size
+    cfg128, cfg256 = _lib.GptqConfig(4, 128, 0, 1), _lib.GptqConfig(4, 256, 0, 1)
+    gsize = lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(cfg128), n, k)
+    if gsize == lib.qmm_repack_bytes(QE.GPTQ.code, C.byref(cfg256), n, k):
+        from mojo_amd import quantize_gptq
+
+        qw, sc, qz, _ = quantize_gptq(gpu(w), QuantizationConfig(quant_method="gptq", bits=4, group_size=128, desc_act=False, sym=True))
+        gp = torch.empty((gsize,), dtype=torch.uint8, device="cuda:0")
+        rhs = (C.c_void_p * 3)(qw.data_ptr(), sc.data_ptr(), qz.data_ptr())
+        _lib.check(lib.qmm_repack(QE.GPTQ.code, C.byref(cfg128), rhs, 3, n, k, C.c_void_p(gp.data_ptr()), gsize, C.c_void_p(s)), "qmm_repack")
+        assert lib.qmm_repack_check(QE.GPTQ.code, C.byref(cfg128), n, k, C.c_void_p(gp.data_ptr()), gsize, C.c_void_p(s)) == 0
+        assert lib.qmm_repack_check(QE.GPTQ.code, C.byref(cfg256), n, k, C.c_void_p(gp.data_ptr()), gsize, C.c_void_p(s)) == -1
+        assert b"group 128" in lib.qmm_last_error() and b"group 256" in lib.qmm_last_error()
