@@ -128,10 +128,14 @@ int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m,
  *   it returns QMM_ERR_UNSUPPORTED.  Bit 1 (QMM_FLAG_ACT_Q8K), Q4_K / Q5_K / Q6_K: the
  *   lhs is quantised to Q8_K blocks (256 wide, fp32 scale) and the products are those of the
  *   integer sub-block dots of the ggml-lineage CPU kernels instead of the default
- *   floating-point ones.  Q4_K with m <= 4 and K <= 16384 takes the integer dots in the kernel;
- *   every other problem writes d8 * code as fp32 rows into the workspace and runs the
- *   floating-point kernels on them (same products, fp32 sums; workspace from
- *   qmm_matmul_workspace_bytes_flags).  Bit 2 (QMM_FLAG_OUT_BF16): `out`
+ *   floating-point ones.  Up to 16 lhs rows go through kernels that form the integer sub-block sums
+ *   themselves (v_dot4_i32_i8, int32 sums per super-block, then (d8 * d) * isum - (d8 * dmin) * msum in fp32),
+ *   in passes of four rows: Q4_K (K <= 16384) quantises the lhs inside the kernel, Q5_K and Q6_K read Q8_K
+ *   codes, scales and 32-code sums that one launch per call writes into the workspace.  The integer sums equal
+ *   the CPU path's bit for bit.  No integer kernel exists beyond 16 rows (or for Q4_K with K > 16384): those
+ *   problems write d8 * code as fp32 rows into the workspace and run the floating-point kernels on them (the
+ *   same products, summed in fp32, not in int32).  Workspace from qmm_matmul_workspace_bytes_flags.
+ *   Bit 2 (QMM_FLAG_OUT_BF16): `out`
  *   points to bf16[m, n] instead of fp32 (the caller's next op takes bf16 activations): the fp32 result is
  *   rounded to nearest even with NaN mapped to the canonical quiet NaN, the reference's narrowing rule
  *   (stdlib/src/builtin/simd.mojo:3279-3300).  The Q4_K decode kernel (m = 1, K <= 16384) stores bf16 itself;

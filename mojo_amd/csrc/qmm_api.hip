@@ -314,14 +314,22 @@ static bool stores_bf16_itself(int encoding, int64_t m, int64_t k, int flags) {
     return encoding == QMM_Q4_K && m == 1 && k % 256 == 0 && k <= 16384 && !(flags & QMM_FLAG_ACT_Q8K) && !qmm::kernel_disabled("q4k_lanes");
 }
 
-// Q8_K activations: Q4_K with up to four lhs rows has a kernel that takes the integer sub-block dots itself; every other
-// problem quantises the lhs, writes d8 * code as fp32 rows into the workspace and runs the floating-point path on those.
-static bool q8k_integer_kernel(int encoding, int64_t m, int64_t k) { return encoding == QMM_Q4_K && m <= 4 && k <= 16384; }
+// Q8_K activations: up to 16 lhs rows go through kernels that take the integer sub-block dots themselves, in passes of four
+// rows (Q4_K: the lhs quantised inside the kernel, K <= 16384; Q5_K and Q6_K: quantised once per call into planes in the
+// workspace).  More rows: the lhs is quantised, d8 * code written as fp32 rows into the workspace, and the floating-point
+// path runs on those (the products of the integer treatment, summed in fp32).
+constexpr int64_t kQ8kIntegerMaxRows = 16;
+static bool q8k_integer_kernel(int encoding, int64_t m, int64_t k) {
+    if (m > kQ8kIntegerMaxRows || k % 256) return false;
+    return encoding == QMM_Q4_K ? k <= 16384 : (encoding == QMM_Q5_K || encoding == QMM_Q6_K);
+}
+static int64_t q8k_integer_workspace(int encoding, int64_t m, int64_t k) { return encoding == QMM_Q4_K ? 0 : qmm::q8k_planes_bytes(m, k); }
 
 int64_t qmm_matmul_workspace_bytes_flags(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k, int flags) {
     int64_t base = qmm_matmul_workspace_bytes(encoding, lhs_dtype, m, n, k);
-    if ((flags & QMM_FLAG_ACT_Q8K) && m > 0 && k > 0 && !q8k_integer_kernel(encoding, m, k))
-        base = up256(m * k * 4) + qmm_matmul_workspace_bytes(encoding, QMM_F32, m, n, k);
+    if ((flags & QMM_FLAG_ACT_Q8K) && m > 0 && k > 0)
+        base = q8k_integer_kernel(encoding, m, k) ? q8k_integer_workspace(encoding, m, k)
+                                                  : up256(m * k * 4) + qmm_matmul_workspace_bytes(encoding, QMM_F32, m, n, k);
     if (!(flags & QMM_FLAG_OUT_BF16) || m <= 0 || n <= 0 || stores_bf16_itself(encoding, m, k, flags)) return base;
     return up256(base) + up256(m * n * 4);
 }
@@ -451,12 +459,26 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     if (flags & QMM_FLAG_ACT_Q8K) {
         if (encoding != QMM_Q4_K && encoding != QMM_Q5_K && encoding != QMM_Q6_K)
             return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q8_K activations go with Q4_K, Q5_K and Q6_K weights");
+        if (q8k_integer_kernel(encoding, m, k) && encoding == QMM_Q4_K) {
+            for (int64_t m0 = 0; m0 < m; m0 += 4) {
+                bool handled = false;
+                hipError_t e = qmm::launch_gemv_q4_k_q8k((const char*)lhs + m0 * k * esz, lhs_dtype, w, (int)std::min<int64_t>(4, m - m0), n, k,
+                                                         out + m0 * n, n, s, &handled);
+                if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K x Q8_K)");
+                if (!handled) return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q4_K x Q8_K shape not taken (M=%lld K=%lld)", (long long)m, (long long)k);
+            }
+            return QMM_OK;
+        }
         if (q8k_integer_kernel(encoding, m, k)) {
-            bool handled = false;
-            hipError_t e = qmm::launch_gemv_q4_k_q8k(lhs, lhs_dtype, w, (int)m, n, k, out, n, s, &handled);
-            if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K x Q8_K)");
-            if (handled) return QMM_OK;
-            return fail(QMM_ERR_UNSUPPORTED, "qmm_matmul: Q4_K x Q8_K shape not taken (M=%lld K=%lld)", (long long)m, (long long)k);
+            if (encoding == QMM_Q5_K && !aligned(w, 16)) return fail(QMM_ERR_INVALID, "qmm_matmul: Q5_K rhs must be 16-byte aligned");
+            const qmm::Q8KPlanes p = qmm::q8k_planes(workspace, m, k);
+            hipError_t e = qmm::launch_quantize_q8_k_planes(lhs, lhs_dtype, m, k, p, s);
+            if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q8_K planes)");
+            for (int64_t m0 = 0; m0 < m; m0 += 4) {
+                e = qmm::launch_gemv_kquant_q8k(encoding, p, m0, (int)std::min<int64_t>(4, m - m0), w, n, k, out + m0 * n, n, s);
+                if (e != hipSuccess) return hip_status(e, "qmm_matmul(K-quant x Q8_K)");
+            }
+            return QMM_OK;
         }
         // the quantised activations as fp32 rows (d8 * code), then the floating-point path on them: the products are those of
         // the integer treatment, summed in fp32

@@ -27,6 +27,18 @@ hipError_t launch_quantize_q8_0(const void* x, int x_dtype, int64_t rows, int64_
                                 void* codes, void* dscale, void* csum, hipStream_t s);
 hipError_t launch_quantize_q8_k(const void* x, int x_dtype, int64_t rows, int64_t k, void* out, hipStream_t s);
 // y fp32[rows, k] = d8 * code of the Q8_K quantisation of x (k a multiple of 256)
+// Q8_K activations as planes (codes [m, k], d8 [m, k / 256], sums of 32 codes [m, k / 32]) and the integer-dot decode kernels
+// for Q5_K and Q6_K weights over them (gemv_kquant_q8k.hip): one pass takes up to four lhs rows.
+struct Q8KPlanes {
+    int8_t* codes;
+    float* d8;
+    int32_t* sums;
+};
+int64_t q8k_planes_bytes(int64_t m, int64_t k);
+Q8KPlanes q8k_planes(void* ws, int64_t m, int64_t k);
+hipError_t launch_quantize_q8_k_planes(const void* x, int x_dtype, int64_t rows, int64_t k, const Q8KPlanes& p, hipStream_t s);
+hipError_t launch_gemv_kquant_q8k(int encoding, const Q8KPlanes& p, int64_t m0, int rows, const uint8_t* w, int64_t n, int64_t k, float* out,
+                                  int64_t ldo, hipStream_t s);
 hipError_t launch_q8k_round_trip(const void* x, int x_dtype, int64_t rows, int64_t k, float* y, hipStream_t s);
 hipError_t launch_quantize_gptq(const float* w, int64_t n, int64_t k, int group, void* qweight,
                                 void* scales, void* qzeros, void* g_idx, hipStream_t s);

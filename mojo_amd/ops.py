@@ -97,7 +97,8 @@ def qmatmul(encoding: QuantizationEncoding, config: Optional[QuantizationConfig]
     ``(qweight int32[K/8, N], scales float16[K/g, N], qzeros int32[K/g, N/8][, g_idx int32[K]])``.
     ``lhs`` is float32 or bfloat16.  Q4_0 quantises ``lhs`` to Q8_0 blocks and
     takes integer block dots; the other encodings use ``lhs`` as given.  ``act_q8k=True`` (Q4_K, Q5_K,
-    Q6_K) quantises ``lhs`` to Q8_K blocks and takes the products of the ggml-lineage CPU kernels' integer sub-block dots instead.
+    Q6_K) quantises ``lhs`` to Q8_K blocks and takes the products of the ggml-lineage CPU kernels' integer sub-block dots instead
+    (integer sums in the kernel up to 16 lhs rows; beyond that the same products summed in fp32).
     ``w_bf16=True`` asks for the reserved mode that rounds the dequantised weights to bfloat16 first; the library
     has no kernel for it and raises ``NotImplementedError``.
 

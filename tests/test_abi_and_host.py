@@ -85,7 +85,8 @@ def test_argument_validation_happens_before_any_launch():
     assert f(1, 0, 1, 4096, 4096, _lib.QMM_FLAG_OUT_BF16) == 0                      # Q4_K decode stores bf16 itself
     assert f(2, 0, 1, 4096, 4096, _lib.QMM_FLAG_OUT_BF16) == 4096 * 4               # Q6_K decode: fp32 result in the workspace
     assert f(1, 0, 4, 4096, 4096, _lib.QMM_FLAG_ACT_Q8K) == 0                       # the integer kernel
-    assert f(2, 0, 4, 4096, 4096, _lib.QMM_FLAG_ACT_Q8K) >= 4 * 4096 * 4            # Q6_K: round-tripped rows
+    assert 4 * 4096 < f(2, 0, 4, 4096, 4096, _lib.QMM_FLAG_ACT_Q8K) < 4 * 4096 * 2  # Q6_K, few rows: Q8_K codes, scales and sums
+    assert f(2, 0, 40, 4096, 4096, _lib.QMM_FLAG_ACT_Q8K) >= 40 * 4096 * 4          # Q6_K, many rows: round-tripped fp32 rows
     assert f(1, 0, 2048, 14336, 4096, 0) == lib.qmm_matmul_workspace_bytes(1, 0, 2048, 14336, 4096)
     # Q5_K / Q6_K prefill: lhs planes and weight planes (2 bytes per weight and plane; Q6_K has two)
     assert lib.qmm_matmul_workspace_bytes(2, 1, 2048, 14336, 4096) >= 2 * 14336 * 4096 * 2
@@ -102,12 +103,12 @@ def test_argument_validation_happens_before_any_launch():
     # is refused.  K = 100 makes a call that got past the size checks fail on the block size instead of reaching a launch.
     both = _lib.QMM_FLAG_ACT_Q8K | _lib.QMM_FLAG_OUT_BF16
     for enc in (4, 2, 1):
-        need = f(enc, 0, 8, 512, 4096, both)
-        assert need >= 8 * 4096 * 4 + 8 * 512 * 4
-        assert lib.qmm_matmul(enc, None, fake, 0, 8, 4096, rhs, 1, 512, fake, ws, need - 1, both, None) == -4
-        assert f(enc, 0, 8, 512, 100, both) >= 8 * 100 * 4 + 8 * 512 * 4
-        assert lib.qmm_matmul(enc, None, fake, 0, 8, 100, rhs, 1, 512, fake, ws, f(enc, 0, 8, 512, 100, both), both, None) == -1
-        assert b"block size" in lib.qmm_last_error()
+        for rows in (8, 40):  # the integer kernels (passes of four rows); the fp32 round trip of the lhs
+            need = f(enc, 0, rows, 512, 4096, both)
+            assert need >= rows * 512 * 4 + (rows * 4096 * 4 if rows > 16 else 0)
+            assert lib.qmm_matmul(enc, None, fake, 0, rows, 4096, rhs, 1, 512, fake, ws, need - 1, both, None) == -4
+            assert lib.qmm_matmul(enc, None, fake, 0, rows, 100, rhs, 1, 512, fake, ws, max(f(enc, 0, rows, 512, 100, both), 1 << 20), both, None) == -1
+            assert b"block size" in lib.qmm_last_error()
     # the normalisation prologue
     g = C.c_void_p(0x3000)
     rn = lib.qmm_matmul_rmsnorm

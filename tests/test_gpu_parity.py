@@ -589,6 +589,55 @@ def test_kquant_matmul_with_q8_k_activations(enc, m, n, k, lhs_bf16):
         assert not O.isclose(got, O.matmul_f32(ENC[enc], a, wq), 1e-4, 1e-5).all()
 
 
+def _kquant_integer_case(enc, m, n, k, bf16, seed):
+    """Inputs on which the fp32 output of the Q8_K-activation path IS a sum of the integer block sums: weight blocks of random
+    bytes with d = 1.0 (and dmin = 1.0; fp16 0x3C00), scale fields kept small (6-bit scales and mins below 16, Q6_K's int8
+    scales in [-8, 7]); lhs values small integers with one +-127 per 256-block, so that every Q8_K scale is +-1 and a code is
+    its value (or minus it).  Then out[i, j] == sum_b d8[i, b] * (isum[i, j, b] - msum[i, j, b]), every term and partial sum an
+    integer below 2^24, which fp32 adds exactly in any order."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    nb = k // 256
+    bpb = {QE.Q4_K: 144, QE.Q5_K: 176, QE.Q6_K: 210}[enc]
+    blocks = rng.integers(0, 256, (n, nb, bpb), dtype=np.uint8)
+    one = np.array([0x00, 0x3C], np.uint8)
+    if enc == QE.Q6_K:
+        blocks[:, :, 192:208] = rng.integers(-8, 8, (n, nb, 16)).astype(np.int8).view(np.uint8)
+        blocks[:, :, 208:210] = one
+    else:
+        blocks[:, :, 0:2] = one
+        blocks[:, :, 2:4] = one
+        blocks[:, :, 4:16] &= 0x0F  # scales / mins of sub-blocks 0..3 below 16; 4..7 keep their low four bits only
+    wq = np.ascontiguousarray(blocks.reshape(n, nb * bpb))
+    a = rng.integers(-7, 8, (m, nb, 256)).astype(np.float32)
+    a[:, 1::3, 40:80] = 0.0
+    peak = rng.integers(0, 256, (m, nb))
+    sign = rng.choice(np.array([-127.0, 127.0], np.float32), (m, nb))
+    np.put_along_axis(a, peak[:, :, None], sign[:, :, None], axis=2)
+    a = np.ascontiguousarray(a.reshape(m, k))
+    aq = O.quantize_q8_k(a)
+    d8 = aq.reshape(m, nb, 292)[:, :, :4].copy().view(np.float32).reshape(m, nb)
+    assert (np.abs(d8) == 1.0).all()
+    isum, msum = O.block_sums_kquant_q8_k(ENC[enc], aq, wq, k)
+    terms = d8[:, None, :].astype(np.int64) * (isum.astype(np.int64) - msum.astype(np.int64))
+    assert np.abs(np.cumsum(np.abs(terms), axis=2)).max() < 2**24
+    lhs = gpu(a).to(torch.bfloat16) if bf16 else gpu(a)
+    return lhs, gpu(wq), terms.sum(axis=2).astype(np.float32)
+
+
+# rows 1..4: one pass of the integer kernels (Q4_K quantises its lhs in the kernel, Q5_K / Q6_K read Q8_K planes made once
+# per call); 7, 16: passes of four; K = 256: a single block; 2304 / 1280: ragged groups of 16 / 4 super-blocks
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("enc,m,n,k", [(QE.Q6_K, 1, 200, 1024), (QE.Q6_K, 4, 130, 256), (QE.Q6_K, 7, 64, 1280), (QE.Q6_K, 16, 33, 512),
+                                       (QE.Q5_K, 1, 200, 1024), (QE.Q5_K, 3, 130, 256), (QE.Q5_K, 7, 64, 2304), (QE.Q5_K, 16, 33, 512),
+                                       (QE.Q4_K, 2, 200, 1024), (QE.Q4_K, 7, 64, 2304), (QE.Q4_K, 16, 33, 256)])
+def test_kquant_production_kernels_give_the_integer_block_sums(enc, m, n, k, bf16):
+    """The integer sub-block sums of the Q8_K-activation kernels (QMM_FLAG_ACT_Q8K, up to 16 lhs rows), read off the fp32 output,
+    equal the oracle's block by block sums bit for bit."""
+    lhs, wq, want = _kquant_integer_case(enc, m, n, k, bf16, seed=51 + m)
+    got = qmatmul(enc, None, lhs, wq, act_q8k=True).cpu().numpy()
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} outputs differ from the integer sums"
+
+
 @pytest.mark.parametrize("enc,m", [(QE.Q6_K, 8), (QE.Q4_K, 8), (QE.Q5_K, 3), (QE.Q4_K, 2)])
 def test_q8_k_activations_with_bf16_output(enc, m):
     """Both flags in one call: the bf16 result is the rounding of the fp32 result of the same call (the Q4_K integer kernel
