@@ -520,10 +520,13 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib"), default="decode",
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib", "mfma_probe", "sweep"),
+                    default="decode",
                     help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill / q6k_prefill / q5k_prefill / q40_prefill: the M=2048 "
                          "GEMM of the same model's gate projection (second target, matrix-core roofline); calib: a plain "
-                         "read and a plain copy of 256 MiB, the yardsticks for the FETCH_SIZE / WRITE_SIZE counters")
+                         "read and a plain copy of 256 MiB, the yardsticks for the FETCH_SIZE / WRITE_SIZE counters; mfma_probe: the "
+                         "matrix-core rate of a register-resident loop by operand data; sweep: Q4_K decode and prefill over shapes "
+                         "the dispatch was not tuned on")
     ap.add_argument("--repacked", action="store_true", help="prefill workloads: weight planes made once (qmm_repack), outside the timed steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip per-shape and secondary-config timings")
@@ -541,6 +544,10 @@ def main() -> int:
     gen.manual_seed(3)
     if args.workload == "calib":
         return calib_main()
+    if args.workload == "mfma_probe":
+        return probe_main()
+    if args.workload == "sweep":
+        return sweep_main(gen)
     if args.workload != "decode":
         return prefill_main(args, gen)
     m = args.m
@@ -595,6 +602,8 @@ def main() -> int:
         extra["one_graph_launch_per_step"]["us_per_step_with_clock_sampler_thread"] = round(d7s * 1e6 / args.steps, 3)
         del small
     roofline_prefill = None if args.no_prefill else prefill_roofline(gen, cu.value, khz.value / 1000.0)
+    if roofline_prefill is not None:
+        roofline_prefill["mfma_probe"] = mfma_probe()
     if not args.no_extra:
         extra.update(extra_timings(layers, acts, gen))
         # the headline once more, after everything else: the same graphs, a short warm-up
@@ -691,6 +700,89 @@ def prefill_roofline(gen, cus: int, nominal_mhz: float):
             "repacked": repacked}
 
 
+def mfma_probe(seconds: float = 0.12):
+    """The matrix-core rate that a register-resident loop of v_mfma_f32_32x32x16_f16 sustains on this part (qmm_mfma_probe: no
+    memory traffic, 8 wavefronts per compute unit), for zeros, for dense random data on both sides, and for random values
+    against integers 0..945 (what the plane GEMMs multiply); each after `seconds` of untimed launches and over `seconds` of
+    timed ones, with the shader clock sampled over launches of its own."""
+    lib = _lib.load()
+    cu = C.c_int32(0)
+    lib.qmm_device_info(C.byref(cu), None)
+    out = torch.empty((cu.value * 512,), dtype=torch.float32, device="cuda:0")
+    s = torch.cuda.current_stream().cuda_stream
+    iters, res = 2000, {}
+    for kind, name in ((0, "zeros"), (2, "random_x_random"), (3, "random_x_integers_0_945")):
+        flops = C.c_int64(0)
+
+        def launch():
+            _lib.check(lib.qmm_mfma_probe(C.c_void_p(out.data_ptr()), out.numel() * 4, kind, iters, C.byref(flops), C.c_void_p(s)), "qmm_mfma_probe")
+
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(8):
+                launch()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        count = 0
+        e0.record()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(8):
+                launch()
+            count += 8
+        e1.record()
+        torch.cuda.synchronize()
+        tf = flops.value * count / (e0.elapsed_time(e1) * 1e-3) / 1e12
+        with ClockSampler() as clk:
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < 0.06:
+                for _ in range(8):
+                    launch()
+                torch.cuda.synchronize()
+        res[name] = {"TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4), "clock_mhz": clk.mhz}
+    return res
+
+
+def probe_main() -> int:
+    print(json.dumps({"metric": "register-resident v_mfma_f32_32x32x16_f16 loop, TFLOP/s by operand data", "unit": "TFLOP/s",
+                      "peak": BF16_PEAK_TFLOPS, "mfma_probe": mfma_probe(0.3)}))
+    return 0
+
+
+SWEEP_SHAPES = [(4096, 11008), (11008, 4096), (32000, 4096), (5120, 5120), (3584, 18944)]  # (N, K): none of them tuned for
+
+
+def sweep_main(gen) -> int:
+    """Q4_K over shapes the dispatch thresholds were not fitted to: decode rows 1 / 4 / 16 as a fraction of the plain read of the
+    same weight bytes (cold: copies rotated beyond the 256 MB cache), prefill rows 512 / 2048 (bf16 lhs) as a fraction of the
+    2.5 PFLOP/s peak.  One JSON line; a cliff in the dispatch shows as a fraction far below its neighbours'."""
+    out = {}
+    for n, k in SWEEP_SHAPES:
+        w0 = make_weight(QE.Q4_K, n, k, gen)
+        copies = max(2, (320 << 20) // w0.numel() + 1)
+        ws = [w0] + [w0.clone() for _ in range(copies - 1)]
+        dev_s, _ = time_graphs([capture([ReadProbe(w) for w in ws])], 20, 3)
+        read_us = dev_s * 1e6 / (20 * copies)
+        row = {"plain_read_us": round(read_us, 2), "plain_read_GB/s": round(w0.numel() / read_us / 1e3, 1)}
+        for m in (1, 4, 16):
+            a = torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen)
+            dev_s, _ = time_graphs([capture([Gemv(QE.Q4_K, w, a) for w in ws])], 20, 3)
+            us = dev_s * 1e6 / (20 * copies)
+            row[f"m{m}"] = {"us": round(us, 2), "GB/s": round(alg_bytes(QE.Q4_K, m, n, k) / us / 1e3, 1), "frac_of_plain_read": round(read_us / us, 3)}
+        del ws
+        for m in (512, 2048):
+            ab = torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen).to(torch.bfloat16)
+            dev_s, _ = time_graphs([capture([Gemv(QE.Q4_K, w0, ab)])], 10, 2)
+            us = dev_s * 1e6 / 10
+            tf = 2.0 * m * n * k / us / 1e6
+            row[f"m{m}"] = {"us": round(us, 1), "TFLOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
+        out[f"{n}x{k}"] = row
+        del w0
+    print(json.dumps({"metric": "Q4_K over untuned shapes: decode as a fraction of the plain read, prefill of the matrix-core peak",
+                      "encoding": "Q4_K", "sweep": out}))
+    return 0
+
+
 def calib_main() -> int:
     """Known-size kernels for scaling the HBM counters: qmm_read_probe reads 256 MiB, a torch copy reads
     and writes 256 MiB.  Each runs three times; buffers are larger than every cache."""
@@ -725,8 +817,6 @@ def prefill_main(args, gen) -> int:
         call, name, kern = GptqMatmul(wg, ab), "GPTQ g128", "gptq_planes_prologue_kernel + gemm_planes_wide_kernel"
     step_text = "one preparation launch (lhs narrowing, weights to fp16 integer planes) + one GEMM launch"
     if args.repacked:
-        if args.workload == "q40_prefill":
-            raise SystemExit("bench.py: Q4_0 has no weight planes that are kept across calls")
         rhs = tuple(call.t[:3]) if args.workload == "gptq_prefill" else (call.w,)
         call = RepackedGemv(call.enc if hasattr(call, "enc") else QE.GPTQ, rhs, ab)
         kern = "planes_prologue_kernel (lhs rows only) + " + kern.split(" + ")[1]

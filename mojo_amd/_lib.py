@@ -27,6 +27,7 @@ SIGNATURES = {
     "qmm_block_params": (_int, [_int, C.POINTER(_i64), C.POINTER(_i64)]),
     "qmm_device_info": (_int, [C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "qmm_read_probe": (_int, [_vp, _i64, _vp]),
+    "qmm_mfma_probe": (_int, [_vp, _i64, _int, _int, C.POINTER(_i64), _vp]),
     "qmm_dequantize": (_int, [_int, _vp, _i64, _i64, _vp, _int, _vp]),
     "qmm_dequantize_gptq": (_int, [C.POINTER(GptqConfig), _vp, _vp, _vp, _vp, _i64, _i64, _vp, _int, _vp]),
     "qmm_quantize": (_int, [_int, _vp, _i64, _i64, _vp, _vp]),

@@ -359,7 +359,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     if (swiglu && (count != 2 || ns[0] != ns[1] || m != 1)) return hipSuccess;
     const bool off = kernel_disabled("q4k_lanes");
     const int nblk = (int)(k / 256);
-    if (off || m > 1 || nblk > 64 || count < 1 || count > kLanesMaxMats) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
+    if (off || m > 1 || nblk > 128 || count < 1 || count > kLanesMaxMats) return hipSuccess;  // (two lhs rows: the small-batch matrix-core kernel is faster)
     LanesMats mats;
     int64_t n = 0;
     for (int j = 0; j < kLanesMaxMats; j++) {
@@ -373,7 +373,7 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     mats.swiglu = swiglu ? 1 : 0;
     mats.out_bf16 = out_bf16 ? 1 : 0;
     if (n > 0x7fffffff) return hipSuccess;
-    const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
+    const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : nblk <= 64 ? 4 : 8;  // (8: the whole workgroup on one row at a time, K up to 32768)
     const int bpw = (nblk + wpr - 1) / wpr;
     const int l = (bpw * 9 + 63) / 64;  // 1..3
     const int mt = m <= 1 ? 1 : 2;
@@ -437,7 +437,8 @@ hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count,
     } while (0)
     if (wpr == 1) QMM_GO0(1);
     else if (wpr == 2) QMM_GO0(2);
-    else QMM_GO0(4);
+    else if (wpr == 4) QMM_GO0(4);
+    else QMM_GO0(8);
 #undef QMM_GO0
 #undef QMM_GO1
 #undef QMM_GO2

@@ -17,6 +17,8 @@ namespace qmm {
 bool kernel_disabled(const char* family);
 
 hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
+// register-resident matrix-core loop (probes.hip): `workgroups` workgroups of 8 wavefronts, out fp32 [workgroups * 512]
+hipError_t launch_mfma_probe(float* out, int workgroups, int kind, int iters, hipStream_t s);
 hipError_t launch_dequant(int enc, const void* rhs, int64_t n, int64_t k, void* out, int out_dtype,
                           hipStream_t s);
 hipError_t launch_dequant_gptq(const void* qweight, const void* scales, const void* qzeros,

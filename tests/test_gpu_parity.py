@@ -491,10 +491,11 @@ def test_leading_dims_broadcast():
 # ------------------------------------------------------------------ Q4_K decode (one lhs row)
 @pytest.mark.parametrize("n,k,lhs_bf16", [(1, 256, False), (7, 512, True), (70000, 256, False), (129, 4096, False),
                                           (300, 4352, True), (50, 8192, False), (33, 9984, False), (40, 16384, True),
-                                          (12, 16640, False), (5000, 3840, False)])
+                                          (12, 16640, False), (5000, 3840, False), (600, 18944, False), (70, 24576, True),
+                                          (9, 33024, False)])
 def test_q4_k_decode_shapes(n, k, lhs_bf16):
-    """One lhs row: rows cut into 1, 2 or 4 parts (K up to 16384; longer rows take the streaming kernel), parts that
-    do not fill a wavefront, fewer rows than wavefronts, many rows per wavefront."""
+    """One lhs row: rows cut into 1, 2, 4 or 8 parts (K up to about 28000, as long as the staged lhs fits the LDS; longer
+    rows take the streaming kernel), parts that do not fill a wavefront, fewer rows than wavefronts, many rows per wavefront."""
     w, a = synth(23, n, k, 1)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
