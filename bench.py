@@ -505,10 +505,21 @@ def cpu_baseline(layer_w, m: int, budget_s: float = 10.0):
 
 
 def measured_traffic(key: str):
-    """HBM bytes per launch from the committed PMC summary (profiles/hbm_traffic.json), or None."""
+    """HBM bytes per launch from the committed PMC summary (profiles/hbm_traffic.json), or None.  The entry names the kernel
+    sources it was measured on (a hash): a figure taken on other sources than the tree's is not reported."""
+    import hashlib
+
+    files = {"decode_m1": ("gemv_q4k_lanes.hip", "lds_stream.h"), "prefill_q4_k": ("gemm_planes.hip", "gemm_tile.h", "gemm_lhs.h")}
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            return json.load(f)[key]["traffic_bytes_per_launch"]
+            entry = json.load(f)[key]
+        h = hashlib.sha256()
+        for name in files[key]:
+            with open(os.path.join(ROOT, "mojo_amd", "csrc", name), "rb") as src:
+                h.update(src.read())
+        if entry.get("source_sha256_16") != h.hexdigest()[:16]:
+            return None
+        return entry["traffic_bytes_per_launch"]
     except (OSError, KeyError, ValueError):
         return None
 
@@ -528,6 +539,8 @@ def main() -> int:
                          "matrix-core rate of a register-resident loop by operand data; sweep: Q4_K decode and prefill over shapes "
                          "the dispatch was not tuned on")
     ap.add_argument("--repacked", action="store_true", help="prefill workloads: weight planes made once (qmm_repack), outside the timed steps")
+    ap.add_argument("--warm-seconds", type=float, default=HEADLINE_WARM_S,
+                    help="decode: least wall time of the headline's warm-up (profiling runs shorten it to keep their traces small)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip per-shape and secondary-config timings")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg (roofline_prefill)")
@@ -561,7 +574,7 @@ def main() -> int:
     # The headline: graphs that hold whole steps (one host launch per rotation of the layers), a warm-up of at least a
     # second, nothing else running in this process while the blocks are timed.
     runner = StepRunner(calls, args.steps)
-    warm_steps = runner.warm(args.warmup, HEADLINE_WARM_S)
+    warm_steps = runner.warm(args.warmup, args.warm_seconds)
     times, wall_s = runner.time(HEADLINE_MIN_MS)
     repeats = len(times)
     dev_s = times[repeats // 2] * 1e-3
@@ -651,7 +664,7 @@ def main() -> int:
         "extra": extra,
     }
     extra["timing"] = (f"ms_per_step is the median of {repeats} timed blocks of exactly {args.steps} steps each, run back to back "
-                       f"after {warm_steps} warm-up steps (at least {args.warmup}, and at least {HEADLINE_WARM_S:.1f} s); a block is "
+                       f"after {warm_steps} warm-up steps (at least {args.warmup}, and at least {args.warm_seconds:.2f} s); a block is "
                        f"{runner.host_launches_per_block} graph launches (a graph holds one step of each of the {args.layers} layers)")
     extra["DEBUG_CLR_GRAPH_PACKET_CAPTURE"] = os.environ.get("DEBUG_CLR_GRAPH_PACKET_CAPTURE")
     if not args.no_cpu:
@@ -691,7 +704,7 @@ def prefill_roofline(gen, cus: int, nominal_mhz: float):
                 "packed_bytes": kept.packed.numel(),
                 "note": "qmm_matmul_repacked on planes made once by qmm_repack, as a host that converts at model load would call it"}
     return {"bound": "mfma", "achieved": round(tf, 2), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(tf / BF16_PEAK_TFLOPS, 4), "kernel": PREFILL_KERNEL, "flops_per_launch": flops,
+            "frac": round(tf / BF16_PEAK_TFLOPS, 4), "traffic": measured_traffic("prefill_q4_k"), "kernel": PREFILL_KERNEL, "flops_per_launch": flops,
             "launch_us": round(us, 2), "clock_mhz_during_kernel": mhz,
             "peak_at_measured_clock": round(peak_at_clock, 1) if peak_at_clock else None,
             "frac_at_measured_clock": round(tf / peak_at_clock, 4) if peak_at_clock else None,
@@ -862,6 +875,10 @@ def extra_timings(layers, acts, gen):
         b = alg_bytes(QE.Q4_K, m, n, k)
         per_shape[f"{name}_{n}x{k}"] = {"us": round(us, 3), "GB/s": round(b / us / 1e3, 1)}
     out["q4_k_per_shape"] = per_shape
+    # the floor under every launch: a kernel that reads 4 KB and does nothing else, 56 of them in a replayed graph
+    tiny = torch.zeros((4096,), dtype=torch.uint8, device="cuda:0")
+    dev_s, _ = time_graphs([capture([ReadProbe(tiny) for _ in range(56)])], 50, 5)
+    out["launch_floor_us_per_kernel_node"] = round(dev_s * 1e6 / (50 * 56), 3)
     # warm cache, labelled as such: one layer (123 MB, inside the 256 MB last-level cache) replayed by itself
     g = capture([Gemv(QE.Q4_K, w, acts[k]) for w, (_, n, k) in zip(layers[0], PROJ)])
     dev_s, _ = time_graphs([g], 100, 10)
