@@ -171,6 +171,7 @@ int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lh
  * QMM_ERR_WORKSPACE (use qmm_matmul with a workspace).  All calls on one GPU share the buffer: calls that
  * can overlap there (different streams, different host threads) race and must be ordered by the caller.
  * Nothing in the buffer is expected to be zero or to survive from one call to the next.
+  * The first call on a device looks the buffer's address up and sets kernel attributes: make it outside graph capture.
  */
 #define QMM_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
 int qmm_matmul_static(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m,

@@ -29,6 +29,8 @@ SETTINGS = [
     {"QMM_DISABLE": "planes_wide,planes_quarters"},
     # ... and Q4_K / GPTQ alone kept off the planes
     {"QMM_DISABLE": "q4k_planes,gptq_planes"},
+    # the plain calls of Q4_K decode and small batch through the kernels that take several matrices
+    {"QMM_DISABLE": "q4k_lanes_plain,q4k_mm_plain"},
 ]
 
 

@@ -99,3 +99,43 @@ def test_static_scratch_rejects_what_does_not_fit():
     rhs = (C.c_void_p * 1)(0x20000)
     assert lib.qmm_matmul_static(1, None, fake, 0, m, k, rhs, 1, n, fake, 0, None) == -4
     assert b"static buffer" in lib.qmm_last_error()
+
+
+def test_static_scratch_inside_a_captured_graph_and_with_bf16_output():
+    """The stated use: after one call outside capture (the first call on a device looks the buffer's address up and sets
+    kernel attributes), the entry point is recorded into a HIP graph and replayed, with the program's own eager work between
+    the replays; every replay equals the eager call bit for bit.  With QMM_FLAG_OUT_BF16 the fp32 result sits in the static
+    buffer on the way."""
+    lib = _lib.load()
+    m, n, k = 12, 130, 2048
+    w, a = synth(61, n, k, m)
+    wq = gpu(O.quantize(O.Q4_K, w))
+    lhs = gpu(a)
+    ptrs = (C.c_void_p * 1)(wq.data_ptr())
+    for flags, dtype in ((0, torch.float32), (_lib.QMM_FLAG_OUT_BF16, torch.bfloat16)):
+        out = torch.zeros((m, n), dtype=dtype, device=DEV)
+
+        def call(stream):
+            rc = lib.qmm_matmul_static(QE.Q4_K.code, None, C.c_void_p(lhs.data_ptr()), _lib.QMM_F32, m, k, ptrs, 1, n,
+                                       C.c_void_p(out.data_ptr()), flags, C.c_void_p(stream))
+            assert rc == 0, lib.qmm_last_error()
+
+        call(torch.cuda.current_stream().cuda_stream)  # outside capture first
+        torch.cuda.synchronize()
+        eager = out.clone()
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                call(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        for i in range(3):
+            out.zero_()
+            other = qmatmul(QE.Q4_K, None, lhs[: 1 + i], wq)  # eager work of the program between the replays
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {i} differs from the eager call (flags {flags})"
+            assert other.shape == (1 + i, n)
+    want = O.matmul_f32(O.Q4_K, a, O.quantize(O.Q4_K, w))
+    assert O.isclose(eager.float().cpu().numpy(), O.bf16_to_f32(O.f32_to_bf16(want)), 1e-2, 1e-3).all()
