@@ -55,6 +55,7 @@ constexpr int kRingBytes = kWaves * kSlots * kSlotBytes;
 constexpr int kAccBytes = kWaves * kMaxTiles * 4 * 64 * 4;
 constexpr int kLdsBytes = kRingBytes + kAccBytes;
 static_assert(4 * kStageBytes + 16 <= kSlotBytes, "four staged lhs rows and their scales fit the free ring slot");
+static_assert(8 * kStageBytes + 32 <= 2 * kSlotBytes, "both super-blocks of four staged lhs rows fit two free ring slots");
 
 typedef __fp16 fp16x2 __attribute__((ext_vector_type(2)));  // what the packed conversion builtin returns
 
@@ -163,10 +164,10 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
         islot = islot == kSlots - 1 ? 0 : islot + 1;
         if (++it_t == my_tiles) { it_t = 0; ig++; }
     };
-    // two items before the conversion (the third slot is its staging area): their loads keep the memory system busy while
-    // the lhs is converted
+    // One item before the first conversion, whose staging area is the other two slots (more loads in front of it only delay
+    // the raw lhs values it waits for); the kernel that reads ready-made lhs planes fills its ring.
     if (total > 0) issue_next();
-    if (total > 1) issue_next();
+    if (!INLINE && total > 1) issue_next();
 
     // lhs operand row of this lane: INLINE: row nn % 8, hi plane for nn < 8, residual for nn >= 8
     const int mrow = min(INLINE ? (nn & 7) : nn, m - 1);
@@ -233,7 +234,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
                             const uint32_t mx = max_abs_bits(x0, x1, x2, x3);
                             mxs[bb * RP + j] = mx;
                             lane_max = max(lane_max, mx);
-                            floor_ok = floor_ok && __builtin_amdgcn_ballot_w64(mx >= 0x3C800000u) != 0;  // some value of it reaches 2^-6
+                            floor_ok = floor_ok & (__builtin_amdgcn_ballot_w64(mx >= 0x3C800000u) != 0);  // some value of it reaches 2^-6
                         }
                     // Every one of them between 2^-6 and 2^15 (activations of ordinary size): the values go to fp16 as they are,
                     // hi + residual carry 22 bits of each, and what is below fp16's normal range (2^-14) is small against the
@@ -247,16 +248,15 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
                         for (int j = 0; j < RP; j++) {
                             float x0, x1, x2, x3;
                             widen(xr[bb][ps * RP + j], x0, x1, x2, x3);
-                            float sc = 1.0f;
                             isc[bb][j] = 1.0f;
                             if (!as_is) {
                                 const uint32_t mxb = mxs[bb * RP + j];
                                 int e = (int)((mxb >> 23) & 0xffu) - 127;
                                 if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite: leave unscaled
-                                sc = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
+                                const float sc = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
                                 isc[bb][j] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+                                x0 *= sc; x1 *= sc; x2 *= sc; x3 *= sc;
                             }
-                            x0 *= sc; x1 *= sc; x2 *= sc; x3 *= sc;
                             // hi part: the value cut to fp16 (toward zero: one instruction converts and packs two);
                             // the residual x - hi is exact in fp32 and is cut to fp16 the same way
                             const fp16x2 c02 = __builtin_amdgcn_cvt_pkrtz(x0, x2), c13 = __builtin_amdgcn_cvt_pkrtz(x1, x3);
@@ -269,20 +269,18 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
                             sp[bb][j] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(sum, sum - (float)sm.x));
                         }
                     }
-#pragma unroll
-                    for (int bb = 0; bb < kRunBlk; bb++) {
-                        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                        for (int j = 0; j < RP; j++) {
-                            uint8_t* st = stg + j * kStageBytes;
-                            *(uint2*)(st + 8 * lane) = make_uint2(hp[bb][j][0], hp[bb][j][1]);
-                            *(uint2*)(st + kPlaneStride + 8 * lane) = make_uint2(lp[bb][j][0], lp[bb][j][1]);
-                            if ((lane & 7) == 0) *(uint32_t*)(st + 2 * kPlaneStride + 4 * (lane >> 3)) = sp[bb][j];
-                            if (lane == 0) *(float*)(stg + RP * kStageBytes + 4 * j) = isc[bb][j];
-                        }
-                        __builtin_amdgcn_wave_barrier();
+                    // The converted values change lanes through LDS: a lane wrote four columns of every row, it reads the
+                    // fragments of one row and plane.  unit u = staged (super-block, row) record.
+                    auto put = [&](uint8_t* area, int u, int bb, int j, float* scales) __attribute__((always_inline)) {
+                        uint8_t* st = area + u * kStageBytes;
+                        *(uint2*)(st + 8 * lane) = make_uint2(hp[bb][j][0], hp[bb][j][1]);
+                        *(uint2*)(st + kPlaneStride + 8 * lane) = make_uint2(lp[bb][j][0], lp[bb][j][1]);
+                        if ((lane & 7) == 0) *(uint32_t*)(st + 2 * kPlaneStride + 4 * (lane >> 3)) = sp[bb][j];
+                        if (lane == 0) scales[u] = isc[bb][j];
+                    };
+                    auto get = [&](const uint8_t* area, int u0, int bb, const float* scales) __attribute__((always_inline)) {
                         if (rr >= ps * RP && rr < ps * RP + RP) {
-                            const uint8_t* st = stg + (rr - ps * RP) * kStageBytes;
+                            const uint8_t* st = area + (u0 + rr - ps * RP) * kStageBytes;
                             const uint8_t* pl = st + (nn >= 8 ? kPlaneStride : 0) + 128 * kg;
 #pragma unroll
                             for (int p = 0; p < 4; p++) {
@@ -299,9 +297,31 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
                         // (with fewer than 4 staged rows every lane takes them: rows past m are dropped at the end)
                         if (RP < 4 || (kg & 1) == ps) {
 #pragma unroll
-                            for (int r = 0; r < RP; r++) bs[bb][r] = *(const float*)(stg + RP * kStageBytes + 4 * r);
+                            for (int r = 0; r < RP; r++) bs[bb][r] = scales[u0 + r];
                         }
+                    };
+                    // First group: only item 0 is in flight (slot 0), slots 1 and 2 take both super-blocks at once.  Later
+                    // groups have one free slot (the next item's): one super-block at a time.
+                    const bool both = grp == 0;
+                    uint8_t* area = both ? ring + kSlotBytes : stg;
+                    float* scales = (float*)(area + (both ? kRunBlk : 1) * RP * kStageBytes);
+                    static_assert(kRunBlk == 2, "the staging below is written for two super-blocks");
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int j = 0; j < RP; j++) put(area, j, 0, j, scales);
+                    if (both) {
+#pragma unroll
+                        for (int j = 0; j < RP; j++) put(area, RP + j, 1, j, scales);
                     }
+                    __builtin_amdgcn_wave_barrier();
+                    get(area, 0, 0, scales);
+                    if (!both) {
+                        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                        for (int j = 0; j < RP; j++) put(area, j, 1, j, scales);
+                        __builtin_amdgcn_wave_barrier();
+                    }
+                    get(area, both ? RP : 0, 1, scales);
                 }
                 // the staged rows are in registers before the next item's load may overwrite the slot
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
