@@ -21,13 +21,10 @@
 // weights again (this path is bound by the per-block fp32 scaling in the vector ALUs, not by the
 // matrix cores: 4 instructions per (lhs row, weight row, block)).
 //
-// Up to 16 lhs rows with K a multiple of 256 take gemm_q4_0_small_kernel instead: the schedule of the
-// Q4_K small-batch kernel (gemv_q4k_mm.hip).  A workgroup of 8 wavefronts walks up to 4 tiles of 16
-// weight rows; wavefront w owns 8 blocks (144 bytes of every row, 16-byte aligned) of each group of 64
-// blocks and keeps the lhs operands of those 8 blocks in registers for all the tiles; the 16 x 144
-// bytes of a (group, tile) item go global -> LDS directly into a private 3-slot ring, two items
-// ahead.  Inside the 144 bytes the block offsets 18 j are compile-time, so the byte alignment of
-// every field is too.
+// Up to 16 lhs rows with K a multiple of 256 take gemm_q4_0_small_kernel instead (described at the kernel): 16
+// wavefronts per workgroup, a ring of 16-row items in LDS shared by the workgroup and loaded row by row, the lhs
+// operands of a wavefront's 8 blocks per 4096 columns in registers.  Inside a wavefront's 144 bytes of a row the block
+// offsets 18 j are compile-time, so the byte alignment of every field is too.
 #include <stdlib.h>
 
 #include <algorithm>
@@ -71,7 +68,9 @@ inline LhsQ8T lhs_q8t(void* ws, int64_t m, int64_t k) {
 
 // One 32-lane group per (padded lhs row, block); same rounding rule as the Q8_0 quantiser:
 // d = amax / 127 stored as fp16, codes = round-half-away(x / d) with the fp32 d.
-template <typename InT>
+// WORDS: the K order of gemm_q4_0_small_kernel inside a block: k-group g holds the elements whose weight nibbles share
+// dword g of the block's 16 code bytes (4 g .. 4 g + 3, then 16 + 4 g .. 16 + 4 g + 3) instead of 8 g .. 8 g + 7.
+template <typename InT, bool WORDS>
 __global__ __launch_bounds__(256) void quantize_q8_0_operand_kernel(const InT* __restrict__ x, int m, int k, int64_t ngroups,
                                                                     int8_t* __restrict__ codes, float* __restrict__ dscale,
                                                                     int32_t* __restrict__ csum) {
@@ -92,12 +91,20 @@ __global__ __launch_bounds__(256) void quantize_q8_0_operand_kernel(const InT* _
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 32);
     const int64_t tile = row >> 4;
-    const int mm = (int)(row & 15), g = l >> 3;
+    const int mm = (int)(row & 15);
+    const int g = WORDS ? (l & 15) >> 2 : l >> 3, pos = WORDS ? (l & 3) + 4 * (l >> 4) : l & 7;
     const int64_t tb = tile * nkb + kb;
-    codes[(tb * 64 + g * 16 + mm) * 8 + (l & 7)] = (int8_t)q;
+    codes[(tb * 64 + g * 16 + mm) * 8 + pos] = (int8_t)q;
     if (l == 0) {
-        dscale[tb * 16 + mm] = h2f(dh);
-        csum[tb * 16 + mm] = sum;
+        if (WORDS) {
+            // one 64-byte record per block: 16 scales as fp16, then 16 times -8 * code sum as int16 (|sum| <= 32 * 127)
+            uint16_t* rec = (uint16_t*)dscale + tb * 32;
+            rec[mm] = dh;
+            rec[16 + mm] = (uint16_t)(int16_t)(-8 * sum);
+        } else {
+            dscale[tb * 16 + mm] = h2f(dh);
+            csum[tb * 16 + mm] = sum;
+        }
     }
 }
 
@@ -225,22 +232,59 @@ __global__ __launch_bounds__(512) void gemm_q4_0_kernel(const uint8_t* __restric
 }
 
 namespace {
-constexpr int kSWaves = 8;                          // wavefronts per workgroup
-constexpr int kSBlk = 8;                            // blocks per wavefront and group: 144 bytes of a row
-constexpr int kSRow = kSBlk * Q4_0_BPB;             // 144
-constexpr int kSPieces = 16 * kSRow / 16;           // 144 pieces of 16 bytes per item
-constexpr int kSLoads = (kSPieces + 63) / 64;       // 3 load instructions per item, the last one by 16 lanes
-constexpr int kSSlot = kSPieces * 16 + 16;          // 2320: one dword of read-ahead past the last row
-constexpr int kSSlots = 3;
+constexpr int kSWaves = 16;                          // wavefronts per workgroup
+constexpr int kSGroup = 128;                         // blocks per group: 4096 columns, 2304 bytes of a row
+constexpr int kSBlk = kSGroup / kSWaves;             // 8 blocks per wavefront and group
+constexpr int kSParts = 1;                           // an item is 1 / kSParts of a group's columns of a tile's 16 rows
+constexpr int kSPartBlk = kSBlk / kSParts;           // blocks per wavefront and item
+constexpr int kSItemBlk = kSGroup / kSParts;         // blocks of an item
+constexpr int kSItemRow = kSItemBlk * Q4_0_BPB;      // bytes of a row of an item: 2304 / kSParts
+constexpr int kSPieces = kSItemRow / 16;             // 16-byte pieces of that
+constexpr int kSLoads = (kSPieces + 63) / 64;        // load instructions per wavefront and item
+constexpr int kSRowLds = kSItemRow + 16;             // rows an odd multiple of 4 dwords apart: 16 rows on 16 bank groups
+constexpr int kSSlot = 16 * kSRowLds;                // one item, 16 rows
+// Items in flight beyond the one being used.  Measured at 16 x 14336 x 4096 (the call with its lhs quantiser, us):
+// whole groups as items, 1 / 2 / 3 in flight: 13.9 / 14.4 / 15.1; half groups, 4 / 6 in flight: 15.0 / 15.8.  Every compute
+// unit asks for its data in the same microsecond, and more requests per compute unit make the first item later.
+constexpr int kSAhead = 1 * kSParts;
+constexpr int kSSlots = kSAhead + kSParts;
 constexpr int kSMaxTiles = 4;
-constexpr int kSRing = kSWaves * kSSlots * kSSlot;
-constexpr int kSLds = kSRing + kSWaves * kSMaxTiles * 4 * 64 * 4;
+constexpr int kSRing = kSSlots * kSSlot;
+constexpr int kSSums = kSWaves * kSMaxTiles * 4 * 64 * 4;     // 65536: the final sums reuse the ring's memory
+constexpr int kSScales = kSBlk * 64;                          // per wavefront: scale / code-sum records of its 8 blocks
+constexpr int kSLds = (kSRing > kSSums ? kSRing : kSSums) + kSWaves * kSScales;
+static_assert(kSItemRow % 16 == 0 && (kSRowLds / 4) % 8 == 4, "whole pieces; row stride an odd multiple of 4 dwords");
+static_assert(kSAhead * kSLoads < 64, "the waits count load instructions in six bits");
+static_assert(kSLds <= 160 * 1024, "LDS of a compute unit");
+
+typedef _Float16 q40_half2 __attribute__((ext_vector_type(2)));
+
+// wait until at most `items` items (kSLoads load instructions each) are outstanding
+__device__ __forceinline__ void q40_wait(int items) {
+    switch (items < kSAhead ? items : kSAhead) {
+        case 0: wait_vmcnt<0>(); break;
+        case 1: wait_vmcnt<kSLoads>(); break;
+        case 2: wait_vmcnt<2 * kSLoads>(); break;
+        case 3: wait_vmcnt<3 * kSLoads>(); break;
+        case 4: wait_vmcnt<4 * kSLoads>(); break;
+        case 5: wait_vmcnt<5 * kSLoads>(); break;
+        case 6: wait_vmcnt<6 * kSLoads>(); break;
+        case 7: wait_vmcnt<7 * kSLoads>(); break;
+        default: wait_vmcnt<kSAhead * kSLoads>(); break;
+    }
+}
 }  // namespace
 
+// A workgroup of 16 wavefronts walks up to 4 tiles of 16 weight rows, in groups of 4096 columns (128 blocks, 2304 bytes
+// of a row).  An item is a tile's 16 rows x one part of a group (the whole group as built).  Loading and arithmetic are cut differently:
+// wavefront w LOADS row w of an item, contiguous bytes, global -> LDS directly into a ring of items shared by the
+// workgroup (whole DRAM pages per instruction), and it COMPUTES a fixed set of 8 blocks per group of all 16 rows,
+// 8 / parts in each part, whose lhs operands it keeps in registers for all tiles; one barrier per item.  Per block: one dword of nibbles per lane (two
+// operand dwords by mask and shift), one matrix-core instruction whose accumulator input is -8 * (code sum), so that it
+// returns isum - 8 asum, and acc += float(that) * (d_w * d_a), the scale product formed from the two fp16 values.
 __global__ __launch_bounds__(64 * kSWaves) void gemm_q4_0_small_kernel(const uint8_t* __restrict__ w,
                                                                       const int8_t* __restrict__ codes,
-                                                                      const float* __restrict__ dscale,
-                                                                      const int32_t* __restrict__ csum,
+                                                                      const float* __restrict__ records,
                                                                       float* __restrict__ out, int m, int n, int k) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -248,124 +292,153 @@ __global__ __launch_bounds__(64 * kSWaves) void gemm_q4_0_small_kernel(const uin
     const int nkb = k >> 5;                       // a multiple of 8
     const int64_t row_bytes = (int64_t)nkb * Q4_0_BPB;
     const int nn = lane & 15, g = lane >> 4;
-    uint8_t* ring = smem + wave * (kSSlots * kSSlot);
+    uint8_t* ring = smem;
     const uint32_t ring_lds = lds_address(ring);
-    float* accs = (float*)(smem + kSRing);        // [kSWaves][kSMaxTiles][4][64]
     const int ntiles = (n + 15) >> 4;
     const int my_tiles = min(kSMaxTiles, (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
-    const int ngrp = (nkb + kSWaves * kSBlk - 1) / (kSWaves * kSBlk);
-    const int total = ngrp * my_tiles;
-    // group gi: blocks [64 gi + 8 wave, + 8) when they exist (K is a multiple of 256, so a share is whole or absent)
-    auto share = [&](int gi, int& first, bool& have) {
-        first = kSWaves * kSBlk * gi + kSBlk * wave;
-        have = first < nkb;
-        first = min(first, nkb - kSBlk);  // (absent: a valid address, the data is not used)
-    };
-    int prow[kSLoads], pidx[kSLoads];
+    const int ngrp = (nkb + kSGroup - 1) / kSGroup;
+    const int total = ngrp * my_tiles * kSParts;
+    // This wavefront's blocks of group gi, part p: [128 gi + (128 / parts) p + (8 / parts) wave, + 8 / parts) when they
+    // exist (K is a multiple of 256, so every run of 8 / parts <= 8 blocks is whole or absent).
+    auto first_block = [&](int gi, int p) { return kSGroup * gi + kSItemBlk * p + kSPartBlk * wave; };
+
+    // lhs operands of the wavefront's 8 blocks of the current group (one 16-row lhs tile).  The codes are a lane's own 8
+    // bytes per block; the scales and code sums are shared by 16 lanes each, and a vector load costs the compute unit's
+    // memory path 64 lanes x its width whatever the lanes ask for, so the 8 records (1 KB) go global -> LDS in one
+    // instruction and are read from there.
+    u32x2 xa[kSBlk];
+    const uint8_t* recs = smem + (kSLds - kSWaves * kSScales) + wave * kSScales;
+    const uint32_t recs_lds = lds_address(recs);
+    auto load_lhs = [&](int gi) {
 #pragma unroll
-    for (int i = 0; i < kSLoads; i++) {
-        const int p = min(lane + 64 * i, kSPieces - 1);
-        prow[i] = p / 9;
-        pidx[i] = p - prow[i] * 9;
-    }
-    auto issue = [&](int gi, int t, int slot) {
+        for (int j = 0; j < kSBlk; j++) {
+            const int kb = min(first_block(gi, j / kSPartBlk) + j % kSPartBlk, nkb - 1);  // (absent: a valid address)
+            hidden_load(xa[j], codes + ((int64_t)kb * 64 + lane) * 8);
+        }
+        // record j of the wavefront (64 bytes) is lanes 4 j .. 4 j + 3 of the load (lanes 0..31)
+        const int j = (lane >> 2) & 7;
+        const int kb = min(first_block(gi, j / kSPartBlk) + j % kSPartBlk, nkb - 1);
+        if (lane < 32) load16_to_lds((const uint8_t*)records + (int64_t)kb * 64 + 16 * (lane & 3), recs_lds);
+    };
+    long aop[kSBlk];
+    q40_half2 dah[kSBlk][2];  // block scales of lhs rows 4 g .. 4 g + 3 (they are fp16 values: the narrowing is exact)
+    int4v c8[kSBlk];          // -8 * code sum of those rows
+    auto take_lhs = [&]() {
+#pragma unroll
+        for (int j = 0; j < kSBlk; j++) {
+            tie(xa[j]);
+            aop[j] = (long)(((uint64_t)xa[j].y << 32) | xa[j].x);
+            const uint2 d = *(const uint2*)(recs + 64 * j + 8 * g), c = *(const uint2*)(recs + 64 * j + 32 + 8 * g);
+            dah[j][0] = __builtin_bit_cast(q40_half2, d.x);
+            dah[j][1] = __builtin_bit_cast(q40_half2, d.y);
+            c8[j][0] = (int)(c.x << 16) >> 16;
+            c8[j][1] = (int)c.x >> 16;
+            c8[j][2] = (int)(c.y << 16) >> 16;
+            c8[j][3] = (int)c.y >> 16;
+        }
+    };
+
+    // this wavefront's row of item (group gi, tile index t, part p) -> ring slot `slot`, row `wave`
+    auto issue = [&](int gi, int t, int p, int slot) {
         const int n0 = ((int)blockIdx.x + t * (int)gridDim.x) * 16;
-        int kb;
-        bool have;
-        share(gi, kb, have);
-        const uint8_t* base = w + (int64_t)kb * Q4_0_BPB;
+        const int kb = min(kSGroup * gi + kSItemBlk * p, nkb - 8);  // (a part past the end of K: a valid address, not used)
+        const int pieces = min(kSItemBlk, nkb - kb) * Q4_0_BPB / 16;  // 9 per 8 blocks
+        const uint8_t* src = w + (int64_t)min(n0 + wave, n - 1) * row_bytes + (int64_t)kb * Q4_0_BPB;
+        const uint32_t dst = ring_lds + slot * kSSlot + wave * kSRowLds;
 #pragma unroll
         for (int i = 0; i < kSLoads; i++) {
-            const uint8_t* src = base + (int64_t)min(n0 + prow[i], n - 1) * row_bytes + 16 * pidx[i];
+            // (lanes past a short last part read its last piece again, into row bytes nobody uses)
             if (i < kSLoads - 1 || lane < kSPieces - 64 * (kSLoads - 1))
-                load16_to_lds_once(src, ring_lds + slot * kSSlot + i * 1024);
+                load16_to_lds_once(src + 16 * min(lane + 64 * i, pieces - 1), dst + i * 1024);
         }
     };
-    int last_issued = -1, ig = 0, it_t = 0, islot = 0;
+    int last_issued = -1, ig = 0, it_t = 0, ip = 0, islot = 0;
     auto issue_next = [&]() {
-        issue(ig, it_t, islot);
+        issue(ig, it_t, ip, islot);
         last_issued++;
         islot = islot == kSSlots - 1 ? 0 : islot + 1;
-        if (++it_t == my_tiles) { it_t = 0; ig++; }
+        if (++ip == kSParts) {
+            ip = 0;
+            if (++it_t == my_tiles) { it_t = 0; ig++; }
+        }
     };
-
-    // lhs operands of the wavefront's 8 blocks of the current group
-    long aop[kSBlk];
-    float4 da[kSBlk], da8[kSBlk];  // block scales of lhs rows 4 g .. 4 g + 3, and -8 * code sum * scale
-
-    int grp = 0, ti = 0, slot = 0;
-    for (int it = 0; it < total; it++) {
-        int kb0;
-        bool have;
-        share(grp, kb0, have);
-        if (ti == 0) {
-            // (ordinary loads: the compiler's waits for them also wait for the items in flight, once per group)
-#pragma unroll
-            for (int j = 0; j < kSBlk; j++) {
-                const int64_t tb = kb0 + j;  // one 16-row lhs tile
-                aop[j] = *(const long*)(codes + (tb * 64 + lane) * 8);
-                da[j] = *(const float4*)(dscale + tb * 16 + 4 * g);
-                const int4v as = *(const int4v*)(csum + tb * 16 + 4 * g);
-                da8[j] = make_float4(-8.0f * (float)as[0] * da[j].x, -8.0f * (float)as[1] * da[j].y,
-                                     -8.0f * (float)as[2] * da[j].z, -8.0f * (float)as[3] * da[j].w);
-            }
-        }
-        while (last_issued < min(it + 2, total - 1)) issue_next();
-        wait_items<kSLoads, 0>(last_issued - it, false);
-        const uint8_t* wrow = ring + slot * kSSlot + nn * kSRow;
-        const uint32_t* l32 = (const uint32_t*)wrow;
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        if (have) {
-#pragma unroll
-            for (int j = 0; j < kSBlk; j++) {
-                // block j at byte 18 j of the row's 144: d, then 16 nibble bytes; this lane's 8 code bytes are the low
-                // nibbles of bytes 8 (g & 1) .. + 7 (g < 2) or their high nibbles
-                constexpr int kUnused = 0;
-                (void)kUnused;
-                const int qoff = Q4_0_BPB * j + 2 + 8 * (g & 1);
-                const int wi = qoff >> 2;                                  // (18 j + 2) / 4 + 2 (g & 1)
-                const uint32_t sh = (uint32_t)((Q4_0_BPB * j + 2) & 3);    // compile-time: 2, 0, 2, 0, ...
-                uint32_t lo, hi;
-                if (sh == 0) {
-                    lo = l32[wi];
-                    hi = l32[wi + 1];
-                } else {
-                    const uint32_t w0 = l32[wi], w1 = l32[wi + 1], w2 = l32[wi + 2];
-                    lo = __builtin_amdgcn_alignbyte(w1, w0, sh);
-                    hi = __builtin_amdgcn_alignbyte(w2, w1, sh);
-                }
-                if (g & 2) {
-                    lo >>= 4;
-                    hi >>= 4;
-                }
-                lo &= 0x0F0F0F0Fu;
-                hi &= 0x0F0F0F0Fu;
-                const long bop = (long)(((uint64_t)hi << 32) | lo);
-                const uint32_t dwv = l32[(Q4_0_BPB * j) >> 2] >> (8 * ((Q4_0_BPB * j) & 3));
-                const float dw = h2f((uint16_t)(dwv & 0xffffu));
-                int4v z = {0, 0, 0, 0};
-                const int4v dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[j], bop, z, 0, 0, 0);
-                // float(dot - 8 asum) * (dw * da), with the -8 asum da part formed once per group
-                acc[0] = fmaf(dw, fmaf((float)dot[0], da[j].x, da8[j].x), acc[0]);
-                acc[1] = fmaf(dw, fmaf((float)dot[1], da[j].y, da8[j].y), acc[1]);
-                acc[2] = fmaf(dw, fmaf((float)dot[2], da[j].z, da8[j].z), acc[2]);
-                acc[3] = fmaf(dw, fmaf((float)dot[3], da[j].w, da8[j].w), acc[3]);
-            }
-        }
-        float* mine = accs + ((wave * kSMaxTiles + ti) * 4) * 64 + lane;
-#pragma unroll
-        for (int r = 0; r < 4; r++) mine[r * 64] = grp == 0 ? acc[r] : mine[r * 64] + acc[r];
-        slot = slot == kSSlots - 1 ? 0 : slot + 1;
-        if (++ti == my_tiles) { ti = 0; grp++; }
+    // Every wavefront's lhs loads (hits in the L2, 72 KB per workgroup) are in the compute unit's memory path before
+    // anybody's weight loads (asking for the first item before them measured 0.1 us slower).
+    if (total > 0) {
+        load_lhs(0);
+        asm volatile("s_barrier" ::: "memory");
+        while (last_issued < min(kSAhead - 1, total - 1)) issue_next();
+        q40_wait(last_issued + 1);  // the lhs operands; the items issued after them stay in flight
+        take_lhs();
     }
+
+    float acc[kSMaxTiles][4];
+#pragma unroll
+    for (int t = 0; t < kSMaxTiles; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+
+    int it = 0, slot = 0;
+    for (int grp = 0; grp < ngrp; grp++) {
+        if (grp > 0) {
+            load_lhs(grp);
+            wait_vmcnt<0>();  // (also the items in flight: once per group of 4096 columns)
+            take_lhs();
+        }
+#pragma unroll
+        for (int ti = 0; ti < kSMaxTiles; ti++) {
+            if (ti >= my_tiles) break;
+#pragma unroll
+            for (int part = 0; part < kSParts; part++) {
+                q40_wait(last_issued - it);  // this wavefront's row of item `it` has landed
+                // every row of the item has landed, and everybody has used item it - 1, whose slot the next load overwrites
+                asm volatile("s_barrier" ::: "memory");
+                while (last_issued < min(it + kSAhead, total - 1)) issue_next();
+                const uint32_t* l32 =
+                    (const uint32_t*)(ring + slot * kSSlot + nn * kSRowLds + wave * (kSPartBlk * Q4_0_BPB));
+                if (first_block(grp, part) < nkb) {
+#pragma unroll
+                    for (int jj = 0; jj < kSPartBlk; jj++) {
+                        // block jj of the wavefront's run at byte 18 jj of it (the run starts on a dword): d, then 16 nibble
+                        // bytes; this lane's operand is dword g of them
+                        const int j = part * kSPartBlk + jj;
+                        const int wi = ((Q4_0_BPB * jj + 2) >> 2) + g;
+                        uint32_t raw;
+                        if (((Q4_0_BPB * jj + 2) & 3) == 0) raw = l32[wi];
+                        else raw = __builtin_amdgcn_alignbyte(l32[wi + 1], l32[wi], 2);
+                        const uint32_t lo = raw & 0x0F0F0F0Fu, hi = (raw >> 4) & 0x0F0F0F0Fu;
+                        const long bop = (long)(((uint64_t)hi << 32) | lo);
+                        const q40_half2 dpair = __builtin_bit_cast(q40_half2, l32[(Q4_0_BPB * jj) >> 2]);
+                        const _Float16 dw = ((Q4_0_BPB * jj) & 2) ? dpair.y : dpair.x;
+                        const int4v dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(aop[j], bop, c8[j], 0, 0, 0);
+                        // (d_w * d_a is exact in fp32; written as a fused multiply-add with 0 so that both fp16 operands
+                        // are taken as they are, v_fma_mix_f32)
+                        acc[ti][0] = fmaf((float)dot[0], fmaf((float)dw, (float)dah[j][0].x, 0.0f), acc[ti][0]);
+                        acc[ti][1] = fmaf((float)dot[1], fmaf((float)dw, (float)dah[j][0].y, 0.0f), acc[ti][1]);
+                        acc[ti][2] = fmaf((float)dot[2], fmaf((float)dw, (float)dah[j][1].x, 0.0f), acc[ti][2]);
+                        acc[ti][3] = fmaf((float)dot[3], fmaf((float)dw, (float)dah[j][1].y, 0.0f), acc[ti][3]);
+                    }
+                }
+                slot = slot == kSSlots - 1 ? 0 : slot + 1;
+                it++;
+            }
+        }
+    }
+    // add the 16 K shares: the ring's memory is free once every wavefront has read its last item
     __syncthreads();
-    for (int pr = wave; pr < my_tiles * 4; pr += kSWaves) {
-        const int t = pr >> 2, r = pr & 3;
+    float* sums = (float*)smem;  // [kSWaves][kSMaxTiles][4][64]
+#pragma unroll
+    for (int t = 0; t < kSMaxTiles; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) sums[((wave * kSMaxTiles + t) * 4 + r) * 64 + lane] = acc[t][r];
+    __syncthreads();
+    {
+        const int t = wave >> 2, r = wave & 3;  // 16 (tile, register) pairs, one per wavefront
         const int col = ((int)blockIdx.x + t * (int)gridDim.x) * 16 + nn, row = 4 * g + r;
         float v = 0.0f;
 #pragma unroll
-        for (int ww = 0; ww < kSWaves; ww++) v += accs[((ww * kSMaxTiles + t) * 4 + r) * 64 + lane];
-        if (row < m && col < n) out[(int64_t)row * n + col] = v;
+        for (int ww = 0; ww < kSWaves; ww++) v += sums[((ww * kSMaxTiles + t) * 4 + r) * 64 + lane];
+        if (t < my_tiles && row < m && col < n) out[(int64_t)row * n + col] = v;
     }
 }
 
@@ -513,18 +586,22 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
                             float* out, void* workspace, hipStream_t s) {
     const LhsQ8T p = lhs_q8t(workspace, m, k);
     const int64_t tiles = (m + 15) / 16, ngroups = tiles * 16 * (k / 32);
+    // Up to 16 lhs rows: the weights are read once and the kernel lives on HBM latency (gemm_q4_0_small_kernel).
+    const bool small = tiles == 1 && k % 256 == 0 && !kernel_disabled("q4_0_small");
     dim3 qgrid((unsigned)((ngroups * 32 + 255) / 256)), qblock(256);
-    if (lhs_dtype == QMM_F32)
-        quantize_q8_0_operand_kernel<float><<<qgrid, qblock, 0, s>>>((const float*)lhs, (int)m, (int)k, ngroups, p.codes,
-                                                                     p.scale, p.sum);
-    else
-        quantize_q8_0_operand_kernel<uint16_t><<<qgrid, qblock, 0, s>>>((const uint16_t*)lhs, (int)m, (int)k, ngroups,
-                                                                        p.codes, p.scale, p.sum);
+#define QMM_Q8_OPERAND(T_, W_)                                                                                        \
+    quantize_q8_0_operand_kernel<T_, W_><<<qgrid, qblock, 0, s>>>((const T_*)lhs, (int)m, (int)k, ngroups, p.codes, p.scale, p.sum)
+    if (lhs_dtype == QMM_F32) {
+        if (small) QMM_Q8_OPERAND(float, true);
+        else QMM_Q8_OPERAND(float, false);
+    } else {
+        if (small) QMM_Q8_OPERAND(uint16_t, true);
+        else QMM_Q8_OPERAND(uint16_t, false);
+    }
+#undef QMM_Q8_OPERAND
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    // Few lhs rows: the weights are read once and the kernel lives on HBM latency, so K is cut eight
-    // ways for more wavefronts in flight; otherwise four.
-    if (tiles == 1 && k % 256 == 0 && !kernel_disabled("q4_0_small")) {
+    if (small) {
         static int cus = 0;
         if (!cus) {
             int dev = 0;
@@ -538,11 +615,10 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
             if (e != hipSuccess) return e;
             lds_set = true;
         }
+        // tiles are dealt round robin: one workgroup per compute unit until that means more than kSMaxTiles each
         const int64_t ntiles = (n + 15) / 16;
-        const int64_t per_wg = std::min<int64_t>(kSMaxTiles, (ntiles + cus - 1) / cus);
-        const int64_t wgs = (ntiles + per_wg - 1) / per_wg;
-        gemm_q4_0_small_kernel<<<dim3((unsigned)wgs), dim3(64 * kSWaves), kSLds, s>>>(w, p.codes, p.scale, p.sum, out, (int)m, (int)n,
-                                                                                   (int)k);
+        const int64_t wgs = std::min<int64_t>(ntiles, std::max<int64_t>(cus, (ntiles + kSMaxTiles - 1) / kSMaxTiles));
+        gemm_q4_0_small_kernel<<<dim3((unsigned)wgs), dim3(64 * kSWaves), kSLds, s>>>(w, p.codes, p.scale, out, (int)m, (int)n, (int)k);
         return hipGetLastError();
     }
     if (tiles > 4 && !kernel_disabled("q4_0_wide")) {
