@@ -53,6 +53,18 @@ __device__ __forceinline__ float ubf3(uint32_t x) { float r; asm("v_cvt_f32_ubyt
 __device__ __forceinline__ float dot4u(float4 x, uint32_t q) {
     return fmaf(x.w, ubf3(q), fmaf(x.z, ubf2(q), fmaf(x.y, ubf1(q), x.x * ubf0(q))));
 }
+// The same dot with the four bytes spread into fp16 lanes first: a byte value q under a zero byte IS the fp16 subnormal
+// q * 2^-24, and v_fma_mix_f32 multiplies it with an fp32 operand exactly: two byte permutes and four mixed fused
+// multiply-adds instead of four conversions and four multiply-adds.  The result is 2^-24 times dot4u's.
+typedef _Float16 q6_half2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot4h(float4 x, uint32_t q) {
+    const q6_half2 p01 = __builtin_bit_cast(q6_half2, __builtin_amdgcn_perm(q, q, 0x0c010c00u));
+    const q6_half2 p23 = __builtin_bit_cast(q6_half2, __builtin_amdgcn_perm(q, q, 0x0c030c02u));
+    float u = fmaf((float)p01.x, x.x, 0.0f);  // (a fused multiply-add with 0: the mixed instruction has no plain multiply)
+    u = fmaf((float)p01.y, x.y, u);
+    u = fmaf((float)p23.x, x.z, u);
+    return fmaf((float)p23.y, x.w, u);
+}
 __device__ __forceinline__ float sbyte(uint32_t x, int shift) { return (float)((int)(x << (24 - shift)) >> 24); }
 
 }  // namespace
@@ -415,8 +427,9 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             x[mi][it][3] = load4(aq, 96);
             const AT* ag = ar + 16 * t;
             const float4 y0 = load4(ag, 0), y1 = load4(ag, 4), y2 = load4(ag, 8), y3 = load4(ag, 12);
-            os[mi][it] = -32.0f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
-                                   ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
+            // (in units of 2^-24 like the dots below: -32 * 2^-24 = -2^-19; the row's sum is scaled back at its end)
+            os[mi][it] = -0x1p-19f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
+                                      ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
             keep += os[mi][it];
         }
     }
@@ -459,10 +472,10 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             const float cg = sbyte(j < 4 ? s0 : s1, 8 * (j & 3));
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) {
-                float u = c1 * dot4u(x[mi][it][0], q1);
-                u = fmaf(c2, dot4u(x[mi][it][1], q2), u);
-                u = fmaf(c3, dot4u(x[mi][it][2], q3), u);
-                u = fmaf(c4, dot4u(x[mi][it][3], q4), u);
+                float u = c1 * dot4h(x[mi][it][0], q1);
+                u = fmaf(c2, dot4h(x[mi][it][1], q2), u);
+                u = fmaf(c3, dot4h(x[mi][it][2], q3), u);
+                u = fmaf(c4, dot4h(x[mi][it][3], q4), u);
                 u = fmaf(cg, os[mi][it], u);
                 v[mi] = lv[it] ? fmaf(d, u, v[mi]) : v[mi];  // (a select: what a missing super-block's lanes read is arbitrary)
             }
@@ -470,7 +483,7 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
             const float sum = wave_sum_dpp_lane63(v[mi]);
-            if (lane == 63) park[ri * MT + mi] = sum;
+            if (lane == 63) park[ri * MT + mi] = sum * 0x1p24f;
         }
     }
     if (wpr > 1) __syncthreads();  // (every wavefront gets here: no early exit above)
@@ -497,7 +510,7 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
         if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipGetLastError();
         cus = prop.multiProcessorCount;
     }
-    const int pc_env = 0, pc = 3;
+    const int pc_env = 0, pc = 3;  // (workgroups per compute unit of the kernels below the vocabulary one)
     const bool lanes_off = kernel_disabled("q6k_lanes");
     // Rows of whole 16-byte pieces (K a multiple of 2048, up to 16384) and enough of them: the kernel with the rows
     // global -> LDS and the activations in registers, one or two lhs rows per pass over the weights (up to 16 rows:
@@ -506,7 +519,10 @@ hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, i
     const int wpr = nblk <= 16 ? 1 : nblk <= 32 ? 2 : 4;
     const int64_t need_parts = (int64_t)cus * 4 * 8;  // below 8 row parts per wavefront of a one-workgroup-per-CU grid the row-at-a-time kernel is faster
     if (k % 2048 == 0 && nblk <= 64 && !((uintptr_t)w & 15) && n * wpr >= need_parts && !lanes_off) {
-        const int ring = 3;
+        // Ring slots and workgroups per compute unit, 128256 x 4096 with one lhs row (us): 3 / 3: 77.9, 2 / 3: 77.8, 2 / 4: 76.9,
+        // 3 / 2: 81.9, 4 / 2: 81.5: the wavefronts per SIMD count (the decode of a row is a chain of LDS reads), a second row
+        // in flight does not.
+        const int ring = m == 1 ? 2 : 3, pc = m == 1 ? 4 : 3;
         const int bpw = nblk / wpr;                                  // 8 .. 16, even
         const int pieces = (12 + bpw * Q6_K_BPB + 15) / 16;
         const int l = (pieces + 63) / 64;                            // 2 .. 4 load instructions per row part
