@@ -132,6 +132,38 @@ def test_prefill_configuration_full_size(kind):
         check_all(other, a.double(), w32, f"{kind} prefill {m}x{n}x{k}, static scratch")
 
 
+@pytest.mark.parametrize("kind", ["Q4_K", "GPTQ"])
+@pytest.mark.parametrize("m,n,k", [(512, 4096, 4096), (512, 4096, 14336), (512, 14336, 4096), (64, 4096, 4096), (200, 1024, 4096)])
+def test_mid_size_prefill_full_size(kind, m, n, k):
+    """A layer's projections with a few hundred lhs rows (a prefill chunk, a wide decode batch): the kernels below the plane
+    GEMM's thresholds, with K cut across workgroups where the tiles are few.  Sampled columns against the oracle's fp64
+    sums, every output against the fp64 product on the GPU."""
+    w, gen = weights(500 + m + n % 89, n, k)
+    a = torch.randn((m, k), dtype=torch.float32, device=DEV, generator=gen).to(torch.bfloat16)
+    a_np = a.float().cpu().numpy()
+    if kind == "Q4_K":
+        packed = quantize(QE.Q4_K, w)
+        got = qmatmul(QE.Q4_K, None, a, packed)
+        idx = np.sort(np.random.default_rng(m + k).choice(n, 24, replace=False))
+        tidx = torch.from_numpy(idx).to(DEV)
+        truth = O.matmul_f64(O.Q4_K, a_np, packed[tidx].cpu().numpy())
+        w32 = dequantize(QE.Q4_K, packed)
+    else:
+        cfg = QuantizationConfig()
+        qw, sc, qz, gi = quantize_gptq(w)
+        got = qmatmul(QE.GPTQ, cfg, a, qw, sc, qz, gi)
+        words = np.sort(np.random.default_rng(m + k).choice(n // 8, 3, replace=False))
+        idx = (words[:, None] * 8 + np.arange(8)[None, :]).reshape(-1)
+        tidx = torch.from_numpy(idx).to(DEV)
+        truth = O.matmul_gptq(a_np, qw[:, tidx].cpu().numpy(), sc[:, tidx].cpu().numpy().view(np.uint16),
+                              np.ascontiguousarray(qz.cpu().numpy()[:, words]), f64=True)
+        w32 = dequantize(QE.GPTQ, qw, sc, qz, gi, config=cfg)
+    assert got.shape == (m, n)
+    ok = O.isclose(got[:, tidx].cpu().numpy(), truth, RTOL, ATOL)
+    assert ok.all(), f"{kind} {m}x{n}x{k}: {(~ok).sum()}/{ok.size} sampled outputs differ from the oracle"
+    check_all(got, a.double(), w32, f"{kind} mid-size prefill {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("m,n,k,bf16", [(16, 14336, 4096, False), (16, 14336, 4096, True), (4, 4096, 14336, False),
                                         (48, 4096, 14336, True), (2, 1024, 4096, True)])
 def test_gptq_small_batch_full_size(m, n, k, bf16):
