@@ -352,7 +352,10 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
             }
         }
         // the slot of item it - 1 is free: its reads fed matrix products whose results are already stored
-        while (last_issued < min(it + 2, total - 1)) issue_next();
+        // (items in flight beyond the one in use: with up to four lhs rows one measures faster than two, 62.2 against 63.3 us for
+        // the seven projections, as in the other small-batch kernels; with eight rows two do, 86.0 against 86.6)
+        constexpr int kAhead = INLINE && MROWS <= 4 ? 1 : 2;
+        while (last_issued < min(it + kAhead, total - 1)) issue_next();
         // item `it` has landed when only the younger loads are outstanding: later items and, if it was
         // issued after this item, the next group's raw lhs
         wait_items<kLoads, NX>(last_issued - it, INLINE && x_after >= it);
