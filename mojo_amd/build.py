@@ -37,6 +37,7 @@ PER_FILE_FLAGS = {
     "gemv_q4k_lanes.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
     "gemv_q4k_mm.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
     "gemm_q4_0.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=12"],
+    "gemv_q4_0.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"],
 }
 
 
