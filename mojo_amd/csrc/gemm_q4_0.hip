@@ -276,12 +276,13 @@ __device__ __forceinline__ void q40_wait(int items) {
 }  // namespace
 
 // A workgroup of 16 wavefronts walks up to 4 tiles of 16 weight rows, in groups of 4096 columns (128 blocks, 2304 bytes
-// of a row).  An item is a tile's 16 rows x one part of a group (the whole group as built).  Loading and arithmetic are cut differently:
-// wavefront w LOADS row w of an item, contiguous bytes, global -> LDS directly into a ring of items shared by the
-// workgroup (whole DRAM pages per instruction), and it COMPUTES a fixed set of 8 blocks per group of all 16 rows,
-// 8 / parts in each part, whose lhs operands it keeps in registers for all tiles; one barrier per item.  Per block: one dword of nibbles per lane (two
-// operand dwords by mask and shift), one matrix-core instruction whose accumulator input is -8 * (code sum), so that it
-// returns isum - 8 asum, and acc += float(that) * (d_w * d_a), the scale product formed from the two fp16 values.
+// of a row).  An item is a tile's 16 rows x one part of a group (the whole group as built).  Loading and arithmetic are
+// cut differently: wavefront w LOADS row w of an item, contiguous bytes, global -> LDS directly into a ring of items
+// shared by the workgroup (whole DRAM pages per instruction), and it COMPUTES a fixed set of 8 blocks per group of all
+// 16 rows, 8 / parts in each part, whose lhs operands it keeps in registers for all tiles; one barrier per item.  Per
+// block: one dword of nibbles per lane (two operand dwords by mask and shift), one matrix-core instruction whose
+// accumulator input is -8 * (code sum), so that it returns isum - 8 asum, and acc += float(that) * (d_w * d_a), the
+// scale product formed from the two fp16 values.
 __global__ __launch_bounds__(64 * kSWaves) void gemm_q4_0_small_kernel(const uint8_t* __restrict__ w,
                                                                       const int8_t* __restrict__ codes,
                                                                       const float* __restrict__ records,
