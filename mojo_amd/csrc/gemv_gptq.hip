@@ -127,16 +127,19 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
     if (m > 4 || group % 32) return hipSuccess;
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const size_t lds = ((size_t)kWaves * mt * group + (size_t)kWaves * mt * 64) * 4;
-    if (lds > 64 * 1024) return hipSuccess;
+    if (lds > (size_t)kLdsPerCu) return hipSuccess;
     dim3 grid((unsigned)((n + 63) / 64)), block(64 * kWaves);
 #define QMM_GPTQ_GO(MT_, ROWS_)                                                                                       \
     do {                                                                                                              \
-        if (a_dtype == QMM_F32)                                                                                       \
+        if (a_dtype == QMM_F32) {                                                                                     \
+            if (lds > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols_kernel<MT_, ROWS_, float>>();                    \
             gemv_gptq_cols_kernel<MT_, ROWS_, float><<<grid, block, lds, s>>>(qweight, scales, qzeros, (const float*)a, \
                                                                              out, m, (int)n, (int)k, group, ldo);    \
-        else                                                                                                          \
+        } else {                                                                                                      \
+            if (lds > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols_kernel<MT_, ROWS_, uint16_t>>();                 \
             gemv_gptq_cols_kernel<MT_, ROWS_, uint16_t><<<grid, block, lds, s>>>(                                     \
                 qweight, scales, qzeros, (const uint16_t*)a, out, m, (int)n, (int)k, group, ldo);                     \
+        }                                                                                                             \
     } while (0)
 #define QMM_GPTQ_MT(ROWS_)                  \
     do {                                    \
