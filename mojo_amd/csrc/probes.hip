@@ -7,6 +7,8 @@
 //   kind 1  1.0 everywhere
 //   kind 2  random values in +-[1, 4) on both sides (dense activations x dense weights)
 //   kind 3  random values in +-[1, 4) x random integers 0..945 (what the plane GEMMs multiply: narrowed activations x sc * q)
+// Kinds 4 and 5 are kinds 0 and 2 with v_mfma_f32_16x16x32_f16 (the small-batch kernels' instruction: half the products
+// per instruction), sixteen independent-enough instructions a round on four accumulator chains as well.
 #include "qmm_internal.h"
 
 namespace qmm {
@@ -77,8 +79,44 @@ __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(float* __restrict__ 
     out[t] = c0[0] + c1[1] + c2[2] + c3[3];
 }
 
+__global__ __launch_bounds__(512, 1) void mfma_probe16_kernel(float* __restrict__ out, int kind, int iters) {
+    typedef float probe_float4 __attribute__((ext_vector_type(4)));
+    union {
+        uint32_t u[4];
+        probe_half8 h;
+    } a[4], b[4];
+    const uint32_t t = blockIdx.x * 512 + threadIdx.x;
+    for (int j = 0; j < 4; j++)
+        for (int i = 0; i < 4; i++) {
+            const uint32_t ra = probe_hash(t * 64 + j * 8 + i), rb = probe_hash(t * 64 + j * 8 + i + 4);
+            a[j].u[i] = kind == 5 ? (ra & 0x87ff87ffu) | 0x3C003C00u : 0u;
+            b[j].u[i] = kind == 5 ? (rb & 0x87ff87ffu) | 0x3C003C00u : 0u;
+        }
+    probe_float4 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            c0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[j].h, c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j].h, b[(j + 1) & 3].h, c1, 0, 0, 0);
+            c2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(j + 1) & 3].h, b[j].h, c2, 0, 0, 0);
+            c3 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(j + 2) & 3].h, b[(j + 3) & 3].h, c3, 0, 0, 0);
+        }
+        if ((i & 63) == 63) {  // keep the sums finite
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                c0[r] *= 1e-6f;
+                c1[r] *= 1e-6f;
+                c2[r] *= 1e-6f;
+                c3[r] *= 1e-6f;
+            }
+        }
+    }
+    out[t] = c0[0] + c1[1] + c2[2] + c3[3];
+}
+
 hipError_t launch_mfma_probe(float* out, int workgroups, int kind, int iters, hipStream_t s) {
-    mfma_probe_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, kind, iters);
+    if (kind >= 4) mfma_probe16_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, kind, iters);
+    else mfma_probe_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, kind, iters);
     return hipGetLastError();
 }
 
