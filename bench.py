@@ -726,7 +726,8 @@ def mfma_probe(seconds: float = 0.12):
     out = torch.empty((cu.value * 512,), dtype=torch.float32, device="cuda:0")
     s = torch.cuda.current_stream().cuda_stream
     iters, res = 2000, {}
-    for kind, name in ((0, "zeros"), (2, "random_x_random"), (3, "random_x_integers_0_945"), (4, "zeros_16x16x32"), (5, "random_x_random_16x16x32")):
+    for kind, name in ((0, "zeros"), (2, "random_x_random"), (3, "random_x_integers_0_945"), (4, "zeros_16x16x32"), (5, "random_x_random_16x16x32"),
+                       (6, "random_x_random_bf16")):
         flops = C.c_int64(0)
 
         def launch():

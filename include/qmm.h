@@ -88,7 +88,8 @@ int qmm_read_probe(const void* buf, int64_t bytes, void* stream);
  * registers (no memory traffic), one workgroup of 8 wavefronts on every compute unit, `iters` rounds of 16 instructions per
  * wavefront.  `kind` selects the operand data: 0 zeros, 1 ones, 2 random values in +-[1, 4) on both sides, 3 such values
  * against random integers 0..945 (what the plane GEMMs multiply); 4 and 5 are kinds 0 and 2 with v_mfma_f32_16x16x32_f16,
- * the instruction of the small-batch kernels.  Timing it gives the matrix-core rate this part sustains
+ * the instruction of the small-batch kernels; 6 is kind 2 with v_mfma_f32_32x32x16_bf16 on bf16 values.  Timing it gives the
+ * matrix-core rate this part sustains
  * on that kind of data, which for dense random data is well below the published peak (the part settles at a lower clock).
  * `out` receives 512 floats per compute unit (checksums; qmm_device_info gives the count), *flops the operations of the
  * launch.  No counterpart in the reference, whose harness times whole kernels (stdlib/docs/bencher/Bench.md).

@@ -114,8 +114,45 @@ __global__ __launch_bounds__(512, 1) void mfma_probe16_kernel(float* __restrict_
     out[t] = c0[0] + c1[1] + c2[2] + c3[3];
 }
 
+// kind 6: v_mfma_f32_32x32x16_bf16 on dense random bf16 values in +-[1, 4)
+__global__ __launch_bounds__(512, 1) void mfma_probe_bf16_kernel(float* __restrict__ out, int iters) {
+    typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+    union {
+        uint32_t u[4];
+        probe_bf16x8 h;
+    } a[4], b[4];
+    const uint32_t t = blockIdx.x * 512 + threadIdx.x;
+    for (int j = 0; j < 4; j++)
+        for (int i = 0; i < 4; i++) {
+            const uint32_t ra = probe_hash(t * 64 + j * 8 + i), rb = probe_hash(t * 64 + j * 8 + i + 4);
+            a[j].u[i] = (ra & 0x80ff80ffu) | 0x3F803F80u;
+            b[j].u[i] = (rb & 0x80ff80ffu) | 0x3F803F80u;
+        }
+    probe_float16 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j].h, b[j].h, c0, 0, 0, 0);
+            c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j].h, b[(j + 1) & 3].h, c1, 0, 0, 0);
+            c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j + 1) & 3].h, b[j].h, c2, 0, 0, 0);
+            c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(j + 2) & 3].h, b[(j + 3) & 3].h, c3, 0, 0, 0);
+        }
+        if ((i & 63) == 63) {  // keep the sums finite
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                c0[r] *= 1e-6f;
+                c1[r] *= 1e-6f;
+                c2[r] *= 1e-6f;
+                c3[r] *= 1e-6f;
+            }
+        }
+    }
+    out[t] = c0[0] + c1[1] + c2[2] + c3[3];
+}
+
 hipError_t launch_mfma_probe(float* out, int workgroups, int kind, int iters, hipStream_t s) {
-    if (kind >= 4) mfma_probe16_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, kind, iters);
+    if (kind == 6) mfma_probe_bf16_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, iters);
+    else if (kind >= 4) mfma_probe16_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, kind, iters);
     else mfma_probe_kernel<<<dim3((unsigned)workgroups), dim3(512), 0, s>>>(out, kind, iters);
     return hipGetLastError();
 }

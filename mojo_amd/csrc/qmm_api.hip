@@ -219,12 +219,12 @@ int qmm_read_probe(const void* buf, int64_t bytes, void* stream) {
 
 int qmm_mfma_probe(void* out, int64_t out_bytes, int kind, int iters, int64_t* flops, void* stream) {
     if (!out || !flops) return fail(QMM_ERR_INVALID, "qmm_mfma_probe: null pointer");
-    if (kind < 0 || kind > 5 || iters < 1 || iters > (1 << 24)) return fail(QMM_ERR_INVALID, "qmm_mfma_probe: kind 0..5, iters 1..2^24");
+    if (kind < 0 || kind > 6 || iters < 1 || iters > (1 << 24)) return fail(QMM_ERR_INVALID, "qmm_mfma_probe: kind 0..6, iters 1..2^24");
     int32_t cus = 0;
     if (int rc = qmm_device_info(&cus, nullptr)) return rc;
     if (!aligned(out, 4) || out_bytes < (int64_t)cus * 512 * 4)
         return fail(QMM_ERR_INVALID, "qmm_mfma_probe: out must hold 512 floats per compute unit (%lld bytes)", (long long)cus * 512 * 4);
-    *flops = (int64_t)cus * 8 * iters * 16 * (kind >= 4 ? 2ll * 16 * 16 * 32 : 2ll * 32 * 32 * 16);
+    *flops = (int64_t)cus * 8 * iters * 16 * (kind == 4 || kind == 5 ? 2ll * 16 * 16 * 32 : 2ll * 32 * 32 * 16);
     return hip_status(qmm::launch_mfma_probe((float*)out, cus, kind, iters, (hipStream_t)stream), "qmm_mfma_probe");
 }
 
