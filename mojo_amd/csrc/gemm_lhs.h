@@ -75,10 +75,13 @@ constexpr int kLhsOrderQ4K = 0, kLhsOrderGPTQ = 1, kLhsOrderQ4K16 = 2, kLhsOrder
 // columns instead of into asum, as `next` further blocks of 256 operand positions: the 32 positions of super-block b are
 // 8 hi, 8 lo, 8 hi, 8 lo parts of its sums (what multiplies a weight-side block of 8 hi, 8 hi, 8 lo, 8 lo table parts to the
 // full hi/lo product), zeros beyond the last super-block.
+// twin_rows > 0 (fp32 lhs): the residual plane is rows twin_rows .. 2 twin_rows - 1 of ONE lhs of twice the rows (a16_lo =
+// a16 + twin_rows * lda), which one pass of a GEMM multiplies like any other rows; their sub-block sums are written as zeros
+// (the min term belongs to the hi rows, which carry the full sums) and their row scales repeat those of the hi rows.
 template <typename AT, int ORDER>
 __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
                                              _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum, float* __restrict__ inv,
-                                             int64_t lda = 0, int next = 0) {
+                                             int64_t lda = 0, int next = 0, int twin_rows = 0) {
     if (lda == 0) lda = k;
     __shared__ uint32_t wmax[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -111,7 +114,10 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
     int e = (int)((mxb >> 23) & 0xffu) - 127;
     if (e < -100 || e > 127) e = 9;  // zero, denormal or non-finite row: leave unscaled
     const float s = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
-    if (tid == 0) inv[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+    if (tid == 0) {
+        inv[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+        if (twin_rows > 0) inv[twin_rows + row] = inv[row];
+    }
     auto emit = [&](int i, float x0, float x1, float x2, float x3) __attribute__((always_inline)) {
         const float h0 = h2f(f2h(x0)), h1 = h2f(f2h(x1)), h2 = h2f(f2h(x2)), h3 = h2f(f2h(x3));
         const int kl = i & 63;
@@ -157,6 +163,10 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
                 _Float16* as = asum + ((int64_t)row * (k >> 8) + blk) * 16;
                 as[j] = (_Float16)sh;
                 as[8 + j] = (_Float16)(sum - sh);
+                if (twin_rows > 0) {
+                    _Float16* az = asum + ((int64_t)(twin_rows + row) * (k >> 8) + blk) * 16;
+                    az[j] = az[8 + j] = (_Float16)0.0f;
+                }
             }
         }
     };
@@ -175,8 +185,8 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
 template <typename AT, int ORDER>
 __global__ __launch_bounds__(256) void prep_lhs_kernel(const AT* __restrict__ a, int k, _Float16* __restrict__ a16,
                                                        _Float16* __restrict__ a16_lo, _Float16* __restrict__ asum,
-                                                       float* __restrict__ inv) {
-    prep_lhs_row<AT, ORDER>((int)blockIdx.x, a, k, a16, a16_lo, asum, inv);
+                                                       float* __restrict__ inv, int twin_rows) {
+    prep_lhs_row<AT, ORDER>((int)blockIdx.x, a, k, a16, a16_lo, asum, inv, 0, 0, twin_rows);
 }
 
 struct LhsPlanes {
@@ -212,15 +222,17 @@ inline LhsPlanes lhs_planes(void* workspace, int lhs_dtype, int64_t m, int64_t k
     return p;
 }
 
+// twin: an fp32 lhs whose planes `p` were laid out as ONE plane of 2 m rows (see prep_lhs_row)
 template <int ORDER>
 inline hipError_t launch_prep_lhs(const void* lhs, int lhs_dtype, int64_t m, int64_t k, const LhsPlanes& p,
-                                  hipStream_t s) {
+                                  hipStream_t s, bool twin = false) {
     if (lhs_dtype == QMM_F32)
-        prep_lhs_kernel<float, ORDER><<<dim3((unsigned)m), dim3(256), 0, s>>>((const float*)lhs, (int)k, p.a16, p.a16_lo,
-                                                                            p.asum, p.inv);
+        prep_lhs_kernel<float, ORDER><<<dim3((unsigned)m), dim3(256), 0, s>>>((const float*)lhs, (int)k, p.a16,
+                                                                            twin ? p.a16 + m * k : p.a16_lo, p.asum, p.inv,
+                                                                            twin ? (int)m : 0);
     else
         prep_lhs_kernel<uint16_t, ORDER><<<dim3((unsigned)m), dim3(256), 0, s>>>((const uint16_t*)lhs, (int)k, p.a16,
-                                                                               nullptr, p.asum, p.inv);
+                                                                               nullptr, p.asum, p.inv, 0);
     return hipGetLastError();
 }
 

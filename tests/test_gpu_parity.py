@@ -728,13 +728,21 @@ def test_q4_k_gemm_bf16_lhs(m, n, k):
     assert_close(got, truth, f"Q4_K GEMM {m}x{n}x{k} vs fp64 truth")
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 128, 512), (33, 64, 256)])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 512), (33, 64, 256), (32, 4096, 4096), (17, 1000, 4096), (100, 2050, 1024),
+                                   (65, 520, 2560)])
 def test_q4_k_gemm_f32_lhs(m, n, k):
+    """fp32 lhs: hi and residual fp16 planes.  From 1024 columns of K on (tiles cut into K shares) the residual plane is the
+    second half of the rows of one lhs and a single pass multiplies both; shorter K takes two passes.  Rows of very different
+    magnitude (the row scales of both halves), ragged m and n."""
     w, a = synth(12, n, k, m)
+    a *= np.logspace(-3, 3, m, dtype=np.float32)[:, None]
     wq = O.quantize(O.Q4_K, w)
-    want = O.matmul_f32(O.Q4_K, a, wq)
-    got = qmatmul(QE.Q4_K, None, gpu(a), gpu(wq))
-    assert_close(got, want, f"Q4_K GEMM fp32 lhs {m}x{n}x{k}")
+    truth = O.matmul_f64(O.Q4_K, a, wq)
+    got = qmatmul(QE.Q4_K, None, gpu(a), gpu(wq)).cpu().numpy()
+    scale = np.abs(truth).max(axis=1, keepdims=True)
+    assert np.all(np.abs(got - truth) <= 1e-4 * scale + 1e-3 * np.abs(truth)), f"Q4_K GEMM fp32 lhs {m}x{n}x{k}"
+    one = qmatmul(QE.Q4_K, None, gpu(a[:1] / np.abs(a[:1]).max()), gpu(wq))
+    assert_close(one, O.matmul_f32(O.Q4_K, a[:1] / np.abs(a[:1]).max(), wq), f"Q4_K fp32 lhs, first row alone {n}x{k}")
 
 
 @pytest.mark.parametrize("m,n,k,bf16", [(512, 16384, 512, True), (500, 18600, 768, True), (300, 32768, 256, True),
