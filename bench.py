@@ -769,7 +769,7 @@ SWEEP_SHAPES = [(4096, 11008), (11008, 4096), (32000, 4096), (5120, 5120), (3584
 
 
 def sweep_main(gen) -> int:
-    """Q4_K over shapes the dispatch thresholds were not fitted to: decode rows 1 / 4 / 16 as a fraction of the plain read of the
+    """Q4_K over shapes the dispatch thresholds were not fitted to: lhs rows 1 / 4 / 16 / 64 (fp32) as a fraction of the plain read of the
     same weight bytes (cold: copies rotated beyond the 256 MB cache), prefill rows 512 / 2048 (bf16 lhs) as a fraction of the
     2.5 PFLOP/s peak.  One JSON line; a cliff in the dispatch shows as a fraction far below its neighbours'."""
     out = {}
@@ -780,7 +780,7 @@ def sweep_main(gen) -> int:
         dev_s, _ = time_graphs([capture([ReadProbe(w) for w in ws])], 20, 3)
         read_us = dev_s * 1e6 / (20 * copies)
         row = {"plain_read_us": round(read_us, 2), "plain_read_GB/s": round(w0.numel() / read_us / 1e3, 1)}
-        for m in (1, 4, 16):
+        for m in (1, 4, 16, 64):
             a = torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen)
             dev_s, _ = time_graphs([capture([Gemv(QE.Q4_K, w, a) for w in ws])], 20, 3)
             us = dev_s * 1e6 / (20 * copies)
