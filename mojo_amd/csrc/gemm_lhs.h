@@ -159,6 +159,10 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
                 _Float16* as = a16 + (int64_t)row * lda + k + blk * 32;
                 as[j] = as[16 + j] = (_Float16)sh;
                 as[8 + j] = as[24 + j] = (_Float16)(sum - sh);
+                if (twin_rows > 0) {
+                    _Float16* az = a16 + (int64_t)(twin_rows + row) * lda + k + blk * 32;
+                    az[j] = az[8 + j] = az[16 + j] = az[24 + j] = (_Float16)0.0f;
+                }
             } else {
                 _Float16* as = asum + ((int64_t)row * (k >> 8) + blk) * 16;
                 as[j] = (_Float16)sh;
@@ -179,7 +183,10 @@ __device__ __forceinline__ void prep_lhs_row(int row, const AT* __restrict__ a, 
     } else {
         for (int i = tid * 4; i < k; i += 1024) emit(i, load_f32(ar, i) * s, load_f32(ar, i + 1) * s, load_f32(ar, i + 2) * s, load_f32(ar, i + 3) * s);
     }
-    for (int i = (k >> 8) * 32 + tid; i < next * 256; i += 256) a16[(int64_t)row * lda + k + i] = (_Float16)0.0f;
+    for (int i = (k >> 8) * 32 + tid; i < next * 256; i += 256) {
+        a16[(int64_t)row * lda + k + i] = (_Float16)0.0f;
+        if (twin_rows > 0) a16[(int64_t)(twin_rows + row) * lda + k + i] = (_Float16)0.0f;
+    }
 }
 
 template <typename AT, int ORDER>

@@ -250,14 +250,14 @@ template <int ENC, typename AT>
 __global__ __launch_bounds__(256) void planes_prologue_kernel(const uint8_t* __restrict__ w, int nblk, int nblk_tile, int tiles_n128,
                                                               uint8_t* __restrict__ planes, float* __restrict__ dtab,
                                                               uint8_t* __restrict__ mtab, int conv, const AT* __restrict__ a, int k,
-                                                              int lhs_ext, int lhs_rows, LhsPlanes p, SplitTiles z) {
+                                                              int lhs_ext, int lhs_rows, LhsPlanes p, SplitTiles z, int twin_rows) {
     const int b = (int)blockIdx.x;
     if (b < conv) {
         const int t = b >> 2, rb = t / tiles_n128;
         planes_from_kquant<ENC>(t - rb * tiles_n128, rb, b & 3, w, z.n, nblk, nblk_tile, planes, dtab, mtab);
     } else if (b < conv + lhs_rows) {
         // (lhs_ext: extension blocks behind each lhs row, as many as the planes have when the wide GEMM follows, else none)
-        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv, (int64_t)k + lhs_ext * 256, lhs_ext);
+        prep_lhs_row<AT, kLhsOrderTile>(b - conv, a, k, p.a16, p.a16_lo, p.asum, p.inv, (int64_t)k + lhs_ext * 256, lhs_ext, twin_rows);
     } else {
         const int e = b - conv - lhs_rows;
         if (z.part) zero_flat(z.out, z.part, (int64_t)z.m * z.n, e);
@@ -1144,7 +1144,7 @@ __global__ __launch_bounds__(256) void gptq_planes_prologue_kernel(const uint32_
     }
 }
 
-bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
+bool gemm_planes_wanted(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (kernel_disabled("kquant_planes") || k % 256 || k < 256) return false;
     if (encoding == QMM_Q4_K) {
         // From three row tiles on (and 160 tiles of 256 x 256) the conversion pass costs less than the plane GEMM gains on the
@@ -1160,7 +1160,14 @@ bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     // 64 rows 88 us, the planes 118 us; beyond 64 rows neither encoding has a kernel that takes more than four rows a pass).
     // Q5_K with 33 to 64 rows where that kernel does not apply (K not a multiple of 512 or beyond 32768) also comes here.
     if (encoding == QMM_Q5_K && m > 32 && (k % 512 || k > 32768 || kernel_disabled("q5k_mm"))) return true;
-    return m > 64;
+    // The small-batch kernels take 16 bf16 or 8 fp32 rows a pass (up to 64 rows), the planes any number in one (an fp32 lhs as
+    // twice the rows) behind a conversion that costs about as much as the passes do per weight.  Microseconds of one pass / of the
+    // planes at 65 rows: 4096 x 4096: Q5_K bf16 9.6 / 35, fp32 13.5 / 46; Q6_K bf16 12.5 / 55, fp32 12.9 / 69; 14336 x 4096: Q5_K
+    // bf16 16.8 / 85, fp32 20.4 / 94; Q6_K bf16 21.6 / 134, fp32 20.8 / 142.
+    const int per_pass = lhs_dtype == QMM_F32 ? 8 : 16;
+    const int64_t passes = (m + per_pass - 1) / per_pass;
+    const bool small = n * k <= ((int64_t)32 << 20);
+    return m > 64 || passes >= (encoding == QMM_Q5_K ? (small ? 4 : 5) : (small ? 6 : 7));
 }
 
 // Very few tiles, or few on a long K: the 256 x 128 plane kernels (one plane, and Q6_K's two) cut every tile in four K quarters (bf16 lhs: one pass), which
@@ -1185,11 +1192,28 @@ int64_t quarter_part_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, in
     return quarter_mode(encoding, lhs_dtype, m, n, k) ? (m * n * 4 + 255) / 256 * 256 : 0;
 }
 
+// An fp32 lhs of up to 256 rows goes through the GEMM as ONE lhs of twice the rows, hi plane on top of residual plane, like a
+// bf16 lhs (one pass, every way of cutting few tiles along K open to it); the GEMM writes into the workspace and the pass
+// that adds K quarters adds the two halves of the rows as well.  Two passes, the second one over whole tiles onto the
+// first one's result, had cost 4096 x 4096 with 65 fp32 rows 110 us (Q5_K) and 176 us (Q6_K) against 31 and 56 us for bf16 rows.
+bool planes_twin(int lhs_dtype, int64_t m) { return lhs_dtype == QMM_F32 && m <= 256 && !kernel_disabled("planes_twin_rows"); }
+// rows and type that the GEMM sees
+int64_t gemm_rows(int lhs_dtype, int64_t m) { return planes_twin(lhs_dtype, m) ? 2 * m : m; }
+int gemm_dtype(int lhs_dtype, int64_t m) { return planes_twin(lhs_dtype, m) ? QMM_BF16 : lhs_dtype; }
+// what follows the lhs planes (and, inside qmm_matmul, the weight planes) in the workspace: the second buffer of the quarter
+// mode, or, for twin rows, the GEMM's result (2 m x n, whole) and that second buffer right behind it
+int64_t planes_tail_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    if (!planes_twin(lhs_dtype, m)) return quarter_part_bytes(encoding, lhs_dtype, m, n, k);
+    return (2 * m * n * 4 * (quarter_mode(encoding, QMM_BF16, 2 * m, n, k) ? 2 : 1) + 255) / 256 * 256;
+}
+
 int64_t gemm_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
-    const int64_t nblk_tile = blocks_per_tile(encoding, m, n, k);
-    const int64_t lhs = (lhs_planes(nullptr, lhs_dtype, m, k, TM, nblk_tile * 256).bytes + 255) / 256 * 256;
-    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile).bytes + quarter_part_bytes(encoding, lhs_dtype, m, n, k);
+    const int64_t me = gemm_rows(lhs_dtype, m);
+    const int dte = gemm_dtype(lhs_dtype, m);
+    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, me, n);
+    const int64_t nblk_tile = blocks_per_tile(encoding, me, n, k);
+    const int64_t lhs = (lhs_planes(nullptr, dte, me, k, TM, nblk_tile * 256).bytes + 255) / 256 * 256;
+    return lhs + plane_space(nullptr, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile).bytes + planes_tail_bytes(encoding, lhs_dtype, m, n, k);
 }
 
 namespace {
@@ -1198,13 +1222,27 @@ namespace {
 // per tile (the super-blocks, then extension blocks if any); convert: they are made from `w` in the preparation launch,
 // otherwise they were made earlier.  wide (not Q6_K): the 256 x 256 tiles, which walk the extension blocks for the min term;
 // the 256 x 128 kernel reads the min operands from ps.mtab and skips the extension blocks if the planes have them.
+// `tail`: the workspace behind the planes (planes_tail_bytes).  m, lhs_dtype: as the caller gave them; nblk_tile and wide: for
+// the rows the GEMM sees (gemm_rows).
 hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, bool convert, int64_t m, int64_t n, int64_t k,
-                             float* out, void* lhs_space, const PlaneSpace& ps, int nblk_tile, bool wide, float* part, hipStream_t s) {
+                             float* out, void* lhs_space, const PlaneSpace& ps, int nblk_tile, bool wide, float* tail, hipStream_t s) {
     const bool q6 = encoding == QMM_Q6_K;
-    if (!quarter_mode(encoding, lhs_dtype, m, n, k)) part = nullptr;
+    const bool twin = planes_twin(lhs_dtype, m);
+    const int64_t m_given = m;
+    float* const out_given = out;
+    const int prep_dtype = lhs_dtype;  // (the narrowing reads the caller's values)
+    if (twin) {
+        m *= 2;
+        lhs_dtype = QMM_BF16;
+        out = tail;
+        tail += m * n;
+    }
+    float* part = quarter_mode(encoding, lhs_dtype, m, n, k) ? tail : nullptr;
     const int nblk = (int)(k / 256), lhs_ext = wide ? nblk_tile - nblk : 0;
     const int64_t lda = (int64_t)(nblk + lhs_ext) * 256;
-    const LhsPlanes p = lhs_planes(lhs_space, lhs_dtype, m, k, TM, lda);
+    LhsPlanes p = lhs_planes(lhs_space, lhs_dtype, m, k, TM, lda);
+    LhsPlanes pp = p;  // as the narrowing launch sees them
+    if (twin) pp.a16_lo = p.a16 + m_given * lda;
     hipError_t e = q6 ? allow_full_lds<gemm_planes2_kernel>() : wide ? hipSuccess : allow_full_lds<gemm_planes_kernel>();
     if (e != hipSuccess) return e;
     const int tiles_m = (int)((m + TM - 1) / TM), tiles_n128 = (int)((n + TN - 1) / TN);
@@ -1228,17 +1266,18 @@ hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const
     }
     const int max_split = z.max_split;
     const int64_t zero_blocks = part ? (m * n + kZeroFlatFloats - 1) / kZeroFlatFloats : (int64_t)max_split * 64;
-    const int64_t conv = convert ? (int64_t)tiles_n128 * nblk * 4 : 0, blocks = conv + m + zero_blocks;
+    const int64_t conv = convert ? (int64_t)tiles_n128 * nblk * 4 : 0, blocks = conv + m_given + zero_blocks;
     if (blocks > INT32_MAX || lda * 2 * 8 > INT32_MAX) return hipErrorInvalidValue;
     const dim3 pgrid((unsigned)blocks);
     auto prologue = [&](auto enc_c) {
         constexpr int ENC = decltype(enc_c)::value;
-        if (lhs_dtype == QMM_F32)
+        if (prep_dtype == QMM_F32)
             planes_prologue_kernel<ENC, float><<<pgrid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv,
-                                                                          (const float*)lhs, (int)k, lhs_ext, (int)m, p, z);
+                                                                          (const float*)lhs, (int)k, lhs_ext, (int)m_given, pp, z,
+                                                                          twin ? (int)m_given : 0);
         else
             planes_prologue_kernel<ENC, uint16_t><<<pgrid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv,
-                                                                             (const uint16_t*)lhs, (int)k, lhs_ext, (int)m, p, z);
+                                                                             (const uint16_t*)lhs, (int)k, lhs_ext, (int)m_given, pp, z, 0);
     };
     if (q6) prologue(std::integral_constant<int, QMM_Q6_K>{});
     else if (encoding == QMM_Q4_K) prologue(std::integral_constant<int, QMM_Q4_K>{});
@@ -1259,6 +1298,8 @@ hipError_t run_kquant_planes(int encoding, const void* lhs, int lhs_dtype, const
             gemm_planes_kernel<<<dim3((unsigned)wg), dim3(512), kPlanesLds, s>>>(ps.planes, ps.dtab, ps.mtab, a, p.asum, p.inv, out, (int)m, (int)n,
                                                                                (int)k, tiles_m, tiles_n, nblk_tile, pass == 0, pass, split, part);
     }
+    // twin rows: the row halves (and the quarter mode's second buffer right behind them: four terms) into the caller's tensor
+    if (twin) return launch_sum_shares(out, out_given, m_given * n, part ? 4 : 2, s);
     if (part) add_part_kernel<<<dim3((unsigned)((m * n + 255) / 256)), dim3(256), 0, s>>>(out, part, m * n);
     return hipGetLastError();
 }
@@ -1278,12 +1319,13 @@ PlaneSpace repacked_space(int encoding, void* base, int64_t n, int64_t k) {
 
 hipError_t launch_gemm_planes(int encoding, const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                               float* out, void* workspace, hipStream_t s) {
-    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, m, n);
-    const int nblk_tile = (int)blocks_per_tile(encoding, m, n, k);
-    const int64_t lhs_bytes = (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)nblk_tile * 256).bytes + 255) / 256 * 256;
+    const int64_t me = gemm_rows(lhs_dtype, m);
+    const bool q6 = encoding == QMM_Q6_K, wide = wide_tiles(encoding, me, n);
+    const int nblk_tile = (int)blocks_per_tile(encoding, me, n, k);
+    const int64_t lhs_bytes = (lhs_planes(nullptr, gemm_dtype(lhs_dtype, m), me, k, TM, (int64_t)nblk_tile * 256).bytes + 255) / 256 * 256;
     const PlaneSpace ps = plane_space((uint8_t*)workspace + lhs_bytes, n, k, q6 ? 2 : 1, !q6 && !wide, nblk_tile);
-    float* part = (float*)((uint8_t*)workspace + lhs_bytes + ps.bytes);
-    return run_kquant_planes(encoding, lhs, lhs_dtype, w, true, m, n, k, out, workspace, ps, nblk_tile, wide, part, s);
+    float* tail = (float*)((uint8_t*)workspace + lhs_bytes + ps.bytes);
+    return run_kquant_planes(encoding, lhs, lhs_dtype, w, true, m, n, k, out, workspace, ps, nblk_tile, wide, tail, s);
 }
 
 // Weight planes kept across calls (the weights of a model are converted once, at load time): the conversion alone, and the
@@ -1301,11 +1343,11 @@ hipError_t launch_repack_planes(int encoding, const uint8_t* w, int64_t n, int64
     const LhsPlanes none{};
     const dim3 grid((unsigned)conv);
     if (encoding == QMM_Q6_K)
-        planes_prologue_kernel<QMM_Q6_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z);
+        planes_prologue_kernel<QMM_Q6_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z, 0);
     else if (encoding == QMM_Q4_K)
-        planes_prologue_kernel<QMM_Q4_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z);
+        planes_prologue_kernel<QMM_Q4_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z, 0);
     else
-        planes_prologue_kernel<QMM_Q5_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z);
+        planes_prologue_kernel<QMM_Q5_K, uint16_t><<<grid, dim3(256), 0, s>>>(w, nblk, nblk_tile, tiles_n128, ps.planes, ps.dtab, ps.mtab, (int)conv, nullptr, (int)k, 0, 0, none, z, 0);
     return hipGetLastError();
 }
 
@@ -1325,14 +1367,15 @@ static int64_t repacked_lhs_bytes(int encoding, int lhs_dtype, int64_t m, int64_
     return (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)repacked_blocks_per_tile(encoding, k) * 256).bytes + 255) / 256 * 256;
 }
 int64_t repacked_planes_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    return repacked_lhs_bytes(encoding, lhs_dtype, m, k) + quarter_part_bytes(encoding, lhs_dtype, m, n, k);
+    return repacked_lhs_bytes(encoding, gemm_dtype(lhs_dtype, m), gemm_rows(lhs_dtype, m), k) + planes_tail_bytes(encoding, lhs_dtype, m, n, k);
 }
 hipError_t launch_gemm_planes_repacked(int encoding, const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k,
                                        float* out, void* workspace, hipStream_t s) {
     const PlaneSpace ps = repacked_space(encoding, const_cast<void*>(packed), n, k);
-    float* part = (float*)((uint8_t*)workspace + repacked_lhs_bytes(encoding, lhs_dtype, m, k));
+    const int64_t me = gemm_rows(lhs_dtype, m);
+    float* tail = (float*)((uint8_t*)workspace + repacked_lhs_bytes(encoding, gemm_dtype(lhs_dtype, m), me, k));
     return run_kquant_planes(encoding, lhs, lhs_dtype, nullptr, false, m, n, k, out, workspace, ps, repacked_blocks_per_tile(encoding, k),
-                             wide_tiles(encoding, m, n), part, s);
+                             wide_tiles(encoding, me, n), tail, s);
 }
 
 // GPTQ through the plane GEMM: groups of 128 or 256 (a scale block is two or four steps), plain groups (no act-order), and

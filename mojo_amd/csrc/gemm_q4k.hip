@@ -370,6 +370,11 @@ __global__ __launch_bounds__(256) void sum_k_shares_kernel(const float* __restri
     out[i] = v;
 }
 
+hipError_t launch_sum_shares(const float* part, float* out, int64_t count, int shares, hipStream_t s) {
+    sum_k_shares_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s>>>(part, out, count, shares, 0);
+    return hipGetLastError();
+}
+
 namespace {
 
 // Shares of K per tile: 1 when the tiles alone fill the machine, otherwise enough for about a thousand

@@ -300,9 +300,11 @@ hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int
     const int64_t ntiles = (n + 15) / 16;
     const dim3 grid((unsigned)std::min<int64_t>(ntiles, cus)), block(64 * kQWaves);
     const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
-    // (K in rounds: the sixteen-row fp32 variant spills in its loop there, two passes of eight rows are faster: 4096 x 14336,
-    // 16 rows: 98 against 112 us; sixteen bf16 rows are one operand set and go as one pass everywhere)
-    const int pass = k == 4096 || a_dtype != QMM_F32 ? 16 : 8;
+    // Sixteen bf16 rows are one operand set and go as one pass everywhere.  Sixteen fp32 rows are two sets (hi parts and
+    // residuals of eight rows each) and the kernel spills registers in its loop: two passes of eight rows are faster unless a
+    // workgroup has many tiles to stream (K = 4096, 16 rows: 4096 rows of weights 26.9 against 36.1 us, 14336: 42.7 against 46.7,
+    // 32000: 64.5 against 60.2, 128256: 192 against 144; K in rounds, 4096 x 14336: 98 against 112 us).
+    const int pass = a_dtype != QMM_F32 || (k == 4096 && ntiles >= 6 * (int64_t)cus) ? 16 : 8;
     for (int m0 = 0; m0 < m; m0 += pass) {
         const int rows = std::min(pass, m - m0);
         const void* am = (const char*)a + (size_t)m0 * k * esz;

@@ -289,8 +289,8 @@ struct OptionalPlanesScope {
     explicit OptionalPlanesScope(bool skip) : prev(g_skip_optional_planes) { g_skip_optional_planes = skip; }
     ~OptionalPlanesScope() { g_skip_optional_planes = prev; }
 };
-static bool kquant_planes(int encoding, int64_t m, int64_t n, int64_t k) {
-    return qmm::gemm_planes_wanted(encoding, m, n, k) && !(encoding == QMM_Q4_K && g_skip_optional_planes);
+static bool kquant_planes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    return qmm::gemm_planes_wanted(encoding, lhs_dtype, m, n, k) && !(encoding == QMM_Q4_K && g_skip_optional_planes);
 }
 static bool gptq_planes(int64_t m, int64_t n, int64_t k, int group) {
     return !g_skip_optional_planes && qmm::gemm_gptq_planes_wanted(m, n, k, group);
@@ -298,7 +298,7 @@ static bool gptq_planes(int64_t m, int64_t n, int64_t k, int group) {
 
 int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (m <= 0 || k <= 0) return 0;
-    if (kquant_planes(encoding, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
+    if (kquant_planes(encoding, lhs_dtype, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (encoding == QMM_Q4_0) {
         const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         const int64_t c = qmm::gemm_q4_0_planes_wanted(m, n, k) ? qmm::gemm_q4_0_planes_workspace_bytes(m, n, k) : 0;
@@ -501,7 +501,7 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     }
     // Q5_K and Q6_K with many lhs rows, Q4_K with more than 512 on large matrices: weights to fp16 integer planes in the workspace,
     // then the matrix cores
-    if (kquant_planes(encoding, m, n, k))
+    if (kquant_planes(encoding, lhs_dtype, m, n, k))
         return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
     // Q5_K with several lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
     if (encoding == QMM_Q5_K && q5k_mm_wanted(m, n, k) && qmm::gemv_q5_k_mm_supported(w, m, n, k))

@@ -12,7 +12,7 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_lanes_rows, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_twin_rows, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
 // Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 
@@ -170,7 +170,9 @@ hipError_t launch_gemm_q4_k_tile(const void* lhs, int lhs_dtype, const uint8_t* 
                                  float* out, void* workspace, hipStream_t s);
 // Q5_K and Q6_K (Q4_K on request) on the matrix cores: a pass that turns the weights into fp16 integer planes in the
 // workspace, then a tile GEMM over them.
-bool gemm_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k);
+// out[i] = part[i] + part[count + i] + ... (`shares` terms, in that order)
+hipError_t launch_sum_shares(const float* part, float* out, int64_t count, int shares, hipStream_t s);
+bool gemm_planes_wanted(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k);
 // GPTQ through the same GEMM (plain groups of 128 or 256 and large problems only)
 bool gemm_gptq_planes_wanted(int64_t m, int64_t n, int64_t k, int group);
 int64_t gemm_gptq_planes_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k);
