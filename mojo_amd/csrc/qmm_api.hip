@@ -98,9 +98,9 @@ bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
 }
 
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    const bool f32 = lhs_dtype == QMM_F32;
-    const double tiles = (double)((m + 127) / 128) * (double)((n + 255) / 256);
-    const double gemm_us = (double)(int64_t)((tiles + 255.0) / 256.0) * ((double)k / 4096.0) * 64.0 * (f32 ? 2.1 : 1.0);
+    const bool f32 = lhs_dtype == QMM_F32, twin = qmm::gemm_gptq_twin(lhs_dtype, m);  // twin: one GEMM pass over 2 m rows, then a small launch
+    const double tiles = (double)(((twin ? 2 * m : m) + 127) / 128) * (double)((n + 255) / 256);
+    const double gemm_us = (double)(int64_t)((tiles + 255.0) / 256.0) * ((double)k / 4096.0) * 64.0 * (f32 && !twin ? 2.1 : 1.0) + (twin ? 5.0 : 0.0);
     const double pass_us = (f32 ? 10.0 : 8.0) + (double)n * (double)k * 0.52 / (f32 ? 1.9e6 : 3.9e6) + (k > 4096 ? 2.0 : 0.0);
     return (double)((m + 15) / 16) * pass_us < gemm_us;
 }
@@ -310,7 +310,7 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
-        const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, k) : 0;
+        const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, n, k) : 0;
         const int64_t c = gptq_planes(m, n, k, 128) ? qmm::gemm_gptq_planes_workspace_bytes(lhs_dtype, m, n, k) : 0;  // (the group size is not known here)
         return std::max(std::max(a, b), c);
     }
