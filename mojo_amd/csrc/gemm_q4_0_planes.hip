@@ -414,8 +414,10 @@ bool gemm_q4_0_planes_wanted(int64_t m, int64_t n, int64_t k) {
     if (k % 256 || k < 256 || kernel_disabled("q4_0_planes")) return false;
     if (force) return m > 16;
     // Measured against the int8 kernels on 1024..14336 x 4096..14336 weights: faster from 80 lhs rows on at every size
-    // (80 rows: 112 against 169 us on 14336 x 4096; 2048 rows: 359 against 674 us).
-    return m > 64;
+    // (80 rows: 112 against 169 us on 14336 x 4096; 2048 rows: 359 against 674 us); on small matrices from 33 rows on, where the
+    // int8 kernel takes a third 16-row tile per workgroup (4096 x 4096: 33 / 64 rows 43 / 49 us against 38 for the planes; 14336 x
+    // 4096: 54 / 56 against 90).
+    return m > 64 || (m > 32 && n * k <= ((int64_t)24 << 20));  // (8192 x 4096: 33 / 64 rows 46 / 50 against 52 / 56 us)
 }
 
 int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k);
