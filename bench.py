@@ -531,13 +531,13 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib", "mfma_probe", "sweep"),
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib", "mfma_probe", "sweep", "ladder"),
                     default="decode",
                     help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill / q6k_prefill / q5k_prefill / q40_prefill: the M=2048 "
                          "GEMM of the same model's gate projection (second target, matrix-core roofline); calib: a plain "
                          "read and a plain copy of 256 MiB, the yardsticks for the FETCH_SIZE / WRITE_SIZE counters; mfma_probe: the "
                          "matrix-core rate of a register-resident loop by operand data; sweep: Q4_K decode and prefill over shapes "
-                         "the dispatch was not tuned on")
+                         "the dispatch was not tuned on; ladder: every encoding over 1 .. 256 lhs rows of both types on two projection shapes")
     ap.add_argument("--repacked", action="store_true", help="prefill workloads: weight planes made once (qmm_repack), outside the timed steps")
     ap.add_argument("--min-ms", type=float, default=HEADLINE_MIN_MS,
                     help="device time the headline's timed blocks cover at least (profiler runs pass a small value to keep their traces short)")
@@ -563,6 +563,8 @@ def main() -> int:
         return probe_main()
     if args.workload == "sweep":
         return sweep_main(gen)
+    if args.workload == "ladder":
+        return ladder_main(gen)
     if args.workload != "decode":
         return prefill_main(args, gen)
     m = args.m
@@ -796,6 +798,35 @@ def sweep_main(gen) -> int:
         del w0
     print(json.dumps({"metric": "Q4_K over untuned shapes: decode as a fraction of the plain read, prefill of the matrix-core peak",
                       "encoding": "Q4_K", "sweep": out}))
+    return 0
+
+
+LADDER_ROWS = (1, 4, 8, 16, 17, 32, 64, 65, 128, 256)
+
+
+def ladder_main(gen) -> int:
+    """Microseconds per qmm_matmul call for every encoding over 1 .. 256 lhs rows, fp32 and bf16, on the q / o and the gate / up
+    shape (six calls per graph on one weight tensor, so the weights come from the last-level cache: the figures compare
+    row counts and lhs types of one shape, not shapes).  One JSON line; a step between neighbouring row counts that is
+    larger than the rows explain is a threshold of the dispatch in the wrong place."""
+    out = {}
+    for enc in (QE.Q4_K, QE.Q5_K, QE.Q6_K, QE.Q4_0, QE.GPTQ):
+        for n, k in ((4096, 4096), (14336, 4096)):
+            if enc == QE.GPTQ:
+                w = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
+            else:
+                w = make_weight(enc, n, k, gen)
+            for dt, name in ((torch.float32, "f32"), (torch.bfloat16, "bf16")):
+                row = {}
+                for m in LADDER_ROWS:
+                    a = torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen).to(dt)
+                    calls = [GptqMatmul(w, a) if enc == QE.GPTQ else Gemv(enc, w, a) for _ in range(6)]
+                    dev_s, _ = time_graphs([capture(calls)], 20, 3)
+                    row[f"m{m}"] = round(dev_s * 1e6 / (20 * len(calls)), 1)
+                    del calls
+                out[f"{enc.name} {n}x{k} {name}"] = row
+            del w
+    print(json.dumps({"metric": "microseconds per call over lhs rows 1 .. 256, every encoding, both lhs types (warm weights)", "ladder": out}))
     return 0
 
 

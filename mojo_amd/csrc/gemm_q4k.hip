@@ -389,11 +389,12 @@ int k_shares(int64_t m, int64_t n, int64_t k, int bm) {
 }  // namespace
 
 namespace {
-// An fp32 lhs on a problem whose tiles are cut into K shares anyway: hi and residual plane as the two halves of one lhs of 2 m
-// rows, one pass of the GEMM instead of two, and the pass that adds the K shares adds the two halves as well (twice the
-// shares of m x n values each).  4096 x 4096 with 32 fp32 rows: 35 -> 20 us.
+// An fp32 lhs on a problem whose tiles are cut into K shares anyway, or of up to 256 rows: hi and residual plane as the two
+// halves of one lhs of 2 m rows, one pass of the GEMM instead of two, and the pass that adds the K shares adds the two halves as
+// well (twice the shares of m x n values each; without K shares it is a launch more and a pass over the weights less).
+// 4096 x 4096 with 32 fp32 rows: 35 -> 20 us; 14336 x 4096 with 256: 157 -> 85.
 bool twin_rows(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    return lhs_dtype == QMM_F32 && k_shares(2 * m, n, k, 64) > 1 && !kernel_disabled("q4k_twin_rows");
+    return lhs_dtype == QMM_F32 && (k_shares(2 * m, n, k, 64) > 1 || m <= 256) && !kernel_disabled("q4k_twin_rows");
 }
 }  // namespace
 
@@ -433,7 +434,7 @@ hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, in
     // persistent workgroups: as many as fit on the device at once (two per compute unit for the 4-wavefront shape)
     const int wg = 8 * min(per_xcd, max(1, cus / 8) * (2 / wm_rows));
     dim3 grid((unsigned)wg), block(256 * wm_rows);
-    float* part = ksplit > 1 ? (float*)((char*)workspace + p.bytes) : nullptr;
+    float* part = ksplit > 1 || twin ? (float*)((char*)workspace + p.bytes) : nullptr;
     float* dst = part ? part : out;
     const int64_t count = m_out * n;
     const int sum_shares = twin ? 2 * ksplit : ksplit;

@@ -729,11 +729,12 @@ def test_q4_k_gemm_bf16_lhs(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 128, 512), (33, 64, 256), (32, 4096, 4096), (17, 1000, 4096), (100, 2050, 1024),
-                                   (65, 520, 2560)])
+                                   (65, 520, 2560), (200, 16500, 512)])
 def test_q4_k_gemm_f32_lhs(m, n, k):
     """fp32 lhs: hi and residual fp16 planes.  From 1024 columns of K on (tiles cut into K shares) the residual plane is the
-    second half of the rows of one lhs and a single pass multiplies both; shorter K takes two passes.  Rows of very different
-    magnitude (the row scales of both halves), ragged m and n."""
+    second half of the rows of one lhs and a single pass multiplies both, and so it is up to 256 rows whatever the tiles (200 x
+    16500: 455 tiles, no K shares); shorter K takes two passes.  Rows of very different magnitude (the row scales of both
+    halves), ragged m and n."""
     w, a = synth(12, n, k, m)
     a *= np.logspace(-3, 3, m, dtype=np.float32)[:, None]
     wq = O.quantize(O.Q4_K, w)
