@@ -302,7 +302,7 @@ bool gemm_gptq_supported(int64_t k, int group) {
 
 // An fp32 lhs of up to 256 rows: hi and residual plane as the two halves of ONE lhs of twice the rows, one pass over the weights
 // into the workspace instead of two onto `out`, and a small launch that adds the halves (4096 x 4096 with 128 rows: 126 -> 70 us).
-bool gemm_gptq_twin(int lhs_dtype, int64_t m) { return lhs_dtype == QMM_F32 && m <= 256 && !kernel_disabled("gptq_twin_rows"); }
+bool gemm_gptq_twin(int lhs_dtype, int64_t m) { return lhs_dtype == QMM_F32 && m <= 256 && twin_rows_allowed() && !kernel_disabled("gptq_twin_rows"); }
 
 int64_t gemm_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     if (gemm_gptq_twin(lhs_dtype, m)) return lhs_planes(nullptr, QMM_BF16, 2 * m, k).bytes + 2 * m * n * 4;

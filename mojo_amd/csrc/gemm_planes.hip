@@ -1196,7 +1196,7 @@ int64_t quarter_part_bytes(int encoding, int lhs_dtype, int64_t m, int64_t n, in
 // bf16 lhs (one pass, every way of cutting few tiles along K open to it); the GEMM writes into the workspace and the pass
 // that adds K quarters adds the two halves of the rows as well.  Two passes, the second one over whole tiles onto the
 // first one's result, had cost 4096 x 4096 with 65 fp32 rows 110 us (Q5_K) and 176 us (Q6_K) against 31 and 56 us for bf16 rows.
-bool planes_twin(int lhs_dtype, int64_t m) { return lhs_dtype == QMM_F32 && m <= 256 && !kernel_disabled("planes_twin_rows"); }
+bool planes_twin(int lhs_dtype, int64_t m) { return lhs_dtype == QMM_F32 && m <= 256 && twin_rows_allowed() && !kernel_disabled("planes_twin_rows"); }
 // rows and type that the GEMM sees
 int64_t gemm_rows(int lhs_dtype, int64_t m) { return planes_twin(lhs_dtype, m) ? 2 * m : m; }
 int gemm_dtype(int lhs_dtype, int64_t m) { return planes_twin(lhs_dtype, m) ? QMM_BF16 : lhs_dtype; }

@@ -394,7 +394,7 @@ namespace {
 // well (twice the shares of m x n values each; without K shares it is a launch more and a pass over the weights less).
 // 4096 x 4096 with 32 fp32 rows: 35 -> 20 us; 14336 x 4096 with 256: 157 -> 85.
 bool twin_rows(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    return lhs_dtype == QMM_F32 && (k_shares(2 * m, n, k, 64) > 1 || m <= 256) && !kernel_disabled("q4k_twin_rows");
+    return lhs_dtype == QMM_F32 && (k_shares(2 * m, n, k, 64) > 1 || m <= 256) && twin_rows_allowed() && !kernel_disabled("q4k_twin_rows");
 }
 }  // namespace
 

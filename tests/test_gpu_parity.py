@@ -806,7 +806,7 @@ def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
     ("Q5_K", 1030, 8200, 2304, False), ("Q4_K", 1600, 8200, 768, True), ("Q4_K", 1540, 10300, 2304, False),
     ("GPTQ128", 1600, 8200, 768, True), ("GPTQ256", 1540, 8200, 768, False), ("GPTQ128", 1536, 11016, 1280, False),
     ("Q4_K", 2000, 14192, 512, True), ("GPTQ128", 1990, 14192, 512, False), ("Q5_K", 1800, 14000, 256, True),
-    ("GPTQ256", 1030, 10296, 1280, True), ("GPTQ128", 2000, 14192, 512, True)])
+    ("GPTQ256", 1030, 10296, 1280, True), ("GPTQ128", 2000, 14192, 512, True), ("Q5_K", 200, 20600, 768, False)])
 def test_plane_gemm_on_256_wide_tiles(kind, m, n, k, bf16):
     """Large problems of the single-plane encodings (from 160 tiles of 256 x 256; Q4_K and GPTQ from 513 lhs rows): the plane GEMM
     that keeps its accumulators in units of the current scale block's scale.  Q4_K / Q5_K carry their min term as extension

@@ -49,6 +49,8 @@ def lhs_rows(seed, m, k, bf16):
     (QE.Q6_K, 1100, 2560, [(300, True, True), (70, True, True), (300, False, True)]),
     (QE.Q4_K, 14080, 768, [(520, True, True), (1600, False, True), (300, True, False), (64, True, True)]),
     (QE.Q4_K, 20600, 256, [(2000, True, True), (300, True, False)]),
+    (QE.Q4_K, 20600, 768, [(200, False, False), (90, False, False)]),
+    (QE.Q5_K, 20600, 768, [(200, False, True), (130, True, True)]),
 ])
 def test_repacked_kquant_matches_oracle_and_qmatmul(enc, n, k, rows):
     """One conversion, many calls.  Q4_K / Q5_K planes carry their min operands both as extension blocks (wide GEMM: 1030 x 8200,
@@ -56,7 +58,9 @@ def test_repacked_kquant_matches_oracle_and_qmatmul(enc, n, k, rows):
     matrix), which then steps over the extension blocks (K = 2304: two of them, one with a single super-block); Q6_K has one
     layout.  Few tiles on K >= 2048 with a bf16 lhs (300 and 70 x 1100 x 2560: 18 and 9 tiles, ten super-blocks) are cut in four K quarters
     of 2, 3, 2 and 3 super-blocks that meet pairwise in two buffers; the fp32 lhs takes halves.  Row counts of the decode kernels are served from the packed tensors.  300 x 20600 (162 tiles of 256 x 256) takes the wide tiles
-    here, 300 x 14080 the 256 x 128 plane kernel, and inside qmatmul both take kernels that unpack as they go: close, not identical."""
+    here, 300 x 14080 the 256 x 128 plane kernel, and inside qmatmul both take kernels that unpack as they go: close, not identical.
+    An fp32 lhs of up to 256 rows goes through the GEMMs as one lhs of twice the rows: 200 x 20600 is then 162 wide tiles (the residual
+    rows' extension blocks are zeros), 90 x 20600 one row tile of the 256 x 128 kernel, 300 x 1100 x 2560 K quarters."""
     wq = kquant_weights(enc, n, k, 7 + n % 5)
     wq_d = gpu(wq)
     weights = repack_weights(enc, None, wq_d)
