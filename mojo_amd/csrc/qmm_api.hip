@@ -363,9 +363,6 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
 int qmm_matmul(int encoding, const qmm_gptq_config* cfg, const void* lhs, int lhs_dtype, int64_t m, int64_t k,
                const void* const* rhs, int n_rhs, int64_t n, float* out, void* workspace, int64_t workspace_bytes,
                int flags, void* stream) {
-    // an fp32 lhs as twice the rows only with a workspace that holds the GEMM's result as well
-    const TwinRowsScope twin(g_skip_twin_rows || (lhs_dtype == QMM_F32 && m > 16 && n > 0 && k > 0 &&
-                                                  (!workspace || workspace_bytes < qmm_matmul_workspace_bytes_flags(encoding, lhs_dtype, m, n, k, flags))));
     // the plane GEMM for Q4_K / GPTQ only with a workspace that holds the planes
     const bool optional = (encoding == QMM_Q4_K || encoding == QMM_GPTQ) && m > 0 && n > 0 && k > 0 && !g_skip_optional_planes;
     const OptionalPlanesScope scope(g_skip_optional_planes ||
@@ -790,14 +787,9 @@ int qmm_matmul_repacked(int encoding, const qmm_gptq_config* cfg, const void* lh
     }
     if (lhs_dtype != QMM_F32 && lhs_dtype != QMM_BF16) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs dtype must be f32 or bf16");
     if (!aligned(lhs, 16) || !aligned(out, 4)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: lhs must be 16-byte aligned");
-    auto bytes_needed = [&] {
-        return encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, n, k)
-               : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
-                                      : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
-    };
-    int64_t need = bytes_needed();
-    const TwinRowsScope twin(g_skip_twin_rows || !workspace || workspace_bytes < need);  // (an fp32 lhs in two passes needs less)
-    need = bytes_needed();
+    const int64_t need = encoding == QMM_Q4_0 ? qmm::repacked_q4_0_workspace_bytes(m, n, k)
+                         : encoding == QMM_GPTQ ? qmm::repacked_gptq_workspace_bytes(lhs_dtype, m, k)
+                                                : qmm::repacked_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (!workspace || workspace_bytes < need)
         return fail(QMM_ERR_WORKSPACE, "qmm_matmul_repacked: workspace of %lld bytes required, %lld given", (long long)need, (long long)workspace_bytes);
     if (!aligned(workspace, 256)) return fail(QMM_ERR_INVALID, "qmm_matmul_repacked: workspace must be 256-byte aligned");

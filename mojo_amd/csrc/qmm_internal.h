@@ -15,8 +15,8 @@ namespace qmm {
 // q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
 // Nothing is disabled by default.
 bool kernel_disabled(const char* family);
-// False while an entry point works with a workspace that is too small for the GEMMs' one-pass treatment of an fp32 lhs (the
-// lhs as twice the rows, the result in the workspace): they then take their two passes.  Per thread.
+// False while qmm_matmul_static serves a problem whose one-pass treatment of an fp32 lhs (the lhs as twice the rows, the
+// result in the workspace) does not fit its scratch: the GEMMs then take their two passes.  Per thread.
 bool twin_rows_allowed();
 
 hipError_t launch_read_probe(const void* buf, int64_t bytes, hipStream_t s);
