@@ -32,6 +32,7 @@
 //     per output row cost a fifth of the tile time).
 #include <stdlib.h>
 
+#include <algorithm>
 #include <type_traits>
 
 #include "gemm_lhs.h"
@@ -360,30 +361,75 @@ __global__ __launch_bounds__(256 * WM, 2 / WM) void gemm_q4_k_kernel(const uint8
     }
 }
 
-// out[i] (+)= part[0][i] + part[1][i] + ... in that order
+// out[i] (+)= part[0][i] + part[1][i] + ... in that order.  VEC: four neighbouring values per thread (count a multiple of 4,
+// 16-byte aligned buffers); the loads of four shares are issued together, the additions keep their order.
+template <bool VEC>
 __global__ __launch_bounds__(256) void sum_k_shares_kernel(const float* __restrict__ part, float* __restrict__ out,
                                                            int64_t count, int ksplit, int accumulate) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= count) return;
-    float v = accumulate ? out[i] : 0.0f;
-    for (int s = 0; s < ksplit; s++) v += part[(int64_t)s * count + i];
-    out[i] = v;
+    if constexpr (VEC) {
+        const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+        if (i >= count) return;
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        float4 v = accumulate ? *(const float4*)(out + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        int s = 0;
+        for (; s + 4 <= ksplit; s += 4) {
+            f32x4 p[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) p[j] = __builtin_nontemporal_load((const f32x4*)(part + (int64_t)(s + j) * count + i));
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v.x += p[j].x;
+                v.y += p[j].y;
+                v.z += p[j].z;
+                v.w += p[j].w;
+            }
+        }
+        for (; s < ksplit; s++) {
+            const f32x4 p = __builtin_nontemporal_load((const f32x4*)(part + (int64_t)s * count + i));
+            v.x += p.x;
+            v.y += p.y;
+            v.z += p.z;
+            v.w += p.w;
+        }
+        *(float4*)(out + i) = v;
+    } else {
+        const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (i >= count) return;
+        float v = accumulate ? out[i] : 0.0f;
+        for (int s = 0; s < ksplit; s++) v += part[(int64_t)s * count + i];
+        out[i] = v;
+    }
 }
 
+namespace {
+void sum_shares(const float* part, float* out, int64_t count, int shares, int accumulate, hipStream_t s) {
+    if (count % 4 == 0 && (((uintptr_t)part | (uintptr_t)out) & 15) == 0)
+        sum_k_shares_kernel<true><<<dim3((unsigned)((count / 4 + 255) / 256)), dim3(256), 0, s>>>(part, out, count, shares, accumulate);
+    else
+        sum_k_shares_kernel<false><<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s>>>(part, out, count, shares, accumulate);
+}
+}  // namespace
+
 hipError_t launch_sum_shares(const float* part, float* out, int64_t count, int shares, hipStream_t s) {
-    sum_k_shares_kernel<<<dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s>>>(part, out, count, shares, 0);
+    sum_shares(part, out, count, shares, 0, s);
     return hipGetLastError();
 }
 
 namespace {
 
-// Shares of K per tile: 1 when the tiles alone fill the machine, otherwise enough for about a thousand
-// work units, each at least two super-blocks long.  A function of the shape only.
+// Shares of K per tile, a function of the shape only: 1 when the tiles alone fill the machine; each share at least two
+// super-blocks long.  Every share is another m x n partial result written and read back, so with several lhs row tiles the aim
+// is about 256 work units (one per compute unit; microseconds with 1024 / 512 / 256 / 128 units aimed at, bf16 lhs: 512 x 4096 x
+// 4096 60.7 / 45.9 / 42.7 / 52.8; 512 x 4096 x 14336 123 / 105 / 107 / 170; 200 x 14336 x 4096 77.6 / 67.7 / 59.9 / 56.7;
+// 96 x 4096 x 14336 57.7 / 49.0 / 43.8 / 60.7).  One row tile (up to 64 rows) has small partial results: as many shares as fit
+// one round of two workgroups per compute unit, sixteen at most (32 rows: 14336 x 4096, 56 tiles, 5 / 8 shares 35.2 / 29.3;
+// 4096 x 14336, 16 tiles, 16 / 28 shares 33.5 / 35.7; 64 rows on 32000 x 4096, 125 tiles, 3 / 5 shares 51.6 / 60.2).
 int k_shares(int64_t m, int64_t n, int64_t k, int bm) {
     const int64_t tiles = ((m + bm - 1) / bm) * ((n + BN - 1) / BN), nblk = k / 256;
     if (tiles >= 256) return 1;
-    const int64_t want = (1024 + tiles - 1) / tiles, cap = nblk / 2 > 1 ? nblk / 2 : 1;
-    return (int)(want < cap ? want : cap);
+    const int64_t cap = nblk / 2 > 1 ? nblk / 2 : 1;
+    const int64_t want = m <= bm ? std::min<int64_t>(512 / tiles, 16) : (256 + tiles - 1) / tiles;
+    return (int)std::max<int64_t>(1, std::min(want, cap));
 }
 
 }  // namespace
@@ -437,17 +483,16 @@ hipError_t launch_gemm_q4_k(const void* lhs, int lhs_dtype, const uint8_t* w, in
     float* part = ksplit > 1 || twin ? (float*)((char*)workspace + p.bytes) : nullptr;
     float* dst = part ? part : out;
     const int64_t count = m_out * n;
-    const int sum_shares = twin ? 2 * ksplit : ksplit;
-    dim3 rgrid((unsigned)((count + 255) / 256)), rblock(256);
+    const int sum_shares_n = twin ? 2 * ksplit : ksplit;
 #define QMM_GEMM_GO(WM_)                                                                                          \
     do {                                                                                                          \
         gemm_q4_k_kernel<WM_><<<grid, block, 0, s>>>(w, p.a16, p.asum, p.inv, dst, (int)m, (int)n, (int)k,       \
                                                      tiles_m, tiles_n, 1, 0, ksplit);                             \
-        if (part) sum_k_shares_kernel<<<rgrid, rblock, 0, s>>>(part, out, count, sum_shares, 0);                  \
+        if (part) sum_shares(part, out, count, sum_shares_n, 0, s);                                               \
         if (p.a16_lo) { /* fp32 lhs: the residual plane, added on top */                                          \
             gemm_q4_k_kernel<WM_><<<grid, block, 0, s>>>(w, p.a16_lo, p.asum, p.inv, dst, (int)m, (int)n,        \
                                                          (int)k, tiles_m, tiles_n, 0, part ? 0 : 1, ksplit);      \
-            if (part) sum_k_shares_kernel<<<rgrid, rblock, 0, s>>>(part, out, count, ksplit, 1);                  \
+            if (part) sum_shares(part, out, count, ksplit, 1, s);                                                 \
         }                                                                                                         \
     } while (0)
     if (wm_rows == 2)
