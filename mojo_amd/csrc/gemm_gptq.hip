@@ -25,6 +25,8 @@
 // use them (a wavefront load covers 32 consecutive columns of two k8 rows: 128-byte runs).
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include <type_traits>
 
 #include "gemm_lhs.h"
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
                                                         const _Float16* __restrict__ a16,
                                                         const _Float16* __restrict__ asum, const float* __restrict__ inv,
                                                         float* __restrict__ out, int m, int n, int k, int tiles_m,
-                                                        int tiles_n) {
+                                                        int tiles_n, int ksplit) {
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][BM * A_STRIDE];
     __shared__ __attribute__((aligned(16))) _Float16 lds_s[BM * 16];
     __shared__ __attribute__((aligned(16))) float lds_inv[BM];
@@ -63,14 +65,20 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 2, wn = wave & 3;
     const int nl = lane & 31, g = lane >> 5;
-    const int nblk = k >> 8;
+    const int nblk_row = k >> 8;  // 256-column blocks of a whole row
 
-    int tile_m, tile_n;
+    // A work unit is a tile's share of K: blocks [kb0, kb0 + nblk); with ksplit > 1 its result goes to slice ks of `out`, then
+    // a [ksplit][m][n] buffer that a later launch adds up.  Every pointer below is moved to the share's first block.
+    int tile_m, tile_n, kb0, nblk;
     {
-        const int total = tiles_m * tiles_n;
+        const int total = tiles_m * tiles_n * ksplit;
         const int per_xcd = (total + 7) / 8;
-        const int o = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-        if (o >= total) return;
+        const int u = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+        if (u >= total) return;
+        const int o = u / ksplit, ks = u - o * ksplit;
+        kb0 = ks * nblk_row / ksplit;
+        nblk = (ks + 1) * nblk_row / ksplit - kb0;
+        out += (int64_t)ks * m * n;
         const int gm = 2, span = gm * tiles_n;
         const int grp = o / span, rem = o - grp * span;
         const int rows_here = min(gm, tiles_m - grp * gm);
@@ -78,6 +86,10 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
         tile_m = grp * gm + rem - tile_n * rows_here;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
+    a16 += (int64_t)kb0 * 256;
+    qweight += (int64_t)kb0 * 32 * n;
+    scales += (int64_t)kb0 * GB * n;
+    qzeros += (int64_t)kb0 * GB * (n >> 3);
 
     const int nsteps = nblk * 4;
     const int a_row = tid >> 2, a_seg = tid & 3;
@@ -149,7 +161,7 @@ __global__ __launch_bounds__(512) void gemm_gptq_kernel(const uint32_t* __restri
         }
     };
     uint4 as_n = make_uint4(0, 0, 0, 0);
-    const uint4* as_src = (const uint4*)(asum + (int64_t)min(m0 + (tid >> 1), m - 1) * nblk * 16 + (tid & 1) * 8);
+    const uint4* as_src = (const uint4*)(asum + ((int64_t)min(m0 + (tid >> 1), m - 1) * nblk_row + kb0) * 16 + (tid & 1) * 8);
     auto as_prefetch = [&](int blk) {
         if (tid < 256) as_n = as_src[min(blk, nblk - 1) * 2];
     };
@@ -304,9 +316,19 @@ bool gemm_gptq_supported(int64_t k, int group) {
 // into the workspace instead of two onto `out`, and a small launch that adds the halves (4096 x 4096 with 128 rows: 126 -> 70 us).
 bool gemm_gptq_twin(int lhs_dtype, int64_t m) { return lhs_dtype == QMM_F32 && m <= 256 && twin_rows_allowed() && !kernel_disabled("gptq_twin_rows"); }
 
+// Shares of K per tile when the tiles leave compute units without work: as many as make about one workgroup per compute unit,
+// each at least two blocks of 256 columns long, sixteen at most (4096 x 4096 with 64 bf16 rows, 16 tiles: 40 -> 21 us).
+int gemm_gptq_k_shares(int64_t m, int64_t n, int64_t k) {
+    const int64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN), nblk = k / 256;
+    if (kernel_disabled("gptq_k_shares")) return 1;
+    return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, 16), nblk / 2));
+}
+
 int64_t gemm_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    if (gemm_gptq_twin(lhs_dtype, m)) return lhs_planes(nullptr, QMM_BF16, 2 * m, k).bytes + 2 * m * n * 4;
-    return lhs_planes(nullptr, lhs_dtype, m, k).bytes;
+    const bool twin = gemm_gptq_twin(lhs_dtype, m);
+    const int64_t me = twin ? 2 * m : m;
+    const int ks = gemm_gptq_k_shares(me, n, k);
+    return lhs_planes(nullptr, twin ? QMM_BF16 : lhs_dtype, me, k).bytes + (twin || ks > 1 ? (int64_t)ks * me * n * 4 : 0);
 }
 
 hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales,
@@ -318,12 +340,12 @@ hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qwei
     const LhsPlanes p = twin ? lhs_planes(workspace, QMM_BF16, 2 * m, k) : lhs_planes(workspace, lhs_dtype, m, k);
     hipError_t e = launch_prep_lhs<kLhsOrderGPTQ>(lhs, lhs_dtype, m, k, p, s, twin);
     if (e != hipSuccess) return e;
-    if (twin) {
-        m *= 2;
-        out = (float*)((char*)workspace + p.bytes);
-    }
+    if (twin) m *= 2;
+    const int ks = gemm_gptq_k_shares(m, n, k);
+    const bool to_workspace = twin || ks > 1;  // partial results [ks][m][n], added up (and the row halves with them) at the end
+    if (to_workspace) out = (float*)((char*)workspace + p.bytes);
     const int tiles_m = (int)((m + BM - 1) / BM), tiles_n = (int)((n + BN - 1) / BN);
-    const int total = tiles_m * tiles_n;
+    const int total = tiles_m * tiles_n * ks;
     const int per_xcd = (total + 7) / 8;
     dim3 grid((unsigned)(per_xcd * 8)), block(512);
 #define QMM_GPTQ_LAUNCH(GB_)                                                                                          \
@@ -331,18 +353,18 @@ hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qwei
         if (twin) { /* both planes as one lhs */                                                                      \
             gemm_gptq_kernel<2, GB_, true, false><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.asum,    \
                                                                          p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
-                                                                         tiles_n);                                   \
+                                                                         tiles_n, ks);                               \
         } else if (lhs_dtype == QMM_F32) { /* main plane, then the residual plane added on top */                     \
             gemm_gptq_kernel<2, GB_, true, false><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.asum,    \
                                                                          p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
-                                                                         tiles_n);                                   \
+                                                                         tiles_n, ks);                               \
             gemm_gptq_kernel<2, GB_, false, true><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16_lo, p.asum, \
                                                                          p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
-                                                                         tiles_n);                                   \
+                                                                         tiles_n, ks);                               \
         } else {                                                                                                      \
             gemm_gptq_kernel<0, GB_, true, false><<<grid, block, 0, s>>>(qweight, scales, qzeros, p.a16, p.asum,    \
                                                                          p.inv, out, (int)m, (int)n, (int)k, tiles_m, \
-                                                                         tiles_n);                                   \
+                                                                         tiles_n, ks);                               \
         }                                                                                                             \
     } while (0)
     if (group == 256) QMM_GPTQ_LAUNCH(1);
@@ -350,7 +372,7 @@ hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qwei
     else if (group == 64) QMM_GPTQ_LAUNCH(4);
     else return hipErrorInvalidValue;
 #undef QMM_GPTQ_LAUNCH
-    if (twin) return launch_sum_shares(out, out_given, m_given * n, 2, s);
+    if (to_workspace) return launch_sum_shares(out, out_given, m_given * n, twin ? 2 * ks : ks, s);
     return hipGetLastError();
 }
 

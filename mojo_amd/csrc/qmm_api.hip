@@ -98,10 +98,16 @@ bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
 }
 
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
-    const bool f32 = lhs_dtype == QMM_F32, twin = qmm::gemm_gptq_twin(lhs_dtype, m);  // twin: one GEMM pass over 2 m rows, then a small launch
-    const double tiles = (double)(((twin ? 2 * m : m) + 127) / 128) * (double)((n + 255) / 256);
-    const double gemm_us = (double)(int64_t)((tiles + 255.0) / 256.0) * ((double)k / 4096.0) * 64.0 * (f32 && !twin ? 2.1 : 1.0) + (twin ? 5.0 : 0.0);
-    const double pass_us = (f32 ? 10.0 : 8.0) + (double)n * (double)k * 0.52 / (f32 ? 1.9e6 : 3.9e6) + (k > 4096 ? 2.0 : 0.0);
+    // Passes of the small-batch kernel (16 rows each) against the GEMM (128 x 256 tiles, cut into K shares when they are few, an
+    // fp32 lhs of up to 256 rows as twice the rows), in microseconds as measured on this part: 4096 x 4096, bf16 / fp32 lhs: a
+    // pass 10.2 / 15.9, the GEMM at 65 .. 256 rows 24 .. 28 / 23 .. 35; 14336 x 4096: a pass 13.0 / 19.6, the GEMM 30 .. 48 / 43 .. 77.
+    const bool f32 = lhs_dtype == QMM_F32, twin = qmm::gemm_gptq_twin(lhs_dtype, m);
+    const int64_t me = twin ? 2 * m : m;
+    const int ks = qmm::gemm_gptq_k_shares(me, n, k);
+    const double tiles = (double)((me + 127) / 128) * (double)((n + 255) / 256);
+    const double rounds = (double)(int64_t)((tiles * ks + 255.0) / 256.0);
+    const double gemm_us = rounds * ((double)k / 4096.0) * 64.0 / ks * (f32 && !twin ? 2.1 : 1.0) + (twin || ks > 1 ? 14.0 : 0.0);
+    const double pass_us = (f32 ? 12.0 : 8.0) + (double)n * (double)k * 0.52 / (f32 ? 3.8e6 : 6.0e6) + (k > 4096 ? 2.0 : 0.0);
     return (double)((m + 15) / 16) * pass_us < gemm_us;
 }
 

@@ -12,7 +12,7 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_lanes_rows, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_twin_rows, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, gptq_k_shares, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
 // Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 // False while qmm_matmul_static serves a problem whose one-pass treatment of an fp32 lhs (the lhs as twice the rows, the
@@ -156,6 +156,7 @@ hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w,
 bool gemm_gptq_supported(int64_t k, int group);
 int64_t gemm_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k);
 bool gemm_gptq_twin(int lhs_dtype, int64_t m);  // an fp32 lhs goes through the GEMM as one lhs of twice the rows
+int gemm_gptq_k_shares(int64_t m, int64_t n, int64_t k);  // K shares per tile of the GEMM (m: the rows it sees)
 hipError_t launch_gemm_gptq(const void* lhs, int lhs_dtype, const uint32_t* qweight, const uint16_t* scales,
                             const uint32_t* qzeros, int64_t m, int64_t n, int64_t k, int group, float* out,
                             void* workspace, hipStream_t s);
