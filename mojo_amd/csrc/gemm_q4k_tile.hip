@@ -463,8 +463,11 @@ bool gemm_q4_k_tile_wanted(int64_t m, int64_t n, int64_t k) {
     static const bool force = getenv("QMM_Q4K_TILE") != nullptr && atoi(getenv("QMM_Q4K_TILE")) == 1;
     if (k % 256 || k < 256 || kernel_disabled("q4k_tile")) return false;
     if (force) return m > 16;
+    // (one round of tiles takes 72 .. 78 us at K = 4096 however many there are; the GEMM with 64-row tiles, microseconds
+    // against this kernel's: 512 x 14336, 224 tiles, 86.5 / 78.5; 512 x 11008, 172 tiles, 80.5 / 72.5; 768 x 8192, 192 tiles,
+    // 80.5 / 73.8; 512 x 8192, 128 tiles, 57.8 / 71.9)
     const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
-    return m > 128 && tiles >= 256;
+    return m > 128 && tiles >= 160;
 }
 
 int64_t gemm_q4_k_tile_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes; }
