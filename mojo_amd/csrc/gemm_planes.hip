@@ -1354,14 +1354,16 @@ hipError_t launch_repack_planes(int encoding, const uint8_t* w, int64_t n, int64
 // With the conversion out of the way the plane GEMMs pay from fewer rows on than inside qmm_matmul.
 // 14336 x 4096: Q5_K 40 lhs rows 39.5 us against 52 us for three passes of the small-batch kernel, Q6_K 53 us against 44 / 66 us
 // for two / three passes of its decode kernel; 4096 x 4096: Q5_K 36 us against 30 us (48 rows) / 40 us (64), Q6_K 45 against 38 / 53.
-// Q4_K against its kernels that unpack as they go: 14336 x 4096, 160 / 256 / 512 rows 53 / 62 / 75 against 68 / 78 / 88 us;
-// 4096 x 4096, 256 / 512 / 1024 rows 41 / 49 / 63 against 35 / 59 / 60 us; 4096 x 14336, 256 / 512 / 1024: 104 / 114 / 159 against 81 / 116 / 180.
+// (Q4_K: below.)
 bool repacked_planes_wanted(int encoding, int64_t m, int64_t n, int64_t k) {
     if (k % 256 || k < 256) return false;
     if (encoding == QMM_Q6_K || encoding == QMM_Q5_K) return m > 48 || (m > 32 && n * k >= ((int64_t)48 << 20));
     if (encoding != QMM_Q4_K) return false;
+    // Against qmm_matmul's kernels that unpack as they go, bf16 lhs, microseconds (those / the planes): 4096 x 4096 with 384 / 1024 /
+    // 2048 rows (64 / 128 / 256 tiles) 37 / 47, 59 / 64, 92 / 86; 14336 x 4096 with 256 / 384 rows (112 / 224 tiles) 59 / 62, 79 / 76;
+    // 4096 x 14336 with 512 / 768 rows (64 / 96 tiles) 102 / 108, 153 / 134; 1024 x 4096 with 2048 rows (64 tiles) 45 / 54.
     const int64_t tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
-    return m > 128 && tiles >= 64;
+    return m > 128 && (tiles >= 200 || (k >= 8192 && tiles >= 96));
 }
 static int64_t repacked_lhs_bytes(int encoding, int lhs_dtype, int64_t m, int64_t k) {
     return (lhs_planes(nullptr, lhs_dtype, m, k, TM, (int64_t)repacked_blocks_per_tile(encoding, k) * 256).bytes + 255) / 256 * 256;
