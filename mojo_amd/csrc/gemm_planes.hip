@@ -1052,10 +1052,7 @@ WideLaunch wide_launch(float* out, int64_t m, int64_t n, int blocks_walked) {
     L.tiles_m = (int)((m + TM - 1) / TM);
     L.tiles_n128 = (int)((n + TN - 1) / TN);
     const int total = L.tiles_m * L.plan.wide_strips, per_xcd = (total + 7) / 8, per_xcd_cus = std::max(1, cus / 8);
-    // Tiles for at most a quarter of the compute units (GPTQ planes kept across calls, few lhs rows): a workgroup per compute
-    // unit, every tile cut in two K halves (4096 x 4096 with 512 rows: 90 -> 60 us; from 112 tiles on the halves lose:
-    // 14336 x 4096 with 512 rows 90 -> 99 us).
-    L.wg = 8 * (total <= 64 && blocks_walked >= 2 ? per_xcd_cus : std::min(per_xcd, per_xcd_cus));
+    L.wg = 8 * std::min(per_xcd, per_xcd_cus);
     L.z = split_tiles(out, m, n, L.tiles_m, L.plan.wide_strips, blocks_walked, L.wg, 2 * TN);
     if (L.plan.narrow_strips) L.z.max_split = 0;
     return L;
@@ -1446,12 +1443,11 @@ hipError_t launch_repack_gptq(const uint32_t* qweight, const uint16_t* scales, c
                                                                                     nullptr, (int)k, 0, LhsPlanes{}, z);
     return hipGetLastError();
 }
-// Against the GEMM that unpacks as it goes (and the small-batch kernel's passes of 16 rows up to 64 rows): 14336 x 4096 with 128 /
-// 256 rows 58 / 69 against 69 / 71 us, 4096 x 4096 with 256 / 512 / 1024 rows 53 / 60 / 74 against 69 / 72 / 74, 4096 x 14336 with
-// 256 / 1024 rows 147 / 173 against 215 / 228; between 65 and 159 tiles the wide tiles lose (14336 x 4096 with 512 rows: 90 against 73 us).
+// Against the GEMM that unpacks as it goes, whose few tiles are cut into K shares (bf16 lhs, microseconds, that GEMM / the planes):
+// 14336 x 4096 with 512 / 1024 / 2048 rows 74 / 74, 129 / 107, 228 / 205; 4096 x 4096 with 256 / 1024 / 2048 rows 31 / 55, 57 / 76,
+// 83 / 83; 4096 x 14336 with 256 / 2048 rows 55 / 149, 263 / 262: the planes serve the problems with enough 256 x 256 tiles.
 bool repacked_gptq_wanted(int64_t m, int64_t n) {
-    const int64_t tiles = ((m + TM - 1) / TM) * ((n + 2 * TN - 1) / (2 * TN));
-    return (m > 256 && wide_tiles(QMM_GPTQ, m, n)) || (m > 96 && tiles <= 64 && !kernel_disabled("planes_wide"));
+    return m > 256 && wide_tiles(QMM_GPTQ, m, n);
 }
 int64_t repacked_gptq_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) { return (lhs_planes(nullptr, lhs_dtype, m, k, TM).bytes + 255) / 256 * 256; }
 hipError_t launch_gemm_gptq_repacked(const void* lhs, int lhs_dtype, const void* packed, int64_t m, int64_t n, int64_t k, int group, float* out,

@@ -84,7 +84,7 @@ def test_repacked_kquant_matches_oracle_and_qmatmul(enc, n, k, rows):
 def test_repacked_gptq_matches_oracle_and_qmatmul(group, n, k, rows):
     """GPTQ planes (q - zero, scale blocks = groups) made once; groups with a zero scale; one and two launches of the wide GEMM, a
     last round of tiles cut in K halves (1536 x 11016), K ending on half a 256-block; few tiles (300 and 120 x 4104: 34 and 17
-    tiles of 256 x 256, every one cut in K halves) where qmatmul takes its GEMM that unpacks as it goes."""
+    tiles of 256 x 256), which the kept planes leave to qmatmul's GEMM that unpacks as it goes (tiles cut into K shares)."""
     w, _ = synth(21, n, k, 1)
     qw, sc, qz, gi = O.quantize_gptq(w, group)
     sc[::2, ::7] = 0
