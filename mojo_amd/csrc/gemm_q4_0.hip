@@ -587,8 +587,11 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
                             float* out, void* workspace, hipStream_t s) {
     const LhsQ8T p = lhs_q8t(workspace, m, k);
     const int64_t tiles = (m + 15) / 16, ngroups = tiles * 16 * (k / 32);
-    // Up to 16 lhs rows: the weights are read once and the kernel lives on HBM latency (gemm_q4_0_small_kernel).
-    const bool small = tiles == 1 && k % 256 == 0 && !kernel_disabled("q4_0_small");
+    // Up to 16 lhs rows a pass: the weights are read once per pass and the kernel lives on HBM latency (gemm_q4_0_small_kernel).
+    // More rows go in passes of 16 (the plane GEMM takes over where it is faster, see gemm_q4_0_planes_wanted): a pass costs 10.6 /
+    // 12.8 / 16.0 us on 4096 x 4096 / 14336 x 4096 / 4096 x 14336, the 17..64-row kernel below 20 / 33 / 57 us up to 32 rows
+    // and 49 / 56 / 165 up to 64.
+    const bool small = k % 256 == 0 && !kernel_disabled("q4_0_small") && (tiles == 1 || !kernel_disabled("q4_0_small_passes"));
     dim3 qgrid((unsigned)((ngroups * 32 + 255) / 256)), qblock(256);
 #define QMM_Q8_OPERAND(T_, W_)                                                                                        \
     quantize_q8_0_operand_kernel<T_, W_><<<qgrid, qblock, 0, s>>>((const T_*)lhs, (int)m, (int)k, ngroups, p.codes, p.scale, p.sum)
@@ -619,7 +622,12 @@ hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, in
         // tiles are dealt round robin: one workgroup per compute unit until that means more than kSMaxTiles each
         const int64_t ntiles = (n + 15) / 16;
         const int64_t wgs = std::min<int64_t>(ntiles, std::max<int64_t>(cus, (ntiles + kSMaxTiles - 1) / kSMaxTiles));
-        gemm_q4_0_small_kernel<<<dim3((unsigned)wgs), dim3(64 * kSWaves), kSLds, s>>>(w, p.codes, p.scale, out, (int)m, (int)n, (int)k);
+        const int64_t nkb = k / 32;
+        for (int64_t t = 0; t < tiles; t++) {  // (codes 512 bytes, records 64 bytes per lhs tile and block)
+            gemm_q4_0_small_kernel<<<dim3((unsigned)wgs), dim3(64 * kSWaves), kSLds, s>>>(
+                w, p.codes + t * nkb * 512, (const float*)((const char*)p.scale + t * nkb * 64), out + t * 16 * n,
+                (int)std::min<int64_t>(16, m - 16 * t), (int)n, (int)k);
+        }
         return hipGetLastError();
     }
     if (tiles > 4 && !kernel_disabled("q4_0_wide")) {

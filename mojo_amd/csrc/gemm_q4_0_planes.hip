@@ -413,11 +413,14 @@ bool gemm_q4_0_planes_wanted(int64_t m, int64_t n, int64_t k) {
     static const bool force = getenv("QMM_Q4_0_PLANES") != nullptr && atoi(getenv("QMM_Q4_0_PLANES")) == 1;
     if (k % 256 || k < 256 || kernel_disabled("q4_0_planes")) return false;
     if (force) return m > 16;
-    // Measured against the int8 kernels on 1024..14336 x 4096..14336 weights: faster from 80 lhs rows on at every size
-    // (80 rows: 112 against 169 us on 14336 x 4096; 2048 rows: 359 against 674 us); on small matrices from 33 rows on, where the
-    // int8 kernel takes a third 16-row tile per workgroup (4096 x 4096: 33 / 64 rows 43 / 49 us against 38 for the planes; 14336 x
-    // 4096: 54 / 56 against 90).
-    return m > 64 || (m > 32 && n * k <= ((int64_t)24 << 20));  // (8192 x 4096: 33 / 64 rows 46 / 50 against 52 / 56 us)
+    // Against passes of the 16-row int8 kernel (one launch that quantises the lhs, then a launch per 16 rows), both in microseconds
+    // as fitted on this part (W: millions of weights).  Measured, 16 / 32 / 64 rows in passes and the planes at 65 rows: 4096 x 4096
+    // 11.4 / 15.6 / 23.9 and 38; 14336 x 4096 12.8 / 22.4 / 41.3 and 90; 4096 x 14336 16.0 / 30.3 / 58.0 and 118; 1024 x 4096
+    // 8.2 / 13.0 / 22 and 33.
+    const double W = (double)n * (double)k * 1e-6;
+    const double passes_us = 3.5 + (double)((m + 15) / 16) * (4.5 + 0.082 * W + (k > 4096 ? 3.0 : 0.0));
+    const double planes_us = 28.0 + 1.0 * W + (k > 4096 ? 28.0 : 0.0) + 0.02 * (double)m;
+    return m > 16 && passes_us > planes_us;
 }
 
 int64_t gemm_q4_0_planes_workspace_bytes(int64_t m, int64_t n, int64_t k);

@@ -317,7 +317,7 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     if (m <= 0 || k <= 0) return 0;
     if (kquant_planes(encoding, lhs_dtype, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (encoding == QMM_Q4_0) {
-        const int64_t a = q8_planes(nullptr, m, k).bytes, b = m >= 5 && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
+        const int64_t a = q8_planes(nullptr, m, k).bytes, b = (m >= 5 || k > 8192) && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         const int64_t c = qmm::gemm_q4_0_planes_wanted(m, n, k) ? qmm::gemm_q4_0_planes_workspace_bytes(m, n, k) : 0;
         return std::max(std::max(a, b), c);
     }
@@ -453,7 +453,11 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
                               "qmm_matmul(GPTQ GEMM)");
         // one pass of the matrix-core small-batch kernel per 16 lhs rows; one row, and two fp32 rows, go to the column
         // kernel (two rows on 14336 x 4096: 12.3 us with a bf16 lhs, 16 us with an fp32 lhs, column kernel 16.5 us)
-        const int mm_min = lhs_dtype == QMM_F32 ? 3 : 2;
+        // a K past 8192: the column kernel walks K with one workgroup per 64 columns, the small-batch kernel splits it
+        // (4096 x 14336, one row: 18.2 -> 13.3 us bf16, 18.2 -> 16.4 us fp32; two fp32 rows 27.5 -> 17.3 us; at K = 8192 the
+        // column kernel still wins on wide matrices: 8192 x 8192 12.3 against 14.0 us)
+        const bool long_k = k > 8192 && !qmm::kernel_disabled("gptq_long_k_mm");
+        const int mm_min = long_k ? 1 : (lhs_dtype == QMM_F32 ? 3 : 2);
         for (int64_t m0 = 0; m0 < m; m0 += 16) {
             int mt = (int)(m - m0 < 16 ? m - m0 : 16);
             bool handled = false;
@@ -539,7 +543,8 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     }
     if (encoding == QMM_Q4_0 && qmm::gemm_q4_0_planes_wanted(m, n, k))
         return hip_status(qmm::launch_gemm_q4_0_planes(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 plane GEMM)");
-    if (encoding == QMM_Q4_0 && m >= 5 && !qmm::kernel_disabled("q4_0_mfma"))
+    // (two rows and more on a K beyond what the decode kernel takes: the matrix-core kernel too, 4096 x 14336 with 4 rows 32 -> 16 us)
+    if (encoding == QMM_Q4_0 && (m >= 5 || (m >= 2 && k > 8192 && k % 256 == 0)) && !qmm::kernel_disabled("q4_0_mfma"))
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0 && m <= 4) {
         // decode: the kernel that quantises the lhs itself (takes K <= 8192)
@@ -759,10 +764,12 @@ int qmm_repack(int encoding, const qmm_gptq_config* cfg, const void* const* rhs,
 }
 
 // Does a call with these rows go through the planes?  Without the packed tensors every row count does.
-constexpr int64_t kQ40RepackedMinRows = 48;  // 14336 x 4096: the plane GEMM 55 us, the int8 kernels 57 us at 48 rows, 59 at 64 (4096 x 4096: 49 against 52 at 64)
+// Q4_0: passes of the 16-row int8 kernel against the kept planes.  4096 x 4096: 28 us against 35 at 64 rows, 41 against 37 at 96;
+// 4096 x 14336: 57 against 83 at 64 rows, 84 against 84 at 96.
+static int64_t q4_0_repacked_min_rows(int64_t k) { return k > 4096 ? 96 : 80; }
 static bool repacked_path(int encoding, int64_t m, int64_t n, int64_t k, bool have_rhs) {
     if (!have_rhs) return true;
-    if (encoding == QMM_Q4_0) return m > kQ40RepackedMinRows;
+    if (encoding == QMM_Q4_0) return m > q4_0_repacked_min_rows(k);
     return encoding == QMM_GPTQ ? qmm::repacked_gptq_wanted(m, n) : qmm::repacked_planes_wanted(encoding, m, n, k);
 }
 

@@ -212,12 +212,14 @@ def _integer_dot_case(m, n, k, one_hot, bf16, seed):
 
 
 # (m, n, k) -> kernel: 1, 4: the decode kernel that quantises the lhs itself; K = 8224: the first-version decode kernel
-# behind the stand-alone quantiser; 5, 16: small-batch int8 matrix-core kernel; 9 with K % 256 != 0, 33, 64: the
-# 16-row-tile kernel (1, 4 tiles per group); 65, 256: the plane GEMM on the fp16 matrix cores (K = 1024, 4096)
+# behind the stand-alone quantiser; 5, 16: small-batch int8 matrix-core kernel, which also serves 33, 64 and 65 rows in
+# passes of 16 (a last pass of one row) and 3 rows on a K past 8192; 9 and 40 with K % 256 != 0: the 16-row-tile kernel
+# (1, 3 tiles per group); 256: the plane GEMM on the fp16 matrix cores
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("one_hot", [True, False])
 @pytest.mark.parametrize("m,n,k", [(1, 200, 4096), (4, 200, 4096), (2, 70, 8224), (5, 200, 4096), (16, 200, 4096),
-                                   (9, 72, 1056), (33, 200, 1024), (64, 72, 4096), (65, 200, 1024), (256, 136, 4096)])
+                                   (9, 72, 1056), (33, 200, 1024), (64, 72, 4096), (65, 200, 1024), (256, 136, 4096),
+                                   (3, 72, 16384), (40, 72, 1056)])
 def test_q4_0_production_kernels_give_the_integer_block_dots(m, n, k, one_hot, bf16):
     """The int8 block dots of every Q4_0 matmul kernel, read off its fp32 output, equal the oracle's bit for bit
     (Q8_0 codes with .5 ties included)."""
@@ -251,10 +253,13 @@ def test_q4_0_decode_shapes(m, n, k, lhs_bf16):
 
 
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(16, 5000, 4096, False), (9, 300, 512, False), (12, 64, 14336, True),
-                                            (5, 4100, 256, False), (16, 16400, 2048, True)])
+                                            (5, 4100, 256, False), (16, 16400, 2048, True), (37, 300, 1024, False),
+                                            (64, 5000, 4096, True), (81, 4100, 2048, False), (3, 200, 14336, False),
+                                            (2, 130, 16384, True)])
 def test_q4_0_small_batch(m, n, k, lhs_bf16):
     """5..16 lhs rows, K a multiple of 256: several 16-row tiles per workgroup, ragged last tile, groups of K in
-    which only some wavefronts have a share."""
+    which only some wavefronts have a share.  More rows go through the same kernel in passes of 16 while that beats making
+    the planes (37: a last pass of five rows; 81: of one), and so do 2..4 rows on a K past 8192."""
     w, a = synth(53, n, k, m)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
@@ -375,11 +380,13 @@ def test_non_finite_lhs_values_stay_in_their_row(enc, m):
 @pytest.mark.parametrize("m,n,k,group,bf16", [
     (2, 72, 256, 128, False), (5, 1000, 1024, 128, False), (8, 8, 4096, 64, False), (13, 136, 4096, 256, True),
     (16, 520, 8192, 128, False), (16, 200, 14336, 128, True), (7, 264, 4352, 64, False), (3, 2048, 2048, 256, True),
-    (33, 96, 4096, 128, False)])
+    (33, 96, 4096, 128, False), (1, 264, 14336, 128, True), (1, 200, 8448, 64, False), (2, 136, 12288, 128, False)])
 def test_gptq_small_batch(m, n, k, group, bf16):
     """2 to 16 lhs rows (and 33 as passes) through the matrix-core small-batch kernel: one to sixteen wavefronts of
     256 k each, K beyond 4096 as launches that add to the output (8192 = 2 x 16, 14336 = 3 x 16 + 8, 4352 = 16 + 1
-    wavefronts), ragged N, N of eight columns, arbitrary zero points, lhs rows of very different magnitude."""
+    wavefronts), ragged N, N of eight columns, arbitrary zero points, lhs rows of very different magnitude.  On a K
+    past 8192 the kernel also serves one row and two fp32 rows (the column kernel walks such a K with one workgroup
+    per 64 columns)."""
     w, a = synth(81, n, k, m)
     a[0] *= 1e-6
     a[m - 1] *= 3e4

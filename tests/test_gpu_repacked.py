@@ -100,24 +100,31 @@ def test_repacked_gptq_matches_oracle_and_qmatmul(group, n, k, rows):
             assert torch.equal(got, qmatmul(QE.GPTQ, cfg, lhs, *rhs)), f"GPTQ {m}x{n}x{k}: differs from qmatmul"
 
 
-@pytest.mark.parametrize("n,k,rows", [(300, 1024, [(70, True), (300, False), (16, True)]), (9300, 768, [(1000, True)]),
-                                      (1100, 2560, [(300, True), (70, False)])])
+@pytest.mark.parametrize("n,k,rows", [(300, 1024, [(70, True, True), (300, False, True), (16, True, True)]),
+                                      (9300, 768, [(1000, True, True)]), (1100, 2560, [(300, True, True), (70, False, True)]),
+                                      (2000, 1024, [(96, True, False), (96, False, False)])])
 def test_repacked_q4_0_matches_oracle_and_qmatmul(n, k, rows):
     """Q4_0: the plane of q - 8 and the block scales made once.  The lhs is quantised to Q8_0 per call as everywhere, so the
-    result is that of the integer block dots: bit-identical with qmatmul above 64 rows (same GEMM), within the bar of the
-    oracle's Q8_0 x Q4_0 product at every row count; without the packed tensor few rows run over the plane too.  1100 x 2560:
-    few tiles on ten groups of 256, cut in four K quarters that meet pairwise in two buffers."""
+    result is that of the integer block dots: bit-identical with qmatmul wherever both run the same kernel (the plane GEMM at
+    many rows, the 16-row int8 kernel at few), within the bar of the oracle's Q8_0 x Q4_0 product at every row count; without
+    the packed tensor few rows run over the plane too.  1100 x 2560: few tiles on ten groups of 256, cut in four K quarters
+    that meet pairwise in two buffers.  2000 x 1024 with 96 rows: the kept plane serves the call, while qmatmul, which would
+    have to make the plane first, takes six passes of the 16-row kernel (another order of the block sums)."""
     w, _ = synth(17, n, k, 1)
     wq = O.quantize(O.Q4_0, w)
     wq_d = gpu(wq)
     weights = repack_weights(QE.Q4_0, None, wq_d)
     alone = repack_weights(QE.Q4_0, None, wq_d, keep_rhs=False)
-    for m, bf16 in rows:
+    for m, bf16, same in rows:
         a, lhs = lhs_rows(60 + m, m, k, bf16)
         want = O.matmul_q4_0(a, wq)
         got = qmatmul_repacked(lhs, weights)
         assert_close(got, want, f"Q4_0 repacked {m}x{n}x{k} bf16={bf16}")
-        assert torch.equal(got, qmatmul(QE.Q4_0, None, lhs, wq_d)), f"Q4_0 {m}x{n}x{k}: differs from qmatmul"
+        per_call = qmatmul(QE.Q4_0, None, lhs, wq_d)
+        if same:
+            assert torch.equal(got, per_call), f"Q4_0 {m}x{n}x{k}: differs from qmatmul"
+        else:
+            assert_close(per_call, want, f"Q4_0 {m}x{n}x{k} bf16={bf16}")
         assert_close(qmatmul_repacked(lhs, alone), want, f"Q4_0 plane only {m}x{n}x{k}")
 
 
