@@ -1159,20 +1159,23 @@ bool gemm_planes_wanted(int encoding, int lhs_dtype, int64_t m, int64_t n, int64
     if (encoding == QMM_Q5_K && m > 32 && (k % 512 || k > 32768 || kernel_disabled("q5k_mm"))) return true;
     // The small-batch kernels take 16 bf16 or 8 fp32 rows a pass (up to 64 rows), the planes any number in one (an fp32 lhs as
     // twice the rows) behind a conversion.  Both sides in microseconds, fitted to this part (W: millions of weights; a K beyond
-    // 4096 costs the small-batch kernels a round per 4096 columns, each with its own narrowing of the lhs, and the planes the
-    // K shares of few tiles).  Measured, one pass / the planes at 65 rows, bf16 and fp32 lhs: Q5_K 4096 x 4096 9.6, 13.5 / 35, 46;
-    // 14336 x 4096 16.9, 20.4 / 85, 94; 4096 x 14336 34.2, 49.7 / 116, 118; Q6_K 12.5, 12.9 / 55, 69; 21.6, 20.8 / 134, 142;
-    // 46.4, 47.9 / 175, 175.
+    // 4096 costs the small-batch kernels a launch that adds the rounds of 4096 columns, and the planes the K shares of few
+    // tiles).  Measured, one pass / the planes at 65 rows, bf16 and fp32 lhs: Q5_K 4096 x 4096 9.6, 13.5 / 35, 46;
+    // 14336 x 4096 16.9, 20.4 / 85, 94; 4096 x 14336 20.2, 24.0 / 116, 118; Q6_K 12.5, 12.9 / 55, 69; 21.6, 20.8 / 134, 142;
+    // 24.4, 24.5 / 175, 175.
     const bool f32 = lhs_dtype == QMM_F32, long_k = k > 4096;
     const double W = (double)n * (double)k * 1e-6;
     const int64_t me = f32 ? 2 * m : m;  // rows of the plane GEMM (more than 128: two wavefront rows of a tile at work)
+    // (a long K: the planes pay for K shares, the more the fewer column tiles there are: at 65 bf16 rows, Q5_K / Q6_K,
+    // 4096 x 8192 65 / 100 us, 2048 x 16384 94 / 146, 4096 x 14336 116 / 175, 8192 x 14336 162 / 250)
+    const double k_over_n = (double)k / (double)n;
     double pass_us, planes_us;
     if (encoding == QMM_Q5_K) {
-        pass_us = (f32 ? 9.0 : 6.0) + W * (f32 ? 0.20 : 0.18) * (long_k ? (f32 ? 3.4 : 2.7) : 1.0);
-        planes_us = 12.0 + 1.15 * W + (f32 ? 4.0 : 0.0) + (me > 128 ? 8.0 : 0.0) + (long_k ? 30.0 : 0.0);
+        pass_us = (f32 ? 9.0 : 6.0) + W * (f32 ? 0.20 : 0.18) + (long_k ? 3.5 : 0.0);
+        planes_us = 12.0 + 1.15 * W + (f32 ? 4.0 : 0.0) + (me > 128 ? 8.0 : 0.0) + (long_k ? std::min(45.0, 9.0 * k_over_n) : 0.0);
     } else {
-        pass_us = (f32 ? 9.5 : 8.5) + W * (f32 ? 0.20 : 0.225) * (long_k ? (f32 ? 3.3 : 2.9) : 1.0);
-        planes_us = 25.0 + 1.85 * W + (f32 ? 2.0 : 0.0) + (me > 128 ? 14.0 : 0.0) + (long_k ? 40.0 : 0.0);
+        pass_us = (f32 ? 9.5 : 8.5) + W * (f32 ? 0.20 : 0.225) + (long_k ? 3.0 : 0.0);
+        planes_us = 25.0 + 1.85 * W + (f32 ? 2.0 : 0.0) + (me > 128 ? 14.0 : 0.0) + (long_k ? std::min(60.0, 11.0 * k_over_n) : 0.0);
     }
     const int64_t passes = (m + (f32 ? 8 : 16) - 1) / (f32 ? 8 : 16);
     return m > 64 || (double)passes * pass_us > planes_us;

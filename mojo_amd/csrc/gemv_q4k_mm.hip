@@ -68,7 +68,10 @@ __device__ __forceinline__ half8 zero_half8() { return pack4(0u, 0u, 0u, 0u); }
 // inv come from prep_lhs_kernel<.., kLhsOrderQ4K16>.
 // MROWS (INLINE): lhs rows converted, 1, 2, 4 or 8 (>= m; rows past m repeat the last one and their results are dropped).
 // PLAIN: one matrix, known at compile time: no matrix lookup per item, a short argument block.
-template <int NPART, bool INLINE, int MROWS, typename AT, bool PLAIN>
+// KPART (with PLAIN): the workgroup takes group blockIdx.y of K only and stores its result as part blockIdx.y of
+// [groups][m][n] at the output pointer (the caller adds the parts in group order): few tiles on a long K then make one
+// workgroup per (share of the tiles, group), which converts its lhs operands once for several tiles.
+template <int NPART, bool INLINE, int MROWS, typename AT, bool PLAIN, bool KPART = false>
 __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict__ a, const _Float16* __restrict__ a16,
                                         const _Float16* __restrict__ a16_lo, const _Float16* __restrict__ asum,
                                         const float* __restrict__ inv, int m, int k) {
@@ -90,8 +93,10 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
     const int n_first = mats.n[0];
     const int my_tiles = min(kMaxTiles, (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x);
     // group g is super-blocks [16 g, 16 g + 16): two per wavefront, or, when 8 or fewer are left, one
-    const int ngrp = (nblk + kRunBlk * kWaves - 1) / (kRunBlk * kWaves);
-    const int total = ngrp * my_tiles;
+    const int ngrp_all = (nblk + kRunBlk * kWaves - 1) / (kRunBlk * kWaves);
+    const int grp0 = KPART ? (int)blockIdx.y : 0;          // first group of this workgroup
+    const int ngrp = KPART ? grp0 + 1 : ngrp_all;          // one past its last
+    const int total = (ngrp - grp0) * my_tiles;
     auto group_share = [&](int g, int& first, int& cnt) {
         const int left = nblk - kRunBlk * kWaves * g;  // > 0
         const int per = left > kWaves ? kRunBlk : 1;
@@ -122,7 +127,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
         x_after = last_issued;
     };
     if constexpr (INLINE) {
-        if (total > 0) load_x(0);
+        if (total > 0) load_x(grp0);
     }
     // piece p = lane + 64 i of an item: row p / 18, 16-byte piece p % 18
     int prow[kLoads], pidx[kLoads];
@@ -157,7 +162,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
     };
 
     // items in flight: it + 1 and it + 2
-    int ig = 0, it_t = 0, islot = 0;  // next item to issue
+    int ig = grp0, it_t = 0, islot = 0;  // next item to issue
     auto issue_next = [&]() {
         issue(ig, it_t, islot);
         last_issued++;
@@ -190,7 +195,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
                 for (int q = 0; q < NPART; q++) fa[bb][p][h][q] = zero_half8();
     }
 
-    int grp = 0, ti = 0, slot = 0;
+    int grp = grp0, ti = 0, slot = 0;
     for (int it = 0; it < total; it++) {
         int gb0, nb;
         group_share(grp, gb0, nb);
@@ -302,7 +307,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
                     };
                     // First group: only item 0 is in flight (slot 0), slots 1 and 2 take both super-blocks at once.  Later
                     // groups have one free slot (the next item's): one super-block at a time.
-                    const bool both = grp == 0;
+                    const bool both = grp == grp0;
                     uint8_t* area = both ? ring + kSlotBytes : stg;
                     float* scales = (float*)(area + (both ? kRunBlk : 1) * RP * kStageBytes);
                     static_assert(kRunBlk == 2, "the staging below is written for two super-blocks");
@@ -414,7 +419,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
         // this wavefront's running sum of the tile over its groups
         float* mine = accs + ((wave * kMaxTiles + ti) * 4) * 64 + lane;
 #pragma unroll
-        for (int r = 0; r < 4; r++) mine[r * 64] = grp == 0 ? acc[r] : mine[r * 64] + acc[r];
+        for (int r = 0; r < 4; r++) mine[r * 64] = grp == grp0 ? acc[r] : mine[r * 64] + acc[r];
 
         slot = slot == kSlots - 1 ? 0 : slot + 1;
         if (++ti == my_tiles) { ti = 0; grp++; }
@@ -425,7 +430,7 @@ __device__ __forceinline__ void mm_body(const MmMats& mats, const AT* __restrict
         const int t = pr >> 2, r = pr & 3;
         const int tile = (int)blockIdx.x + t * (int)gridDim.x;
         int n = n_first, tile0 = 0;
-        float* out = out_first;
+        float* out = KPART ? out_first + (int64_t)grp0 * m * n_first : out_first;
         if (!single) {
             int j = 0;
             while (j + 1 < mats.count && tile >= mats.tile_end[j]) j++;
@@ -454,7 +459,7 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_kernel(const MmMats mats, co
 }
 
 // The plain call with up to 8 lhs rows: one matrix [n, k], lhs converted in the kernel.  Nine dwords of arguments.
-template <int MROWS, typename AT>
+template <int MROWS, typename AT, bool KPART = false>
 __global__ __launch_bounds__(512) void gemv_q4_k_mm_plain_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
                                                                  float* __restrict__ out, int n, int m, int k) {
     asm volatile("" ::"s"(w), "s"(a), "s"(out), "s"(n), "s"(m), "s"(k));  // (all arguments in the first batch of scalar loads)
@@ -467,16 +472,51 @@ __global__ __launch_bounds__(512) void gemv_q4_k_mm_plain_kernel(const uint8_t* 
         mats.tile_end[j] = (n + 15) >> 4;
     }
     mats.count = 1;
-    mm_body<1, true, MROWS, AT, true>(mats, a, nullptr, nullptr, nullptr, nullptr, m, k);
+    mm_body<1, true, MROWS, AT, true, KPART>(mats, a, nullptr, nullptr, nullptr, nullptr, m, k);
 }
+
+namespace {
+// Up to 8 lhs rows, few tiles, a K beyond 4096: the groups of K side by side in the grid (KPART).  Measured, 4096 x 14336 with
+// 4 fp32 rows: one workgroup per tile that walks the 3.5 groups and converts the lhs for each 16.3 us.
+struct KParts {
+    int groups;       // 1: not wanted
+    int64_t per, gx;  // tiles per workgroup, workgroups across the tiles
+};
+KParts k_parts(int lhs_dtype, int64_t m, int64_t n, int64_t k, int cus) {
+    const int64_t ntiles = (n + 15) / 16, groups = (k / 256 + kRunBlk * kWaves - 1) / (kRunBlk * kWaves);
+    const KParts none = {1, 0, 0};
+    if (m < 2 || m > 8 || groups < 2 || ntiles > cus || kernel_disabled("q4k_mm_k_parts")) return none;
+    const bool heavy = m > 4 && lhs_dtype == QMM_F32;  // eight fp32 rows: the conversion is two thirds of a workgroup's time
+    // two groups: the launch that adds the parts costs what one conversion of up to four rows saves (4096 x 8192, 4 rows: 10.4
+    // against 9.8 us; 8 fp32 rows 13.0 against 14.0)
+    if (groups == 2 && !heavy) return none;
+    // One workgroup per compute unit at most (a few more would run behind all the others), and nearly all of them in use:
+    // 4096 x 14336 (64 x 4 workgroups of 4 tiles) 4 rows 16.3 -> 13.5 us, 2048 x 16384 16.7 -> 10.0; but 4096 x 11008
+    // (64 x 3 of 4 tiles) 13.1 -> 14.3, with 8 fp32 rows 19.3 -> 16.7.
+    const int64_t across = std::max<int64_t>(1, cus / groups), per = (ntiles + across - 1) / across;
+    if (per > kMaxTiles) return none;
+    const int64_t gx = (ntiles + per - 1) / per;
+    if (gx * groups * 10 < (int64_t)cus * (heavy ? 7 : 9)) return none;
+    return {(int)groups, per, gx};
+}
+}  // namespace
 
 int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k) {
     return m <= 8 ? 0 : lhs_planes(nullptr, lhs_dtype, m, k).bytes;
 }
 
+// The plain call (launch_gemv_q4_k_mm): with up to 8 rows, the parts of K of a matrix of few tiles (on a part of 256 compute
+// units; the launch does not cut K on any other).
+int64_t gemv_q4_k_mm_plain_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    if (m > 8) return gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k);
+    const int groups = k_parts(lhs_dtype, m, n, k, 256).groups;
+    return groups > 1 ? (int64_t)groups * m * n * 4 : 0;
+}
+
 // count matrices [ns[j], k] that share the lhs (count = 1: the plain call); out[j] is fp32 [m, ns[j]], dense.
+// k_parts_ok: the workspace holds gemv_q4_k_mm_plain_workspace_bytes (the plain call only).
 hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
-                                       float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s) {
+                                       float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s, bool k_parts_ok) {
     if (count < 1 || count > kLanesMaxMats) return hipErrorInvalidValue;
     MmMats mats;
     int64_t ntiles = 0;
@@ -507,6 +547,13 @@ hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count
             e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
             if (e != hipSuccess) return e;
         }
+        const void* kfns[6] = {(const void*)gemv_q4_k_mm_plain_kernel<2, float, true>, (const void*)gemv_q4_k_mm_plain_kernel<4, float, true>,
+                               (const void*)gemv_q4_k_mm_plain_kernel<8, float, true>, (const void*)gemv_q4_k_mm_plain_kernel<2, uint16_t, true>,
+                               (const void*)gemv_q4_k_mm_plain_kernel<4, uint16_t, true>, (const void*)gemv_q4_k_mm_plain_kernel<8, uint16_t, true>};
+        for (const void* fn : kfns) {
+            e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return e;
+        }
         const void* fns[10] = {(const void*)gemv_q4_k_mm_kernel<1, true, 1, float>, (const void*)gemv_q4_k_mm_kernel<1, true, 2, float>,
                                (const void*)gemv_q4_k_mm_kernel<1, true, 4, float>, (const void*)gemv_q4_k_mm_kernel<1, true, 8, float>,
                                (const void*)gemv_q4_k_mm_kernel<1, true, 1, uint16_t>, (const void*)gemv_q4_k_mm_kernel<1, true, 2, uint16_t>,
@@ -525,6 +572,27 @@ hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count
     dim3 grid((unsigned)wgs), block(64 * kWaves);
     if (m <= 8) {
         const bool plain = count == 1 && !kernel_disabled("q4k_mm_plain");
+        // few tiles on a long K: a workgroup per (share of the tiles, group of K), the groups' results added by a launch of
+        // their own in group order
+        const KParts kp = plain && k_parts_ok && workspace && cus == 256 ? k_parts(lhs_dtype, m, ns[0], k, cus) : KParts{1, 0, 0};
+        const int groups = kp.groups;
+        if (groups > 1) {
+            const dim3 kgrid((unsigned)kp.gx, (unsigned)groups);
+            float* part = (float*)workspace;
+#define QMM_MM_KPART(MR_)                                                                                             \
+    do {                                                                                                              \
+        if (lhs_dtype == QMM_F32)                                                                                     \
+            gemv_q4_k_mm_plain_kernel<MR_, float, true><<<kgrid, block, kLdsBytes, s>>>(ws[0], (const float*)lhs, part, (int)ns[0], (int)m, (int)k); \
+        else                                                                                                          \
+            gemv_q4_k_mm_plain_kernel<MR_, uint16_t, true><<<kgrid, block, kLdsBytes, s>>>(ws[0], (const uint16_t*)lhs, part, (int)ns[0], (int)m, (int)k); \
+    } while (0)
+            if (m == 2) QMM_MM_KPART(2);
+            else if (m <= 4) QMM_MM_KPART(4);
+            else QMM_MM_KPART(8);
+#undef QMM_MM_KPART
+            e = hipGetLastError();
+            return e != hipSuccess ? e : launch_sum_shares(part, outs[0], m * ns[0], groups, s);
+        }
 #define QMM_MM_INLINE(MR_)                                                                                            \
     do {                                                                                                              \
         if (plain && lhs_dtype == QMM_F32)                                                                            \
@@ -557,7 +625,7 @@ hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count
 
 hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                float* out, void* workspace, hipStream_t s) {
-    return launch_gemv_q4_k_mm_grouped(lhs, lhs_dtype, 1, &w, &n, &out, m, k, workspace, s);
+    return launch_gemv_q4_k_mm_grouped(lhs, lhs_dtype, 1, &w, &n, &out, m, k, workspace, s, true);
 }
 
 }  // namespace qmm

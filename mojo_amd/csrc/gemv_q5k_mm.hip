@@ -84,8 +84,10 @@ __device__ __forceinline__ void v_stream16_to_lds(uint32_t lane_offset, const vo
 // bf16 rows need no residual rows and are one set (sixteen fp32 rows would be two sets of eight, each with its own operands
 // and sums; the launcher does not use that: it spills).  A lane holds rows 4 (lane / 16) + r of a set; accumulator registers
 // that hold no wanted lhs row are not computed.
-// ROUNDS: K beyond 4096, walked in rounds of 16 super-blocks; without it everything about rounds is constant.
-template <int MROWS, typename AT, bool ROUNDS>
+// ROUNDS: K other than 4096 in rounds of 16 super-blocks; 0: a single whole round, everything about rounds is constant; 1: the
+// workgroup walks the rounds one after the other and adds to its own output; 2: round blockIdx.y only, its result stored as
+// part blockIdx.y of [rounds][m][ldo] at `out` (the caller adds the parts in round order).
+template <int MROWS, typename AT, int ROUNDS>
 __global__ __launch_bounds__(64 * kVWaves) void gemv_q5_k_mm_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
                                                                    float* __restrict__ out, int m, int n, int k, int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -135,7 +137,8 @@ __global__ __launch_bounds__(64 * kVWaves) void gemv_q5_k_mm_kernel(const uint8_
     int it = 0;  // tiles done, over all rounds: its parity picks the buffer of the partial results
 
     const int rounds = ROUNDS ? (nblk + 15) >> 4 : 1;
-    for (int round = 0; round < rounds; round++) {
+    const int round0 = ROUNDS == 2 ? (int)blockIdx.y : 0, round1 = ROUNDS == 2 ? round0 + 1 : rounds;
+    for (int round = round0; round < round1; round++) {
     const bool have = ROUNDS ? 16 * round + 2 * wave < nblk : true;            // this wavefront has super-blocks in the round
     const int nw = ROUNDS ? min(kVWaves, (nblk - 16 * round) >> 1) : kVWaves;  // wavefronts that have
     if (have && my_tiles > 0) issue(round, 0, 0);
@@ -307,8 +310,8 @@ __global__ __launch_bounds__(64 * kVWaves) void gemv_q5_k_mm_kernel(const uint8_
             for (int ww = 0; ww < kVWaves; ww++)
                 if (ww < nw) v += HI16 ? src[ww * 512] : src[ww * 512 + 0] + src[ww * 512 + 32];  // hi rows, residual rows (8 further)
             if (row < m && n0 + col < n) {
-                float* o = out + (int64_t)row * ldo + n0 + col;
-                *o = ROUNDS && round ? *o + v : v;
+                float* o = out + (ROUNDS == 2 ? (int64_t)round * m * ldo : 0) + (int64_t)row * ldo + n0 + col;
+                *o = ROUNDS == 1 && round ? *o + v : v;
             }
         }
     }
@@ -321,9 +324,10 @@ bool gemv_q5_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k) {
 }
 
 // Any number of lhs rows in passes of 16 (bf16) or 8 (fp32); out is fp32 [m, ldo].  The caller checks
-// gemv_q5_k_mm_supported.
+// gemv_q5_k_mm_supported.  workspace: gemv_kquant_mm_workspace_bytes(m, n, k) bytes, or null (the rounds of a long K then
+// run one after the other in each workgroup).
 hipError_t launch_gemv_q5_k_mm(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
-                               hipStream_t s) {
+                               void* workspace, hipStream_t s) {
     static int cus = 0;
     if (!cus) {
         int dev = 0;
@@ -331,7 +335,11 @@ hipError_t launch_gemv_q5_k_mm(const void* a, int a_dtype, const uint8_t* w, int
             cus = 256;
     }
     const int64_t ntiles = (n + 15) / 16;
-    const dim3 grid((unsigned)std::min<int64_t>(ntiles, cus)), block(64 * kVWaves);
+    // A long K: a workgroup per (share of the tiles, round), so that it converts its lhs operands once and streams several
+    // tiles behind them; the rounds' results go to the workspace and are added in round order by a launch of their own.
+    const int rounds = (int)(((k >> 8) + 15) / 16);
+    const bool side_by_side = rounds > 1 && workspace && ldo == n && !kernel_disabled("kquant_mm_rounds_grid");
+    const dim3 grid((unsigned)std::min<int64_t>(ntiles, side_by_side ? std::max(1, cus / rounds) : cus), side_by_side ? rounds : 1), block(64 * kVWaves);
     const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
     // (sixteen fp32 rows would be two operand sets of 64 registers each: the compiler spills 700 bytes; two passes of eight)
     const int pass = a_dtype != QMM_F32 ? 16 : 8;
@@ -342,13 +350,17 @@ hipError_t launch_gemv_q5_k_mm(const void* a, int a_dtype, const uint8_t* w, int
 #define QMM_Q5MM(MR_, AT_)                                                                                              \
     do {                                                                                                                \
         if (k == 4096) {                                                                                                \
-            hipError_t e_ = allow_full_lds<gemv_q5_k_mm_kernel<MR_, AT_, false>>();                                     \
+            hipError_t e_ = allow_full_lds<gemv_q5_k_mm_kernel<MR_, AT_, 0>>();                                         \
             if (e_ != hipSuccess) return e_;                                                                            \
-            gemv_q5_k_mm_kernel<MR_, AT_, false><<<grid, block, kVLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+            gemv_q5_k_mm_kernel<MR_, AT_, 0><<<grid, block, kVLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+        } else if (side_by_side) {                                                                                      \
+            hipError_t e_ = allow_full_lds<gemv_q5_k_mm_kernel<MR_, AT_, 2>>();                                         \
+            if (e_ != hipSuccess) return e_;                                                                            \
+            gemv_q5_k_mm_kernel<MR_, AT_, 2><<<grid, block, kVLds, s>>>(w, (const AT_*)am, (float*)workspace, rows, (int)n, (int)k, ldo); \
         } else {                                                                                                        \
-            hipError_t e_ = allow_full_lds<gemv_q5_k_mm_kernel<MR_, AT_, true>>();                                      \
+            hipError_t e_ = allow_full_lds<gemv_q5_k_mm_kernel<MR_, AT_, 1>>();                                         \
             if (e_ != hipSuccess) return e_;                                                                            \
-            gemv_q5_k_mm_kernel<MR_, AT_, true><<<grid, block, kVLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+            gemv_q5_k_mm_kernel<MR_, AT_, 1><<<grid, block, kVLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
         }                                                                                                               \
     } while (0)
 #define QMM_Q5MM_AT(MR_)                               \
@@ -362,7 +374,8 @@ hipError_t launch_gemv_q5_k_mm(const void* a, int a_dtype, const uint8_t* w, int
         else QMM_Q5MM(16, uint16_t);
 #undef QMM_Q5MM_AT
 #undef QMM_Q5MM
-        const hipError_t e = hipGetLastError();
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess && side_by_side) e = launch_sum_shares((const float*)workspace, om, (int64_t)rows * n, rounds, s);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;

@@ -87,8 +87,10 @@ __device__ __forceinline__ void stream16_to_lds(uint32_t lane_offset, const void
 // MROWS: lhs rows of the pass, 1, 2, 4, 8 or 16 (>= m; rows past m are zero operands and their results are dropped).  Sixteen
 // rows are two sets of eight, each with its own operands and sums, multiplied with the same decoded weights.
 // Accumulator registers that hold no wanted lhs row are not computed: a lane holds rows 4 (lane / 16) + r of a set.
-// ROUNDS: K beyond 4096 (or 2048), walked in rounds of 16 super-blocks; without it everything about rounds is constant.
-template <int MROWS, typename AT, bool ROUNDS>
+// ROUNDS: K beyond 4096 (or 2048) in rounds of 16 super-blocks; 0: a single round, everything about rounds is constant; 1: the
+// workgroup walks the rounds one after the other and adds to its own output; 2: round blockIdx.y only, its result stored as
+// part blockIdx.y of [rounds][m][ldo] at `out` (the caller adds the parts in round order).
+template <int MROWS, typename AT, int ROUNDS>
 __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_t* __restrict__ w, const AT* __restrict__ a,
                                                                    float* __restrict__ out, int m, int n, int k, int64_t ldo) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -142,7 +144,8 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
     // K in rounds of 16 super-blocks (4096 columns); a last round of 8 keeps wavefronts 0..3 busy.  Results of the rounds
     // after the first are added to what the same thread stored before.
     const int rounds = ROUNDS ? (nblk + 15) >> 4 : 1;
-    for (int round = 0; round < rounds; round++) {
+    const int round0 = ROUNDS == 2 ? (int)blockIdx.y : 0, round1 = ROUNDS == 2 ? round0 + 1 : rounds;
+    for (int round = round0; round < round1; round++) {
     const bool have = ROUNDS ? 16 * round + 2 * wave < nblk : true;            // this wavefront has super-blocks in the round
     const int nw = ROUNDS ? min(kQWaves, (nblk - 16 * round) >> 1) : kQWaves;  // wavefronts that have
     if (have && my_tiles > 0) issue(round, 0, 0);
@@ -276,8 +279,8 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
             for (int ww = 0; ww < kQWaves; ww++)
                 if (ww < nw) v += HI16 ? src[ww * 512] : src[ww * 512 + 0] + src[ww * 512 + 32];  // hi rows, residual rows (8 further)
             if (row < m && n0 + col < n) {
-                float* o = out + (int64_t)row * ldo + n0 + col;
-                *o = ROUNDS && round ? *o + v : v;
+                float* o = out + (ROUNDS == 2 ? (int64_t)round * m * ldo : 0) + (int64_t)row * ldo + n0 + col;
+                *o = ROUNDS == 1 && round ? *o + v : v;
             }
         }
     }
@@ -288,9 +291,18 @@ bool gemv_q6_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k) {
     return !kernel_disabled("q6k_mm") && m >= 1 && m <= 64 && k >= 2048 && k % 2048 == 0 && k <= 16384 && n >= 1 && n <= 0x7fffffff && ((uintptr_t)w & 15) == 0;
 }
 
+// K beyond 4096 with the rounds side by side in the grid (this kernel and the Q5_K one): room for the rounds' results of one
+// pass of up to 16 lhs rows.
+int64_t gemv_kquant_mm_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+    if (k <= 4096 || k % 512 || k > 32768 || m < 1 || m > 64) return 0;
+    return ((k >> 8) + 15) / 16 * std::min<int64_t>(m, 16) * n * 4;
+}
+
 // Any number of lhs rows in passes of 16 (K = 4096) or 8; out is fp32 [m, ldo].  The caller checks gemv_q6_k_mm_supported.
+// workspace: gemv_kquant_mm_workspace_bytes(m, n, k) bytes, or null (the rounds of a long K then run one after the other
+// in each workgroup).
 hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
-                               hipStream_t s) {
+                               void* workspace, hipStream_t s) {
     static int cus = 0;
     if (!cus) {
         int dev = 0;
@@ -298,7 +310,11 @@ hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int
             cus = 256;
     }
     const int64_t ntiles = (n + 15) / 16;
-    const dim3 grid((unsigned)std::min<int64_t>(ntiles, cus)), block(64 * kQWaves);
+    // A long K: a workgroup per (share of the tiles, round), so that it converts its lhs operands once and streams several
+    // tiles behind them; the rounds' results go to the workspace and are added in round order by a launch of their own.
+    const int rounds = (int)(((k >> 8) + 15) / 16);
+    const bool side_by_side = rounds > 1 && workspace && ldo == n && !kernel_disabled("kquant_mm_rounds_grid");
+    const dim3 grid((unsigned)std::min<int64_t>(ntiles, side_by_side ? std::max(1, cus / rounds) : cus), side_by_side ? rounds : 1), block(64 * kQWaves);
     const size_t esz = a_dtype == QMM_F32 ? 4 : 2;
     // Sixteen bf16 rows are one operand set and go as one pass everywhere.  Sixteen fp32 rows are two sets (hi parts and
     // residuals of eight rows each) and the kernel spills registers in its loop: two passes of eight rows are faster unless a
@@ -312,13 +328,17 @@ hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int
 #define QMM_Q6MM(MR_, AT_)                                                                                          \
     do {                                                                                                            \
         if (k == 4096) {                                                                                            \
-            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, false>>();                                 \
+            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, 0>>();                                     \
             if (e_ != hipSuccess) return e_;                                                                        \
-            gemv_q6_k_mm_kernel<MR_, AT_, false><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+            gemv_q6_k_mm_kernel<MR_, AT_, 0><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+        } else if (side_by_side) {                                                                                  \
+            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, 2>>();                                     \
+            if (e_ != hipSuccess) return e_;                                                                        \
+            gemv_q6_k_mm_kernel<MR_, AT_, 2><<<grid, block, kQLds, s>>>(w, (const AT_*)am, (float*)workspace, rows, (int)n, (int)k, ldo); \
         } else {                                                                                                    \
-            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, true>>();                                  \
+            hipError_t e_ = allow_full_lds<gemv_q6_k_mm_kernel<MR_, AT_, 1>>();                                     \
             if (e_ != hipSuccess) return e_;                                                                        \
-            gemv_q6_k_mm_kernel<MR_, AT_, true><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
+            gemv_q6_k_mm_kernel<MR_, AT_, 1><<<grid, block, kQLds, s>>>(w, (const AT_*)am, om, rows, (int)n, (int)k, ldo); \
         }                                                                                                           \
     } while (0)
 #define QMM_Q6MM_AT(MR_)                               \
@@ -333,7 +353,8 @@ hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int
         else QMM_Q6MM_AT(16);
 #undef QMM_Q6MM_AT
 #undef QMM_Q6MM
-        const hipError_t e = hipGetLastError();
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess && side_by_side) e = launch_sum_shares((const float*)workspace, om, (int64_t)rows * n, rounds, s);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;

@@ -71,17 +71,17 @@ bool q4k_lanes_rows_wins(int64_t n, int64_t k) {
 
 // Q6_K (K a multiple of 2048 up to 16384): the small-batch matrix-core kernel, or passes of the decode kernel (one or two
 // lhs rows each)?
-bool q6k_mm_wanted(int64_t m, int64_t n) {
+bool q6k_mm_wanted(int64_t m, int64_t n, int64_t k) {
     // Measured, small-batch kernel / decode-kernel passes, fp32 lhs: 128256 rows: 1 lhs row 87 / 78 us, 2 87 / 113, 4 95 / 225,
     // 8 98 / 449, 16 144 / 895; 14336 rows: 1 17.0 / 14.8, 2 17.5 / 20.6, 4 19.5 / 40.8, 8 21.6 / 81.7, 16 46.7 / 162;
     // 4096 rows: 2 10.3 / 9.6, 4 11.7 / 15.2, 8 13.8 / 32.9, 16 36 / 52; 1024 rows: 2 9.8 / 6.1, 4 11.2 / 7.7, 8 13.2 / 21.9,
-    // 16 29 / 38; 4096 x 14336 (four rounds over K): 2 33 / 24, 4 39 / 47, 8 49 / 93, 16 98 / 186.  (Its fixed cost is the
-    // conversion of the lhs in every workgroup and round.)  QMM_Q6K_MM=1 sends every shape there.
+    // 16 29 / 38; 4096 x 14336 (four rounds over K, side by side): 1 19.2 / 16.1, 2 20.0 / 22.4, 4 22.1 / 47.  (Its fixed cost is
+    // the conversion of the lhs in every workgroup and round.)  QMM_Q6K_MM=1 sends every shape there.
     static const bool forced = [] {
         const char* e = getenv("QMM_Q6K_MM");
         return e && e[0] == '1';
     }();
-    return forced || m >= 5 || (m >= 3 && n >= 2048) || (m == 2 && n >= 8192);
+    return forced || m >= 5 || (m >= 3 && n >= 2048) || (m == 2 && (n >= 8192 || (k > 8192 && n >= 2048)));
 }
 
 // Q5_K: the small-batch matrix-core kernel, or passes of the decode kernel (up to four lhs rows each)?
@@ -89,12 +89,13 @@ bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
     // Measured, small-batch kernel / decode-kernel passes, fp32 lhs (bf16 lhs: the small-batch kernel is 10-20 % faster, and
     // sixteen bf16 rows cost what eight do): 14336 x 4096: 2 lhs rows 17.5 / 17.5 us, 4 19.2 / 27.2, 8 20.9 / 53.6, 16 41.5 / 106;
     // 4096 x 4096: 4 11.9 / 11.4, 8 14.3 / 22.1; 1024 x 4096: 4 11.6 / 7.8, 8 13.9 / 15.3; 4096 x 14336: 2 34.4 / 33.1, 4 40.4 / 65.4,
-    // 8 50.2 / 130.  QMM_Q5K_MM=1 sends every shape the kernel takes there.
+    // 8 50.2 / 130; with the rounds of a long K side by side: 2 19.9 / 32.1, 4 21.6 / 65.  QMM_Q5K_MM=1 sends every shape the kernel
+    // takes there.
     static const bool forced = [] {
         const char* e = getenv("QMM_Q5K_MM");
         return e && e[0] == '1';
     }();
-    return forced || m >= 5 || (m >= 3 && n * k >= ((int64_t)32 << 20));
+    return forced || m >= 5 || (m >= 3 && n * k >= ((int64_t)32 << 20)) || (m >= 2 && k > 8192 && n >= 2048);
 }
 
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
@@ -322,10 +323,11 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
         return std::max(std::max(a, b), c);
     }
     if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) {  // lhs planes from 9 rows on; partial sums of K chunks
-        const int64_t a = qmm::gemv_q4_k_mm_workspace_bytes(lhs_dtype, m, k), b = m >= 2 ? qmm::gemv_q4_k_kc_workspace_bytes(m, n, k) : 0;
+        const int64_t a = qmm::gemv_q4_k_mm_plain_workspace_bytes(lhs_dtype, m, n, k), b = m >= 2 ? qmm::gemv_q4_k_kc_workspace_bytes(m, n, k) : 0;
         return a > b ? a : b;
     }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
+    if (encoding == QMM_Q5_K || encoding == QMM_Q6_K) return qmm::gemv_kquant_mm_workspace_bytes(m, n, k);  // rounds of a long K side by side
     if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
         const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, n, k) : 0;
         const int64_t c = gptq_planes(m, n, k, 128) ? qmm::gemm_gptq_planes_workspace_bytes(lhs_dtype, m, n, k) : 0;  // (the group size is not known here)
@@ -526,7 +528,7 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
     // Q5_K with several lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
     if (encoding == QMM_Q5_K && q5k_mm_wanted(m, n, k) && qmm::gemv_q5_k_mm_supported(w, m, n, k))
-        return hip_status(qmm::launch_gemv_q5_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, s), "qmm_matmul(Q5_K small batch)");
+        return hip_status(qmm::launch_gemv_q5_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s), "qmm_matmul(Q5_K small batch)");
     if (encoding == QMM_Q5_K) {
         // a decode-shaped kernel; a pass takes as many lhs rows as fit its LDS copy of the lhs
         const int64_t ngroups = (k / 256 + 15) / 16;
@@ -568,14 +570,19 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
 
     // 2..4 lhs rows on a small matrix: the decode kernel with one sub-block per lane (the activations of four rows fit a
     // lane's registers)
-    if (encoding == QMM_Q4_K && m >= 2 && m <= 4 && q4k_lanes_rows_wins(n, k)) {
+    // (not with 3 or 4 rows where the matrix-core kernel cuts a long K over the grid: 1024 x 14336 with 4 fp32 rows 23.4 -> 10.5 us,
+    // bf16 rows 13.6 -> 10.0)
+    const bool q4k_mm_cuts_k = encoding == QMM_Q4_K && m >= 2 && m <= 8 && !qmm::kernel_disabled("q4k_mm") &&
+                               qmm::gemv_q4_k_mm_plain_workspace_bytes(lhs_dtype, m, n, k) > 0;
+    if (encoding == QMM_Q4_K && m >= 2 && m <= 4 && q4k_lanes_rows_wins(n, k) && !(m >= 3 && q4k_mm_cuts_k)) {
         bool handled = false;
         hipError_t e = qmm::launch_gemv_q4_k_lanes_rows(lhs, lhs_dtype, w, (int)m, n, k, out, n, s, &handled);
         if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K decode, 2..4 rows)");
         if (handled) return QMM_OK;
     }
-    // 2..16 lhs rows on few weight rows and long K: the small-batch kernel that cuts K across workgroups
-    if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && q4k_kc_wins(lhs_dtype, m, n, k) && qmm::gemv_q4_k_kc_supported(w, k)) {
+    // 2..16 lhs rows on few weight rows and long K: the small-batch kernel that cuts K across workgroups (up to 8 rows the
+    // matrix-core kernel below does so itself where its grid then fills the part: 4096 x 14336 with 8 bf16 rows 20.6 -> 15.6 us)
+    if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && q4k_kc_wins(lhs_dtype, m, n, k) && !q4k_mm_cuts_k && qmm::gemv_q4_k_kc_supported(w, k)) {
         bool handled = false;
         hipError_t e = qmm::launch_gemv_q4_k_kc(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s, &handled);
         if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K small batch, K chunks)");
@@ -588,8 +595,8 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");
 
     // Q6_K with 2..64 lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
-    if (encoding == QMM_Q6_K && q6k_mm_wanted(m, n) && qmm::gemv_q6_k_mm_supported(w, m, n, k))
-        return hip_status(qmm::launch_gemv_q6_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, s), "qmm_matmul(Q6_K small batch)");
+    if (encoding == QMM_Q6_K && q6k_mm_wanted(m, n, k) && qmm::gemv_q6_k_mm_supported(w, m, n, k))
+        return hip_status(qmm::launch_gemv_q6_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s), "qmm_matmul(Q6_K small batch)");
 
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         int mt = (int)(m - m0 < 16 ? m - m0 : 16);

@@ -12,7 +12,7 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_lanes_rows, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_twin_rows, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_small_passes, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, gptq_k_shares, gptq_long_k_mm, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_small_passes, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, gptq_k_shares, gptq_long_k_mm, kquant_mm_rounds_grid, q4k_mm_k_parts, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
 // Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 // False while qmm_matmul_static serves a problem whose one-pass treatment of an fp32 lhs (the lhs as twice the rows, the
@@ -95,7 +95,7 @@ struct MmMats {
     int count;
 };
 hipError_t launch_gemv_q4_k_mm_grouped(const void* lhs, int lhs_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
-                                       float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s);
+                                       float* const* outs, int64_t m, int64_t k, void* workspace, hipStream_t s, bool k_parts = false);
 hipError_t launch_gemv_q4_k_lanes_grouped(const void* a, int a_dtype, int count, const uint8_t* const* ws, const int64_t* ns,
                                           float* const* outs, int m, int64_t k, int64_t ldo, hipStream_t s, bool* handled,
                                           bool swiglu = false, bool out_bf16 = false);
@@ -118,12 +118,14 @@ hipError_t launch_gemv_q6_k(const void* a, int a_dtype, const uint8_t* w, int m,
 // matrix-core kernel (gemv_q5k_mm.hip).
 bool gemv_q5_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemv_q5_k_mm(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
-                               hipStream_t s);
+                               void* workspace, hipStream_t s);
+// Both small-batch K-quant kernels on a K beyond 4096: bytes for the results of the rounds of K, which then run side by side.
+int64_t gemv_kquant_mm_workspace_bytes(int64_t m, int64_t n, int64_t k);
 // Q6_K, up to 64 lhs rows (passes of 16 or 8), K a multiple of 2048 up to 16384, 16-byte aligned weights: the small-batch
 // matrix-core kernel (gemv_q6k_mm.hip).
 bool gemv_q6_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,
-                               hipStream_t s);
+                               void* workspace, hipStream_t s);
 hipError_t launch_gemv_q6_k_rows(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k,
                                  float* out, int64_t ldo, hipStream_t s, bool* handled);
 int64_t gemm_q4_0_workspace_bytes(int64_t m, int64_t k);
@@ -151,6 +153,7 @@ int64_t gemv_q4_k_kc_workspace_bytes(int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemv_q4_k_kc(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out,
                                int64_t ldo, void* workspace, hipStream_t s, bool* handled);
 int64_t gemv_q4_k_mm_workspace_bytes(int lhs_dtype, int64_t m, int64_t k);
+int64_t gemv_q4_k_mm_plain_workspace_bytes(int lhs_dtype, int64_t m, int64_t n, int64_t k);  // launch_gemv_q4_k_mm
 hipError_t launch_gemv_q4_k_mm(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                                float* out, void* workspace, hipStream_t s);
 bool gemm_gptq_supported(int64_t k, int group);

@@ -19,8 +19,9 @@ CASES = {
     "Q4_K": [(1, 300, 4096, False), (2, 130, 2048, True), (4, 200, 4096, False), (12, 64, 8192, False), (16, 72, 512, True),
              (40, 300, 1024, True), (1, 70, 32768, False), (200, 260, 512, True), (3, 1100, 8192, False), (1030, 8200, 512, True)],
     "Q4_0": [(1, 200, 4096, False), (4, 200, 4096, True), (9, 72, 1056, False), (16, 200, 4096, False), (80, 136, 1024, True), (80, 300, 2560, True)],
-    "Q6_K": [(1, 8200, 2048, False), (1, 300, 4096, True), (4, 200, 4096, False), (16, 72, 512, False), (70, 136, 1024, True), (8, 600, 4096, False), (70, 300, 2560, True)],
-    "Q5_K": [(2, 300, 4096, False), (6, 200, 4096, True), (16, 72, 1024, False), (1030, 8200, 512, True), (70, 300, 2560, True)],
+    "Q6_K": [(1, 8200, 2048, False), (1, 300, 4096, True), (4, 200, 4096, False), (16, 72, 512, False), (70, 136, 1024, True), (8, 600, 4096, False), (70, 300, 2560, True), (6, 520, 8192, True)],
+    "Q5_K": [(2, 300, 4096, False), (6, 200, 4096, True), (16, 72, 1024, False), (1030, 8200, 512, True), (70, 300, 2560, True),
+             (12, 520, 6144, False)],
     "GPTQ": [(1, 264, 1024, False), (4, 264, 1024, True), (16, 264, 1024, False), (40, 264, 1024, True), (1030, 8200, 512, True)],
 }
 
