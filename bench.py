@@ -805,13 +805,13 @@ LADDER_ROWS = (1, 4, 8, 16, 17, 32, 64, 65, 128, 256)
 
 
 def ladder_main(gen) -> int:
-    """Microseconds per qmm_matmul call for every encoding over 1 .. 256 lhs rows, fp32 and bf16, on the q / o and the gate / up
-    shape (six calls per graph on one weight tensor, so the weights come from the last-level cache: the figures compare
+    """Microseconds per qmm_matmul call for every encoding over 1 .. 256 lhs rows, fp32 and bf16, on the q / o, the gate / up and
+    the down shape (six calls per graph on one weight tensor, so the weights come from the last-level cache: the figures compare
     row counts and lhs types of one shape, not shapes).  One JSON line; a step between neighbouring row counts that is
     larger than the rows explain is a threshold of the dispatch in the wrong place."""
     out = {}
     for enc in (QE.Q4_K, QE.Q5_K, QE.Q6_K, QE.Q4_0, QE.GPTQ):
-        for n, k in ((4096, 4096), (14336, 4096)):
+        for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
             if enc == QE.GPTQ:
                 w = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
             else:

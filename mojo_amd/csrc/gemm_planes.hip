@@ -1155,8 +1155,18 @@ bool gemm_planes_wanted(int encoding, int lhs_dtype, int64_t m, int64_t n, int64
     // Up to these row counts the passes of the small-batch kernels (16 lhs rows a pass) cost less than the conversion pass plus
     // a GEMM whose 256-row tiles are mostly empty (14336 x 4096, Q5_K: 48 rows 52 us, 64 rows 69 us, the planes 65 us; Q6_K:
     // 64 rows 88 us, the planes 118 us; beyond 64 rows neither encoding has a kernel that takes more than four rows a pass).
-    // Q5_K with 33 to 64 rows where that kernel does not apply (K not a multiple of 512 or beyond 32768) also comes here.
-    if (encoding == QMM_Q5_K && m > 32 && (k % 512 || k > 32768 || kernel_disabled("q5k_mm"))) return true;
+    // Where the small-batch kernel does not take the K (Q5_K: a multiple of 512 up to 32768; Q6_K: of 2048 up to 16384), the
+    // alternative is the decode kernel once per one or two lhs rows, at about the cost of a one-row call each time (us, W in
+    // millions of weights: 5 + 0.2 W): 4096 x 11008 with 16 / 32 rows 198 / 401 us (Q5_K), 195 / 398 (Q6_K), the planes 88 /
+    // 152; 8192 x 28672, Q6_K, 64 rows 3810 against 500.
+    const bool mm_takes_k = encoding == QMM_Q5_K ? (k % 512 == 0 && k <= 32768 && !kernel_disabled("q5k_mm"))
+                                                 : (k % 2048 == 0 && k <= 16384 && !kernel_disabled("q6k_mm"));
+    if (!mm_takes_k) {
+        const double W = (double)n * (double)k * 1e-6, row_us = 5.0 + 0.2 * W;
+        const double planes_us = (encoding == QMM_Q5_K ? 12.0 + 1.15 * W : 25.0 + 1.85 * W) +
+                                 (k > 4096 ? std::min(encoding == QMM_Q5_K ? 45.0 : 60.0, (encoding == QMM_Q5_K ? 9.0 : 11.0) * (double)k / (double)n) : 0.0);
+        return m > 4 && 0.9 * (double)m * row_us > planes_us;
+    }
     // The small-batch kernels take 16 bf16 or 8 fp32 rows a pass (up to 64 rows), the planes any number in one (an fp32 lhs as
     // twice the rows) behind a conversion.  Both sides in microseconds, fitted to this part (W: millions of weights; a K beyond
     // 4096 costs the small-batch kernels a launch that adds the rounds of 4096 columns, and the planes the K shares of few

@@ -56,6 +56,11 @@ bool q4k_kc_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     return m >= (lhs_dtype == QMM_F32 ? 9 : 5) && n <= 4096 && k > 4096;
 }
 
+static bool q4k_gemm_from_9_rows(int encoding, int lhs_dtype, int64_t m, int64_t n, int64_t k) {
+    return encoding == QMM_Q4_K && lhs_dtype == QMM_F32 && m > 8 && m <= 16 && k > 4096 && k % 256 == 0 && n * k >= ((int64_t)128 << 20) &&
+           !q4k_kc_wins(lhs_dtype, m, n, k);
+}
+
 // Q4_K with 2..4 lhs rows: the decode kernel with one sub-block per lane, or the small-batch matrix-core kernel?
 bool q4k_lanes_rows_wins(int64_t n, int64_t k) {
     // The decode kernel pays per weight (its decode runs on the vector units once per row group), the matrix-core kernel
@@ -95,7 +100,9 @@ bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
         const char* e = getenv("QMM_Q5K_MM");
         return e && e[0] == '1';
     }();
-    return forced || m >= 5 || (m >= 3 && n * k >= ((int64_t)32 << 20)) || (m >= 2 && k > 8192 && n >= 2048);
+    // Other shapes: 5120 x 5120 with 4 rows 21 / 29.8; 32000 x 4096 with 2 rows 28 / 32.2; 8192 x 28672 with one row 50 / 61.
+    return forced || m >= 5 || (m >= 3 && (n * k >= ((int64_t)32 << 20) || (k > 4096 && n >= 2048))) ||
+           (m >= 2 && ((k > 8192 && n >= 2048) || n * k >= ((int64_t)96 << 20))) || (k > 16384 && n >= 2048);
 }
 
 bool gptq_small_batch_wins(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
@@ -318,13 +325,14 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     if (m <= 0 || k <= 0) return 0;
     if (kquant_planes(encoding, lhs_dtype, m, n, k)) return qmm::gemm_planes_workspace_bytes(encoding, lhs_dtype, m, n, k);
     if (encoding == QMM_Q4_0) {
-        const int64_t a = q8_planes(nullptr, m, k).bytes, b = (m >= 5 || k > 8192) && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
+        const int64_t a = q8_planes(nullptr, m, k).bytes, b = (m >= 5 || k > 4096) && k % 32 == 0 ? qmm::gemm_q4_0_workspace_bytes(m, k) : 0;
         const int64_t c = qmm::gemm_q4_0_planes_wanted(m, n, k) ? qmm::gemm_q4_0_planes_workspace_bytes(m, n, k) : 0;
         return std::max(std::max(a, b), c);
     }
     if (encoding == QMM_Q4_K && m <= 16 && k % 256 == 0) {  // lhs planes from 9 rows on; partial sums of K chunks
         const int64_t a = qmm::gemv_q4_k_mm_plain_workspace_bytes(lhs_dtype, m, n, k), b = m >= 2 ? qmm::gemv_q4_k_kc_workspace_bytes(m, n, k) : 0;
-        return a > b ? a : b;
+        const int64_t c = q4k_gemm_from_9_rows(encoding, lhs_dtype, m, n, k) ? qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k) : 0;
+        return std::max(std::max(a, b), c);
     }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     if (encoding == QMM_Q5_K || encoding == QMM_Q6_K) return qmm::gemv_kquant_mm_workspace_bytes(m, n, k);  // rounds of a long K side by side
@@ -546,7 +554,8 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     if (encoding == QMM_Q4_0 && qmm::gemm_q4_0_planes_wanted(m, n, k))
         return hip_status(qmm::launch_gemm_q4_0_planes(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 plane GEMM)");
     // (two rows and more on a K beyond what the decode kernel takes: the matrix-core kernel too, 4096 x 14336 with 4 rows 32 -> 16 us)
-    if (encoding == QMM_Q4_0 && (m >= 5 || (m >= 2 && k > 8192 && k % 256 == 0)) && !qmm::kernel_disabled("q4_0_mfma"))
+    // (three and four rows on a K beyond 4096 as well: 8192 x 8192 with 4 rows 34.8 -> 14.4 us, 5120 x 5120 18.1 -> 12.2)
+    if (encoding == QMM_Q4_0 && (m >= 5 || (m >= 2 && k > 8192 && k % 256 == 0) || (m >= 3 && k > 4096 && k % 256 == 0)) && !qmm::kernel_disabled("q4_0_mfma"))
         return hip_status(qmm::launch_gemm_q4_0(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_0 int8 MFMA)");
     if (encoding == QMM_Q4_0 && m <= 4) {
         // decode: the kernel that quantises the lhs itself (takes K <= 8192)
@@ -588,7 +597,11 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         if (e != hipSuccess) return hip_status(e, "qmm_matmul(Q4_K small batch, K chunks)");
         if (handled) return QMM_OK;
     }
-    // 3..16 lhs rows: the small-batch matrix-core kernel; more: the prefill kernel
+    // 3..16 lhs rows: the small-batch matrix-core kernel; more: the prefill kernel (which also takes 9..16 fp32 rows on a large
+    // matrix with a long K, where the small-batch kernel works through two planes of a prepared lhs: 28672 x 8192 with 16 rows
+    // 70 us against 61 for 32 rows, 8192 x 28672 94 against 76)
+    if (q4k_gemm_from_9_rows(encoding, lhs_dtype, m, n, k))
+        return hip_status(qmm::launch_gemm_q4_k(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K GEMM)");
     if (encoding == QMM_Q4_K && m >= 2 && m <= 16 && !qmm::kernel_disabled("q4k_mm"))
         return hip_status(qmm::launch_gemv_q4_k_mm(lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(Q4_K small batch)");
     if (encoding == QMM_Q4_K && m > 16)

@@ -255,11 +255,11 @@ def test_q4_0_decode_shapes(m, n, k, lhs_bf16):
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(16, 5000, 4096, False), (9, 300, 512, False), (12, 64, 14336, True),
                                             (5, 4100, 256, False), (16, 16400, 2048, True), (37, 300, 1024, False),
                                             (64, 5000, 4096, True), (81, 4100, 2048, False), (3, 200, 14336, False),
-                                            (2, 130, 16384, True)])
+                                            (2, 130, 16384, True), (3, 200, 5120, False), (4, 130, 8192, True)])
 def test_q4_0_small_batch(m, n, k, lhs_bf16):
     """5..16 lhs rows, K a multiple of 256: several 16-row tiles per workgroup, ragged last tile, groups of K in
     which only some wavefronts have a share.  More rows go through the same kernel in passes of 16 while that beats making
-    the planes (37: a last pass of five rows; 81: of one), and so do 2..4 rows on a K past 8192."""
+    the planes (37: a last pass of five rows; 81: of one), and so do 2..4 rows on a K past 8192 and 3, 4 rows on one past 4096."""
     w, a = synth(53, n, k, m)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
@@ -294,7 +294,7 @@ def test_kquant_matmul_bf16_lhs(enc):
 
 
 @pytest.mark.parametrize("m,n,k,bf16", [(1, 4099, 4096, False), (1, 1030, 4096, True), (3, 777, 14336, False), (1, 130, 32768, False),
-                                        (4, 2050, 1280, True), (7, 300, 8192, False)])
+                                        (4, 2050, 1280, True), (7, 300, 8192, False), (1, 2100, 28672, False)])
 def test_q5_k_decode_shapes(m, n, k, bf16):
     """Q5_K through its kernel's variants: activations in registers (one row, K <= 4096), from the LDS copy,
     several groups of 16 super-blocks with a partial last one, row counts that leave wavefronts unequal work,
@@ -764,9 +764,9 @@ def test_q4_k_gemm_bf16_lhs(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 128, 512), (33, 64, 256), (32, 4096, 4096), (17, 1000, 4096), (100, 2050, 1024),
-                                   (65, 520, 2560), (200, 16500, 512)])
+                                   (65, 520, 2560), (200, 16500, 512), (12, 16400, 8192)])
 def test_q4_k_gemm_f32_lhs(m, n, k):
-    """fp32 lhs: hi and residual fp16 planes.  From 1024 columns of K on (tiles cut into K shares) the residual plane is the
+    """fp32 lhs: hi and residual fp16 planes (12 x 16400 x 8192: the GEMM from nine rows on, a large matrix with a long K).  From 1024 columns of K on (tiles cut into K shares) the residual plane is the
     second half of the rows of one lhs and a single pass multiplies both, and so it is up to 256 rows whatever the tiles (200 x
     16500: 455 tiles, no K shares); shorter K takes two passes.  Rows of very different magnitude (the row scales of both
     halves), ragged m and n."""
@@ -805,9 +805,10 @@ def test_q4_k_gemm_tile_kernel(m, n, k, bf16):
 @pytest.mark.parametrize("enc,m,n,k,bf16", [
     (QE.Q6_K, 65, 130, 512, True), (QE.Q6_K, 300, 257, 1024, False), (QE.Q6_K, 1000, 9300, 768, True), (QE.Q6_K, 256, 128, 256, True),
     (QE.Q5_K, 65, 130, 512, True), (QE.Q5_K, 33, 130, 768, True), (QE.Q5_K, 300, 257, 1024, False), (QE.Q5_K, 1000, 9300, 768, True), (QE.Q5_K, 520, 8200, 256, False),
-    (QE.Q5_K, 40, 24, 36864, True)])
+    (QE.Q5_K, 40, 24, 36864, True), (QE.Q5_K, 20, 520, 2816, True), (QE.Q6_K, 16, 300, 5120, False), (QE.Q6_K, 12, 264, 18432, True)])
 def test_q5_k_q6_k_prefill_on_the_matrix_cores(enc, m, n, k, bf16):
-    """Q5_K and Q6_K above 64 lhs rows (Q5_K above 32 where its small-batch kernel does not take K): the weights become fp16 integer planes (Q5_K sc * q; Q6_K two planes,
+    """Q5_K and Q6_K above 64 lhs rows (from a few rows on where the small-batch kernel does not take K: Q5_K on 2816 and 36864
+    columns, Q6_K on 5120 and 18432): the weights become fp16 integer planes (Q5_K sc * q; Q6_K two planes,
     (16 hi) * q and lo * q with sc = 16 hi + lo) and a tile GEMM multiplies them.  Ragged edges in m and n, one super-block,
     a last round of tiles cut in two K halves (292 tiles; for Q6_K the cut falls between or inside the planes), fp32 lhs
     (second pass on the residual), a K beyond what the Q5_K decode kernel takes; a third of the blocks carry random bytes
