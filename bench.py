@@ -531,7 +531,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers of weights to rotate over")
     ap.add_argument("--m", type=int, default=1, help="lhs rows of the headline workload (1 or 4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib", "mfma_probe", "sweep", "ladder"),
+    ap.add_argument("--workload", choices=("decode", "prefill", "gptq_prefill", "q6k_prefill", "q5k_prefill", "q40_prefill", "calib", "mfma_probe", "sweep", "ladder", "ladder_other"),
                     default="decode",
                     help="decode: the headline Q4_K GEMV set; prefill / gptq_prefill / q6k_prefill / q5k_prefill / q40_prefill: the M=2048 "
                          "GEMM of the same model's gate projection (second target, matrix-core roofline); calib: a plain "
@@ -565,6 +565,8 @@ def main() -> int:
         return sweep_main(gen)
     if args.workload == "ladder":
         return ladder_main(gen)
+    if args.workload == "ladder_other":
+        return ladder_main(gen, LADDER_OTHER_SHAPES, LADDER_OTHER_ROWS)
     if args.workload != "decode":
         return prefill_main(args, gen)
     m = args.m
@@ -802,23 +804,28 @@ def sweep_main(gen) -> int:
 
 
 LADDER_ROWS = (1, 4, 8, 16, 17, 32, 64, 65, 128, 256)
+LADDER_SHAPES = ((4096, 4096), (14336, 4096), (4096, 14336))
+# projection shapes of other models (Llama-2-7B, 13B-like, 70B), a vocabulary of 32000, a K that is no multiple of 512 or 2048
+LADDER_OTHER_SHAPES = ((11008, 4096), (4096, 11008), (5120, 5120), (8192, 8192), (32000, 4096), (28672, 8192), (8192, 28672))
+LADDER_OTHER_ROWS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
 
-def ladder_main(gen) -> int:
+def ladder_main(gen, shapes=LADDER_SHAPES, rows=LADDER_ROWS) -> int:
     """Microseconds per qmm_matmul call for every encoding over 1 .. 256 lhs rows, fp32 and bf16, on the q / o, the gate / up and
     the down shape (six calls per graph on one weight tensor, so the weights come from the last-level cache: the figures compare
     row counts and lhs types of one shape, not shapes).  One JSON line; a step between neighbouring row counts that is
-    larger than the rows explain is a threshold of the dispatch in the wrong place."""
+    larger than the rows explain is a threshold of the dispatch in the wrong place.  ladder_other: the same over shapes
+    that no threshold was fitted on."""
     out = {}
     for enc in (QE.Q4_K, QE.Q5_K, QE.Q6_K, QE.Q4_0, QE.GPTQ):
-        for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
+        for n, k in shapes:
             if enc == QE.GPTQ:
                 w = quantize_gptq(torch.randn((n, k), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02)
             else:
                 w = make_weight(enc, n, k, gen)
             for dt, name in ((torch.float32, "f32"), (torch.bfloat16, "bf16")):
                 row = {}
-                for m in LADDER_ROWS:
+                for m in rows:
                     a = torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen).to(dt)
                     calls = [GptqMatmul(w, a) if enc == QE.GPTQ else Gemv(enc, w, a) for _ in range(6)]
                     dev_s, _ = time_graphs([capture(calls)], 20, 3)

@@ -1155,12 +1155,12 @@ bool gemm_planes_wanted(int encoding, int lhs_dtype, int64_t m, int64_t n, int64
     // Up to these row counts the passes of the small-batch kernels (16 lhs rows a pass) cost less than the conversion pass plus
     // a GEMM whose 256-row tiles are mostly empty (14336 x 4096, Q5_K: 48 rows 52 us, 64 rows 69 us, the planes 65 us; Q6_K:
     // 64 rows 88 us, the planes 118 us; beyond 64 rows neither encoding has a kernel that takes more than four rows a pass).
-    // Where the small-batch kernel does not take the K (Q5_K: a multiple of 512 up to 32768; Q6_K: of 2048 up to 16384), the
+    // Where the small-batch kernel does not take the K (Q5_K: a multiple of 512 up to 32768; Q6_K: of 2048 up to 32768), the
     // alternative is the decode kernel once per one or two lhs rows, at about the cost of a one-row call each time (us, W in
     // millions of weights: 5 + 0.2 W): 4096 x 11008 with 16 / 32 rows 198 / 401 us (Q5_K), 195 / 398 (Q6_K), the planes 88 /
     // 152; 8192 x 28672, Q6_K, 64 rows 3810 against 500.
     const bool mm_takes_k = encoding == QMM_Q5_K ? (k % 512 == 0 && k <= 32768 && !kernel_disabled("q5k_mm"))
-                                                 : (k % 2048 == 0 && k <= 16384 && !kernel_disabled("q6k_mm"));
+                                                 : (k % 2048 == 0 && k <= 32768 && !kernel_disabled("q6k_mm"));
     if (!mm_takes_k) {
         const double W = (double)n * (double)k * 1e-6, row_us = 5.0 + 0.2 * W;
         const double planes_us = (encoding == QMM_Q5_K ? 12.0 + 1.15 * W : 25.0 + 1.85 * W) +

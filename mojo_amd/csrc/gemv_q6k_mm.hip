@@ -1,4 +1,4 @@
-// Q6_K with up to 16 lhs rows a pass on the matrix cores, K a multiple of 2048 up to 16384: the weight rows are decoded
+// Q6_K with up to 16 lhs rows a pass on the matrix cores, K a multiple of 2048 up to 32768: the weight rows are decoded
 // once for all lhs rows of a pass, and the per-16 int8 scales are applied to a 16 x 16 block of results at a time.
 //
 // Arithmetic.  A Q6_K weight is d * sc * q with q = (ql nibble | qh bits << 4) - 32 and sc an int8 per 16 weights.  The
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(64 * kQWaves) void gemv_q6_k_mm_kernel(const uint8_
 }
 
 bool gemv_q6_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k) {
-    return !kernel_disabled("q6k_mm") && m >= 1 && m <= 64 && k >= 2048 && k % 2048 == 0 && k <= 16384 && n >= 1 && n <= 0x7fffffff && ((uintptr_t)w & 15) == 0;
+    return !kernel_disabled("q6k_mm") && m >= 1 && m <= 64 && k >= 2048 && k % 2048 == 0 && k <= 32768 && n >= 1 && n <= 0x7fffffff && ((uintptr_t)w & 15) == 0;
 }
 
 // K beyond 4096 with the rounds side by side in the grid (this kernel and the Q5_K one): room for the rounds' results of one

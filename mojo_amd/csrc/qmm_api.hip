@@ -74,7 +74,7 @@ bool q4k_lanes_rows_wins(int64_t n, int64_t k) {
     return forced || n <= 1024 || n * k <= ((int64_t)8 << 20);
 }
 
-// Q6_K (K a multiple of 2048 up to 16384): the small-batch matrix-core kernel, or passes of the decode kernel (one or two
+// Q6_K (K a multiple of 2048 up to 32768): the small-batch matrix-core kernel, or passes of the decode kernel (one or two
 // lhs rows each)?
 bool q6k_mm_wanted(int64_t m, int64_t n, int64_t k) {
     // Measured, small-batch kernel / decode-kernel passes, fp32 lhs: 128256 rows: 1 lhs row 87 / 78 us, 2 87 / 113, 4 95 / 225,
@@ -86,7 +86,8 @@ bool q6k_mm_wanted(int64_t m, int64_t n, int64_t k) {
         const char* e = getenv("QMM_Q6K_MM");
         return e && e[0] == '1';
     }();
-    return forced || m >= 5 || (m >= 3 && n >= 2048) || (m == 2 && (n >= 8192 || (k > 8192 && n >= 2048)));
+    // (a K beyond 16384, which the decode kernel with the rows global -> LDS does not take: from one bf16 row on)
+    return forced || m >= 5 || (m >= 3 && n >= 2048) || (m == 2 && (n >= 8192 || (k > 8192 && n >= 2048))) || (k > 16384 && n >= 2048);
 }
 
 // Q5_K: the small-batch matrix-core kernel, or passes of the decode kernel (up to four lhs rows each)?

@@ -121,7 +121,7 @@ hipError_t launch_gemv_q5_k_mm(const void* a, int a_dtype, const uint8_t* w, int
                                void* workspace, hipStream_t s);
 // Both small-batch K-quant kernels on a K beyond 4096: bytes for the results of the rounds of K, which then run side by side.
 int64_t gemv_kquant_mm_workspace_bytes(int64_t m, int64_t n, int64_t k);
-// Q6_K, up to 64 lhs rows (passes of 16 or 8), K a multiple of 2048 up to 16384, 16-byte aligned weights: the small-batch
+// Q6_K, up to 64 lhs rows (passes of 16 or 8), K a multiple of 2048 up to 32768, 16-byte aligned weights: the small-batch
 // matrix-core kernel (gemv_q6k_mm.hip).
 bool gemv_q6_k_mm_supported(const void* w, int64_t m, int64_t n, int64_t k);
 hipError_t launch_gemv_q6_k_mm(const void* a, int a_dtype, const uint8_t* w, int m, int64_t n, int64_t k, float* out, int64_t ldo,

@@ -1081,7 +1081,8 @@ def test_q6_k_decode_vocabulary_shapes(m, n, k, lhs_bf16):
                                             (20, 300, 4096, False), (40, 130, 4096, True), (64, 72, 4096, False),
                                             (4, 300, 14336, False), (8, 130, 8192, True), (5, 2100, 2048, False),
                                             (16, 77, 6144, False), (6, 40, 16384, True), (16, 300, 14336, True), (13, 50, 2048, True),
-                                            (4, 4200, 14336, True), (2, 2100, 14336, False), (20, 1100, 8192, False)])
+                                            (4, 4200, 14336, True), (2, 2100, 14336, False), (20, 1100, 8192, False),
+                                            (4, 2100, 28672, False), (1, 2064, 20480, True)])
 def test_q6_k_small_batch_matrix_core_kernel(m, n, k, lhs_bf16):
     """Q6_K with 2..64 lhs rows on K = 4096: weight rows decoded once for all lhs rows (codes as exact fp16 integers, one
     matrix-core instruction per 16-weight scale group and set of eight lhs rows; sixteen bf16 rows are one set without
