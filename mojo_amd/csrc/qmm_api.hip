@@ -336,7 +336,9 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
         return std::max(std::max(a, b), c);
     }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
-    if (encoding == QMM_Q5_K || encoding == QMM_Q6_K) return qmm::gemv_kquant_mm_workspace_bytes(m, n, k);  // rounds of a long K side by side
+    // (the small-batch kernels with the rounds of a long K side by side; the decode kernels need nothing)
+    if (encoding == QMM_Q5_K) return q5k_mm_wanted(m, n, k) && k % 512 == 0 ? qmm::gemv_kquant_mm_workspace_bytes(m, n, k) : 0;
+    if (encoding == QMM_Q6_K) return q6k_mm_wanted(m, n, k) && k % 2048 == 0 ? qmm::gemv_kquant_mm_workspace_bytes(m, n, k) : 0;
     if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
         const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, n, k) : 0;
         const int64_t c = gptq_planes(m, n, k, 128) ? qmm::gemm_gptq_planes_workspace_bytes(lhs_dtype, m, n, k) : 0;  // (the group size is not known here)

@@ -79,6 +79,13 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.qmm_matmul_workspace_bytes(1, 0, 8, 4096, 4096) == 0  # up to 8 rows the kernel narrows the lhs itself
     assert lib.qmm_matmul_workspace_bytes(1, 0, 12, 4096, 4096) >= 2 * 12 * 4096 * 2  # fp16 hi and residual planes
     assert lib.qmm_matmul_workspace_bytes(1, 1, 2048, 14336, 4096) >= 2048 * 4096 * 2
+    # one-row decode of the K-quants needs none on any projection shape; a few rows on a long K hold the partial results of
+    # the parts of K that lie side by side in the grid (Q4_K: four groups of 4096 columns; Q6_K: four rounds)
+    for enc in (1, 2, 4):
+        for n, k in ((4096, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
+            assert lib.qmm_matmul_workspace_bytes(enc, 0, 1, n, k) == 0, (enc, n, k)
+    assert lib.qmm_matmul_workspace_bytes(1, 0, 4, 4096, 14336) == 4 * 4 * 4096 * 4
+    assert lib.qmm_matmul_workspace_bytes(2, 0, 4, 4096, 14336) == 4 * 4 * 4096 * 4
     # flags that change the workspace: a bf16 result that the kernel does not store itself goes through an fp32 copy; Q8_K
     # activations outside the integer kernel go through fp32 rows of d8 * code
     f = lib.qmm_matmul_workspace_bytes_flags
