@@ -1,4 +1,4 @@
-// Q4_0 decode kernel (m <= 4 lhs rows, K <= 8192): weight rows streamed global -> LDS with 16-byte loads, the
+// Q4_0 decode kernel (m <= 4 lhs rows, K <= 8192; one lhs row: K up to 14528): weight rows streamed global -> LDS with 16-byte loads, the
 // Q8_0 quantisation of the lhs done in the kernel, v_dot4_i32_i8 block dots.
 //
 // A Q4_0 block is 18 bytes (fp16 d, 16 bytes of nibbles), so blocks are only 2-byte aligned.  A
@@ -41,15 +41,17 @@ __device__ __forceinline__ void wait_rows(int rows) {
 }  // namespace
 
 // BPL: blocks per lane (k <= 2048 * BPL).  L = load instructions per row = pieces of 16 bytes / 64, for the
-// longest row BPL allows plus one piece of misalignment.  RING: LDS slots per wavefront.
+// longest row BPL allows plus one piece of misalignment (LROW: given instead, for the rows of a K beyond 8192, whose slots
+// would not fit the LDS at the full length BPL allows).  RING: LDS slots per wavefront.  Six and eight blocks per lane hold
+// one workgroup per compute unit (LDS) and are built for it.
 // NORM: the lhs rows are RMS-normalised first, y = x * rsqrt(mean(x^2) + eps) * gamma in fp32 (rounded to bf16 when the
 // lhs is bf16: what a bf16 normalisation node would hand over), and y is what gets quantised.
-template <int MT, int BPL, int RING, typename AT, bool NORM>
-__global__ __launch_bounds__(64 * kWaves, 2) void gemv_q4_0_stream_kernel(const uint8_t* __restrict__ w,
+template <int MT, int BPL, int RING, typename AT, bool NORM, int LROW = 0>
+__global__ __launch_bounds__(64 * kWaves, BPL > 4 ? 1 : 2) void gemv_q4_0_stream_kernel(const uint8_t* __restrict__ w,
                                                                          const AT* __restrict__ a,
                                                                          float* __restrict__ out, int m, int n, int k,
                                                                          int64_t ldo, const float* __restrict__ gamma, float eps) {
-    constexpr int L = (72 * BPL + 1 + 63) / 64;
+    constexpr int L = LROW ? LROW : (72 * BPL + 1 + 63) / 64;
     constexpr int kSlot = L * 1024;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -269,7 +271,10 @@ hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w,
     if (gamma && ((uintptr_t)gamma & 15)) return hipSuccess;  // (the kernel reads gamma in 16-byte pieces)
     const int nblk = (int)(k / 32);
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
-    const int bpl = nblk <= 128 ? 2 : nblk <= 256 ? 4 : 0;
+    // one lhs row on a K beyond 8192: six or eight blocks per lane, rows of up to seven / eight KB (K <= 12288 / 14528)
+    const int64_t row_pieces = ((int64_t)nblk * Q4_0_BPB + 15 + 15) / 16;  // with the worst misalignment
+    const int bpl = nblk <= 128 ? 2 : nblk <= 256 ? 4 : (mt == 1 && !gamma && nblk <= 384 && row_pieces <= 7 * 64) ? 6
+                  : (mt == 1 && !gamma && nblk <= 512 && row_pieces <= 8 * 64) ? 8 : 0;
     if (!bpl || mt * bpl > 8) return hipSuccess;  // the codes of the lane's blocks must fit its registers
     static int cus = 0;
     if (!cus) {
@@ -278,8 +283,8 @@ hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w,
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
     }
-    const int L = (72 * bpl + 1 + 63) / 64;
-    const int ring = bpl == 2 ? 4 : 3;  // LDS: 8 wavefronts x ring x L KB
+    const int L = bpl == 6 ? 7 : bpl == 8 ? 8 : (72 * bpl + 1 + 63) / 64;
+    const int ring = bpl == 2 ? 4 : bpl == 4 ? 3 : 2;  // LDS: 8 wavefronts x ring x L KB
     const size_t lds = (size_t)kWaves * ring * L * 1024 + (size_t)kWaves * kMaxRows * mt * 4 + (size_t)mt * nblk * 40 + 128;  // (the last 128 bytes: the row norms' partial sums)
     int64_t wgs = cus;  // one workgroup of 8 wavefronts per compute unit
     if (wgs * kWaves > n) wgs = (n + kWaves - 1) / kWaves;
@@ -303,7 +308,23 @@ hipError_t launch_gemv_q4_0_stream(const void* a, int a_dtype, const uint8_t* w,
             else QMM_GO2(MT_, BPL_, RING_, uint16_t, false);              \
         }                                                                 \
     } while (0)
-    if (bpl == 2) {
+    if (bpl > 4) {
+#define QMM_GO_LONG(BPL_, L_)                                                                                         \
+    do {                                                                                                              \
+        if (a_dtype == QMM_F32) {                                                                                     \
+            hipError_t e_ = allow_full_lds<gemv_q4_0_stream_kernel<1, BPL_, 2, float, false, L_>>();                  \
+            if (e_ != hipSuccess) return e_;                                                                          \
+            gemv_q4_0_stream_kernel<1, BPL_, 2, float, false, L_><<<grid, block, lds, s>>>(w, (const float*)a, out, m, (int)n, (int)k, ldo, nullptr, 0.0f); \
+        } else {                                                                                                      \
+            hipError_t e_ = allow_full_lds<gemv_q4_0_stream_kernel<1, BPL_, 2, uint16_t, false, L_>>();               \
+            if (e_ != hipSuccess) return e_;                                                                          \
+            gemv_q4_0_stream_kernel<1, BPL_, 2, uint16_t, false, L_><<<grid, block, lds, s>>>(w, (const uint16_t*)a, out, m, (int)n, (int)k, ldo, nullptr, 0.0f); \
+        }                                                                                                             \
+    } while (0)
+        if (bpl == 6) QMM_GO_LONG(6, 7);
+        else QMM_GO_LONG(8, 8);
+#undef QMM_GO_LONG
+    } else if (bpl == 2) {
         if (mt == 1) QMM_GO(1, 2, 4);
         else if (mt == 2) QMM_GO(2, 2, 4);
         else QMM_GO(4, 2, 4);

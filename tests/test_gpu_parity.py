@@ -219,7 +219,7 @@ def _integer_dot_case(m, n, k, one_hot, bf16, seed):
 @pytest.mark.parametrize("one_hot", [True, False])
 @pytest.mark.parametrize("m,n,k", [(1, 200, 4096), (4, 200, 4096), (2, 70, 8224), (5, 200, 4096), (16, 200, 4096),
                                    (9, 72, 1056), (33, 200, 1024), (64, 72, 4096), (65, 200, 1024), (256, 136, 4096),
-                                   (3, 72, 16384), (40, 72, 1056)])
+                                   (3, 72, 16384), (40, 72, 1056), (1, 200, 14336)])
 def test_q4_0_production_kernels_give_the_integer_block_dots(m, n, k, one_hot, bf16):
     """The int8 block dots of every Q4_0 matmul kernel, read off its fp32 output, equal the oracle's bit for bit
     (Q8_0 codes with .5 ties included)."""
@@ -239,10 +239,12 @@ def test_q4_0_matmul(m, n, k):
 
 @pytest.mark.parametrize("m,n,k,lhs_bf16", [(2, 1000, 8192, False), (4, 300, 4096, True), (1, 5001, 2048, False),
                                             (1, 70000, 256, False), (3, 9, 4128, False), (2, 64, 8224, True),
-                                            (4, 33, 8192, False)])
+                                            (4, 33, 8192, False), (1, 4099, 14336, False), (1, 300, 11008, True),
+                                            (1, 70, 14528, False), (1, 130, 14560, True), (1, 9, 8224, False)])
 def test_q4_0_decode_shapes(m, n, k, lhs_bf16):
     """Q4_0 decode: rows at every 2-byte alignment, K up to 8192 in the kernel that quantises the lhs itself
-    (K past that and 4 rows at K = 8192 through the Q8_0 planes), many rows per wavefront, bf16 lhs."""
+    (more rows on a longer K through the Q8_0 planes), many rows per wavefront, bf16 lhs.  One lhs row: that kernel up to
+    K = 14528 with six or eight blocks per lane (8224, 11008 / 14336, 14528; 14560 is past it)."""
     w, a = synth(52, n, k, m)
     if lhs_bf16:
         a = O.bf16_to_f32(O.f32_to_bf16(a))
