@@ -425,11 +425,24 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             x[mi][it][1] = load4(aq, 32);
             x[mi][it][2] = load4(aq, 64);
             x[mi][it][3] = load4(aq, 96);
-            const AT* ag = ar + 16 * t;
-            const float4 y0 = load4(ag, 0), y1 = load4(ag, 4), y2 = load4(ag, 8), y3 = load4(ag, 12);
+            // The sum of group t = 8 h + j (columns 128 h + 16 j .. + 15) from the quartets already loaded, not from loads of its
+            // own (a wavefront's lhs loads are half of its start-up: 32 KB through the compute unit's load path for 16 KB of
+            // values): those 16 columns are quartet j / 2 of the four lanes 4 (j % 2) .. + 3 of this half row.  Quartet sums,
+            // added over each aligned group of four lanes; the other group of the eight is a mirror away.
+            float qs[4], qo[4];
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++) {
+                const float4 q = x[mi][it][c4];
+                qs[c4] = (q.x + q.y) + (q.z + q.w);
+                qs[c4] += dpp_move<0xB1>(qs[c4]);
+                qs[c4] += dpp_move<0x4E>(qs[c4]);
+                qo[c4] = dpp_move<0x141>(qs[c4]);
+            }
+            const int cj = j >> 1;
+            const float mine = cj == 0 ? qs[0] : cj == 1 ? qs[1] : cj == 2 ? qs[2] : qs[3];
+            const float othr = cj == 0 ? qo[0] : cj == 1 ? qo[1] : cj == 2 ? qo[2] : qo[3];
             // (in units of 2^-24 like the dots below: -32 * 2^-24 = -2^-19; the row's sum is scaled back at its end)
-            os[mi][it] = -0x1p-19f * (((y0.x + y0.y) + (y0.z + y0.w)) + ((y1.x + y1.y) + (y1.z + y1.w)) +
-                                      ((y2.x + y2.y) + (y2.z + y2.w)) + ((y3.x + y3.y) + (y3.z + y3.w)));
+            os[mi][it] = -0x1p-19f * ((j & 1) == (j >> 2) ? mine : othr);
             keep += os[mi][it];
         }
     }
