@@ -481,8 +481,11 @@ __global__ __launch_bounds__(256) void gemv_q6_k_lanes_kernel(const uint8_t* __r
             const uint32_t q3 = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
             const uint32_t q4 = ((B >> 4) & 0x0F0F0F0Fu) | ((H >> 2) & 0x30303030u);
             // the int8 scales of the four quartets and of this lane's 16-column group; d once at the end
-            const float c1 = sbyte(s0, sc_shift), c2 = sbyte(s0, sc_shift + 16), c3 = sbyte(s1, sc_shift), c4 = sbyte(s1, sc_shift + 16);
-            const float cg = sbyte(j < 4 ? s0 : s1, 8 * (j & 3));
+            // (one shift per dword, then sign-extending byte selects: a conversion instruction each)
+            const uint32_t t0 = s0 >> sc_shift, t1 = s1 >> sc_shift, tg = (j < 4 ? s0 : s1) >> (8 * (j & 3));
+            const float c1 = (float)(signed char)(t0 & 0xffu), c2 = (float)(signed char)((t0 >> 16) & 0xffu);
+            const float c3 = (float)(signed char)(t1 & 0xffu), c4 = (float)(signed char)((t1 >> 16) & 0xffu);
+            const float cg = (float)(signed char)(tg & 0xffu);
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) {
                 float u = c1 * dot4h(x[mi][it][0], q1);
