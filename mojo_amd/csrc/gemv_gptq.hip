@@ -120,12 +120,161 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols_kernel(const uint3
     }
 }
 
+// The same product for matrices of few columns (N / 64 workgroups would leave most compute units idle): a wavefront covers 16
+// columns and four k8 rows per load instruction (lane l: column l % 16, row l / 16 of every four: 64 contiguous bytes per row),
+// so N / 16 workgroups; consecutive column blocks run on one XCD, whose L2 then sees both halves of a 128-byte line.  A lane
+// takes NR = group / 32 words per group; the loads of G groups go out together (what is in flight per wavefront sets the
+// bandwidth), their activations are parked side by side.  The four row lanes of a column meet in the final sum, in lane order.
+template <int MT, int NR, int G, typename AT>
+__global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uint32_t* __restrict__ qweight,
+                                                                       const uint16_t* __restrict__ scales,
+                                                                       const uint32_t* __restrict__ qzeros,
+                                                                       const AT* __restrict__ a, float* __restrict__ out,
+                                                                       int m, int n, int k, int64_t ldo, int per_xcd) {
+    extern __shared__ __attribute__((aligned(16))) float gsm[];
+    constexpr int GROUP = 32 * NR;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cl = lane & 15, kr = lane >> 4;
+    const int ngroups = k / GROUP;
+    float* red = gsm;                                               // [kWaves][MT][64]
+    float* mine = gsm + kWaves * MT * 64 + wave * (G * MT * GROUP);  // this wavefront's copy of G groups' activations: [G][MT][GROUP]
+    const int cb = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (cb * 16 >= n) return;  // (the whole workgroup: the grid is rounded up to eight times per_xcd)
+    const int col = cb * 16 + cl;
+    const int ccol = min(col, n - 1);
+    const int zshift = 4 * (ccol & 7);
+    float acc[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
+
+    for (int g0 = wave * G; g0 < ngroups; g0 += kWaves * G) {
+        uint32_t x[G][NR];
+        float sc[G], nz[G];
+#pragma unroll
+        for (int gi = 0; gi < G; gi++) {
+            const int g = min(g0 + gi, ngroups - 1);
+            const int64_t k8 = (int64_t)g * (4 * NR);
+#pragma unroll
+            for (int j = 0; j < NR; j++) x[gi][j] = (qweight + (k8 + 4 * j + kr) * n)[ccol];
+            // (a group past the end repeats the last one with scale 0; the zero-point term once per column, in row lane 0)
+            sc[gi] = g0 + gi < ngroups ? h2f(scales[(int64_t)g * n + ccol]) : 0.0f;
+            nz[gi] = kr == 0 ? -(float)(((qzeros[(int64_t)g * (n >> 3) + (ccol >> 3)] >> zshift) & 0xFu) + 1u) : 0.0f;
+        }
+        float gsum[G][MT];
+#pragma unroll
+        for (int gi = 0; gi < G; gi++) {
+            const int g = min(g0 + gi, ngroups - 1);
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+                const AT* ar = a + (int64_t)min(mi, m - 1) * k + (int64_t)g * GROUP;
+                float s = 0.0f;
+                for (int i = lane; i < GROUP; i += 64) {
+                    const float v = act(ar, i);
+                    mine[(gi * MT + mi) * GROUP + i] = v;
+                    s += v;
+                }
+                gsum[gi][mi] = wave_sum(s);
+            }
+        }
+#pragma unroll
+        for (int gi = 0; gi < G; gi++) {
+            float part[MT];
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) part[mi] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NR; j++) {
+                const uint32_t qe = x[gi][j] & 0x0F0F0F0Fu, qo = (x[gi][j] >> 4) & 0x0F0F0F0Fu;  // k 0,2,4,6 / k 1,3,5,7
+                const float w0 = gub0(qe), w2 = gub1(qe), w4 = gub2(qe), w6 = gub3(qe);
+                const float w1 = gub0(qo), w3 = gub1(qo), w5 = gub2(qo), w7 = gub3(qo);
+#pragma unroll
+                for (int mi = 0; mi < MT; mi++) {
+                    const float4* ap = (const float4*)(mine + (gi * MT + mi) * GROUP + (4 * j + kr) * 8);  // four addresses per wavefront
+                    const float4 a0 = ap[0], a1 = ap[1];
+                    float t = part[mi];
+                    t = fmaf(w0, a0.x, t);
+                    t = fmaf(w1, a0.y, t);
+                    t = fmaf(w2, a0.z, t);
+                    t = fmaf(w3, a0.w, t);
+                    t = fmaf(w4, a1.x, t);
+                    t = fmaf(w5, a1.y, t);
+                    t = fmaf(w6, a1.z, t);
+                    part[mi] = fmaf(w7, a1.w, t);
+                }
+            }
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) acc[mi] = fmaf(sc[gi], fmaf(nz[gi], gsum[gi][mi], part[mi]), acc[mi]);
+        }
+    }
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) red[(wave * MT + mi) * 64 + lane] = acc[mi];
+    __syncthreads();
+    if (tid < 16 && cb * 16 + tid < n) {
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+            if (mi < m) {
+                float v = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; w++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) v += red[(w * MT + mi) * 64 + 16 * r + tid];
+                out[(int64_t)mi * ldo + cb * 16 + tid] = v;
+            }
+        }
+    }
+}
+
+// Up to 4096 columns (a quarter of the compute units with 64 columns each): 4096 x 4096 with one row 6.9 -> 6.2 us, two fp32
+// rows 9.2 -> 6.6, 4096 x 14336 16.4 -> 10.7.  More columns fill the part with 64 each, whose row loads are whole cache
+// lines: 11008 x 4096 7.3 us against 16.4 here, 8192 x 8192 12.3 against 14.7.
+bool gemv_gptq_cols16_wanted(int64_t n, int group) {
+    return (group == 64 || group == 128 || group == 256) && n <= 4096 && n % 8 == 0 && !kernel_disabled("gptq_cols16");
+}
+
 hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                  const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                                  int64_t ldo, hipStream_t s, bool* handled) {
     *handled = false;
     if (m > 4 || group % 32) return hipSuccess;
     const int mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
+    // few columns: the kernel with 16 columns per workgroup
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    if (gemv_gptq_cols16_wanted(n, group)) {
+        const int gq = mt == 1 ? 4 : mt == 2 ? 2 : 1;
+        const size_t lds16 = ((size_t)kWaves * gq * mt * group + (size_t)kWaves * mt * 64) * 4;
+        const int per_xcd = (int)(((n + 15) / 16 + 7) / 8);
+        dim3 grid16((unsigned)(8 * per_xcd)), block16(64 * kWaves);
+#define QMM_GPTQ16(MT_, NR_, G_)                                                                                      \
+    do {                                                                                                              \
+        if (a_dtype == QMM_F32) {                                                                                     \
+            if (lds16 > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols16_kernel<MT_, NR_, G_, float>>();              \
+            gemv_gptq_cols16_kernel<MT_, NR_, G_, float><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const float*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
+        } else {                                                                                                      \
+            if (lds16 > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols16_kernel<MT_, NR_, G_, uint16_t>>();           \
+            gemv_gptq_cols16_kernel<MT_, NR_, G_, uint16_t><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const uint16_t*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
+        }                                                                                                             \
+    } while (0)
+#define QMM_GPTQ16_NR(NR_)                      \
+    do {                                        \
+        if (mt == 1) QMM_GPTQ16(1, NR_, 4);     \
+        else if (mt == 2) QMM_GPTQ16(2, NR_, 2); \
+        else QMM_GPTQ16(4, NR_, 1);             \
+    } while (0)
+        if (lds16 <= (size_t)kLdsPerCu) {
+            if (group == 64) QMM_GPTQ16_NR(2);
+            else if (group == 128) QMM_GPTQ16_NR(4);
+            else QMM_GPTQ16_NR(8);
+            *handled = true;
+            return hipGetLastError();
+        }
+#undef QMM_GPTQ16_NR
+#undef QMM_GPTQ16
+    }
     const size_t lds = ((size_t)kWaves * mt * group + (size_t)kWaves * mt * 64) * 4;
     if (lds > (size_t)kLdsPerCu) return hipSuccess;
     dim3 grid((unsigned)((n + 63) / 64)), block(64 * kWaves);

@@ -470,7 +470,10 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
         // (4096 x 14336, one row: 18.2 -> 13.3 us bf16, 18.2 -> 16.4 us fp32; two fp32 rows 27.5 -> 17.3 us; at K = 8192 the
         // column kernel still wins on wide matrices: 8192 x 8192 12.3 against 14.0 us)
         const bool long_k = k > 8192 && !qmm::kernel_disabled("gptq_long_k_mm");
-        const int mm_min = long_k ? 1 : (lhs_dtype == QMM_F32 ? 3 : 2);
+        // (... unless the matrix has few columns: the column kernel with 16 per workgroup, 4096 x 14336 10.7 us)
+        // (few columns and K up to 8192: two rows of either type there too, 4096 x 4096 with two bf16 rows 8.2 -> 6.5 us)
+        const bool cols16 = qmm::gemv_gptq_cols16_wanted(n, cfg->group_size);
+        const int mm_min = long_k ? (cols16 ? 2 : 1) : (lhs_dtype == QMM_F32 || cols16 ? 3 : 2);
         for (int64_t m0 = 0; m0 < m; m0 += 16) {
             int mt = (int)(m - m0 < 16 ? m - m0 : 16);
             bool handled = false;

@@ -12,7 +12,7 @@ namespace qmm {
 // Kernel families switched off by the environment variable QMM_DISABLE (a comma-separated list of names, read once
 // per process), for tests and triage: a disabled family reports that it does not take a shape, and the next kernel
 // in the dispatch order serves it.  Names: q4k_lanes, q4k_lanes_rows, q4k_stream, q4k_mm, q4k_kc, q4k_tile, q4k_gemm64, q4k_twin_rows, q4k_rows_v2,
-// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_small_passes, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, gptq_k_shares, gptq_long_k_mm, kquant_mm_rounds_grid, q4k_mm_k_parts, q4k_planes, gptq_planes, gptq_mm, gptq_cols.
+// q4_0_stream, q4_0_mfma, q4_0_small, q4_0_small_passes, q4_0_wide, q4_0_planes, q6k_lanes, q6k_slab, q6k_staged, kquant_planes, planes_wide, planes_192, planes_quarters, planes_twin_rows, gptq_twin_rows, gptq_k_shares, gptq_long_k_mm, kquant_mm_rounds_grid, q4k_mm_k_parts, q4k_planes, gptq_planes, gptq_mm, gptq_cols, gptq_cols16.
 // Nothing is disabled by default.
 bool kernel_disabled(const char* family);
 // False while qmm_matmul_static serves a problem whose one-pass treatment of an fp32 lhs (the lhs as twice the rows, the
@@ -137,6 +137,7 @@ hipError_t launch_gemm_q4_0_planes(const void* lhs, int lhs_dtype, const uint8_t
                                    void* workspace, hipStream_t s);
 hipError_t launch_gemm_q4_0(const void* lhs, int lhs_dtype, const uint8_t* w, int64_t m, int64_t n, int64_t k,
                             float* out, void* workspace, hipStream_t s);
+bool gemv_gptq_cols16_wanted(int64_t n, int group);  // the decode kernel with 16 columns per workgroup serves this matrix
 hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
                                  const uint32_t* qzeros, int m, int64_t n, int64_t k, int group, float* out,
                                  int64_t ldo, hipStream_t s, bool* handled);

@@ -33,6 +33,8 @@ SETTINGS = [
     {"QMM_DISABLE": "q4k_lanes_plain,q4k_mm_plain"},
     # the small-batch kernels of Q5_K and Q6_K with the rounds of a long K one after the other in each workgroup
     {"QMM_DISABLE": "kquant_mm_rounds_grid"},
+    # GPTQ decode on few columns through the kernel with 64 columns per workgroup
+    {"QMM_DISABLE": "gptq_cols16"},
 ]
 
 

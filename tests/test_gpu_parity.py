@@ -349,7 +349,8 @@ def test_q5_k_small_batch_matrix_core_kernel(m, n, k, bf16):
     assert O.isclose(got.cpu().numpy()[big], want[big], RTOL, ATOL).all()
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256), (1, 14336, 4096), (3, 200, 14336)])
+@pytest.mark.parametrize("m,n,k", [(1, 256, 1024), (4, 520, 512), (16, 64, 4096), (18, 64, 256), (1, 14336, 4096), (3, 200, 14336),
+                                   (1, 4096, 14336), (2, 1000, 8192), (1, 8, 4096), (2, 4104, 1024)])
 def test_gptq_matmul(m, n, k):
     w, a = synth(5, n, k, m)
     qw, sc, qz, gi = O.quantize_gptq(w)
