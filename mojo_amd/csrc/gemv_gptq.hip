@@ -120,28 +120,29 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols_kernel(const uint3
     }
 }
 
-// The same product for matrices of few columns (N / 64 workgroups would leave most compute units idle): a wavefront covers 16
-// columns and four k8 rows per load instruction (lane l: column l % 16, row l / 16 of every four: 64 contiguous bytes per row),
-// so N / 16 workgroups; consecutive column blocks run on one XCD, whose L2 then sees both halves of a 128-byte line.  A lane
-// takes NR = group / 32 words per group; the loads of G groups go out together (what is in flight per wavefront sets the
-// bandwidth), their activations are parked side by side.  The four row lanes of a column meet in the final sum, in lane order.
-template <int MT, int NR, int G, typename AT>
+// The same product for matrices of few columns (N / 64 workgroups would leave most compute units idle): a wavefront covers CW =
+// 16 or 32 columns and KR = 64 / CW k8 rows per load instruction (lane l: column l % CW, row l / CW of every KR: 64 or 128
+// contiguous bytes per row), so N / CW workgroups; consecutive column blocks run on one XCD, whose L2 then sees both halves of a
+// 128-byte line.  A lane takes NR = group / (8 KR) words per group; the loads of G groups go out together (what is in flight per
+// wavefront sets the bandwidth), their activations are parked side by side.  The KR row lanes of a column meet in the final sum,
+// in lane order.
+template <int MT, int NR, int G, int CW, typename AT>
 __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uint32_t* __restrict__ qweight,
                                                                        const uint16_t* __restrict__ scales,
                                                                        const uint32_t* __restrict__ qzeros,
                                                                        const AT* __restrict__ a, float* __restrict__ out,
                                                                        int m, int n, int k, int64_t ldo, int per_xcd) {
     extern __shared__ __attribute__((aligned(16))) float gsm[];
-    constexpr int GROUP = 32 * NR;
+    constexpr int KR = 64 / CW, GROUP = 8 * KR * NR;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int cl = lane & 15, kr = lane >> 4;
+    const int cl = lane % CW, kr = lane / CW;
     const int ngroups = k / GROUP;
     float* red = gsm;                                               // [kWaves][MT][64]
     float* mine = gsm + kWaves * MT * 64 + wave * (G * MT * GROUP);  // this wavefront's copy of G groups' activations: [G][MT][GROUP]
     const int cb = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
-    if (cb * 16 >= n) return;  // (the whole workgroup: the grid is rounded up to eight times per_xcd)
-    const int col = cb * 16 + cl;
+    if (cb * CW >= n) return;  // (the whole workgroup: the grid is rounded up to eight times per_xcd)
+    const int col = cb * CW + cl;
     const int ccol = min(col, n - 1);
     const int zshift = 4 * (ccol & 7);
     float acc[MT];
@@ -154,9 +155,9 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uin
 #pragma unroll
         for (int gi = 0; gi < G; gi++) {
             const int g = min(g0 + gi, ngroups - 1);
-            const int64_t k8 = (int64_t)g * (4 * NR);
+            const int64_t k8 = (int64_t)g * (KR * NR);
 #pragma unroll
-            for (int j = 0; j < NR; j++) x[gi][j] = (qweight + (k8 + 4 * j + kr) * n)[ccol];
+            for (int j = 0; j < NR; j++) x[gi][j] = (qweight + (k8 + KR * j + kr) * n)[ccol];
             // (a group past the end repeats the last one with scale 0; the zero-point term once per column, in row lane 0)
             sc[gi] = g0 + gi < ngroups ? h2f(scales[(int64_t)g * n + ccol]) : 0.0f;
             nz[gi] = kr == 0 ? -(float)(((qzeros[(int64_t)g * (n >> 3) + (ccol >> 3)] >> zshift) & 0xFu) + 1u) : 0.0f;
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uin
                 const float w1 = gub0(qo), w3 = gub1(qo), w5 = gub2(qo), w7 = gub3(qo);
 #pragma unroll
                 for (int mi = 0; mi < MT; mi++) {
-                    const float4* ap = (const float4*)(mine + (gi * MT + mi) * GROUP + (4 * j + kr) * 8);  // four addresses per wavefront
+                    const float4* ap = (const float4*)(mine + (gi * MT + mi) * GROUP + (KR * j + kr) * 8);  // KR addresses per wavefront
                     const float4 a0 = ap[0], a1 = ap[1];
                     float t = part[mi];
                     t = fmaf(w0, a0.x, t);
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uin
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) red[(wave * MT + mi) * 64 + lane] = acc[mi];
     __syncthreads();
-    if (tid < 16 && cb * 16 + tid < n) {
+    if (tid < CW && cb * CW + tid < n) {
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
             if (mi < m) {
@@ -217,8 +218,8 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uin
 #pragma unroll
                 for (int w = 0; w < kWaves; w++)
 #pragma unroll
-                    for (int r = 0; r < 4; r++) v += red[(w * MT + mi) * 64 + 16 * r + tid];
-                out[(int64_t)mi * ldo + cb * 16 + tid] = v;
+                    for (int r = 0; r < KR; r++) v += red[(w * MT + mi) * 64 + CW * r + tid];
+                out[(int64_t)mi * ldo + cb * CW + tid] = v;
             }
         }
     }
@@ -229,6 +230,10 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uin
 // lines: 11008 x 4096 7.3 us against 16.4 here, 8192 x 8192 12.3 against 14.7.
 bool gemv_gptq_cols16_wanted(int64_t n, int group) {
     return (group == 64 || group == 128 || group == 256) && n <= 4096 && n % 8 == 0 && !kernel_disabled("gptq_cols16");
+}
+// ... and up to 8192 columns with 32 per workgroup (whole cache lines per row)
+static bool gemv_gptq_cols32_wanted(int64_t n, int group) {
+    return (group == 64 || group == 128 || group == 256) && n > 4096 && n <= 8192 && n % 8 == 0 && !kernel_disabled("gptq_cols16");
 }
 
 hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
@@ -244,26 +249,35 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
     }
-    if (gemv_gptq_cols16_wanted(n, group)) {
+    const bool c32 = gemv_gptq_cols32_wanted(n, group);
+    if (gemv_gptq_cols16_wanted(n, group) || c32) {
         const int gq = mt == 1 ? 4 : mt == 2 ? 2 : 1;
         const size_t lds16 = ((size_t)kWaves * gq * mt * group + (size_t)kWaves * mt * 64) * 4;
-        const int per_xcd = (int)(((n + 15) / 16 + 7) / 8);
+        const int cw = c32 ? 32 : 16;
+        const int per_xcd = (int)(((n + cw - 1) / cw + 7) / 8);
         dim3 grid16((unsigned)(8 * per_xcd)), block16(64 * kWaves);
-#define QMM_GPTQ16(MT_, NR_, G_)                                                                                      \
+#define QMM_GPTQ16(MT_, NR_, G_, CW_)                                                                                 \
     do {                                                                                                              \
         if (a_dtype == QMM_F32) {                                                                                     \
-            if (lds16 > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols16_kernel<MT_, NR_, G_, float>>();              \
-            gemv_gptq_cols16_kernel<MT_, NR_, G_, float><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const float*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
+            if (lds16 > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols16_kernel<MT_, NR_, G_, CW_, float>>();         \
+            gemv_gptq_cols16_kernel<MT_, NR_, G_, CW_, float><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const float*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
         } else {                                                                                                      \
-            if (lds16 > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols16_kernel<MT_, NR_, G_, uint16_t>>();           \
-            gemv_gptq_cols16_kernel<MT_, NR_, G_, uint16_t><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const uint16_t*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
+            if (lds16 > 64 * 1024) (void)allow_full_lds<gemv_gptq_cols16_kernel<MT_, NR_, G_, CW_, uint16_t>>();      \
+            gemv_gptq_cols16_kernel<MT_, NR_, G_, CW_, uint16_t><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const uint16_t*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
         }                                                                                                             \
     } while (0)
-#define QMM_GPTQ16_NR(NR_)                      \
-    do {                                        \
-        if (mt == 1) QMM_GPTQ16(1, NR_, 4);     \
-        else if (mt == 2) QMM_GPTQ16(2, NR_, 2); \
-        else QMM_GPTQ16(4, NR_, 1);             \
+    /* (NR_: words per lane and group with 16 columns; with 32 columns twice as many) */
+#define QMM_GPTQ16_NR(NR_)                                      \
+    do {                                                        \
+        if (c32) {                                              \
+            if (mt == 1) QMM_GPTQ16(1, 2 * NR_, 4, 32);         \
+            else if (mt == 2) QMM_GPTQ16(2, 2 * NR_, 2, 32);    \
+            else QMM_GPTQ16(4, 2 * NR_, 1, 32);                 \
+        } else {                                                \
+            if (mt == 1) QMM_GPTQ16(1, NR_, 4, 16);             \
+            else if (mt == 2) QMM_GPTQ16(2, NR_, 2, 16);        \
+            else QMM_GPTQ16(4, NR_, 1, 16);                     \
+        }                                                       \
     } while (0)
         if (lds16 <= (size_t)kLdsPerCu) {
             if (group == 64) QMM_GPTQ16_NR(2);
