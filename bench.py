@@ -812,7 +812,7 @@ LADDER_OTHER_ROWS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
 def ladder_main(gen, shapes=LADDER_SHAPES, rows=LADDER_ROWS) -> int:
     """Microseconds per qmm_matmul call for every encoding over 1 .. 256 lhs rows, fp32 and bf16, on the q / o, the gate / up and
-    the down shape (six calls per graph on one weight tensor, so the weights come from the last-level cache: the figures compare
+    the down shape (24 calls per graph on one weight tensor, so the weights come from the last-level cache: the figures compare
     row counts and lhs types of one shape, not shapes).  One JSON line; a step between neighbouring row counts that is
     larger than the rows explain is a threshold of the dispatch in the wrong place.  ladder_other: the same over shapes
     that no threshold was fitted on."""
@@ -827,9 +827,11 @@ def ladder_main(gen, shapes=LADDER_SHAPES, rows=LADDER_ROWS) -> int:
                 row = {}
                 for m in rows:
                     a = torch.randn((m, k), dtype=torch.float32, device="cuda:0", generator=gen).to(dt)
-                    calls = [GptqMatmul(w, a) if enc == QE.GPTQ else Gemv(enc, w, a) for _ in range(6)]
-                    dev_s, _ = time_graphs([capture(calls)], 20, 3)
-                    row[f"m{m}"] = round(dev_s * 1e6 / (20 * len(calls)), 1)
+                    # (24 calls per graph: a graph launch costs the host about 20 us plus 3 us per kernel node, so six calls
+                    # per graph would put a floor of 6 us under every figure)
+                    calls = [GptqMatmul(w, a) if enc == QE.GPTQ else Gemv(enc, w, a) for _ in range(24)]
+                    dev_s, _ = time_graphs([capture(calls)], 10, 2)
+                    row[f"m{m}"] = round(dev_s * 1e6 / (10 * len(calls)), 1)
                     del calls
                 out[f"{enc.name} {n}x{k} {name}"] = row
             del w
@@ -1118,6 +1120,25 @@ def extra_timings(layers, acts, gen):
     us = dev_s * 1e6 / 10
     tf = 2 * 2048 * 14336 * 4096 / us / 1e6
     out["q4_0_prefill_m2048"] = {"us": round(us, 1), "TOP/s": round(tf, 1), "frac_of_2500": round(tf / BF16_PEAK_TFLOPS, 4)}
+    del g, ab32
+    # the headline's step in the other encodings (one fp32 row, seven qmm_matmul launches per layer, three layers rotated: more
+    # than the last-level cache holds): what a model stored in that encoding pays per layer
+    if m == 1:
+        a1 = {kk: torch.randn((1, kk), dtype=torch.float32, device="cuda:0", generator=gen) for kk in (4096, 14336)}
+        for enc, tag in ((QE.Q4_0, "q4_0"), (QE.Q6_K, "q6_k"), (QE.Q5_K, "q5_k"), (QE.GPTQ, "gptq_g128")):
+            cs, sb = [], 0.0
+            for _ in range(3):
+                if enc == QE.GPTQ:
+                    cs += [GptqMatmul(quantize_gptq(torch.randn((nn, kk), dtype=torch.float32, device="cuda:0", generator=gen) * 0.02), a1[kk])
+                           for _, nn, kk in PROJ]
+                else:
+                    cs += [Gemv(enc, make_weight(enc, nn, kk, gen), a1[kk]) for _, nn, kk in PROJ]
+            for _, nn, kk in PROJ:
+                sb += (nn * kk * 0.5176 + 4 * kk + 4 * nn) if enc == QE.GPTQ else alg_bytes(enc, 1, nn, kk)
+            # (one graph of two rotations, 42 kernel nodes: a host launch per step would be the limiter)
+            dev_s, _ = time_graphs([capture(cs + cs)], 20, 3)
+            out[f"{tag}_m1_seven_projections"] = {"us_per_step": round(dev_s * 1e6 / 120, 2), "GB/s": round(sb * 120 / dev_s / 1e9, 1)}
+            del cs
     return out
 
 

@@ -120,12 +120,13 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols_kernel(const uint3
     }
 }
 
-// The same product for matrices of few columns (N / 64 workgroups would leave most compute units idle): a wavefront covers CW =
-// 16 or 32 columns and KR = 64 / CW k8 rows per load instruction (lane l: column l % CW, row l / CW of every KR: 64 or 128
-// contiguous bytes per row), so N / CW workgroups; consecutive column blocks run on one XCD, whose L2 then sees both halves of a
-// 128-byte line.  A lane takes NR = group / (8 KR) words per group; the loads of G groups go out together (what is in flight per
-// wavefront sets the bandwidth), their activations are parked side by side.  The KR row lanes of a column meet in the final sum,
-// in lane order.
+// The same product for matrices of few columns (N / 64 workgroups would leave most compute units idle): a wavefront covers CW
+// columns and KR = 64 / CW k8 rows per load instruction (lane l: column l % CW, row l / CW of every KR: CW * 4 contiguous bytes
+// per row), so N / CW workgroups; consecutive column blocks run on one XCD, whose L2 then sees both halves of a 128-byte line.
+// A lane takes NR = group / (8 KR) words per group; a wavefront has the loads of G groups in flight at a time.  The KR row lanes
+// of a column meet in the final sum, in lane order.  Built with CW = 16 and G = 1: one-row calls on weights that no cache holds,
+// 4096 x 4096 8.5 us with 64 columns per workgroup, 6.4 with 16, 9.8 with 32; 4096 x 14336 22.6 / 15.3 / 20.1; more groups in
+// flight leave wavefronts without work and are slower (G = 4: 8.7 us on 4096 x 4096, 5.5 against 3.0 on 1024 x 1024).
 template <int MT, int NR, int G, int CW, typename AT>
 __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uint32_t* __restrict__ qweight,
                                                                        const uint16_t* __restrict__ scales,
@@ -225,15 +226,11 @@ __global__ __launch_bounds__(64 * kWaves) void gemv_gptq_cols16_kernel(const uin
     }
 }
 
-// Up to 4096 columns (a quarter of the compute units with 64 columns each): 4096 x 4096 with one row 6.9 -> 6.2 us, two fp32
-// rows 9.2 -> 6.6, 4096 x 14336 16.4 -> 10.7.  More columns fill the part with 64 each, whose row loads are whole cache
-// lines: 11008 x 4096 7.3 us against 16.4 here, 8192 x 8192 12.3 against 14.7.
+// Up to 4096 columns (a quarter of the compute units with 64 columns each).  More columns fill the part with 64 each, whose
+// row loads are whole cache lines (weights from memory, one row: 5120 x 5120 10.0 us either way, 11008 x 4096 9.1 against
+// 12.1 here, 14336 x 4096 9.7 against 13.9, 28672 x 8192 30 against 44).
 bool gemv_gptq_cols16_wanted(int64_t n, int group) {
     return (group == 64 || group == 128 || group == 256) && n <= 4096 && n % 8 == 0 && !kernel_disabled("gptq_cols16");
-}
-// ... and up to 8192 columns with 32 per workgroup (whole cache lines per row)
-static bool gemv_gptq_cols32_wanted(int64_t n, int group) {
-    return (group == 64 || group == 128 || group == 256) && n > 4096 && n <= 8192 && n % 8 == 0 && !kernel_disabled("gptq_cols16");
 }
 
 hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qweight, const uint16_t* scales,
@@ -249,12 +246,9 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
     }
-    const bool c32 = gemv_gptq_cols32_wanted(n, group);
-    if (gemv_gptq_cols16_wanted(n, group) || c32) {
-        const int gq = mt == 1 ? 4 : mt == 2 ? 2 : 1;
-        const size_t lds16 = ((size_t)kWaves * gq * mt * group + (size_t)kWaves * mt * 64) * 4;
-        const int cw = c32 ? 32 : 16;
-        const int per_xcd = (int)(((n + cw - 1) / cw + 7) / 8);
+    if (gemv_gptq_cols16_wanted(n, group)) {
+        const size_t lds16 = ((size_t)kWaves * mt * group + (size_t)kWaves * mt * 64) * 4;
+        const int per_xcd = (int)(((n + 15) / 16 + 7) / 8);
         dim3 grid16((unsigned)(8 * per_xcd)), block16(64 * kWaves);
 #define QMM_GPTQ16(MT_, NR_, G_, CW_)                                                                                 \
     do {                                                                                                              \
@@ -266,18 +260,11 @@ hipError_t launch_gemv_gptq_cols(const void* a, int a_dtype, const uint32_t* qwe
             gemv_gptq_cols16_kernel<MT_, NR_, G_, CW_, uint16_t><<<grid16, block16, lds16, s>>>(qweight, scales, qzeros, (const uint16_t*)a, out, m, (int)n, (int)k, ldo, per_xcd); \
         }                                                                                                             \
     } while (0)
-    /* (NR_: words per lane and group with 16 columns; with 32 columns twice as many) */
-#define QMM_GPTQ16_NR(NR_)                                      \
-    do {                                                        \
-        if (c32) {                                              \
-            if (mt == 1) QMM_GPTQ16(1, 2 * NR_, 4, 32);         \
-            else if (mt == 2) QMM_GPTQ16(2, 2 * NR_, 2, 32);    \
-            else QMM_GPTQ16(4, 2 * NR_, 1, 32);                 \
-        } else {                                                \
-            if (mt == 1) QMM_GPTQ16(1, NR_, 4, 16);             \
-            else if (mt == 2) QMM_GPTQ16(2, NR_, 2, 16);        \
-            else QMM_GPTQ16(4, NR_, 1, 16);                     \
-        }                                                       \
+#define QMM_GPTQ16_NR(NR_)                      \
+    do {                                        \
+        if (mt == 1) QMM_GPTQ16(1, NR_, 1, 16); \
+        else if (mt == 2) QMM_GPTQ16(2, NR_, 1, 16); \
+        else QMM_GPTQ16(4, NR_, 1, 16);         \
     } while (0)
         if (lds16 <= (size_t)kLdsPerCu) {
             if (group == 64) QMM_GPTQ16_NR(2);

@@ -464,16 +464,15 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
             return hip_status(qmm::launch_gemm_gptq(lhs, lhs_dtype, (const uint32_t*)rhs[0], (const uint16_t*)rhs[1],
                                                     (const uint32_t*)rhs[2], m, n, k, cfg->group_size, out, workspace, s),
                               "qmm_matmul(GPTQ GEMM)");
-        // one pass of the matrix-core small-batch kernel per 16 lhs rows; one row, and two fp32 rows, go to the column
-        // kernel (two rows on 14336 x 4096: 12.3 us with a bf16 lhs, 16 us with an fp32 lhs, column kernel 16.5 us)
-        // a K past 8192: the column kernel walks K with one workgroup per 64 columns, the small-batch kernel splits it
-        // (4096 x 14336, one row: 18.2 -> 13.3 us bf16, 18.2 -> 16.4 us fp32; two fp32 rows 27.5 -> 17.3 us; at K = 8192 the
-        // column kernel still wins on wide matrices: 8192 x 8192 12.3 against 14.0 us)
+        // One pass of the matrix-core small-batch kernel per 16 lhs rows; the fewest rows go to the column kernels (weights from the
+        // last-level cache, us).  More than 4096 columns, 64 per workgroup: one row, and two fp32 rows (14336 x 4096 with two rows:
+        // 12.3 bf16 / 16 fp32 in the small-batch kernel, 16.5 in the column kernel); on a K past 8192 not even one (that kernel walks
+        // K with one workgroup per 64 columns, the small-batch kernel splits it: 8192 x 28672 30 against 37).  Up to 4096 columns,
+        // 16 per workgroup: one and two rows at any K (4096 x 4096: 4.2 / 5.9 against 6.7 / 8.0; 4096 x 14336: 9.0 / 14.2 against
+        // 13.0 / 17.0), three and four fp32 rows up to K = 4096 (9.1 / 9.7 against 11.1 / 11.5).
         const bool long_k = k > 8192 && !qmm::kernel_disabled("gptq_long_k_mm");
-        // (... unless the matrix has few columns: the column kernel with 16 per workgroup, 4096 x 14336 10.7 us)
-        // (few columns and K up to 8192: two rows of either type there too, 4096 x 4096 with two bf16 rows 8.2 -> 6.5 us)
-        const bool cols16 = qmm::gemv_gptq_cols16_wanted(n, cfg->group_size);
-        const int mm_min = long_k ? (cols16 ? 2 : 1) : (lhs_dtype == QMM_F32 || cols16 ? 3 : 2);
+        const bool cols16 = qmm::gemv_gptq_cols16_wanted(n, cfg->group_size) && !qmm::kernel_disabled("gptq_cols");
+        const int mm_min = cols16 ? (lhs_dtype == QMM_F32 && k <= 4096 ? 5 : 3) : long_k ? 1 : (lhs_dtype == QMM_F32 ? 3 : 2);
         for (int64_t m0 = 0; m0 < m; m0 += 16) {
             int mt = (int)(m - m0 < 16 ? m - m0 : 16);
             bool handled = false;
