@@ -91,7 +91,7 @@ bool q6k_mm_wanted(int64_t m, int64_t n, int64_t k) {
 }
 
 // Q5_K: the small-batch matrix-core kernel, or passes of the decode kernel (up to four lhs rows each)?
-bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
+bool q5k_mm_wanted(int lhs_dtype, int64_t m, int64_t n, int64_t k) {
     // Measured, small-batch kernel / decode-kernel passes, fp32 lhs (bf16 lhs: the small-batch kernel is 10-20 % faster, and
     // sixteen bf16 rows cost what eight do): 14336 x 4096: 2 lhs rows 17.5 / 17.5 us, 4 19.2 / 27.2, 8 20.9 / 53.6, 16 41.5 / 106;
     // 4096 x 4096: 4 11.9 / 11.4, 8 14.3 / 22.1; 1024 x 4096: 4 11.6 / 7.8, 8 13.9 / 15.3; 4096 x 14336: 2 34.4 / 33.1, 4 40.4 / 65.4,
@@ -102,7 +102,9 @@ bool q5k_mm_wanted(int64_t m, int64_t n, int64_t k) {
         return e && e[0] == '1';
     }();
     // Other shapes: 5120 x 5120 with 4 rows 21 / 29.8; 32000 x 4096 with 2 rows 28 / 32.2; 8192 x 28672 with one row 50 / 61.
-    return forced || m >= 5 || (m >= 3 && (n * k >= ((int64_t)32 << 20) || (k > 4096 && n >= 2048))) ||
+    // (three and four bf16 rows from 16 Mi weights on: 4096 x 4096 8.8 / 9.1 against 10.6 / 10.8)
+    const int64_t min3 = lhs_dtype == QMM_BF16 ? ((int64_t)16 << 20) : ((int64_t)32 << 20);
+    return forced || m >= 5 || (m >= 3 && (n * k >= min3 || (k > 4096 && n >= 2048))) ||
            (m >= 2 && ((k > 8192 && n >= 2048) || n * k >= ((int64_t)96 << 20))) || (k > 16384 && n >= 2048);
 }
 
@@ -337,7 +339,7 @@ int64_t qmm_matmul_workspace_bytes(int encoding, int lhs_dtype, int64_t m, int64
     }
     if (encoding == QMM_Q4_K && m > 16 && k % 256 == 0) return qmm::gemm_q4_k_workspace_bytes(lhs_dtype, m, n, k);
     // (the small-batch kernels with the rounds of a long K side by side; the decode kernels need nothing)
-    if (encoding == QMM_Q5_K) return q5k_mm_wanted(m, n, k) && k % 512 == 0 ? qmm::gemv_kquant_mm_workspace_bytes(m, n, k) : 0;
+    if (encoding == QMM_Q5_K) return q5k_mm_wanted(lhs_dtype, m, n, k) && k % 512 == 0 ? qmm::gemv_kquant_mm_workspace_bytes(m, n, k) : 0;
     if (encoding == QMM_Q6_K) return q6k_mm_wanted(m, n, k) && k % 2048 == 0 ? qmm::gemv_kquant_mm_workspace_bytes(m, n, k) : 0;
     if (encoding == QMM_GPTQ && k % 256 == 0) {  // small-batch kernel: partial sums of the K chunks; GEMM: lhs planes
         const int64_t a = qmm::gemv_gptq_mm_workspace_bytes(m, n, k), b = m > 16 ? qmm::gemm_gptq_workspace_bytes(lhs_dtype, m, n, k) : 0;
@@ -540,7 +542,7 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     if (kquant_planes(encoding, lhs_dtype, m, n, k))
         return hip_status(qmm::launch_gemm_planes(encoding, lhs, lhs_dtype, w, m, n, k, out, workspace, s), "qmm_matmul(K-quant planes GEMM)");
     // Q5_K with several lhs rows: the small-batch matrix-core kernel (passes of 16 or 8 rows)
-    if (encoding == QMM_Q5_K && q5k_mm_wanted(m, n, k) && qmm::gemv_q5_k_mm_supported(w, m, n, k))
+    if (encoding == QMM_Q5_K && q5k_mm_wanted(lhs_dtype, m, n, k) && qmm::gemv_q5_k_mm_supported(w, m, n, k))
         return hip_status(qmm::launch_gemv_q5_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s), "qmm_matmul(Q5_K small batch)");
     if (encoding == QMM_Q5_K) {
         // a decode-shaped kernel; a pass takes as many lhs rows as fit its LDS copy of the lhs
@@ -616,8 +618,11 @@ static int matmul_f32(int encoding, const qmm_gptq_config* cfg, const void* lhs,
     if (encoding == QMM_Q6_K && q6k_mm_wanted(m, n, k) && qmm::gemv_q6_k_mm_supported(w, m, n, k))
         return hip_status(qmm::launch_gemv_q6_k_mm(lhs, lhs_dtype, w, (int)m, n, k, out, n, workspace, s), "qmm_matmul(Q6_K small batch)");
 
-    for (int64_t m0 = 0; m0 < m; m0 += 16) {
-        int mt = (int)(m - m0 < 16 ? m - m0 : 16);
+    // (Q6_K with more than four rows on a long K that is no multiple of 2048: passes of four rows through the kernel that stages
+    // the lhs, not the first-version kernel on all of them: 4096 x 11008 with 8 rows 102 -> 73 us)
+    const int64_t pass = encoding == QMM_Q6_K && m > 4 && k % 2048 != 0 && k > 8192 ? 4 : 16;
+    for (int64_t m0 = 0; m0 < m; m0 += pass) {
+        int mt = (int)(m - m0 < pass ? m - m0 : pass);
         const void* a = (const char*)lhs + m0 * k * esz;
         hipError_t e = encoding == QMM_Q4_K ? qmm::launch_gemv_q4_k(a, lhs_dtype, w, mt, n, k, out + m0 * n, n, s)
                                             : qmm::launch_gemv_q6_k(a, lhs_dtype, w, mt, n, k, out + m0 * n, n, s);
